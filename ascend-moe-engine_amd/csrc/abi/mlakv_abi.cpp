@@ -1,0 +1,614 @@
+// The thin C ABI (include/mlakv.h): argument validation, status codes and error text around
+// the kernel launchers and the host classes. Nothing here touches data.
+#include "mlakv.h"
+
+#include <hip/hip_runtime.h>
+
+#include <cmath>
+#include <cstdarg>
+#include <cstdio>
+#include <cstdlib>
+#include <cstring>
+#include <memory>
+#include <mutex>
+#include <string>
+
+#include "../kernels/kernels.h"
+#include "abi_common.h"
+#include "moe_hip/kv_cache_manager.hpp"
+#include "moe_hip/static_arena.hpp"
+
+namespace mlakv_abi {
+
+static thread_local std::string g_last_error;
+
+mlakvStatus Fail(mlakvStatus code, const char* format, ...) {
+  char buffer[1024];
+  va_list args;
+  va_start(args, format);
+  std::vsnprintf(buffer, sizeof(buffer), format, args);
+  va_end(args);
+  g_last_error = buffer;
+  return code;
+}
+
+mlakvStatus FailText(mlakvStatus code, const std::string& text) {
+  g_last_error = text;
+  return code;
+}
+
+const char* LastError() { return g_last_error.c_str(); }
+
+int ComputeUnits() {
+  static const int units = [] {
+    int count = 0;
+    if (hipGetDeviceCount(&count) != hipSuccess || count <= 0) return 256;  // MI355X figure, for planning without a device
+    int device = 0;
+    hipDeviceProp_t prop;
+    if (hipGetDevice(&device) != hipSuccess || hipGetDeviceProperties(&prop, device) != hipSuccess) return 256;
+    return prop.multiProcessorCount > 0 ? prop.multiProcessorCount : 256;
+  }();
+  return units;
+}
+
+mlakvStatus CheckView(const mlakvCacheView* cache, const char* who) {
+  if (cache == nullptr) return Fail(MLAKV_ERR_PARAM_NULLPTR, "%s: cache view is null", who);
+  if (cache->latent == nullptr || cache->rope == nullptr) return Fail(MLAKV_ERR_PARAM_NULLPTR, "%s: cache planes are null", who);
+  if (cache->latent_dim != mlakv::kLatentDim || cache->rope_dim != mlakv::kRopeDim) {
+    return Fail(MLAKV_ERR_PARAM_INVALID, "%s: kernels are built for latent %d + rope %d, got %d + %d", who, mlakv::kLatentDim,
+                mlakv::kRopeDim, cache->latent_dim, cache->rope_dim);
+  }
+  if (cache->dtype != MLAKV_DTYPE_BF16 && cache->dtype != MLAKV_DTYPE_FP8_E4M3) {
+    return Fail(MLAKV_ERR_PARAM_INVALID, "%s: unknown cache dtype %d", who, cache->dtype);
+  }
+  if (cache->dtype == MLAKV_DTYPE_FP8_E4M3 && cache->scale == nullptr) {
+    return Fail(MLAKV_ERR_PARAM_NULLPTR, "%s: an FP8 cache needs its scale plane", who);
+  }
+  if (cache->block_size <= 0 || cache->num_blocks <= 0 || cache->num_layers <= 0) {
+    return Fail(MLAKV_ERR_PARAM_INVALID, "%s: block_size %d, num_blocks %d, num_layers %d must be positive", who,
+                cache->block_size, cache->num_blocks, cache->num_layers);
+  }
+  const int64_t strides[] = {cache->latent_layer_stride, cache->latent_block_stride, cache->latent_row_stride,
+                             cache->rope_layer_stride,   cache->rope_block_stride,   cache->rope_row_stride};
+  for (int64_t stride : strides) {
+    if (stride % 16 != 0) {
+      return Fail(MLAKV_ERR_PARAM_INVALID, "%s: cache stride %lld is not a multiple of 16 bytes", who, static_cast<long long>(stride));
+    }
+  }
+  if (reinterpret_cast<uintptr_t>(cache->latent) % 16 != 0 || reinterpret_cast<uintptr_t>(cache->rope) % 16 != 0) {
+    return Fail(MLAKV_ERR_PARAM_INVALID, "%s: cache plane addresses must be 16-byte aligned", who);
+  }
+  if (cache->scale != nullptr && (reinterpret_cast<uintptr_t>(cache->scale) % 4 != 0 || cache->scale_layer_stride % 4 != 0 ||
+                                  cache->scale_block_stride % 4 != 0)) {
+    return Fail(MLAKV_ERR_PARAM_INVALID, "%s: scale plane must be 4-byte aligned", who);
+  }
+  return MLAKV_SUCCESS;
+}
+
+mlakvStatus CheckLayers(const mlakvCacheView* cache, int32_t begin, int32_t count, const char* who) {
+  if (begin < 0 || count < 0 || begin + count > cache->num_layers) {
+    return Fail(MLAKV_ERR_PARAM_INVALID, "%s: layers [%d, %d) outside the cache's %d layers", who, begin, begin + count,
+                cache->num_layers);
+  }
+  return MLAKV_SUCCESS;
+}
+
+mlakv::Plane PlaneAt(void* base, int64_t layer_stride, int64_t block_stride, int64_t row_stride, int32_t layer) {
+  mlakv::Plane plane;
+  plane.base = base == nullptr ? nullptr : static_cast<char*>(base) + static_cast<int64_t>(layer) * layer_stride;
+  plane.layer_stride = layer_stride;
+  plane.block_stride = block_stride;
+  plane.row_stride = row_stride;
+  return plane;
+}
+
+void FillPlanes(const mlakvCacheView* cache, int32_t layer, mlakv::Plane* latent, mlakv::Plane* rope, mlakv::Plane* scale) {
+  *latent = PlaneAt(cache->latent, cache->latent_layer_stride, cache->latent_block_stride, cache->latent_row_stride, layer);
+  *rope = PlaneAt(cache->rope, cache->rope_layer_stride, cache->rope_block_stride, cache->rope_row_stride, layer);
+  *scale = PlaneAt(cache->scale, cache->scale_layer_stride, cache->scale_block_stride, 4, layer);
+}
+
+mlakvStatus HipFail(hipError_t status, const char* who) {
+  return Fail(MLAKV_ERR_RUNTIME, "%s: %s", who, hipGetErrorString(status));
+}
+
+bool Aligned16(const void* pointer) { return reinterpret_cast<uintptr_t>(pointer) % 16 == 0; }
+
+}  // namespace mlakv_abi
+
+using namespace mlakv_abi;
+
+extern "C" {
+
+const char* mlakvGetLastError(void) { return LastError(); }
+
+int32_t mlakvDeviceCount(void) {
+  int count = 0;
+  if (hipGetDeviceCount(&count) != hipSuccess) return 0;
+  return count;
+}
+
+// ---- kernels ----------------------------------------------------------------------
+
+mlakvStatus mlakvAppend(const mlakvCacheView* cache, int32_t layer_begin, int32_t layer_count, const void* latent_src,
+                        int64_t latent_src_layer_stride, int64_t latent_src_row_stride, const void* rope_src,
+                        int64_t rope_src_layer_stride, int64_t rope_src_row_stride, const int32_t* slot_mapping,
+                        int32_t num_tokens, void* stream) {
+  if (mlakvStatus s = CheckView(cache, "mlakvAppend")) return s;
+  if (mlakvStatus s = CheckLayers(cache, layer_begin, layer_count, "mlakvAppend")) return s;
+  if (num_tokens < 0) return Fail(MLAKV_ERR_PARAM_INVALID, "mlakvAppend: negative token count");
+  if (num_tokens == 0 || layer_count == 0) return MLAKV_SUCCESS;
+  if (latent_src == nullptr || rope_src == nullptr || slot_mapping == nullptr) {
+    return Fail(MLAKV_ERR_PARAM_NULLPTR, "mlakvAppend: source rows and slot mapping are required");
+  }
+  if (!Aligned16(latent_src) || !Aligned16(rope_src) || latent_src_row_stride % 16 != 0 || rope_src_row_stride % 16 != 0 ||
+      latent_src_layer_stride % 16 != 0 || rope_src_layer_stride % 16 != 0) {
+    return Fail(MLAKV_ERR_PARAM_INVALID, "mlakvAppend: source rows must be 16-byte aligned with 16-byte-multiple strides");
+  }
+  mlakv::AppendArgs args{};
+  FillPlanes(cache, layer_begin, &args.latent, &args.rope, &args.scale);
+  args.latent_src = {const_cast<char*>(static_cast<const char*>(latent_src)), latent_src_layer_stride, latent_src_row_stride};
+  args.rope_src = {const_cast<char*>(static_cast<const char*>(rope_src)), rope_src_layer_stride, rope_src_row_stride};
+  args.slots = slot_mapping;
+  args.num_tokens = num_tokens;
+  args.num_layers = layer_count;
+  args.num_blocks = cache->num_blocks;
+  args.block_size = cache->block_size;
+  args.fp8 = cache->dtype == MLAKV_DTYPE_FP8_E4M3;
+  const hipError_t status = mlakv::LaunchAppend(args, static_cast<hipStream_t>(stream));
+  return status == hipSuccess ? MLAKV_SUCCESS : HipFail(status, "mlakvAppend");
+}
+
+mlakvStatus mlakvGather(const mlakvCacheView* cache, int32_t layer_begin, int32_t layer_count, const int32_t* block_table,
+                        int32_t table_stride, const int32_t* seq_lens, const int32_t* cu_seq_lens, int32_t batch,
+                        int32_t max_seq_len, void* latent_dst, int64_t latent_dst_layer_stride,
+                        int64_t latent_dst_row_stride, void* rope_dst, int64_t rope_dst_layer_stride,
+                        int64_t rope_dst_row_stride, void* stream) {
+  if (mlakvStatus s = CheckView(cache, "mlakvGather")) return s;
+  if (mlakvStatus s = CheckLayers(cache, layer_begin, layer_count, "mlakvGather")) return s;
+  if (batch < 0 || max_seq_len < 0 || table_stride < 0) return Fail(MLAKV_ERR_PARAM_INVALID, "mlakvGather: negative size");
+  if (batch == 0 || layer_count == 0 || max_seq_len == 0) return MLAKV_SUCCESS;
+  if (block_table == nullptr || seq_lens == nullptr || cu_seq_lens == nullptr || latent_dst == nullptr || rope_dst == nullptr) {
+    return Fail(MLAKV_ERR_PARAM_NULLPTR, "mlakvGather: block table, lengths and destinations are required");
+  }
+  if (static_cast<int64_t>(table_stride) * cache->block_size < max_seq_len) {
+    return Fail(MLAKV_ERR_PARAM_INVALID, "mlakvGather: a table row of %d blocks cannot address %d tokens", table_stride, max_seq_len);
+  }
+  if (batch > 65535 || layer_count > 65535) return Fail(MLAKV_ERR_PARAM_INVALID, "mlakvGather: batch/layers exceed the launch grid");
+  if (!Aligned16(latent_dst) || !Aligned16(rope_dst) || latent_dst_row_stride % 16 != 0 || rope_dst_row_stride % 16 != 0 ||
+      latent_dst_layer_stride % 16 != 0 || rope_dst_layer_stride % 16 != 0) {
+    return Fail(MLAKV_ERR_PARAM_INVALID, "mlakvGather: destination rows must be 16-byte aligned with 16-byte-multiple strides");
+  }
+  mlakv::GatherArgs args{};
+  FillPlanes(cache, layer_begin, &args.latent, &args.rope, &args.scale);
+  args.latent_dst = {static_cast<char*>(latent_dst), latent_dst_layer_stride, latent_dst_row_stride};
+  args.rope_dst = {static_cast<char*>(rope_dst), rope_dst_layer_stride, rope_dst_row_stride};
+  args.block_table = block_table;
+  args.table_stride = table_stride;
+  args.seq_lens = seq_lens;
+  args.cu_seq_lens = cu_seq_lens;
+  args.batch = batch;
+  args.max_seq_len = max_seq_len;
+  args.num_layers = layer_count;
+  args.num_blocks = cache->num_blocks;
+  args.block_size = cache->block_size;
+  args.fp8 = cache->dtype == MLAKV_DTYPE_FP8_E4M3;
+  const hipError_t status = mlakv::LaunchGather(args, static_cast<hipStream_t>(stream));
+  return status == hipSuccess ? MLAKV_SUCCESS : HipFail(status, "mlakvGather");
+}
+
+mlakvStatus mlakvCopyBlocks(const mlakvCacheView* cache, int32_t layer_begin, int32_t layer_count, const int32_t* moves,
+                            int32_t num_moves, void* stream) {
+  if (mlakvStatus s = CheckView(cache, "mlakvCopyBlocks")) return s;
+  if (mlakvStatus s = CheckLayers(cache, layer_begin, layer_count, "mlakvCopyBlocks")) return s;
+  if (num_moves < 0) return Fail(MLAKV_ERR_PARAM_INVALID, "mlakvCopyBlocks: negative move count");
+  if (num_moves == 0 || layer_count == 0) return MLAKV_SUCCESS;
+  if (moves == nullptr) return Fail(MLAKV_ERR_PARAM_NULLPTR, "mlakvCopyBlocks: moves is null");
+  if (layer_count > 65535) return Fail(MLAKV_ERR_PARAM_INVALID, "mlakvCopyBlocks: layers exceed the launch grid");
+  mlakv::CopyBlocksArgs args{};
+  FillPlanes(cache, layer_begin, &args.latent, &args.rope, &args.scale);
+  args.moves = moves;
+  args.num_moves = num_moves;
+  args.num_layers = layer_count;
+  args.num_blocks = cache->num_blocks;
+  args.block_size = cache->block_size;
+  const int32_t element = cache->dtype == MLAKV_DTYPE_BF16 ? 2 : 1;
+  args.latent_row_bytes = element * cache->latent_dim;
+  args.rope_row_bytes = element * cache->rope_dim;
+  args.has_scale = cache->dtype == MLAKV_DTYPE_FP8_E4M3;
+  const hipError_t status = mlakv::LaunchCopyBlocks(args, static_cast<hipStream_t>(stream));
+  return status == hipSuccess ? MLAKV_SUCCESS : HipFail(status, "mlakvCopyBlocks");
+}
+
+mlakvStatus mlakvAttnPlanInit(int32_t batch, int32_t heads, int32_t max_seq_len, int32_t block_size, int32_t dtype,
+                              mlakvAttnPlan* plan) {
+  if (plan == nullptr) return Fail(MLAKV_ERR_PARAM_NULLPTR, "mlakvAttnPlanInit: plan is null");
+  if (batch <= 0 || batch > 65535) return Fail(MLAKV_ERR_PARAM_INVALID, "mlakvAttnPlanInit: batch %d outside [1, 65535]", batch);
+  if (heads <= 0 || heads % 16 != 0 || heads > 128) {
+    return Fail(MLAKV_ERR_PARAM_INVALID, "mlakvAttnPlanInit: heads %d must be a multiple of 16 up to 128", heads);
+  }
+  if (max_seq_len <= 0 || block_size <= 0) return Fail(MLAKV_ERR_PARAM_INVALID, "mlakvAttnPlanInit: sizes must be positive");
+  if (dtype != MLAKV_DTYPE_BF16 && dtype != MLAKV_DTYPE_FP8_E4M3) {
+    return Fail(MLAKV_ERR_PARAM_INVALID, "mlakvAttnPlanInit: unknown cache dtype %d", dtype);
+  }
+  const int max_tiles = (max_seq_len + mlakv::kTileTokens - 1) / mlakv::kTileTokens;
+  const int head_groups = (heads + 63) / 64;
+  // One workgroup occupies a whole CU (two 72 KB tile buffers), so aim for one chunk per CU.
+  int chunks_wanted = ComputeUnits() / (batch * head_groups);
+  if (chunks_wanted < 1) chunks_wanted = 1;
+  int chunk_tiles = (max_tiles + chunks_wanted - 1) / chunks_wanted;
+  if (chunk_tiles < 2) chunk_tiles = max_tiles < 2 ? 1 : 2;  // amortise the query load over at least two tiles
+  if (const char* forced = std::getenv("MLAKV_ATTN_CHUNK_TILES")) {
+    const int value = std::atoi(forced);
+    if (value > 0) chunk_tiles = value;
+  }
+  if (chunk_tiles > max_tiles) chunk_tiles = max_tiles;
+  plan->batch = batch;
+  plan->heads = heads;
+  plan->max_seq_len = max_seq_len;
+  plan->block_size = block_size;
+  plan->dtype = dtype;
+  plan->chunk_tiles = chunk_tiles;
+  plan->max_chunks = (max_tiles + chunk_tiles - 1) / chunk_tiles;
+  plan->reserved = 0;
+  if (plan->max_chunks > 1) {
+    const uint64_t rows = static_cast<uint64_t>(batch) * plan->max_chunks * heads;
+    plan->workspace_bytes = rows * mlakv::kLatentDim * sizeof(float) + ((rows * sizeof(float) + 255) & ~255ull);
+  } else {
+    plan->workspace_bytes = 0;
+  }
+  return MLAKV_SUCCESS;
+}
+
+mlakvStatus mlakvAttnDecode(const mlakvAttnPlan* plan, const mlakvCacheView* cache, int32_t layer, const void* q_latent,
+                            int64_t q_latent_seq_stride, int64_t q_latent_head_stride, const void* q_rope,
+                            int64_t q_rope_seq_stride, int64_t q_rope_head_stride, const int32_t* block_table,
+                            int32_t table_stride, const int32_t* seq_lens, double scale, void* out, int64_t out_seq_stride,
+                            int64_t out_head_stride, float* lse, void* workspace, uint64_t workspace_bytes, void* stream) {
+  if (plan == nullptr) return Fail(MLAKV_ERR_PARAM_NULLPTR, "mlakvAttnDecode: plan is null");
+  if (mlakvStatus s = CheckView(cache, "mlakvAttnDecode")) return s;
+  if (mlakvStatus s = CheckLayers(cache, layer, 1, "mlakvAttnDecode")) return s;
+  if (q_latent == nullptr || q_rope == nullptr || block_table == nullptr || seq_lens == nullptr || out == nullptr) {
+    return Fail(MLAKV_ERR_PARAM_NULLPTR, "mlakvAttnDecode: query, block table, lengths and output are required");
+  }
+  if (plan->dtype != cache->dtype || plan->block_size != cache->block_size) {
+    return Fail(MLAKV_ERR_PARAM_INVALID, "mlakvAttnDecode: the plan was made for dtype %d / block %d, the cache has %d / %d",
+                plan->dtype, plan->block_size, cache->dtype, cache->block_size);
+  }
+  if (!(scale > 0.0) || !std::isfinite(scale)) return Fail(MLAKV_ERR_PARAM_INVALID, "mlakvAttnDecode: a positive softmax scale is required");
+  if (static_cast<int64_t>(table_stride) * cache->block_size < plan->max_seq_len) {
+    return Fail(MLAKV_ERR_PARAM_INVALID, "mlakvAttnDecode: a table row of %d blocks cannot address %d tokens", table_stride,
+                plan->max_seq_len);
+  }
+  if (!Aligned16(q_latent) || !Aligned16(q_rope) || q_latent_seq_stride % 16 != 0 || q_latent_head_stride % 16 != 0 ||
+      q_rope_seq_stride % 16 != 0 || q_rope_head_stride % 16 != 0) {
+    return Fail(MLAKV_ERR_PARAM_INVALID, "mlakvAttnDecode: query rows must be 16-byte aligned with 16-byte-multiple strides");
+  }
+  if (!Aligned16(out) || out_seq_stride % 16 != 0 || out_head_stride % 16 != 0) {
+    return Fail(MLAKV_ERR_PARAM_INVALID, "mlakvAttnDecode: output rows must be 16-byte aligned with 16-byte-multiple strides");
+  }
+  if (plan->workspace_bytes > 0) {
+    if (workspace == nullptr) return Fail(MLAKV_ERR_PARAM_NULLPTR, "mlakvAttnDecode: the plan needs %llu workspace bytes",
+                                          static_cast<unsigned long long>(plan->workspace_bytes));
+    if (workspace_bytes < plan->workspace_bytes || !Aligned16(workspace)) {
+      return Fail(MLAKV_ERR_PARAM_INVALID, "mlakvAttnDecode: workspace of %llu bytes (16-byte aligned) needed, %llu given",
+                  static_cast<unsigned long long>(plan->workspace_bytes), static_cast<unsigned long long>(workspace_bytes));
+    }
+  }
+  static std::once_flag prepared;
+  static hipError_t prepare_status = hipSuccess;
+  std::call_once(prepared, [] { prepare_status = mlakv::PrepareAttnKernels(); });
+  if (prepare_status != hipSuccess) return HipFail(prepare_status, "mlakvAttnDecode (kernel attributes)");
+
+  mlakv::AttnArgs args{};
+  FillPlanes(cache, layer, &args.latent, &args.rope, &args.scale);
+  args.q_latent = static_cast<const char*>(q_latent);
+  args.q_latent_seq_stride = q_latent_seq_stride;
+  args.q_latent_head_stride = q_latent_head_stride;
+  args.q_rope = static_cast<const char*>(q_rope);
+  args.q_rope_seq_stride = q_rope_seq_stride;
+  args.q_rope_head_stride = q_rope_head_stride;
+  args.block_table = block_table;
+  args.table_stride = table_stride;
+  args.seq_lens = seq_lens;
+  args.out = static_cast<char*>(out);
+  args.out_seq_stride = out_seq_stride;
+  args.out_head_stride = out_head_stride;
+  args.lse = lse;
+  const uint64_t rows = static_cast<uint64_t>(plan->batch) * plan->max_chunks * plan->heads;
+  args.partial_out = static_cast<float*>(workspace);
+  args.partial_lse = workspace == nullptr ? nullptr : static_cast<float*>(workspace) + rows * mlakv::kLatentDim;
+  args.scale_log2 = static_cast<float>(scale * 1.4426950408889634);
+  args.batch = plan->batch;
+  args.heads = plan->heads;
+  args.num_blocks = cache->num_blocks;
+  args.block_size = cache->block_size;
+  args.chunk_tiles = plan->chunk_tiles;
+  args.max_chunks = plan->max_chunks;
+  args.fp8 = cache->dtype == MLAKV_DTYPE_FP8_E4M3;
+  const hipError_t status = mlakv::LaunchAttnDecode(args, static_cast<hipStream_t>(stream));
+  return status == hipSuccess ? MLAKV_SUCCESS : HipFail(status, "mlakvAttnDecode");
+}
+
+}  // extern "C"
+
+// ---- arena and KV cache handles -------------------------------------------------------
+
+struct mlakvArena {
+  std::unique_ptr<moe_hip::IDeviceBackend> backend;
+  std::unique_ptr<moe_hip::StaticMemoryArena> arena;
+};
+
+struct mlakvKvCache {
+  mlakvArena* owner = nullptr;
+  std::unique_ptr<moe_hip::KvCacheManager> manager;
+};
+
+namespace {
+// Runs `body`, mapping a contract refusal (KvError) to MLAKV_ERR_CONTRACT.
+template <typename Body>
+mlakvStatus Guard(const char* who, Body body) {
+  try {
+    body();
+    return MLAKV_SUCCESS;
+  } catch (const moe_hip::KvError& error) {
+    return FailText(MLAKV_ERR_CONTRACT, std::string(who) + ": " + error.what());
+  } catch (const std::exception& error) {
+    return FailText(MLAKV_ERR_RUNTIME, std::string(who) + ": " + error.what());
+  }
+}
+}  // namespace
+
+extern "C" {
+
+mlakvStatus mlakvArenaCreate(int32_t backend, mlakvArena** arena) {
+  if (arena == nullptr) return Fail(MLAKV_ERR_PARAM_NULLPTR, "mlakvArenaCreate: output is null");
+  *arena = nullptr;
+  if (backend != MLAKV_BACKEND_HIP && backend != MLAKV_BACKEND_HOST) {
+    return Fail(MLAKV_ERR_PARAM_INVALID, "mlakvArenaCreate: unknown backend %d", backend);
+  }
+  auto handle = std::make_unique<mlakvArena>();
+  const mlakvStatus status = Guard("mlakvArenaCreate", [&] {
+    if (backend == MLAKV_BACKEND_HIP) handle->backend = std::make_unique<moe_hip::HipDeviceBackend>();
+    else handle->backend = std::make_unique<moe_hip::HostDeviceBackend>();
+    handle->arena = std::make_unique<moe_hip::StaticMemoryArena>(*handle->backend);
+  });
+  if (status != MLAKV_SUCCESS) return status == MLAKV_ERR_CONTRACT ? MLAKV_ERR_RUNTIME : status;
+  *arena = handle.release();
+  return MLAKV_SUCCESS;
+}
+
+void mlakvArenaDestroy(mlakvArena* arena) {
+  if (arena == nullptr) return;
+  arena->arena.reset();
+  arena->backend.reset();
+  delete arena;
+}
+
+#define MLAKV_NEED(pointer, who) \
+  if ((pointer) == nullptr) return Fail(MLAKV_ERR_PARAM_NULLPTR, who ": null argument")
+
+mlakvStatus mlakvArenaReserve(mlakvArena* arena, const char* name, size_t bytes, size_t align, size_t* handle) {
+  MLAKV_NEED(arena, "mlakvArenaReserve");
+  MLAKV_NEED(name, "mlakvArenaReserve");
+  return Guard("mlakvArenaReserve", [&] {
+    const size_t h = arena->arena->Reserve(name, bytes, align);
+    if (handle != nullptr) *handle = h;
+  });
+}
+
+mlakvStatus mlakvArenaCommit(mlakvArena* arena) {
+  MLAKV_NEED(arena, "mlakvArenaCommit");
+  return Guard("mlakvArenaCommit", [&] { arena->arena->Commit(); });
+}
+
+mlakvStatus mlakvArenaAddress(const mlakvArena* arena, size_t handle, void** address) {
+  MLAKV_NEED(arena, "mlakvArenaAddress");
+  MLAKV_NEED(address, "mlakvArenaAddress");
+  return Guard("mlakvArenaAddress", [&] { *address = arena->arena->Address(handle); });
+}
+
+mlakvStatus mlakvArenaBytes(const mlakvArena* arena, size_t handle, size_t* bytes) {
+  MLAKV_NEED(arena, "mlakvArenaBytes");
+  MLAKV_NEED(bytes, "mlakvArenaBytes");
+  return Guard("mlakvArenaBytes", [&] { *bytes = arena->arena->Bytes(handle); });
+}
+
+mlakvStatus mlakvArenaOffset(const mlakvArena* arena, size_t handle, size_t* offset) {
+  MLAKV_NEED(arena, "mlakvArenaOffset");
+  MLAKV_NEED(offset, "mlakvArenaOffset");
+  return Guard("mlakvArenaOffset", [&] { *offset = arena->arena->Offset(handle); });
+}
+
+mlakvStatus mlakvArenaNoteWorkspace(mlakvArena* arena, uint64_t bytes) {
+  MLAKV_NEED(arena, "mlakvArenaNoteWorkspace");
+  return Guard("mlakvArenaNoteWorkspace", [&] { arena->arena->NoteWorkspace(bytes); });
+}
+
+mlakvStatus mlakvArenaCommitWorkspace(mlakvArena* arena) {
+  MLAKV_NEED(arena, "mlakvArenaCommitWorkspace");
+  return Guard("mlakvArenaCommitWorkspace", [&] { arena->arena->CommitWorkspace(); });
+}
+
+mlakvStatus mlakvArenaAssertWorkspaceFits(const mlakvArena* arena, uint64_t bytes, const char* what) {
+  MLAKV_NEED(arena, "mlakvArenaAssertWorkspaceFits");
+  return Guard("mlakvArenaAssertWorkspaceFits", [&] { arena->arena->AssertWorkspaceFits(bytes, what ? what : "plan"); });
+}
+
+mlakvStatus mlakvArenaSeal(mlakvArena* arena) {
+  MLAKV_NEED(arena, "mlakvArenaSeal");
+  return Guard("mlakvArenaSeal", [&] { arena->arena->Seal(); });
+}
+
+mlakvStatus mlakvArenaValidateAlignment(const mlakvArena* arena) {
+  MLAKV_NEED(arena, "mlakvArenaValidateAlignment");
+  return Guard("mlakvArenaValidateAlignment", [&] {
+    MOE_HIP_REQUIRE(arena->arena->committed(), "ValidateAlignment needs the arena to be committed first");
+    arena->arena->ValidateAlignment();
+  });
+}
+
+void* mlakvArenaWorkspace(const mlakvArena* arena) { return arena ? arena->arena->workspace() : nullptr; }
+uint64_t mlakvArenaWorkspaceBytes(const mlakvArena* arena) { return arena ? arena->arena->workspace_bytes() : 0; }
+size_t mlakvArenaTotalBytes(const mlakvArena* arena) { return arena ? arena->arena->arena_bytes() : 0; }
+size_t mlakvArenaReservedBytes(const mlakvArena* arena) { return arena ? arena->arena->reserved_bytes() : 0; }
+size_t mlakvArenaReservationCount(const mlakvArena* arena) { return arena ? arena->arena->reservations().size() : 0; }
+int32_t mlakvArenaSealed(const mlakvArena* arena) { return arena && arena->arena->sealed() ? 1 : 0; }
+uint64_t mlakvArenaDeviceAllocationCount(const mlakvArena* arena) { return arena ? arena->backend->DeviceAllocationCount() : 0; }
+
+size_t mlakvArenaDescribeLedger(const mlakvArena* arena, char* buffer, size_t capacity) {
+  if (arena == nullptr) return 0;
+  const std::string text = arena->arena->DescribeLedger();
+  if (buffer != nullptr && capacity > 0) {
+    const size_t n = text.size() < capacity - 1 ? text.size() : capacity - 1;
+    std::memcpy(buffer, text.data(), n);
+    buffer[n] = '\0';
+  }
+  return text.size();
+}
+
+// ---- KV cache manager ---------------------------------------------------------------
+
+mlakvStatus mlakvKvCacheCreate(mlakvArena* arena, const mlakvKvConfig* config, mlakvKvCache** cache) {
+  MLAKV_NEED(arena, "mlakvKvCacheCreate");
+  MLAKV_NEED(config, "mlakvKvCacheCreate");
+  MLAKV_NEED(cache, "mlakvKvCacheCreate");
+  *cache = nullptr;
+  if (config->dtype != MLAKV_DTYPE_BF16 && config->dtype != MLAKV_DTYPE_FP8_E4M3) {
+    return Fail(MLAKV_ERR_PARAM_INVALID, "mlakvKvCacheCreate: unknown cache dtype %d", config->dtype);
+  }
+  auto handle = std::make_unique<mlakvKvCache>();
+  handle->owner = arena;
+  const mlakvStatus status = Guard("mlakvKvCacheCreate", [&] {
+    moe_hip::KvCacheConfig c;
+    c.num_layers = config->num_layers;
+    c.block_size = config->block_size;
+    c.max_context_len = config->max_context_len;
+    c.max_batch = config->max_batch;
+    c.pool_blocks = config->pool_blocks;
+    c.mla.kv_lora_rank = config->kv_lora_rank;
+    c.mla.qk_rope_head_dim = config->qk_rope_head_dim;
+    c.dtype = static_cast<moe_hip::KvDtype>(config->dtype);
+    c.fused_rows = config->fused_rows != 0;
+    c.seed = config->seed;
+    c.shuffle = config->shuffle != 0;
+    handle->manager = std::make_unique<moe_hip::KvCacheManager>(*arena->arena, c);
+  });
+  if (status != MLAKV_SUCCESS) return status;
+  *cache = handle.release();
+  return MLAKV_SUCCESS;
+}
+
+void mlakvKvCacheDestroy(mlakvKvCache* cache) { delete cache; }
+
+mlakvStatus mlakvKvCacheBind(mlakvKvCache* cache) {
+  MLAKV_NEED(cache, "mlakvKvCacheBind");
+  return Guard("mlakvKvCacheBind", [&] { cache->manager->Bind(); });
+}
+
+mlakvStatus mlakvKvCacheGetView(const mlakvKvCache* cache, mlakvCacheView* view) {
+  MLAKV_NEED(cache, "mlakvKvCacheGetView");
+  MLAKV_NEED(view, "mlakvKvCacheGetView");
+  if (!cache->manager->bound()) return Fail(MLAKV_ERR_CONTRACT, "mlakvKvCacheGetView: the cache is not bound yet");
+  const moe_hip::KvCacheView& v = cache->manager->view();
+  view->latent = v.latent.base;
+  view->latent_layer_stride = v.latent.layer_stride;
+  view->latent_block_stride = v.latent.block_stride;
+  view->latent_row_stride = v.latent.row_stride;
+  view->rope = v.rope.base;
+  view->rope_layer_stride = v.rope.layer_stride;
+  view->rope_block_stride = v.rope.block_stride;
+  view->rope_row_stride = v.rope.row_stride;
+  view->scale = v.scale.base;
+  view->scale_layer_stride = v.scale.layer_stride;
+  view->scale_block_stride = v.scale.block_stride;
+  view->num_layers = v.num_layers;
+  view->num_blocks = v.num_blocks;
+  view->block_size = v.block_size;
+  view->latent_dim = v.latent_dim;
+  view->rope_dim = v.rope_dim;
+  view->dtype = static_cast<int32_t>(v.dtype);
+  return MLAKV_SUCCESS;
+}
+
+int64_t mlakvKvCacheNumBlocks(const mlakvKvCache* cache) { return cache ? cache->manager->num_blocks() : 0; }
+int64_t mlakvKvCachePoolBlocks(const mlakvKvCache* cache) { return cache ? cache->manager->pool_blocks() : 0; }
+
+mlakvStatus mlakvKvCacheAddSequence(mlakvKvCache* cache, int64_t seq, int64_t context_len) {
+  MLAKV_NEED(cache, "mlakvKvCacheAddSequence");
+  return Guard("mlakvKvCacheAddSequence", [&] { cache->manager->AddSequence(seq, context_len); });
+}
+
+mlakvStatus mlakvKvCacheAppendToken(mlakvKvCache* cache, int64_t seq, int32_t* slot) {
+  MLAKV_NEED(cache, "mlakvKvCacheAppendToken");
+  return Guard("mlakvKvCacheAppendToken", [&] {
+    const int32_t s = cache->manager->AppendToken(seq);
+    if (slot != nullptr) *slot = s;
+  });
+}
+
+mlakvStatus mlakvKvCacheFreeSequence(mlakvKvCache* cache, int64_t seq) {
+  MLAKV_NEED(cache, "mlakvKvCacheFreeSequence");
+  return Guard("mlakvKvCacheFreeSequence", [&] { cache->manager->FreeSequence(seq); });
+}
+
+mlakvStatus mlakvKvCacheCompact(mlakvKvCache* cache, int32_t* moves, int64_t* num_moves, void* stream) {
+  MLAKV_NEED(cache, "mlakvKvCacheCompact");
+  return Guard("mlakvKvCacheCompact", [&] {
+    const auto planned = cache->manager->Compact(stream);
+    if (moves != nullptr) {
+      for (size_t i = 0; i < planned.size(); ++i) {
+        moves[2 * i] = planned[i].first;
+        moves[2 * i + 1] = planned[i].second;
+      }
+    }
+    if (num_moves != nullptr) *num_moves = static_cast<int64_t>(planned.size());
+  });
+}
+
+mlakvStatus mlakvKvCacheUploadStep(mlakvKvCache* cache, void* stream) {
+  MLAKV_NEED(cache, "mlakvKvCacheUploadStep");
+  return Guard("mlakvKvCacheUploadStep", [&] { cache->manager->UploadStep(stream); });
+}
+
+mlakvStatus mlakvKvCacheGetStats(const mlakvKvCache* cache, mlakvKvStats* stats) {
+  MLAKV_NEED(cache, "mlakvKvCacheGetStats");
+  MLAKV_NEED(stats, "mlakvKvCacheGetStats");
+  const moe_hip::PagedAttentionStats s = cache->manager->stats();
+  stats->total_blocks_allocated = s.total_blocks_allocated;
+  stats->active_context_tokens = s.active_context_tokens;
+  stats->block_size = s.block_size;
+  stats->kv_cache_utilization = s.kv_cache_utilization;
+  return MLAKV_SUCCESS;
+}
+
+const int32_t* mlakvKvCacheHostBlockTable(const mlakvKvCache* cache) { return cache ? cache->manager->host_block_table() : nullptr; }
+const int32_t* mlakvKvCacheHostSlotMapping(const mlakvKvCache* cache) { return cache ? cache->manager->host_slot_mapping() : nullptr; }
+const int32_t* mlakvKvCacheHostSeqLens(const mlakvKvCache* cache) { return cache ? cache->manager->host_seq_lens() : nullptr; }
+int64_t mlakvKvCacheFreeBlocks(const mlakvKvCache* cache) { return cache ? cache->manager->pool().free_blocks() : 0; }
+
+int64_t mlakvKvCacheFreeList(const mlakvKvCache* cache, int32_t* out) {
+  if (cache == nullptr) return 0;
+  const std::vector<int32_t> list = cache->manager->pool().FreeList();
+  if (out != nullptr) std::memcpy(out, list.data(), list.size() * sizeof(int32_t));
+  return static_cast<int64_t>(list.size());
+}
+
+int32_t* mlakvKvCacheDeviceBlockTable(const mlakvKvCache* cache) { return cache ? cache->manager->device_block_table() : nullptr; }
+int32_t* mlakvKvCacheDeviceSlotMapping(const mlakvKvCache* cache) { return cache ? cache->manager->device_slot_mapping() : nullptr; }
+int32_t* mlakvKvCacheDeviceSeqLens(const mlakvKvCache* cache) { return cache ? cache->manager->device_seq_lens() : nullptr; }
+int32_t* mlakvKvCacheDeviceCuSeqLens(const mlakvKvCache* cache) { return cache ? cache->manager->device_cu_seq_lens() : nullptr; }
+
+int64_t mlakvNumBlocks(int64_t max_context_len, int64_t block_size) {
+  if (block_size <= 0 || max_context_len < block_size) return -1;
+  return moe_hip::DivideUp(max_context_len, block_size);
+}
+
+uint64_t mlakvBackboneDeviceBytes(int64_t kv_lora_rank, int64_t qk_rope_head_dim, int64_t block_size, int64_t max_context_len) {
+  moe_hip::MlaGeometry mla;
+  mla.kv_lora_rank = kv_lora_rank;
+  mla.qk_rope_head_dim = qk_rope_head_dim;
+  return moe_hip::BackboneDeviceBytes(mla, block_size, max_context_len);
+}
+
+}  // extern "C"

@@ -1,0 +1,100 @@
+// Internal launch interface between the C ABI and the gfx950 kernels. Host code fills
+// these parameter blocks after validating shapes; the launchers only enqueue.
+#pragma once
+
+#include <hip/hip_runtime.h>
+
+#include <cstdint>
+
+namespace mlakv {
+
+// Address of row (layer, block, slot) = base + layer*layer_stride + block*block_stride + slot*row_stride.
+struct Plane {
+  char* base;
+  int64_t layer_stride;
+  int64_t block_stride;
+  int64_t row_stride;
+};
+
+// Token rows outside the cache: address = base + layer*layer_stride + row*row_stride.
+struct Rows {
+  char* base;
+  int64_t layer_stride;
+  int64_t row_stride;
+};
+
+struct AppendArgs {
+  Plane latent, rope, scale;  // cache planes, already offset to the first layer of the launch
+  Rows latent_src, rope_src;  // bf16 sources
+  const int32_t* slots;
+  int32_t num_tokens;
+  int32_t num_layers;
+  int32_t num_blocks;
+  int32_t block_size;
+  bool fp8;
+};
+
+struct GatherArgs {
+  Plane latent, rope, scale;
+  Rows latent_dst, rope_dst;  // bf16 destinations
+  const int32_t* block_table;
+  int32_t table_stride;  // int32 elements per sequence
+  const int32_t* seq_lens;
+  const int32_t* cu_seq_lens;
+  int32_t batch;
+  int32_t max_seq_len;
+  int32_t num_layers;
+  int32_t num_blocks;
+  int32_t block_size;
+  bool fp8;
+};
+
+struct CopyBlocksArgs {
+  Plane latent, rope, scale;
+  const int32_t* moves;  // (src, dst) pairs
+  int32_t num_moves;
+  int32_t num_layers;
+  int32_t num_blocks;
+  int32_t block_size;
+  int32_t latent_row_bytes;
+  int32_t rope_row_bytes;
+  bool has_scale;
+};
+
+struct AttnArgs {
+  Plane latent, rope, scale;  // offset to the layer of the launch; layer_stride unused
+  const char* q_latent;
+  int64_t q_latent_seq_stride, q_latent_head_stride;
+  const char* q_rope;
+  int64_t q_rope_seq_stride, q_rope_head_stride;
+  const int32_t* block_table;
+  int32_t table_stride;
+  const int32_t* seq_lens;
+  char* out;
+  int64_t out_seq_stride, out_head_stride;
+  float* lse;            // optional
+  float* partial_out;    // workspace: [batch][max_chunks][heads][512] fp32
+  float* partial_lse;    // workspace: [batch][max_chunks][heads] fp32, log2 domain
+  float scale_log2;      // softmax scale * log2(e)
+  int32_t batch;
+  int32_t heads;
+  int32_t num_blocks;
+  int32_t block_size;
+  int32_t chunk_tiles;
+  int32_t max_chunks;
+  bool fp8;
+};
+
+// MLA geometry the kernels are specialised for (include/moe/core/config.hpp:78-109 defaults).
+constexpr int kLatentDim = 512;
+constexpr int kRopeDim = 64;
+constexpr int kTileTokens = 64;
+
+hipError_t LaunchAppend(const AppendArgs& args, hipStream_t stream);
+hipError_t LaunchGather(const GatherArgs& args, hipStream_t stream);
+hipError_t LaunchCopyBlocks(const CopyBlocksArgs& args, hipStream_t stream);
+hipError_t LaunchAttnDecode(const AttnArgs& args, hipStream_t stream);
+// One-time per-process kernel attribute setup (dynamic LDS above 64 KB).
+hipError_t PrepareAttnKernels();
+
+}  // namespace mlakv

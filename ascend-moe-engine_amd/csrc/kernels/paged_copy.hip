@@ -1,0 +1,358 @@
+// Paged KV data movement for gfx950: append (scatter of token rows into physical blocks),
+// block-table gather, compaction block copy; bf16 byte copies and the FP8-E4M3 row-scaled
+// variants (quantize on append, dequantize on gather).
+//
+// All three are HBM-bound. One wavefront owns one work item (a token row for append, a
+// run of rows of one physical block for gather/compaction); every lane moves 16 bytes per
+// access (global_load/store_dwordx4), so a 1024-byte latent row is exactly one wave access
+// and eight 128-byte rope rows are another. The block-table entry and all row bases are
+// wave-uniform, so the address arithmetic stays in scalar registers.
+#include "kernels.h"
+
+namespace mlakv {
+namespace {
+
+typedef __attribute__((ext_vector_type(4))) unsigned int u32x4;
+typedef __attribute__((ext_vector_type(2))) unsigned int u32x2;
+typedef __attribute__((ext_vector_type(2))) float f32x2;
+
+constexpr int kWave = 64;
+constexpr int kWavesPerGroup = 4;
+constexpr int kThreads = kWave * kWavesPerGroup;
+
+__device__ __forceinline__ u32x4 Load16(const char* p) {
+  return __builtin_nontemporal_load(reinterpret_cast<const u32x4*>(p));
+}
+__device__ __forceinline__ void Store16(char* p, u32x4 v) {
+  __builtin_nontemporal_store(v, reinterpret_cast<u32x4*>(p));
+}
+__device__ __forceinline__ u32x2 Load8(const char* p) {
+  return __builtin_nontemporal_load(reinterpret_cast<const u32x2*>(p));
+}
+__device__ __forceinline__ void Store8(char* p, u32x2 v) {
+  __builtin_nontemporal_store(v, reinterpret_cast<u32x2*>(p));
+}
+__device__ __forceinline__ int Uniform(int v) { return __builtin_amdgcn_readfirstlane(v); }
+
+// Copies `nrows` rows of CH 16-byte chunks with one wavefront; U accesses in flight.
+template <int CH>
+__device__ __forceinline__ void CopyRows(const char* src, int64_t src_row_stride, char* dst, int64_t dst_row_stride,
+                                         int nrows, int lane) {
+  static_assert(CH <= kWave && (kWave % CH) == 0, "a row is at most one wave access");
+  constexpr int kRowsPerAccess = kWave / CH;
+  constexpr int U = 8;
+  const int sub = lane / CH;
+  const int chunk = lane % CH;
+  const char* s = src + sub * src_row_stride + chunk * 16;
+  char* d = dst + sub * dst_row_stride + chunk * 16;
+  int r = 0;
+  for (; r + kRowsPerAccess * U <= nrows; r += kRowsPerAccess * U) {
+    u32x4 v[U];
+#pragma unroll
+    for (int u = 0; u < U; ++u) v[u] = Load16(s + static_cast<int64_t>(r + u * kRowsPerAccess) * src_row_stride);
+#pragma unroll
+    for (int u = 0; u < U; ++u) Store16(d + static_cast<int64_t>(r + u * kRowsPerAccess) * dst_row_stride, v[u]);
+  }
+  if (r < nrows) {
+    u32x4 v[U];
+#pragma unroll
+    for (int u = 0; u < U; ++u) {
+      const int row = r + u * kRowsPerAccess;
+      if (row + sub < nrows) v[u] = Load16(s + static_cast<int64_t>(row) * src_row_stride);
+    }
+#pragma unroll
+    for (int u = 0; u < U; ++u) {
+      const int row = r + u * kRowsPerAccess;
+      if (row + sub < nrows) Store16(d + static_cast<int64_t>(row) * dst_row_stride, v[u]);
+    }
+  }
+}
+
+// ---- number formats ---------------------------------------------------------
+
+__device__ __forceinline__ float Bf16ToF32(unsigned int bits16) { return __builtin_bit_cast(float, bits16 << 16); }
+
+// Round to nearest even; inputs here are finite.
+__device__ __forceinline__ unsigned int F32ToBf16(float v) {
+  unsigned int bits = __builtin_bit_cast(unsigned int, v);
+  bits += 0x7fffu + ((bits >> 16) & 1u);
+  return bits >> 16;
+}
+
+// OCP E4M3FN encode: round to nearest even, saturate to +-448, subnormal grid 2^-9 below 2^-6.
+__device__ __forceinline__ unsigned int E4m3Encode(float v) {
+  const unsigned int bits = __builtin_bit_cast(unsigned int, v);
+  const unsigned int sign = (bits >> 24) & 0x80u;
+  const unsigned int mag_bits = bits & 0x7fffffffu;
+  if (mag_bits > 0x7f800000u) return sign | 0x7fu;
+  const float mag = __builtin_bit_cast(float, mag_bits);
+  if (mag >= 448.0f) return sign | 0x7eu;
+  if (mag < 0.015625f) return sign | static_cast<unsigned int>(static_cast<int>(__builtin_rintf(mag * 512.0f)));
+  const unsigned int rounded = mag_bits + 0x7ffffu + ((mag_bits >> 20) & 1u);
+  const int exponent = static_cast<int>(rounded >> 23) - 120;
+  const unsigned int mantissa = (rounded >> 20) & 7u;
+  if (exponent > 15 || (exponent == 15 && mantissa == 7u)) return sign | 0x7eu;
+  return sign | (static_cast<unsigned int>(exponent) << 3) | mantissa;
+}
+
+// Eight E4M3 codes -> eight bf16, each decoded value times `scale`, rounded to nearest even.
+__device__ __forceinline__ u32x4 Dequant8(u32x2 codes, float scale) {
+  const f32x2 a = __builtin_amdgcn_cvt_pk_f32_fp8(static_cast<int>(codes.x), false);
+  const f32x2 b = __builtin_amdgcn_cvt_pk_f32_fp8(static_cast<int>(codes.x), true);
+  const f32x2 c = __builtin_amdgcn_cvt_pk_f32_fp8(static_cast<int>(codes.y), false);
+  const f32x2 d = __builtin_amdgcn_cvt_pk_f32_fp8(static_cast<int>(codes.y), true);
+  u32x4 out;
+  out.x = F32ToBf16(a.x * scale) | (F32ToBf16(a.y * scale) << 16);
+  out.y = F32ToBf16(b.x * scale) | (F32ToBf16(b.y * scale) << 16);
+  out.z = F32ToBf16(c.x * scale) | (F32ToBf16(c.y * scale) << 16);
+  out.w = F32ToBf16(d.x * scale) | (F32ToBf16(d.y * scale) << 16);
+  return out;
+}
+
+// ---- append -----------------------------------------------------------------
+
+// One wavefront per (token, layer). bf16: 64 lanes move the latent row, 8 lanes the rope row.
+__global__ __launch_bounds__(kThreads) void AppendBf16Kernel(AppendArgs a) {
+  const int lane = threadIdx.x & (kWave - 1);
+  const int token = blockIdx.x * kWavesPerGroup + (threadIdx.x >> 6);
+  const int layer = blockIdx.y;
+  if (token >= a.num_tokens) return;
+  const int slot = Uniform(a.slots[token]);
+  if (slot < 0) return;
+  const int block = slot / a.block_size;
+  const int in_block = slot - block * a.block_size;
+  if (block >= a.num_blocks) return;
+  const char* latent_src = a.latent_src.base + layer * a.latent_src.layer_stride + token * a.latent_src.row_stride;
+  const char* rope_src = a.rope_src.base + layer * a.rope_src.layer_stride + token * a.rope_src.row_stride;
+  char* latent_dst = a.latent.base + layer * a.latent.layer_stride + block * a.latent.block_stride +
+                     in_block * a.latent.row_stride;
+  char* rope_dst = a.rope.base + layer * a.rope.layer_stride + block * a.rope.block_stride + in_block * a.rope.row_stride;
+  static_assert(kLatentDim * 2 / 16 == kWave, "one latent row is one wave access");
+  const u32x4 v = Load16(latent_src + lane * 16);
+  u32x4 r;
+  if (lane < kRopeDim * 2 / 16) r = Load16(rope_src + lane * 16);
+  Store16(latent_dst + lane * 16, v);
+  if (lane < kRopeDim * 2 / 16) Store16(rope_dst + lane * 16, r);
+}
+
+// Quantize-on-append: per-row absmax over latent+rope by wave shuffles, scale = absmax/448,
+// code = e4m3(x / scale). Each lane quantizes the 8 latent values it loaded (8-byte store);
+// lanes 0..7 also the rope values.
+__global__ __launch_bounds__(kThreads) void AppendFp8Kernel(AppendArgs a) {
+  const int lane = threadIdx.x & (kWave - 1);
+  const int token = blockIdx.x * kWavesPerGroup + (threadIdx.x >> 6);
+  const int layer = blockIdx.y;
+  if (token >= a.num_tokens) return;
+  const int slot = Uniform(a.slots[token]);
+  if (slot < 0) return;
+  const int block = slot / a.block_size;
+  const int in_block = slot - block * a.block_size;
+  if (block >= a.num_blocks) return;
+  const char* latent_src = a.latent_src.base + layer * a.latent_src.layer_stride + token * a.latent_src.row_stride;
+  const char* rope_src = a.rope_src.base + layer * a.rope_src.layer_stride + token * a.rope_src.row_stride;
+  const bool has_rope = lane < kRopeDim * 2 / 16;
+  const u32x4 lv = Load16(latent_src + lane * 16);
+  u32x4 rv = {0u, 0u, 0u, 0u};
+  if (has_rope) rv = Load16(rope_src + lane * 16);
+  float x[8], y[8];
+#pragma unroll
+  for (int i = 0; i < 4; ++i) {
+    x[2 * i] = Bf16ToF32(lv[i] & 0xffffu);
+    x[2 * i + 1] = Bf16ToF32(lv[i] >> 16);
+    y[2 * i] = Bf16ToF32(rv[i] & 0xffffu);
+    y[2 * i + 1] = Bf16ToF32(rv[i] >> 16);
+  }
+  float absmax = 0.0f;
+#pragma unroll
+  for (int i = 0; i < 8; ++i) absmax = fmaxf(absmax, fmaxf(fabsf(x[i]), fabsf(y[i])));
+#pragma unroll
+  for (int offset = 32; offset >= 1; offset >>= 1) absmax = fmaxf(absmax, __shfl_xor(absmax, offset));
+  const float scale = absmax == 0.0f ? 1.0f : absmax / 448.0f;
+  u32x2 lq = {0u, 0u}, rq = {0u, 0u};
+#pragma unroll
+  for (int i = 0; i < 4; ++i) {
+    lq.x |= E4m3Encode(x[i] / scale) << (8 * i);
+    lq.y |= E4m3Encode(x[4 + i] / scale) << (8 * i);
+    rq.x |= E4m3Encode(y[i] / scale) << (8 * i);
+    rq.y |= E4m3Encode(y[4 + i] / scale) << (8 * i);
+  }
+  char* latent_dst = a.latent.base + layer * a.latent.layer_stride + block * a.latent.block_stride +
+                     in_block * a.latent.row_stride;
+  char* rope_dst = a.rope.base + layer * a.rope.layer_stride + block * a.rope.block_stride + in_block * a.rope.row_stride;
+  Store8(latent_dst + lane * 8, lq);
+  if (has_rope) Store8(rope_dst + lane * 8, rq);
+  if (lane == 0) {
+    float* scale_dst = reinterpret_cast<float*>(a.scale.base + layer * a.scale.layer_stride + block * a.scale.block_stride) + in_block;
+    *scale_dst = scale;
+  }
+}
+
+// ---- gather -----------------------------------------------------------------
+
+// Work item (one wavefront) = `rows_per_item` consecutive token slots of one logical block of
+// one sequence in one layer. grid = (items / 4, batch, layers).
+struct GatherItem {
+  int seq, layer, physical_block, row0, nrows;
+  int64_t out_row0;
+  bool valid;
+};
+
+__device__ __forceinline__ GatherItem ResolveGatherItem(const GatherArgs& g, int rows_per_item) {
+  GatherItem item;
+  item.valid = false;
+  const int wave_item = blockIdx.x * kWavesPerGroup + (threadIdx.x >> 6);
+  item.seq = blockIdx.y;
+  item.layer = blockIdx.z;
+  const int seq_len = Uniform(g.seq_lens[item.seq]);
+  const int items_per_block = g.block_size / rows_per_item;
+  const int logical_block = wave_item / items_per_block;
+  item.row0 = (wave_item - logical_block * items_per_block) * rows_per_item;
+  const int position0 = logical_block * g.block_size + item.row0;
+  if (position0 >= seq_len) return item;
+  item.nrows = min(rows_per_item, seq_len - position0);
+  item.physical_block = Uniform(g.block_table[static_cast<int64_t>(item.seq) * g.table_stride + logical_block]);
+  if (static_cast<unsigned>(item.physical_block) >= static_cast<unsigned>(g.num_blocks)) return item;
+  item.out_row0 = static_cast<int64_t>(Uniform(g.cu_seq_lens[item.seq])) + position0;
+  item.valid = true;
+  return item;
+}
+
+__global__ __launch_bounds__(kThreads) void GatherBf16Kernel(GatherArgs g, int rows_per_item) {
+  const GatherItem item = ResolveGatherItem(g, rows_per_item);
+  if (!item.valid) return;
+  const int lane = threadIdx.x & (kWave - 1);
+  const char* latent_src = g.latent.base + item.layer * g.latent.layer_stride +
+                           item.physical_block * g.latent.block_stride + item.row0 * g.latent.row_stride;
+  char* latent_dst = g.latent_dst.base + item.layer * g.latent_dst.layer_stride + item.out_row0 * g.latent_dst.row_stride;
+  CopyRows<kLatentDim * 2 / 16>(latent_src, g.latent.row_stride, latent_dst, g.latent_dst.row_stride, item.nrows, lane);
+  const char* rope_src = g.rope.base + item.layer * g.rope.layer_stride + item.physical_block * g.rope.block_stride +
+                         item.row0 * g.rope.row_stride;
+  char* rope_dst = g.rope_dst.base + item.layer * g.rope_dst.layer_stride + item.out_row0 * g.rope_dst.row_stride;
+  CopyRows<kRopeDim * 2 / 16>(rope_src, g.rope.row_stride, rope_dst, g.rope_dst.row_stride, item.nrows, lane);
+}
+
+// FP8 rows: each lane decodes 8 codes (8-byte load) to 8 bf16 (16-byte store).
+__global__ __launch_bounds__(kThreads) void GatherFp8Kernel(GatherArgs g, int rows_per_item) {
+  const GatherItem item = ResolveGatherItem(g, rows_per_item);
+  if (!item.valid) return;
+  const int lane = threadIdx.x & (kWave - 1);
+  const char* latent_src = g.latent.base + item.layer * g.latent.layer_stride +
+                           item.physical_block * g.latent.block_stride + item.row0 * g.latent.row_stride;
+  const char* rope_src = g.rope.base + item.layer * g.rope.layer_stride + item.physical_block * g.rope.block_stride +
+                         item.row0 * g.rope.row_stride;
+  const float* scales = reinterpret_cast<const float*>(g.scale.base + item.layer * g.scale.layer_stride +
+                                                       item.physical_block * g.scale.block_stride) + item.row0;
+  char* latent_dst = g.latent_dst.base + item.layer * g.latent_dst.layer_stride + item.out_row0 * g.latent_dst.row_stride;
+  char* rope_dst = g.rope_dst.base + item.layer * g.rope_dst.layer_stride + item.out_row0 * g.rope_dst.row_stride;
+  constexpr int U = 4;
+  // latent: one row (512 codes) per wave access
+  for (int r = 0; r < item.nrows; r += U) {
+    u32x2 codes[U];
+    float scale[U];
+#pragma unroll
+    for (int u = 0; u < U; ++u) {
+      if (r + u < item.nrows) {
+        codes[u] = Load8(latent_src + static_cast<int64_t>(r + u) * g.latent.row_stride + lane * 8);
+        scale[u] = scales[r + u];
+      }
+    }
+#pragma unroll
+    for (int u = 0; u < U; ++u) {
+      if (r + u < item.nrows) Store16(latent_dst + static_cast<int64_t>(r + u) * g.latent_dst.row_stride + lane * 16, Dequant8(codes[u], scale[u]));
+    }
+  }
+  // rope: eight rows (64 codes each) per wave access
+  const int sub = lane >> 3, chunk = lane & 7;
+  for (int r = 0; r < item.nrows; r += 8) {
+    const int row = r + sub;
+    if (row < item.nrows) {
+      const u32x2 codes = Load8(rope_src + static_cast<int64_t>(row) * g.rope.row_stride + chunk * 8);
+      Store16(rope_dst + static_cast<int64_t>(row) * g.rope_dst.row_stride + chunk * 16, Dequant8(codes, scales[row]));
+    }
+  }
+}
+
+// ---- compaction copy ----------------------------------------------------------
+
+// Work item = `rows_per_item` slots of one (src, dst) block pair in one layer.
+template <int LATENT_CH, int ROPE_CH>
+__global__ __launch_bounds__(kThreads) void CopyBlocksKernel(CopyBlocksArgs c, int rows_per_item) {
+  const int lane = threadIdx.x & (kWave - 1);
+  const int wave_item = blockIdx.x * kWavesPerGroup + (threadIdx.x >> 6);
+  const int layer = blockIdx.y;
+  const int items_per_block = c.block_size / rows_per_item;
+  const int move = wave_item / items_per_block;
+  if (move >= c.num_moves) return;
+  const int row0 = (wave_item - move * items_per_block) * rows_per_item;
+  const int src = Uniform(c.moves[2 * move]);
+  const int dst = Uniform(c.moves[2 * move + 1]);
+  if (static_cast<unsigned>(src) >= static_cast<unsigned>(c.num_blocks) ||
+      static_cast<unsigned>(dst) >= static_cast<unsigned>(c.num_blocks)) return;
+  char* latent = c.latent.base + layer * c.latent.layer_stride + row0 * c.latent.row_stride;
+  CopyRows<LATENT_CH>(latent + src * c.latent.block_stride, c.latent.row_stride, latent + dst * c.latent.block_stride,
+                      c.latent.row_stride, rows_per_item, lane);
+  char* rope = c.rope.base + layer * c.rope.layer_stride + row0 * c.rope.row_stride;
+  CopyRows<ROPE_CH>(rope + src * c.rope.block_stride, c.rope.row_stride, rope + dst * c.rope.block_stride,
+                    c.rope.row_stride, rows_per_item, lane);
+  if (c.has_scale) {
+    char* scale = c.scale.base + layer * c.scale.layer_stride + row0 * 4;
+    for (int r = lane; r < rows_per_item; r += kWave) {
+      reinterpret_cast<float*>(scale + dst * c.scale.block_stride)[r] =
+          reinterpret_cast<const float*>(scale + src * c.scale.block_stride)[r];
+    }
+  }
+}
+
+// Largest divisor of block_size that is at most `want` (work-item granularity).
+int RowsPerItem(int block_size, int want) {
+  int rows = block_size < want ? block_size : want;
+  while (block_size % rows != 0) --rows;
+  return rows;
+}
+
+int DivUp(int a, int b) { return (a + b - 1) / b; }
+
+}  // namespace
+
+hipError_t LaunchAppend(const AppendArgs& args, hipStream_t stream) {
+  if (args.num_tokens <= 0 || args.num_layers <= 0) return hipSuccess;
+  const dim3 grid(DivUp(args.num_tokens, kWavesPerGroup), args.num_layers);
+  if (args.fp8) {
+    hipLaunchKernelGGL(AppendFp8Kernel, grid, dim3(kThreads), 0, stream, args);
+  } else {
+    hipLaunchKernelGGL(AppendBf16Kernel, grid, dim3(kThreads), 0, stream, args);
+  }
+  return hipGetLastError();
+}
+
+hipError_t LaunchGather(const GatherArgs& args, hipStream_t stream) {
+  if (args.batch <= 0 || args.num_layers <= 0 || args.max_seq_len <= 0) return hipSuccess;
+  // 16-row items keep more than 8 waves per CU busy even when the batch holds few blocks.
+  const int rows_per_item = RowsPerItem(args.block_size, 16);
+  const int items_per_block = args.block_size / rows_per_item;
+  const int blocks = DivUp(args.max_seq_len, args.block_size);
+  const dim3 grid(DivUp(blocks * items_per_block, kWavesPerGroup), args.batch, args.num_layers);
+  if (args.fp8) {
+    hipLaunchKernelGGL(GatherFp8Kernel, grid, dim3(kThreads), 0, stream, args, rows_per_item);
+  } else {
+    hipLaunchKernelGGL(GatherBf16Kernel, grid, dim3(kThreads), 0, stream, args, rows_per_item);
+  }
+  return hipGetLastError();
+}
+
+hipError_t LaunchCopyBlocks(const CopyBlocksArgs& args, hipStream_t stream) {
+  if (args.num_moves <= 0 || args.num_layers <= 0) return hipSuccess;
+  const int rows_per_item = RowsPerItem(args.block_size, 16);
+  const int items_per_block = args.block_size / rows_per_item;
+  const dim3 grid(DivUp(args.num_moves * items_per_block, kWavesPerGroup), args.num_layers);
+  if (args.latent_row_bytes == kLatentDim * 2 && args.rope_row_bytes == kRopeDim * 2) {
+    hipLaunchKernelGGL((CopyBlocksKernel<64, 8>), grid, dim3(kThreads), 0, stream, args, rows_per_item);
+  } else if (args.latent_row_bytes == kLatentDim && args.rope_row_bytes == kRopeDim) {
+    hipLaunchKernelGGL((CopyBlocksKernel<32, 4>), grid, dim3(kThreads), 0, stream, args, rows_per_item);
+  } else {
+    return hipErrorInvalidValue;
+  }
+  return hipGetLastError();
+}
+
+}  // namespace mlakv

@@ -1,0 +1,250 @@
+/*
+ * mlakv.h -- thin C ABI over the gfx950 HIP kernels of the paged MLA KV-cache path:
+ * static-arena block reservation, per-layer latent KV append, block-table gather,
+ * compaction copy and absorbed-MLA decode attention.
+ *
+ * Plain pointers and sizes only. Every device pointer is an address the caller owns
+ * (the arena below hands them out); `stream` is a hipStream_t passed as void*.
+ * All strides are in BYTES unless a parameter says otherwise. Every function returns
+ * a status and never throws; mlakvGetLastError() returns the text of the most recent
+ * failure on the calling thread.
+ *
+ * Each entry point cites the interface of the reference engine (fxslava/ascend-moe-engine,
+ * paths relative to its tree) that it stands in for.
+ */
+#ifndef MLAKV_H_
+#define MLAKV_H_
+
+#include <stddef.h>
+#include <stdint.h>
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+typedef int32_t mlakvStatus;
+/* Status codes follow the aclnn convention the reference checks against
+ * (include/moe/core/op_table.hpp:142-147). */
+#define MLAKV_SUCCESS 0
+#define MLAKV_ERR_PARAM_NULLPTR 161001
+#define MLAKV_ERR_PARAM_INVALID 161002
+#define MLAKV_ERR_RUNTIME 361001
+/* A refusal of the arena's phase contract (the reference throws Dsv4Error,
+ * include/moe/core/error.hpp:38-77; the mock's contract code, mock/mock_descriptor.cpp:40-44). */
+#define MLAKV_ERR_CONTRACT 100001
+
+#define MLAKV_DTYPE_BF16 0
+#define MLAKV_DTYPE_FP8_E4M3 1
+
+const char* mlakvGetLastError(void);
+/* Number of HIP devices visible; 0 without a GPU. Never fails. */
+int32_t mlakvDeviceCount(void);
+
+/* ------------------------------------------------------------------------- */
+/* Paged cache geometry                                                       */
+/* ------------------------------------------------------------------------- */
+
+/* One paged MLA cache: a latent plane and a rope plane, each
+ * [layer][physical block][slot][dim] (src/memory/static_arena_manager.cpp:315-318, :571-578),
+ * plus, for FP8 rows, one fp32 scale per slot. A fused 576-element row is the special
+ * case rope = latent + latent_dim elements with both row strides equal to the fused row. */
+typedef struct mlakvCacheView {
+  void* latent;
+  int64_t latent_layer_stride, latent_block_stride, latent_row_stride;
+  void* rope;
+  int64_t rope_layer_stride, rope_block_stride, rope_row_stride;
+  void* scale; /* fp32 [layer][block][slot]; NULL for bf16 */
+  int64_t scale_layer_stride, scale_block_stride;
+  int32_t num_layers;
+  int32_t num_blocks; /* physical blocks per layer */
+  int32_t block_size; /* token slots per block */
+  int32_t latent_dim; /* 512: kv_lora_rank, include/moe/core/config.hpp:78-109 */
+  int32_t rope_dim;   /* 64: qk_rope_head_dim */
+  int32_t dtype;      /* MLAKV_DTYPE_* */
+} mlakvCacheView;
+
+/* ------------------------------------------------------------------------- */
+/* Kernels                                                                    */
+/* ------------------------------------------------------------------------- */
+
+/* Append: replaces the launch of stage `kv_cache_write` = aclnnScatterPaKvCache
+ * (src/pipeline/pipeline.cpp:226-234, :415; contract include/moe/core/op_table.hpp:339-372).
+ * For every layer l in [layer_begin, layer_begin+layer_count) and token t with
+ * slot_mapping[t] >= 0:  cache[l][slot/bs][slot%bs] = (latent_src[l][t], rope_src[l][t]).
+ * Sources are bf16; an FP8 cache quantizes on append (E4M3, one fp32 scale per row =
+ * absmax/448, 1 for a zero row). The reference launches one layer per call
+ * (layer_count = 1); the batched form exists because 43 launches of 36 KB are
+ * launch-bound. */
+mlakvStatus mlakvAppend(const mlakvCacheView* cache, int32_t layer_begin, int32_t layer_count,
+                        const void* latent_src, int64_t latent_src_layer_stride, int64_t latent_src_row_stride,
+                        const void* rope_src, int64_t rope_src_layer_stride, int64_t rope_src_row_stride,
+                        const int32_t* slot_mapping, int32_t num_tokens, void* stream);
+
+/* Gather: the paged read that the reference leaves implicit inside its attention
+ * operator (addressing as in third_party/ops_transformer/attention/quant_lightning_indexer/
+ * op_kernel/arch35/quant_lightning_indexer_service_cube.h:243-270):
+ *   dst[l][cu_seq_lens[b] + i] = cache[l][block_table[b][i / bs]][i % bs],  i < seq_lens[b].
+ * Output rows are bf16 (FP8 caches are dequantized: e4m3 * scale). cu_seq_lens has
+ * batch+1 entries (exclusive prefix sum of seq_lens); max_seq_len bounds every seq_lens[b]
+ * and sizes the launch. table_stride is in int32 elements. */
+mlakvStatus mlakvGather(const mlakvCacheView* cache, int32_t layer_begin, int32_t layer_count,
+                        const int32_t* block_table, int32_t table_stride, const int32_t* seq_lens,
+                        const int32_t* cu_seq_lens, int32_t batch, int32_t max_seq_len, void* latent_dst,
+                        int64_t latent_dst_layer_stride, int64_t latent_dst_row_stride, void* rope_dst,
+                        int64_t rope_dst_layer_stride, int64_t rope_dst_row_stride, void* stream);
+
+/* Compaction copy: cache[l][dst_block] = cache[l][src_block] for every (src, dst) pair
+ * in `moves` (device int32[2 * num_moves]) and every layer. Sources and destinations must
+ * be disjoint sets, which the block pool's plan guarantees. No reference counterpart
+ * (the reference never recycles a block). */
+mlakvStatus mlakvCopyBlocks(const mlakvCacheView* cache, int32_t layer_begin, int32_t layer_count,
+                            const int32_t* moves, int32_t num_moves, void* stream);
+
+/* Decode attention: replaces the plan + launch of stage `attention` =
+ * aclnnFusedInferAttentionScoreV5 (src/pipeline/pipeline.cpp:235-249, :416; contract
+ * include/moe/core/op_table.hpp:375-454; constants include/moe/core/config.hpp:193-201).
+ *   s_i = scale * (q_latent[b,h] . c_i + q_rope[b,h] . r_i), p = softmax_i(s),
+ *   out[b,h] = sum_i p_i c_i     over the seq_lens[b] cached rows of sequence b,
+ * one query token per sequence, `heads` query heads sharing one latent KV head.
+ * The plan fixes shapes and the workspace; the launch only enqueues. */
+typedef struct mlakvAttnPlan {
+  int32_t batch;
+  int32_t heads;           /* multiple of 16, at most 128 */
+  int32_t max_seq_len;
+  int32_t block_size;
+  int32_t dtype;           /* cache dtype */
+  int32_t chunk_tiles;     /* 64-token tiles per workgroup; chosen by the plan */
+  int32_t max_chunks;      /* ceil(ceil(max_seq_len / 64) / chunk_tiles) */
+  int32_t reserved;
+  uint64_t workspace_bytes;
+} mlakvAttnPlan;
+
+mlakvStatus mlakvAttnPlanInit(int32_t batch, int32_t heads, int32_t max_seq_len, int32_t block_size, int32_t dtype,
+                              mlakvAttnPlan* plan);
+
+/* q strides: bytes between sequences / between heads. out is bf16 [batch, heads, latent_dim]
+ * with its own strides; lse (optional) is fp32 [batch, heads], natural log of the softmax
+ * denominator. workspace must hold plan->workspace_bytes. */
+mlakvStatus mlakvAttnDecode(const mlakvAttnPlan* plan, const mlakvCacheView* cache, int32_t layer,
+                            const void* q_latent, int64_t q_latent_seq_stride, int64_t q_latent_head_stride,
+                            const void* q_rope, int64_t q_rope_seq_stride, int64_t q_rope_head_stride,
+                            const int32_t* block_table, int32_t table_stride, const int32_t* seq_lens, double scale,
+                            void* out, int64_t out_seq_stride, int64_t out_head_stride, float* lse, void* workspace,
+                            uint64_t workspace_bytes, void* stream);
+
+/* ------------------------------------------------------------------------- */
+/* Static arena (host)                                                        */
+/* ------------------------------------------------------------------------- */
+
+/* The three-phase single-allocation arena, same calls and refusals as the reference's
+ * StaticMemoryArena (include/moe/memory/static_arena.hpp:79-181, src/memory/static_arena.cpp):
+ * Reserve :88-102, Commit :108-118, Address/Bytes :120-129, NoteWorkspace/CommitWorkspace/
+ * AssertWorkspaceFits :270-295, Seal :301-304, ValidateAlignment :310-332, DescribeLedger :334-348.
+ * A refusal returns MLAKV_ERR_CONTRACT where the reference throws. */
+typedef struct mlakvArena mlakvArena;
+#define MLAKV_BACKEND_HIP 0   /* hipMalloc / hipMemset on the current device */
+#define MLAKV_BACKEND_HOST 1  /* 4096-aligned host memory: the counterpart of the reference's
+                                 SimulatedDeviceOps (src/core/device_ops.cpp:268-440), for
+                                 exercising the arena and block pool without a GPU. Kernels
+                                 never run on it. */
+mlakvStatus mlakvArenaCreate(int32_t backend, mlakvArena** arena);
+void mlakvArenaDestroy(mlakvArena* arena);
+mlakvStatus mlakvArenaReserve(mlakvArena* arena, const char* name, size_t bytes, size_t align, size_t* handle);
+mlakvStatus mlakvArenaCommit(mlakvArena* arena);
+mlakvStatus mlakvArenaAddress(const mlakvArena* arena, size_t handle, void** address);
+mlakvStatus mlakvArenaBytes(const mlakvArena* arena, size_t handle, size_t* bytes);
+mlakvStatus mlakvArenaOffset(const mlakvArena* arena, size_t handle, size_t* offset);
+mlakvStatus mlakvArenaNoteWorkspace(mlakvArena* arena, uint64_t bytes);
+mlakvStatus mlakvArenaCommitWorkspace(mlakvArena* arena);
+mlakvStatus mlakvArenaAssertWorkspaceFits(const mlakvArena* arena, uint64_t bytes, const char* what);
+mlakvStatus mlakvArenaSeal(mlakvArena* arena);
+mlakvStatus mlakvArenaValidateAlignment(const mlakvArena* arena);
+void* mlakvArenaWorkspace(const mlakvArena* arena);
+uint64_t mlakvArenaWorkspaceBytes(const mlakvArena* arena);
+size_t mlakvArenaTotalBytes(const mlakvArena* arena);
+size_t mlakvArenaReservedBytes(const mlakvArena* arena);
+size_t mlakvArenaReservationCount(const mlakvArena* arena);
+int32_t mlakvArenaSealed(const mlakvArena* arena);
+/* Device allocations served so far by the arena's backend; the zero-allocation-per-step
+ * invariant is checked by watching it (include/moe/core/device_allocator.hpp:47-50). */
+uint64_t mlakvArenaDeviceAllocationCount(const mlakvArena* arena);
+/* Writes the ledger text (NUL-terminated, truncated to capacity); returns the full length. */
+size_t mlakvArenaDescribeLedger(const mlakvArena* arena, char* buffer, size_t capacity);
+
+/* ------------------------------------------------------------------------- */
+/* KV cache manager (host): reservations, block pool, per-step metadata       */
+/* ------------------------------------------------------------------------- */
+
+/* The KV part of the reference's StaticArenaManager (src/memory/static_arena_manager.cpp:
+ * num_blocks :192-201, reservations :298-300 and :315-318, per-layer strides
+ * src/pipeline/pipeline.cpp:390-395, slot mapping :515-519, diagnostics :134-136 and :532-534),
+ * generalised from one sequence with identity paging to a batch over a shared pool of
+ * physical blocks with a free list, recycling and compaction. */
+typedef struct mlakvKvConfig {
+  int64_t num_layers;       /* 43: include/moe/core/config.hpp:38 */
+  int64_t block_size;       /* RuntimeConfig::block_size */
+  int64_t max_context_len;  /* RuntimeConfig::max_context_len */
+  int64_t max_batch;        /* 1 in the reference (kTokensPerStep) */
+  int64_t pool_blocks;      /* physical blocks per layer; 0 = max_batch * ceil(max_context_len / block_size) */
+  int64_t kv_lora_rank;     /* 512 */
+  int64_t qk_rope_head_dim; /* 64 */
+  int32_t dtype;            /* MLAKV_DTYPE_* */
+  int32_t fused_rows;       /* 0: two planes as in the reference; 1: one plane of 576-element rows */
+  uint64_t seed;            /* free-list shuffle seed */
+  int32_t shuffle;          /* 0: free list in id order (identity paging for one sequence) */
+  int32_t reserved;
+} mlakvKvConfig;
+
+typedef struct mlakvKvStats { /* include/moe/diagnostics/inference_stats.hpp:21-28 */
+  uint64_t total_blocks_allocated;
+  uint64_t active_context_tokens;
+  uint64_t block_size;
+  double kv_cache_utilization;
+} mlakvKvStats;
+
+typedef struct mlakvKvCache mlakvKvCache;
+/* RESERVE phase: records kv.block_table, kv.slot_mapping, kv.seq_lens, kv.cu_seq_lens,
+ * kv.compaction_moves, kv.latent_cache, kv.rope_cache (and kv.scale_cache for FP8) in `arena`. */
+mlakvStatus mlakvKvCacheCreate(mlakvArena* arena, const mlakvKvConfig* config, mlakvKvCache** cache);
+void mlakvKvCacheDestroy(mlakvKvCache* cache);
+/* After mlakvArenaCommit: resolves the reservations to addresses. */
+mlakvStatus mlakvKvCacheBind(mlakvKvCache* cache);
+mlakvStatus mlakvKvCacheGetView(const mlakvKvCache* cache, mlakvCacheView* view);
+int64_t mlakvKvCacheNumBlocks(const mlakvKvCache* cache);      /* per sequence: ceil(max_ctx / bs) */
+int64_t mlakvKvCachePoolBlocks(const mlakvKvCache* cache);
+mlakvStatus mlakvKvCacheAddSequence(mlakvKvCache* cache, int64_t seq, int64_t context_len);
+/* Bookkeeping for one decode step of sequence `seq`: the slot of its next token
+ * (slot = table[pos / bs] * bs + pos % bs; identity paging gives slot = position,
+ * src/pipeline/pipeline.cpp:517). */
+mlakvStatus mlakvKvCacheAppendToken(mlakvKvCache* cache, int64_t seq, int32_t* slot);
+mlakvStatus mlakvKvCacheFreeSequence(mlakvKvCache* cache, int64_t seq);
+/* Plans the defragmentation (live blocks to ids [0, n_live)), rewrites the host tables and
+ * free list, writes the (src, dst) pairs to `moves` (capacity 2 * pool_blocks, may be NULL)
+ * and, when the arena is on the HIP backend, uploads them and enqueues the copy kernel. */
+mlakvStatus mlakvKvCacheCompact(mlakvKvCache* cache, int32_t* moves, int64_t* num_moves, void* stream);
+/* Enqueues the H2D copy of this step's metadata (block table, slot mapping, seq_lens,
+ * cu_seq_lens) from the pinned mirror; the batched form of the reference's 4-byte
+ * slot mailbox copy (src/pipeline/pipeline.cpp:515-519). On the host backend it is a memcpy. */
+mlakvStatus mlakvKvCacheUploadStep(mlakvKvCache* cache, void* stream);
+mlakvStatus mlakvKvCacheGetStats(const mlakvKvCache* cache, mlakvKvStats* stats);
+/* Host mirrors (valid until the cache is destroyed). */
+const int32_t* mlakvKvCacheHostBlockTable(const mlakvKvCache* cache);  /* [max_batch][num_blocks] */
+const int32_t* mlakvKvCacheHostSlotMapping(const mlakvKvCache* cache); /* [max_batch], -1 = no token this step */
+const int32_t* mlakvKvCacheHostSeqLens(const mlakvKvCache* cache);     /* [max_batch], 0 for unused */
+int64_t mlakvKvCacheFreeBlocks(const mlakvKvCache* cache);
+int64_t mlakvKvCacheFreeList(const mlakvKvCache* cache, int32_t* out); /* head first; returns length */
+/* Device addresses inside the arena (NULL before Bind). */
+int32_t* mlakvKvCacheDeviceBlockTable(const mlakvKvCache* cache);
+int32_t* mlakvKvCacheDeviceSlotMapping(const mlakvKvCache* cache);
+int32_t* mlakvKvCacheDeviceSeqLens(const mlakvKvCache* cache);
+int32_t* mlakvKvCacheDeviceCuSeqLens(const mlakvKvCache* cache);
+
+/* Pure arithmetic mirrors, usable without any allocation. */
+int64_t mlakvNumBlocks(int64_t max_context_len, int64_t block_size); /* -1 = refused */
+uint64_t mlakvBackboneDeviceBytes(int64_t kv_lora_rank, int64_t qk_rope_head_dim, int64_t block_size,
+                                  int64_t max_context_len); /* static_arena_manager.cpp:205-241 */
+
+#ifdef __cplusplus
+}
+#endif
+#endif /* MLAKV_H_ */

@@ -1,0 +1,218 @@
+/*
+ * kv_oracle.h -- CPU restatement of the paged MLA KV-cache path. TEST INFRASTRUCTURE ONLY.
+ *
+ * This library is the checker for the HIP implementation. Nothing in the shipped
+ * product may link, load or call it: only the test suite, the smoke entry and the
+ * cpu_baseline leg of the benchmark do, and there only to produce expected values
+ * or a CPU timing.
+ *
+ * Every function names the reference file:line it follows (paths relative to the
+ * reference tree). Where the reference has no counterpart (batched block pool,
+ * FP8 rows, compaction, attention numerics -- its operators are closed binaries and
+ * its mock executes nothing) the header says so and names what pins the function
+ * instead.
+ *
+ * PARITY STATUS
+ *   pinned by the reference itself (oracle/_ref probe + golden ledger):
+ *     kvo_align_up, kvo_divide_up, kvo_num_blocks, kvo_backbone_device_bytes,
+ *     kvo_kv_reservation_bytes, kvo_arena_*, kvo_kv_stats
+ *   pinned by closed form / brute force / library routine (no reference numerics exist):
+ *     kvo_slot, kvo_append_rows, kvo_gather_rows (memcpy identities),
+ *     kvo_splitmix64 (published known answers), kvo_pool_* (invariants, brute force),
+ *     kvo_e4m3_* and kvo_bf16_* (torch CPU casts, exhaustive decode table),
+ *     kvo_mla_decode (float64 torch softmax on small inputs, special cases)
+ *   parity unpinned against the reference's device results: append bytes, gathered
+ *     bytes and attention values as produced by CANN's aclnnScatterPaKvCache /
+ *     aclnnFusedInferAttentionScoreV5 (CANN 9.2.0-beta.2, closed, absent).
+ */
+#ifndef KV_ORACLE_H_
+#define KV_ORACLE_H_
+
+#include <stddef.h>
+#include <stdint.h>
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+#define KVO_OK 0
+#define KVO_REFUSED 1
+
+#define KVO_DTYPE_BF16 0
+#define KVO_DTYPE_FP8_E4M3 1
+
+/* ---- layout arithmetic --------------------------------------------------- */
+
+/* src/memory/expert_layout.cpp:27 */
+size_t kvo_align_up(size_t value, size_t alignment);
+/* src/memory/static_arena_manager.cpp:183 */
+int64_t kvo_divide_up(int64_t value, int64_t divisor);
+/* src/memory/static_arena_manager.cpp:192-201; -1 when the reference constructor refuses. */
+int64_t kvo_num_blocks(int64_t max_context_len, int64_t block_size);
+/* src/memory/static_arena_manager.cpp:205-241 */
+uint64_t kvo_backbone_device_bytes(int64_t kv_lora_rank, int64_t qk_rope_head_dim, int64_t block_size,
+                                   int64_t max_context_len);
+
+/* Sizes of the four KV reservations, src/memory/static_arena_manager.cpp:298-300, :315-318.
+ * `tokens_per_step` is 1 in the reference (kTokensPerStep); a batch generalises it. */
+typedef struct kvo_kv_reservation_bytes_t {
+  uint64_t block_table;
+  uint64_t slot_mapping;
+  uint64_t latent_cache;
+  uint64_t rope_cache;
+} kvo_kv_reservation_bytes_t;
+void kvo_kv_reservation_bytes(int64_t num_layers, int64_t tokens_per_step, int64_t num_blocks, int64_t block_size,
+                              int64_t kv_lora_rank, int64_t qk_rope_head_dim, kvo_kv_reservation_bytes_t* out);
+
+/* KV diagnostics, src/pipeline/pipeline.cpp:134-136 and :532-534. */
+typedef struct kvo_kv_stats_t {
+  uint64_t total_blocks_allocated;
+  uint64_t active_context_tokens;
+  uint64_t block_size;
+  double kv_cache_utilization;
+} kvo_kv_stats_t;
+void kvo_kv_stats(int64_t num_layers, int64_t num_blocks, int64_t block_size, int64_t position, kvo_kv_stats_t* out);
+
+/* ---- static arena (src/memory/static_arena.cpp) -------------------------- */
+
+typedef struct kvo_arena kvo_arena;
+kvo_arena* kvo_arena_new(void);
+void kvo_arena_delete(kvo_arena* arena);
+/* :88-102 */
+int kvo_arena_reserve(kvo_arena* arena, const char* name, size_t bytes, size_t align, size_t* handle);
+/* :108-118; `base` plays the address the single device allocation returned. */
+int kvo_arena_commit(kvo_arena* arena, uintptr_t base);
+/* :120-129 */
+int kvo_arena_address(const kvo_arena* arena, size_t handle, uintptr_t* address);
+int kvo_arena_bytes(const kvo_arena* arena, size_t handle, size_t* bytes);
+int kvo_arena_offset(const kvo_arena* arena, size_t handle, size_t* offset);
+/* :270-295 */
+int kvo_arena_note_workspace(kvo_arena* arena, uint64_t bytes);
+int kvo_arena_commit_workspace(kvo_arena* arena);
+int kvo_arena_workspace_fits(const kvo_arena* arena, uint64_t bytes);
+uint64_t kvo_arena_workspace_bytes(const kvo_arena* arena);
+/* :301-304 */
+int kvo_arena_seal(kvo_arena* arena);
+int kvo_arena_sealed(const kvo_arena* arena);
+/* :310-332 */
+int kvo_arena_validate(const kvo_arena* arena);
+size_t kvo_arena_total_bytes(const kvo_arena* arena);
+size_t kvo_arena_reserved_bytes(const kvo_arena* arena);
+size_t kvo_arena_count(const kvo_arena* arena);
+int kvo_arena_allocations(const kvo_arena* arena);
+
+/* ---- paged addressing ---------------------------------------------------- */
+
+/* slot = table[pos / bs] * bs + pos % bs. Paged addressing as in
+ * third_party/ops_transformer/attention/quant_lightning_indexer/op_kernel/arch35/
+ * quant_lightning_indexer_service_cube.h:243-270; with an identity table this is the
+ * reference's slot = position (src/pipeline/pipeline.cpp:517). */
+int64_t kvo_slot(const int32_t* table_row, int64_t position, int64_t block_size);
+
+/* Scatter of token rows into one plane of one layer: for each t with slots[t] >= 0,
+ * plane[slot/bs][slot%bs][:] = src[t][:] (contract of aclnnScatterPaKvCache mode "Norm",
+ * include/moe/core/op_table.hpp:339-372). All strides in bytes. */
+void kvo_append_rows(uint8_t* plane, int64_t block_stride, int64_t row_stride, int64_t block_size,
+                     const uint8_t* src, int64_t src_row_stride, int64_t row_bytes, const int32_t* slots,
+                     int64_t num_tokens);
+
+/* Block-table gather of one plane of one layer into packed per-sequence rows:
+ * dst[cu(b) + i][:] = plane[table[b][i/bs]][i%bs][:], i < seq_lens[b]. */
+void kvo_gather_rows(const uint8_t* plane, int64_t block_stride, int64_t row_stride, int64_t block_size,
+                     const int32_t* table, int64_t table_stride, const int32_t* seq_lens, int64_t batch,
+                     uint8_t* dst, int64_t dst_row_stride, int64_t row_bytes);
+
+/* Block copy used by compaction: plane[dst_block] = plane[src_block] for each move. */
+void kvo_copy_blocks(uint8_t* plane, int64_t block_stride, int64_t block_bytes, const int32_t* moves,
+                     int64_t num_moves);
+
+/* ---- number formats ------------------------------------------------------ */
+
+uint16_t kvo_bf16_from_f32(float value); /* round to nearest even; NaN stays NaN */
+float kvo_bf16_to_f32(uint16_t bits);
+/* OCP FP8 E4M3FN: bias 7, no infinities, 0x7f/0xff NaN, max finite 448
+ * (reference constant kSwigluMaxDtypeValue, include/moe/core/config.hpp:191). Encode rounds
+ * to nearest even and saturates finite inputs to +-448. */
+uint8_t kvo_e4m3_from_f32(float value);
+float kvo_e4m3_to_f32(uint8_t code);
+/* scale = absmax(row)/448 in fp32; 1.0 for an all-zero row. */
+float kvo_fp8_row_scale(const uint16_t* latent_bf16, int64_t latent_dim, const uint16_t* rope_bf16,
+                        int64_t rope_dim);
+
+/* Quantize-on-append: one fp32 scale per token row over latent+rope, code = e4m3(x / scale). */
+void kvo_append_rows_fp8(uint8_t* latent_plane, int64_t latent_block_stride, int64_t latent_row_stride,
+                         uint8_t* rope_plane, int64_t rope_block_stride, int64_t rope_row_stride,
+                         float* scale_plane, int64_t scale_block_stride /* in floats */, int64_t block_size,
+                         const uint16_t* latent_src, int64_t latent_src_row_stride /* elements */,
+                         const uint16_t* rope_src, int64_t rope_src_row_stride /* elements */, int64_t latent_dim,
+                         int64_t rope_dim, const int32_t* slots, int64_t num_tokens);
+
+/* Dequantizing gather: bf16(e4m3_to_f32(code) * scale). */
+void kvo_gather_rows_fp8(const uint8_t* latent_plane, int64_t latent_block_stride, int64_t latent_row_stride,
+                         const uint8_t* rope_plane, int64_t rope_block_stride, int64_t rope_row_stride,
+                         const float* scale_plane, int64_t scale_block_stride, int64_t block_size,
+                         const int32_t* table, int64_t table_stride, const int32_t* seq_lens, int64_t batch,
+                         uint16_t* latent_dst, int64_t latent_dst_row_stride /* elements */, uint16_t* rope_dst,
+                         int64_t rope_dst_row_stride /* elements */, int64_t latent_dim, int64_t rope_dim);
+
+/* ---- absorbed-MLA decode attention --------------------------------------- */
+
+/* Per sequence b and head h (contract of aclnnFusedInferAttentionScoreV5 as the reference
+ * plans it, src/pipeline/pipeline.cpp:235-249; include/moe/core/op_table.hpp:375-454):
+ *   s_i = scale * (q_lat[b,h] . c_i + q_rope[b,h] . r_i),  p = softmax_i(s),  o[b,h] = sum_i p_i c_i
+ * with c_i the latent row (K and V alias it) and r_i the rope row of token i < seq_lens[b],
+ * reached through the block table. Accumulation in double (accum_f32 == 0) or float.
+ * q strides in elements. out is fp32 [batch, heads, latent_dim]; lse (optional) is
+ * log(sum exp(s_i)) per (b,h). A sequence of length 0 yields zeros and lse = -inf. */
+typedef struct kvo_cache_view_t {
+  const void* latent;      /* layer base */
+  int64_t latent_block_stride, latent_row_stride; /* bytes */
+  const void* rope;
+  int64_t rope_block_stride, rope_row_stride;     /* bytes */
+  const float* scale;      /* fp8 only */
+  int64_t scale_block_stride;                     /* floats */
+  int64_t block_size;
+  int64_t latent_dim, rope_dim;
+  int32_t dtype;           /* KVO_DTYPE_* */
+} kvo_cache_view_t;
+
+void kvo_mla_decode(const uint16_t* q_latent, int64_t q_latent_seq_stride, int64_t q_latent_head_stride,
+                    const uint16_t* q_rope, int64_t q_rope_seq_stride, int64_t q_rope_head_stride,
+                    const kvo_cache_view_t* cache, const int32_t* table, int64_t table_stride,
+                    const int32_t* seq_lens, int64_t batch, int64_t heads, double scale, float* out, float* lse,
+                    int accum_f32);
+
+/* ---- block pool: free list, block tables, recycling, compaction ---------- */
+/* No reference counterpart (the reference is one sequence with identity paging and
+ * never writes its block table, src/memory/static_arena_manager.cpp:298). Semantics:
+ *   - the free list is a FIFO queue over physical block ids, initialised 0..P-1 and,
+ *     when `shuffle` is set, permuted by Fisher-Yates driven by SplitMix64(seed):
+ *     for i = P-1 .. 1: j = next() % (i+1); swap(list[i], list[j]);
+ *   - a sequence takes blocks from the head in logical order; freeing a sequence
+ *     returns its blocks to the tail in logical order;
+ *   - unused table entries are 0 (the arena is zero-filled);
+ *   - compaction moves every live block with id >= n_live into the free ids < n_live,
+ *     pairing the highest live id with the lowest hole; afterwards the free list is
+ *     n_live..P-1 ascending. */
+uint64_t kvo_splitmix64(uint64_t* state);
+
+typedef struct kvo_pool kvo_pool;
+kvo_pool* kvo_pool_new(int64_t num_blocks, int64_t block_size, int64_t max_seqs, int64_t max_blocks_per_seq,
+                       uint64_t seed, int shuffle);
+void kvo_pool_delete(kvo_pool* pool);
+int kvo_pool_add_sequence(kvo_pool* pool, int64_t seq, int64_t context_len);
+int kvo_pool_append_token(kvo_pool* pool, int64_t seq, int32_t* slot);
+int kvo_pool_free_sequence(kvo_pool* pool, int64_t seq);
+/* moves = (src, dst) pairs, capacity 2 * num_blocks int32. */
+int kvo_pool_compact(kvo_pool* pool, int32_t* moves, int64_t* num_moves);
+const int32_t* kvo_pool_table(const kvo_pool* pool);
+int64_t kvo_pool_seq_len(const kvo_pool* pool, int64_t seq);
+int64_t kvo_pool_free_blocks(const kvo_pool* pool);
+int64_t kvo_pool_live_blocks(const kvo_pool* pool);
+/* free list snapshot, head first; returns its length. */
+int64_t kvo_pool_free_list(const kvo_pool* pool, int32_t* out);
+
+#ifdef __cplusplus
+}
+#endif
+#endif /* KV_ORACLE_H_ */

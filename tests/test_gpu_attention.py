@@ -1,0 +1,171 @@
+"""GPU parity: absorbed-MLA decode attention through the C ABI against the CPU oracle
+(float64 accumulation). Tolerance, from the target statement: 2e-2 relative for bf16 KV,
+6e-2 for FP8 KV, measured as max|gpu - oracle| / max|oracle| per test and element-wise as
+|gpu - oracle| <= tol * (|oracle| + max|oracle|)."""
+import math
+
+import numpy as np
+import pytest
+import torch
+
+import kv_testing as kt
+import oracle_ffi as orc
+
+pytestmark = pytest.mark.gpu
+
+LATENT, ROPE = kt.LATENT, kt.ROPE
+SCALE = 1.0 / math.sqrt(192.0)  # 1/sqrt(qk_nope + qk_rope), reference pipeline.cpp:238
+TOL_BF16, TOL_FP8 = 2e-2, 6e-2
+
+
+def _fill_cache(cache, ctxs, table, seed, outliers=0.0):
+    total = sum(ctxs)
+    latent_src = kt.randn_bf16((cache.layers, total, LATENT), seed=seed, outlier_fraction=outliers).cuda()
+    rope_src = kt.randn_bf16((cache.layers, total, ROPE), seed=seed + 1, outlier_fraction=outliers).cuda()
+    kt.append(cache, latent_src, rope_src, kt.dev_i32(kt.slots_for(table, ctxs, cache.block_size)))
+    torch.cuda.synchronize()
+    return latent_src, rope_src
+
+
+def _assert_close(got_bf16, expected_f32, tol):
+    got = got_bf16.float().cpu().numpy()
+    assert np.isfinite(got).all()
+    peak = np.abs(expected_f32).max()
+    err = np.abs(got - expected_f32)
+    assert err.max() <= tol * peak, f"max err {err.max():.4g} vs {tol} * {peak:.4g}"
+    assert (err <= tol * (np.abs(expected_f32) + peak)).all()
+    return err.max() / peak
+
+
+@pytest.mark.parametrize("bs", [16, 64, 128])
+@pytest.mark.parametrize("heads", [16, 64, 128])
+def test_attention_matches_oracle_ragged(bs, heads, monkeypatch):
+    ctxs = [1, 63, 64, 65, 200, 333]
+    blocks = sum(-(-c // bs) for c in ctxs) + 4
+    pool = kt.build_tables(ctxs, bs, blocks, seed=31)
+    table = pool.table()
+    cache = kt.PagedCache(2, blocks, bs)
+    _fill_cache(cache, ctxs, table, seed=40)
+    q = kt.randn_bf16((len(ctxs), heads, LATENT + ROPE), seed=50).cuda()
+    expected, expected_lse = kt.oracle_attention(cache, 1, q, table, ctxs, SCALE)
+    for chunk_tiles in (None, 1, 2, 100):  # planner's choice, many chunks, single chunk (direct path)
+        if chunk_tiles is None:
+            monkeypatch.delenv("MLAKV_ATTN_CHUNK_TILES", raising=False)
+        else:
+            monkeypatch.setenv("MLAKV_ATTN_CHUNK_TILES", str(chunk_tiles))
+        out, lse, plan = kt.attention(cache, 1, q, kt.dev_i32(table), kt.dev_i32(ctxs), SCALE)
+        _assert_close(out, expected, TOL_BF16)
+        assert np.abs(lse.cpu().numpy() - expected_lse).max() <= 2e-2
+
+
+def test_attention_special_cases():
+    bs, heads = 64, 64
+    # (a) context of one token: softmax is 1, output is exactly that latent row
+    # (b) all rows identical: output equals the row
+    # (c) one dominant score: output tends to that row
+    ctxs = [1, 150, 130]
+    blocks = 8
+    pool = kt.build_tables(ctxs, bs, blocks, seed=3)
+    table = pool.table()
+    cache = kt.PagedCache(1, blocks, bs)
+    total = sum(ctxs)
+    latent = kt.randn_bf16((1, total, LATENT), seed=60)
+    rope = kt.randn_bf16((1, total, ROPE), seed=61)
+    latent[0, 1:151] = latent[0, 1]
+    rope[0, 1:151] = rope[0, 1]
+    q = kt.randn_bf16((3, heads, LATENT + ROPE), seed=62)
+    # sequence 2: make token 17 dominate for every head by aligning it with +-q is impossible for all
+    # heads at once, so use a shared query for all heads and a row parallel to it.
+    q[2, :, :] = q[2, 0, :]
+    base = 151
+    latent[0, base + 17] = (q[2, 0, :LATENT].float() * 4).to(torch.bfloat16)
+    rope[0, base + 17] = (q[2, 0, LATENT:].float() * 4).to(torch.bfloat16)
+    latent, rope = latent.cuda(), rope.cuda()
+    kt.append(cache, latent, rope, kt.dev_i32(kt.slots_for(table, ctxs, bs)))
+    out, lse, _ = kt.attention(cache, 0, q.cuda(), kt.dev_i32(table), kt.dev_i32(ctxs), SCALE)
+    assert torch.equal(out[0], latent[0, 0].expand(heads, LATENT))  # (a) exact
+    assert torch.allclose(out[1].float(), latent[0, 1].float().expand(heads, LATENT), rtol=2 ** -7, atol=1e-6)  # (b)
+    dominant = latent[0, base + 17].float()
+    assert (out[2].float() - dominant).abs().max() <= 2e-2 * dominant.abs().max()  # (c)
+    expected, _ = kt.oracle_attention(cache, 0, q.cuda(), table, ctxs, SCALE)
+    _assert_close(out, expected, TOL_BF16)
+
+
+def test_attention_invariant_under_physical_block_permutation():
+    bs, heads = 64, 64
+    ctxs = [257, 100]
+    blocks = 12
+    outs = []
+    for seed in (1, 2):
+        pool = kt.build_tables(ctxs, bs, blocks, seed=seed)
+        table = pool.table()
+        cache = kt.PagedCache(1, blocks, bs)
+        _fill_cache(cache, ctxs, table, seed=70)
+        q = kt.randn_bf16((2, heads, LATENT + ROPE), seed=71).cuda()
+        out, lse, _ = kt.attention(cache, 0, q, kt.dev_i32(table), kt.dev_i32(ctxs), SCALE)
+        outs.append((out, lse, table))
+    assert not np.array_equal(outs[0][2], outs[1][2])
+    assert torch.equal(outs[0][0], outs[1][0])  # same logical order -> bitwise identical
+    assert torch.equal(outs[0][1], outs[1][1])
+
+
+def test_attention_empty_sequence_gives_zeros(monkeypatch):
+    bs, heads = 64, 64
+    ctxs = [0, 70, 0]
+    blocks = 4
+    pool = kt.build_tables(ctxs, bs, blocks, seed=4)
+    table = pool.table()
+    cache = kt.PagedCache(1, blocks, bs)
+    _fill_cache(cache, ctxs, table, seed=80)
+    q = kt.randn_bf16((3, heads, LATENT + ROPE), seed=81).cuda()
+    for chunk_tiles in ("1", "100"):
+        monkeypatch.setenv("MLAKV_ATTN_CHUNK_TILES", chunk_tiles)
+        out, lse, _ = kt.attention(cache, 0, q, kt.dev_i32(table), kt.dev_i32(ctxs), SCALE, max_seq_len=128)
+        assert (out[0] == 0).all() and (out[2] == 0).all()
+        assert torch.isinf(lse[0]).all() and (lse[0] < 0).all()
+        expected, _ = kt.oracle_attention(cache, 0, q, table, ctxs, SCALE)
+        _assert_close(out, expected, TOL_BF16)
+
+
+@pytest.mark.parametrize("bs", [16, 64])
+def test_attention_fp8_kv_matches_oracle(bs):
+    heads = 64
+    ctxs = [5, 64, 129, 700]
+    blocks = sum(-(-c // bs) for c in ctxs) + 2
+    pool = kt.build_tables(ctxs, bs, blocks, seed=9)
+    table = pool.table()
+    cache = kt.PagedCache(1, blocks, bs, fp8=True)
+    _fill_cache(cache, ctxs, table, seed=90, outliers=0.01)
+    q = kt.randn_bf16((len(ctxs), heads, LATENT + ROPE), seed=91).cuda()
+    out, lse, _ = kt.attention(cache, 0, q, kt.dev_i32(table), kt.dev_i32(ctxs), SCALE)
+    expected, expected_lse = kt.oracle_attention(cache, 0, q, table, ctxs, SCALE)
+    _assert_close(out, expected, TOL_FP8)
+    assert np.abs(lse.cpu().numpy() - expected_lse).max() <= 6e-2
+
+
+def test_config3_full_size_against_oracle_sample_and_torch():
+    """BASELINE config 3: batch 32, 64 heads, context 2048, block 64, shuffled table. Every
+    sequence is checked against a float32 torch evaluation of the same formula on the GPU
+    (library routine); four sequences are checked against the float64 oracle."""
+    batch, heads, ctx, bs = 32, 64, 2048, 64
+    ctxs = [ctx] * batch
+    blocks = batch * (ctx // bs) + 16
+    pool = kt.build_tables(ctxs, bs, blocks, seed=77)
+    table = pool.table()
+    cache = kt.PagedCache(1, blocks, bs)
+    gen = torch.Generator(device="cuda").manual_seed(3)
+    latent_src = torch.randn(1, batch * ctx, LATENT, generator=gen, device="cuda").to(torch.bfloat16)
+    rope_src = torch.randn(1, batch * ctx, ROPE, generator=gen, device="cuda").to(torch.bfloat16)
+    kt.append(cache, latent_src, rope_src, kt.dev_i32(kt.slots_for(table, ctxs, bs)))
+    q = torch.randn(batch, heads, LATENT + ROPE, generator=gen, device="cuda").to(torch.bfloat16)
+    out, lse, plan = kt.attention(cache, 0, q, kt.dev_i32(table), kt.dev_i32(ctxs), SCALE)
+    k = torch.cat([latent_src[0], rope_src[0]], dim=-1).float().view(batch, ctx, LATENT + ROPE)
+    v = latent_src[0].float().view(batch, ctx, LATENT)
+    scores = torch.einsum("bhd,btd->bht", q.float(), k) * SCALE
+    ref = torch.einsum("bht,btd->bhd", torch.softmax(scores, dim=-1), v)
+    peak = ref.abs().max().item()
+    assert (out.float() - ref).abs().max().item() <= TOL_BF16 * peak
+    assert (lse - torch.logsumexp(scores, dim=-1)).abs().max().item() <= 2e-2
+    sample = [0, 7, 19, 31]
+    expected, _ = kt.oracle_attention(cache, 0, q[sample], table[sample], [ctx] * len(sample), SCALE)
+    _assert_close(out[sample], expected, TOL_BF16)

@@ -1,0 +1,316 @@
+"""GPU parity: append / gather / compaction through the C ABI against the CPU oracle.
+Bit-exact for block tables, append offsets and gathered bytes (bf16 and FP8 codes/scales)."""
+import ctypes as C
+
+import numpy as np
+import pytest
+import torch
+
+import kv_testing as kt
+import mlakv_ffi as ffi
+import oracle_ffi as orc
+
+pytestmark = pytest.mark.gpu
+
+LATENT, ROPE = kt.LATENT, kt.ROPE
+
+
+def _oracle_planes(layers, blocks, bs, fp8=False):
+    e = 1 if fp8 else 2
+    latent = [np.zeros(blocks * bs * LATENT * e, dtype=np.uint8) for _ in range(layers)]
+    rope = [np.zeros(blocks * bs * ROPE * e, dtype=np.uint8) for _ in range(layers)]
+    scale = [np.zeros(blocks * bs, dtype=np.float32) for _ in range(layers)] if fp8 else None
+    return latent, rope, scale
+
+
+def _oracle_append_bf16(latent, rope, bs, latent_src, rope_src, slots):
+    for layer in range(len(latent)):
+        ls = kt.u8(latent_src[layer]).reshape(-1)
+        rs = kt.u8(rope_src[layer]).reshape(-1)
+        orc.append_rows(latent[layer], bs * LATENT * 2, LATENT * 2, bs, ls, LATENT * 2, LATENT * 2, slots)
+        orc.append_rows(rope[layer], bs * ROPE * 2, ROPE * 2, bs, rs, ROPE * 2, ROPE * 2, slots)
+
+
+def test_config1_identity_paging_append_then_gather():
+    """BASELINE config 1: one layer, block 64, one sequence with identity paging; 128 prompt rows
+    appended one per step, one decode row, gather of all 129 rows, byte comparison. Runs on the
+    arena + KV cache manager (HIP backend), so the reservations and diagnostics are exercised too."""
+    bs, max_ctx = 64, 8192
+    arena = ffi.Arena(ffi.BACKEND_HIP)
+    cache = ffi.KvCache(arena, num_layers=1, block_size=bs, max_context_len=max_ctx, max_batch=1)
+    arena.commit()
+    assert arena.device_allocations == 1
+    cache.bind()
+    arena.seal()
+    view = cache.view()
+    lib = ffi.load()
+    cache.add_sequence(0, 0)
+    rows = kt.randn_bf16((129, LATENT + ROPE), seed=1).cuda()
+    latent_src = rows[:, :LATENT].contiguous()
+    rope_src = rows[:, LATENT:].contiguous()
+    allocations_before = arena.device_allocations
+    for position in range(129):
+        slot = cache.append_token(0)
+        assert slot == position  # identity paging: slot = position (reference pipeline.cpp:517)
+        cache.upload_step(kt.stream_ptr())
+        ffi.check(lib.mlakvAppend(C.byref(view), 0, 1, latent_src[position].data_ptr(), 0, LATENT * 2,
+                                  rope_src[position].data_ptr(), 0, ROPE * 2, cache.device_slot_mapping, 1,
+                                  kt.stream_ptr()))
+    assert arena.device_allocations == allocations_before  # zero allocations inside the steps
+    torch.cuda.synchronize()
+    stats = cache.stats()
+    assert stats.active_context_tokens == 129
+    assert stats.kv_cache_utilization == 0.0157470703125  # reference docs/preflight-verification.md:42-45
+    assert stats.total_blocks_allocated == 128
+    latent_out = torch.zeros(129, LATENT, dtype=torch.bfloat16, device="cuda")
+    rope_out = torch.zeros(129, ROPE, dtype=torch.bfloat16, device="cuda")
+    ffi.check(lib.mlakvGather(C.byref(view), 0, 1, cache.device_block_table, cache.num_blocks, cache.device_seq_lens,
+                              cache.device_cu_seq_lens, 1, 129, latent_out.data_ptr(), 0, LATENT * 2,
+                              rope_out.data_ptr(), 0, ROPE * 2, kt.stream_ptr()))
+    torch.cuda.synchronize()
+    # oracle: memcpy append at slot = position into a zeroed plane, then gather through the table
+    blocks = cache.pool_blocks
+    lat, rop, _ = _oracle_planes(1, blocks, bs)
+    slots = np.arange(129, dtype=np.int32)
+    orc.append_rows(lat[0], bs * LATENT * 2, LATENT * 2, bs, kt.u8(latent_src).reshape(-1), LATENT * 2, LATENT * 2, slots)
+    orc.append_rows(rop[0], bs * ROPE * 2, ROPE * 2, bs, kt.u8(rope_src).reshape(-1), ROPE * 2, ROPE * 2, slots)
+    table = cache.host_block_table()
+    assert list(table[0, :3]) == [0, 1, 2]
+    exp_latent = orc.gather_rows(lat[0], bs * LATENT * 2, LATENT * 2, bs, table, [129], LATENT * 2)
+    exp_rope = orc.gather_rows(rop[0], bs * ROPE * 2, ROPE * 2, bs, table, [129], ROPE * 2)
+    assert kt.u8(latent_out).reshape(-1).tobytes() == exp_latent.tobytes()
+    assert kt.u8(rope_out).reshape(-1).tobytes() == exp_rope.tobytes()
+    assert kt.u8(latent_out).reshape(-1).tobytes() == kt.u8(latent_src).reshape(-1).tobytes()
+    cache.close()
+    arena.close()
+
+
+@pytest.mark.parametrize("fused", [False, True])
+@pytest.mark.parametrize("bs", [16, 64, 128])
+def test_append_gather_shuffled_ragged_batch(fused, bs):
+    layers = 3
+    ctxs = [0, 1, bs - 1, bs, bs + 1, 3 * bs + 7, 5 * bs]
+    need = sum(-(-c // bs) for c in ctxs)
+    blocks = need + 5
+    pool = kt.build_tables(ctxs, bs, blocks, seed=7)
+    table = pool.table()
+    total = sum(ctxs)
+    cache = kt.PagedCache(layers, blocks, bs, fused=fused)
+    latent_src = kt.randn_bf16((layers, total, LATENT), seed=2).cuda()
+    rope_src = kt.randn_bf16((layers, total, ROPE), seed=3).cuda()
+    slots = kt.slots_for(table, ctxs, bs)
+    kt.append(cache, latent_src, rope_src, kt.dev_i32(slots))
+    torch.cuda.synchronize()
+    lat, rop, _ = _oracle_planes(layers, blocks, bs)
+    _oracle_append_bf16(lat, rop, bs, latent_src, rope_src, slots)
+    for layer in range(layers):  # planes bit-exact, including the untouched (zero) slots
+        assert kt.u8(cache.latent[layer].contiguous()).reshape(-1).tobytes() == lat[layer].tobytes()
+        assert kt.u8(cache.rope[layer].contiguous()).reshape(-1).tobytes() == rop[layer].tobytes()
+    for fused_out in (False, True):
+        got_latent, got_rope = kt.gather(cache, kt.dev_i32(table), kt.dev_i32(ctxs), fused_out=fused_out)
+        for layer in range(layers):
+            exp_latent = orc.gather_rows(lat[layer], bs * LATENT * 2, LATENT * 2, bs, table, ctxs, LATENT * 2)
+            exp_rope = orc.gather_rows(rop[layer], bs * ROPE * 2, ROPE * 2, bs, table, ctxs, ROPE * 2)
+            assert kt.u8(got_latent[layer].contiguous()).reshape(-1).tobytes() == exp_latent.tobytes()
+            assert kt.u8(got_rope[layer].contiguous()).reshape(-1).tobytes() == exp_rope.tobytes()
+        # gather o append = identity on the logical sequences
+        assert torch.equal(got_latent.contiguous(), latent_src)
+        assert torch.equal(got_rope.contiguous(), rope_src)
+
+
+def test_append_skips_negative_slots_and_layer_window():
+    layers, bs, blocks = 4, 64, 6
+    cache = kt.PagedCache(layers, blocks, bs)
+    latent_src = kt.randn_bf16((2, 5, LATENT), seed=4).cuda()
+    rope_src = kt.randn_bf16((2, 5, ROPE), seed=5).cuda()
+    slots = np.array([3, -1, 200, -1, 64], dtype=np.int32)
+    kt.append(cache, latent_src, rope_src, kt.dev_i32(slots), layer_begin=1, layer_count=2)
+    torch.cuda.synchronize()
+    lat, rop, _ = _oracle_planes(layers, blocks, bs)
+    _oracle_append_bf16(lat[1:3], rop[1:3], bs, latent_src, rope_src, slots)
+    for layer in range(layers):
+        assert kt.u8(cache.latent[layer].contiguous()).reshape(-1).tobytes() == lat[layer].tobytes()
+        assert kt.u8(cache.rope[layer].contiguous()).reshape(-1).tobytes() == rop[layer].tobytes()
+
+
+def test_compaction_copy_keeps_gathered_bytes():
+    layers, bs = 2, 64
+    ctxs = [130, 64, 300, 17, 200]
+    blocks = 24
+    pool = kt.build_tables(ctxs, bs, blocks, seed=11)
+    cache = kt.PagedCache(layers, blocks, bs)
+    total = sum(ctxs)
+    latent_src = kt.randn_bf16((layers, total, LATENT), seed=6).cuda()
+    rope_src = kt.randn_bf16((layers, total, ROPE), seed=7).cuda()
+    kt.append(cache, latent_src, rope_src, kt.dev_i32(kt.slots_for(pool.table(), ctxs, bs)))
+    # sequences 1 and 3 finish; their blocks return to the free list
+    assert pool.free_sequence(1) == orc.OK and pool.free_sequence(3) == orc.OK
+    live_ctxs = [130, 0, 300, 0, 200]
+    before_latent, before_rope = kt.gather(cache, kt.dev_i32(pool.table()), kt.dev_i32(live_ctxs))
+    lat = [kt.u8(cache.latent[l].contiguous()).reshape(-1).copy() for l in range(layers)]
+    moves = pool.compact()
+    assert moves, "the shuffled pool must need moves"
+    live = pool.live_blocks
+    table = pool.table()
+    used = sorted(int(table[s, i]) for s, n in enumerate(live_ctxs) for i in range(-(-n // bs)))
+    assert used == list(range(live))  # live blocks occupy [0, n_live)
+    lib = ffi.load()
+    moves_dev = kt.dev_i32(np.asarray(moves, dtype=np.int32).reshape(-1))
+    ffi.check(lib.mlakvCopyBlocks(C.byref(cache.view), 0, layers, moves_dev.data_ptr(), len(moves), kt.stream_ptr()))
+    torch.cuda.synchronize()
+    for l in range(layers):  # plane equals the oracle's block copies
+        orc.copy_blocks(lat[l], bs * LATENT * 2, bs * LATENT * 2, moves)
+        assert kt.u8(cache.latent[l].contiguous()).reshape(-1).tobytes() == lat[l].tobytes()
+    after_latent, after_rope = kt.gather(cache, kt.dev_i32(table), kt.dev_i32(live_ctxs))
+    assert torch.equal(before_latent, after_latent) and torch.equal(before_rope, after_rope)
+
+
+def test_kv_cache_manager_matches_oracle_pool_and_compacts_on_device():
+    bs, layers, batch = 64, 2, 6
+    ctxs = [100, 64, 129, 1, 250, 63]
+    arena = ffi.Arena(ffi.BACKEND_HIP)
+    cache = ffi.KvCache(arena, num_layers=layers, block_size=bs, max_context_len=512, max_batch=batch, pool_blocks=20,
+                        seed=99, shuffle=1)
+    arena.commit()
+    cache.bind()
+    view = cache.view()
+    pool = orc.Pool(20, bs, batch, 8, seed=99, shuffle=True)
+    for s, n in enumerate(ctxs):
+        cache.add_sequence(s, n)
+        assert pool.add_sequence(s, n) == orc.OK
+    assert np.array_equal(cache.host_block_table(), pool.table())
+    total = sum(ctxs)
+    latent_src = kt.randn_bf16((layers, total, LATENT), seed=8).cuda()
+    rope_src = kt.randn_bf16((layers, total, ROPE), seed=9).cuda()
+    lib = ffi.load()
+    slots = kt.dev_i32(kt.slots_for(pool.table(), ctxs, bs))
+    ffi.check(lib.mlakvAppend(C.byref(view), 0, layers, latent_src.data_ptr(), total * LATENT * 2, LATENT * 2,
+                              rope_src.data_ptr(), total * ROPE * 2, ROPE * 2, slots.data_ptr(), total, kt.stream_ptr()))
+    cache.free_sequence(2)
+    cache.free_sequence(5)
+    pool.free_sequence(2)
+    pool.free_sequence(5)
+    moves = cache.compact(kt.stream_ptr())
+    assert moves == pool.compact()
+    assert np.array_equal(cache.host_block_table(), pool.table())
+    assert cache.free_list() == pool.free_list()
+    cache.upload_step(kt.stream_ptr())
+    live = [100, 64, 0, 1, 250, 0]
+    rows = sum(live)
+    latent_out = torch.zeros(layers, rows, LATENT, dtype=torch.bfloat16, device="cuda")
+    rope_out = torch.zeros(layers, rows, ROPE, dtype=torch.bfloat16, device="cuda")
+    ffi.check(lib.mlakvGather(C.byref(view), 0, layers, cache.device_block_table, cache.num_blocks,
+                              cache.device_seq_lens, cache.device_cu_seq_lens, batch, 512, latent_out.data_ptr(),
+                              rows * LATENT * 2, LATENT * 2, rope_out.data_ptr(), rows * ROPE * 2, ROPE * 2,
+                              kt.stream_ptr()))
+    torch.cuda.synchronize()
+    starts = np.concatenate([[0], np.cumsum(ctxs)])
+    keep = np.concatenate([np.arange(starts[s], starts[s] + ctxs[s]) for s in (0, 1, 3, 4)])
+    assert torch.equal(latent_out, latent_src[:, keep]) and torch.equal(rope_out, rope_src[:, keep])
+    cache.close()
+    arena.close()
+
+
+# ---- FP8 rows ---------------------------------------------------------------------------
+
+
+@pytest.mark.parametrize("bs", [16, 64])
+def test_fp8_quantize_on_append_and_dequant_gather_bit_exact(bs):
+    layers = 2
+    ctxs = [1, bs + 3, 4 * bs, 0, 77]
+    blocks = sum(-(-c // bs) for c in ctxs) + 3
+    pool = kt.build_tables(ctxs, bs, blocks, seed=21)
+    table = pool.table()
+    total = sum(ctxs)
+    cache = kt.PagedCache(layers, blocks, bs, fp8=True)
+    latent_src = kt.randn_bf16((layers, total, LATENT), seed=10, outlier_fraction=0.01).cuda()
+    rope_src = kt.randn_bf16((layers, total, ROPE), seed=11, outlier_fraction=0.01).cuda()
+    latent_src[0, 0] = 0  # an all-zero row: scale must be 1, codes 0
+    rope_src[0, 0] = 0
+    slots = kt.slots_for(table, ctxs, bs)
+    kt.append(cache, latent_src, rope_src, kt.dev_i32(slots))
+    torch.cuda.synchronize()
+    lat, rop, scl = _oracle_planes(layers, blocks, bs, fp8=True)
+    for layer in range(layers):
+        orc.append_rows_fp8(lat[layer], rop[layer], scl[layer], bs, kt.bits16(latent_src[layer]),
+                            kt.bits16(rope_src[layer]), slots)
+        assert cache.scale_np(layer).tobytes() == scl[layer].tobytes()
+        assert cache.latent_np(layer).tobytes() == lat[layer].tobytes()
+        assert cache.rope_np(layer).tobytes() == rop[layer].tobytes()
+    assert scl[0][slots[0]] == 1.0
+    got_latent, got_rope = kt.gather(cache, kt.dev_i32(table), kt.dev_i32(ctxs))
+    for layer in range(layers):
+        exp_latent, exp_rope = orc.gather_rows_fp8(lat[layer], rop[layer], scl[layer], bs, table, ctxs)
+        assert kt.bits16(got_latent[layer]).tobytes() == exp_latent.tobytes()
+        assert kt.bits16(got_rope[layer]).tobytes() == exp_rope.tobytes()
+    # round-trip bound: |x - dequant| <= scale * 2^-4 * 448 / ... per element; e4m3 keeps 3 mantissa
+    # bits, so the relative error of a normal code is at most 2^-4 and the absolute error in the
+    # subnormal range at most scale * 2^-10 (plus the bf16 rounding of the result, 2^-9 relative).
+    x = latent_src.float()
+    y = got_latent.float()
+    scale = (torch.maximum(latent_src.float().abs().amax(-1), rope_src.float().abs().amax(-1)) / 448.0).unsqueeze(-1)
+    bound = torch.maximum(x.abs() * (2.0 ** -4 + 2.0 ** -8), scale * 2.0 ** -9)
+    assert bool(((x - y).abs() <= bound).all())
+
+
+def test_fp8_compaction_moves_codes_and_scales():
+    layers, bs, blocks = 2, 64, 12
+    ctxs = [100, 64, 129]
+    pool = kt.build_tables(ctxs, bs, blocks, seed=5)
+    cache = kt.PagedCache(layers, blocks, bs, fp8=True)
+    total = sum(ctxs)
+    latent_src = kt.randn_bf16((layers, total, LATENT), seed=12).cuda()
+    rope_src = kt.randn_bf16((layers, total, ROPE), seed=13).cuda()
+    kt.append(cache, latent_src, rope_src, kt.dev_i32(kt.slots_for(pool.table(), ctxs, bs)))
+    pool.free_sequence(1)
+    live = [100, 0, 129]
+    before = kt.gather(cache, kt.dev_i32(pool.table()), kt.dev_i32(live))
+    moves = pool.compact()
+    lib = ffi.load()
+    moves_dev = kt.dev_i32(np.asarray(moves, dtype=np.int32).reshape(-1))
+    ffi.check(lib.mlakvCopyBlocks(C.byref(cache.view), 0, layers, moves_dev.data_ptr(), len(moves), kt.stream_ptr()))
+    after = kt.gather(cache, kt.dev_i32(pool.table()), kt.dev_i32(live))
+    assert torch.equal(before[0], after[0]) and torch.equal(before[1], after[1])
+
+
+# ---- full-size property checks (BASELINE config 2 shape) ---------------------------------------
+
+
+def test_config2_full_size_round_trip():
+    """43 layers, batch 32, contexts uniform in [128, 2048], block 64, shuffled free list: the
+    gathered rows must equal the appended rows for every layer (gather o append = identity)."""
+    layers, batch, bs = 43, 32, 64
+    rng = np.random.default_rng(2)
+    ctxs = [int(v) for v in rng.integers(128, 2049, size=batch)]
+    blocks = sum(-(-(c + 1) // bs) for c in ctxs) + 64
+    pool = kt.build_tables(ctxs, bs, blocks, seed=1234, max_blocks=33)
+    cache = kt.PagedCache(layers, blocks, bs)
+    total = sum(ctxs)
+    gen = torch.Generator(device="cuda").manual_seed(5)
+    latent_src = torch.randn(layers, total, LATENT, generator=gen, device="cuda", dtype=torch.float32).to(torch.bfloat16)
+    rope_src = torch.randn(layers, total, ROPE, generator=gen, device="cuda", dtype=torch.float32).to(torch.bfloat16)
+    kt.append(cache, latent_src, rope_src, kt.dev_i32(kt.slots_for(pool.table(), ctxs, bs)))
+    # one decode step: one more row per sequence per layer
+    step_latent = torch.randn(layers, batch, LATENT, generator=gen, device="cuda", dtype=torch.float32).to(torch.bfloat16)
+    step_rope = torch.randn(layers, batch, ROPE, generator=gen, device="cuda", dtype=torch.float32).to(torch.bfloat16)
+    step_slots = []
+    for s in range(batch):
+        status, slot = pool.append_token(s)
+        assert status == orc.OK
+        step_slots.append(slot)
+    kt.append(cache, step_latent, step_rope, kt.dev_i32(step_slots))
+    new_ctxs = [c + 1 for c in ctxs]
+    got_latent, got_rope = kt.gather(cache, kt.dev_i32(pool.table()), kt.dev_i32(new_ctxs))
+    starts = np.concatenate([[0], np.cumsum(new_ctxs)])
+    old_starts = np.concatenate([[0], np.cumsum(ctxs)])
+    for s in range(batch):
+        a, b = int(starts[s]), int(starts[s + 1])
+        oa, ob = int(old_starts[s]), int(old_starts[s + 1])
+        assert torch.equal(got_latent[:, a:b - 1], latent_src[:, oa:ob])
+        assert torch.equal(got_rope[:, a:b - 1], rope_src[:, oa:ob])
+        assert torch.equal(got_latent[:, b - 1], step_latent[:, s])
+        assert torch.equal(got_rope[:, b - 1], step_rope[:, s])
+    # slots never written stay zero: checksum of the whole pool equals checksum of the sources
+    pool_sum = cache.latent.view(torch.int16).to(torch.int64).sum().item()
+    src_sum = latent_src.view(torch.int16).to(torch.int64).sum().item() + step_latent.view(torch.int16).to(torch.int64).sum().item()
+    assert pool_sum == src_sum
