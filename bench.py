@@ -1,0 +1,323 @@
+#!/usr/bin/env python3
+"""Benchmark of the paged MLA KV-cache hot path on one MI355X.
+
+A step is one pass of the hot path over one batch of synthetic input, for the workload the
+headline metric is quoted on (BASELINE.json configs[1]):
+    43 layers, batch 32, contexts uniform in [128, 2048], block 64, seeded-shuffled free list,
+    bf16 rows of 576 elements (512 latent + 64 rope); per step: host block-pool bookkeeping,
+    metadata upload, append of one row per sequence per layer, gather of every sequence's
+    full context into contiguous [sum ctx, 576] rows per layer.
+`value` is algorithmic bytes per step / wall time per step with all inputs resident in HBM.
+The decode-attention configuration (configs[2]: batch 32, 64 heads, context 2048) is timed in
+the same run and reported under "attention" (us per launch and fraction of the HBM roofline);
+launches rotate over 8 layer slices (604 MB) so the 256 MB Infinity Cache cannot hold the KV.
+
+Prints ONE JSON line. Everything goes through the C ABI (include/mlakv.h); the CPU oracle is
+used only for the cpu_baseline leg.
+"""
+import argparse
+import ctypes as C
+import json
+import math
+import os
+import sys
+import time
+
+ROOT = os.path.dirname(os.path.abspath(__file__))
+sys.path.insert(0, os.path.join(ROOT, "ascend-moe-engine_amd", "python"))
+sys.path.insert(0, os.path.join(ROOT, "oracle"))
+
+HBM_PEAK_GBPS = 8000.0      # MI355X HBM3E, published
+MFMA_BF16_PEAK_TFLOPS = 2500.0
+LATENT, ROPE, ROW = 512, 64, 576
+ROW_BYTES = ROW * 2
+
+
+def parse_args():
+    p = argparse.ArgumentParser()
+    p.add_argument("--gpus", type=int, default=1)
+    p.add_argument("--steps", type=int, default=20)
+    p.add_argument("--warmup", type=int, default=5)
+    p.add_argument("--no-cpu-baseline", action="store_true")
+    p.add_argument("--no-attention", action="store_true")
+    p.add_argument("--split-out", action="store_true", help="gather into separate latent/rope planes instead of 576-wide rows")
+    return p.parse_args()
+
+
+def stream_ptr(torch):
+    return C.c_void_p(torch.cuda.current_stream().cuda_stream)
+
+
+def bench_append_gather(args, torch, np, ffi):
+    lib = ffi.load()
+    layers, batch, bs, max_ctx = 43, 32, 64, 2048 + 128
+    rng = np.random.default_rng(20251125)
+    ctxs = [int(v) for v in rng.integers(128, 2049, size=batch)]
+    total_steps = args.warmup + args.steps
+    pool_blocks = sum(-(-(c + total_steps) // bs) for c in ctxs) + 32
+    arena = ffi.Arena(ffi.BACKEND_HIP)
+    cache = ffi.KvCache(arena, num_layers=layers, block_size=bs, max_context_len=max_ctx, max_batch=batch,
+                        pool_blocks=pool_blocks, seed=20251125, shuffle=1)
+    arena.commit()
+    cache.bind()
+    arena.seal()
+    view = cache.view()
+    for s, n in enumerate(ctxs):
+        cache.add_sequence(s, n)
+    gen = torch.Generator(device="cuda").manual_seed(1)
+    # prefill the pool with N(0,1) rows so the gather reads real data
+    total = sum(ctxs)
+    table = cache.host_block_table()
+    slots = np.concatenate([table[s, np.arange(n) // bs].astype(np.int64) * bs + np.arange(n) % bs
+                            for s, n in enumerate(ctxs)]).astype(np.int32)
+    slots_dev = torch.as_tensor(slots, device="cuda")
+    for layer in range(layers):
+        lat = torch.randn(total, LATENT, generator=gen, device="cuda").to(torch.bfloat16)
+        rop = torch.randn(total, ROPE, generator=gen, device="cuda").to(torch.bfloat16)
+        ffi.check(lib.mlakvAppend(C.byref(view), layer, 1, lat.data_ptr(), 0, LATENT * 2, rop.data_ptr(), 0, ROPE * 2,
+                                  slots_dev.data_ptr(), total, stream_ptr(torch)))
+        torch.cuda.synchronize()
+    step_latent = torch.randn(layers, batch, LATENT, generator=gen, device="cuda").to(torch.bfloat16)
+    step_rope = torch.randn(layers, batch, ROPE, generator=gen, device="cuda").to(torch.bfloat16)
+    rows_cap = total + batch * total_steps
+    if args.split_out:
+        out_latent = torch.empty(layers, rows_cap, LATENT, dtype=torch.bfloat16, device="cuda")
+        out_rope = torch.empty(layers, rows_cap, ROPE, dtype=torch.bfloat16, device="cuda")
+        dst = (out_latent.data_ptr(), rows_cap * LATENT * 2, LATENT * 2, out_rope.data_ptr(), rows_cap * ROPE * 2, ROPE * 2)
+    else:
+        out = torch.empty(layers, rows_cap, ROW, dtype=torch.bfloat16, device="cuda")
+        dst = (out.data_ptr(), rows_cap * ROW_BYTES, ROW_BYTES, out.data_ptr() + LATENT * 2, rows_cap * ROW_BYTES, ROW_BYTES)
+    allocations_before = arena.device_allocations
+    gather_events, append_events = [], []
+
+    def step(timed):
+        for s in range(batch):
+            cache.append_token(s)
+        cache.upload_step(stream_ptr(torch))
+        ev = [torch.cuda.Event(enable_timing=True) for _ in range(3)] if timed else None
+        if timed:
+            ev[0].record()
+        ffi.check(lib.mlakvAppend(C.byref(view), 0, layers, step_latent.data_ptr(), batch * LATENT * 2, LATENT * 2,
+                                  step_rope.data_ptr(), batch * ROPE * 2, ROPE * 2, cache.device_slot_mapping, batch,
+                                  stream_ptr(torch)))
+        if timed:
+            ev[1].record()
+        ffi.check(lib.mlakvGather(C.byref(view), 0, layers, cache.device_block_table, cache.num_blocks,
+                                  cache.device_seq_lens, cache.device_cu_seq_lens, batch, max_ctx, dst[0], dst[1], dst[2],
+                                  dst[3], dst[4], dst[5], stream_ptr(torch)))
+        if timed:
+            ev[2].record()
+            append_events.append((ev[0], ev[1]))
+            gather_events.append((ev[1], ev[2]))
+
+    for _ in range(args.warmup):
+        step(False)
+    torch.cuda.synchronize()
+    rows_per_step = []
+    t0 = time.perf_counter()
+    for i in range(args.steps):
+        step(True)
+        rows_per_step.append(total + batch * (args.warmup + i + 1))
+    torch.cuda.synchronize()
+    elapsed = time.perf_counter() - t0
+    assert arena.device_allocations == allocations_before, "a step allocated device memory"
+
+    blocks_per_step = []
+    lens = cache.host_seq_lens()
+    # algorithmic bytes: append 2*R*row + 4*R; gather 2*sum(ctx)*row + 4*sum(ceil(ctx/bs)), per layer
+    def gather_bytes(rows, final_lens, back):
+        nblk = sum(-(-(int(l) - back) // bs) for l in final_lens)
+        return layers * (2 * rows * ROW_BYTES + 4 * nblk)
+    append_bytes = layers * (2 * batch * ROW_BYTES + 4 * batch)
+    g_bytes = [gather_bytes(rows_per_step[i], lens, args.steps - 1 - i) for i in range(args.steps)]
+    total_bytes = sum(g_bytes) + append_bytes * args.steps
+    gather_ms = [a.elapsed_time(b) for a, b in gather_events]
+    append_ms = [a.elapsed_time(b) for a, b in append_events]
+    gather_gbps = sum(g_bytes) / (sum(gather_ms) * 1e-3) / 1e9
+    result = {
+        "value": total_bytes / elapsed / 1e9,
+        "ms_per_step": elapsed / args.steps * 1e3,
+        "gather_ms": sum(gather_ms) / len(gather_ms),
+        "append_ms": sum(append_ms) / len(append_ms),
+        "gather_gbps": gather_gbps,
+        "append_gbps": append_bytes / (sum(append_ms) / len(append_ms) * 1e-3) / 1e9,
+        "bytes_per_step": total_bytes / args.steps,
+        "gather_bytes_per_launch": sum(g_bytes) / args.steps,
+        "mean_ctx": sum(rows_per_step) / len(rows_per_step) / batch,
+        "ctxs": ctxs, "pool_blocks": pool_blocks, "seed": 20251125,
+    }
+    cache.close()
+    arena.close()
+    return result
+
+
+def bench_attention(args, torch, np, ffi, fp8=False, batch=32, ctx=2048, heads=64, slices=8, iters=None):
+    lib = ffi.load()
+    bs = 64
+    blocks_per_seq = -(-ctx // bs)
+    pool_blocks = batch * blocks_per_seq + 8
+    arena = ffi.Arena(ffi.BACKEND_HIP)
+    cache = ffi.KvCache(arena, num_layers=slices, block_size=bs, max_context_len=ctx, max_batch=batch,
+                        pool_blocks=pool_blocks, seed=7, shuffle=1, dtype=ffi.DTYPE_FP8_E4M3 if fp8 else ffi.DTYPE_BF16)
+    plan = ffi.AttnPlan()
+    ffi.check(lib.mlakvAttnPlanInit(batch, heads, ctx, bs, cache.config.dtype, C.byref(plan)))
+    arena.note_workspace(int(plan.workspace_bytes))
+    arena.commit()
+    arena.commit_workspace()
+    cache.bind()
+    arena.seal()
+    view = cache.view()
+    for s in range(batch):
+        cache.add_sequence(s, ctx)
+    cache.upload_step(stream_ptr(torch))
+    table = cache.host_block_table()
+    slots = np.concatenate([table[s, np.arange(ctx) // bs].astype(np.int64) * bs + np.arange(ctx) % bs
+                            for s in range(batch)]).astype(np.int32)
+    slots_dev = torch.as_tensor(slots, device="cuda")
+    gen = torch.Generator(device="cuda").manual_seed(2)
+    for layer in range(slices):
+        lat = torch.randn(batch * ctx, LATENT, generator=gen, device="cuda").to(torch.bfloat16)
+        rop = torch.randn(batch * ctx, ROPE, generator=gen, device="cuda").to(torch.bfloat16)
+        ffi.check(lib.mlakvAppend(C.byref(view), layer, 1, lat.data_ptr(), 0, LATENT * 2, rop.data_ptr(), 0, ROPE * 2,
+                                  slots_dev.data_ptr(), batch * ctx, stream_ptr(torch)))
+        torch.cuda.synchronize()
+    q = torch.randn(slices, batch, heads, ROW, generator=gen, device="cuda").to(torch.bfloat16)
+    out = torch.empty(slices, batch, heads, LATENT, dtype=torch.bfloat16, device="cuda")
+
+    def launch(i):
+        k = i % slices
+        ffi.check(lib.mlakvAttnDecode(C.byref(plan), C.byref(view), k, q[k].data_ptr(), heads * ROW_BYTES, ROW_BYTES,
+                                      q[k].data_ptr() + LATENT * 2, heads * ROW_BYTES, ROW_BYTES,
+                                      cache.device_block_table, cache.num_blocks, cache.device_seq_lens,
+                                      1.0 / math.sqrt(192.0), out[k].data_ptr(), heads * LATENT * 2, LATENT * 2, None,
+                                      arena.workspace, arena.workspace_bytes, stream_ptr(torch)))
+
+    iters = iters or max(args.steps * 8, 64)
+    for i in range(16):
+        launch(i)
+    torch.cuda.synchronize()
+    start, stop = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+    start.record()
+    for i in range(iters):
+        launch(i)
+    stop.record()
+    torch.cuda.synchronize()
+    us = start.elapsed_time(stop) * 1e3 / iters
+    kv_row = 580 if fp8 else ROW_BYTES
+    algorithmic = batch * ctx * kv_row + batch * heads * ROW * 2 + batch * heads * LATENT * 2 + 4 * batch * blocks_per_seq
+    flops = 2.0 * batch * heads * ctx * (ROW + LATENT)
+    result = {
+        "us_per_step": us,
+        "workload": f"configs[{3 if fp8 else 2}]-shape: 1 layer per launch, batch {batch}, {heads} heads, ctx {ctx}, block 64, "
+                    f"{'fp8 e4m3 + fp32 row scale' if fp8 else 'bf16'} KV, shuffled table, {slices} rotating layer slices",
+        "roofline": {"bound": "hbm", "achieved": algorithmic / (us * 1e-6) / 1e9, "peak": HBM_PEAK_GBPS, "unit": "GB/s",
+                     "frac": algorithmic / (us * 1e-6) / 1e9 / HBM_PEAK_GBPS, "traffic": None},
+        "algorithmic_bytes": algorithmic,
+        "mfma_tflops": flops / (us * 1e-6) / 1e12,
+        "mfma_frac_of_bf16_peak": flops / (us * 1e-6) / 1e12 / MFMA_BF16_PEAK_TFLOPS,
+        "chunk_tiles": int(plan.chunk_tiles), "max_chunks": int(plan.max_chunks),
+        "workspace_bytes": int(plan.workspace_bytes), "launches_timed": iters,
+    }
+    cache.close()
+    arena.close()
+    return result
+
+
+def cpu_baseline(np, ag):
+    """The CPU oracle (a port: the reference has no CPU numerics for this path) on one core, on a
+    bounded sample of the same workload: the append+gather step of 4 of the 43 layers."""
+    import oracle_ffi as orc
+    bs, batch = 64, len(ag["ctxs"])
+    sample_layers = 4
+    ctxs = [c + 1 for c in ag["ctxs"]]
+    pool = orc.Pool(ag["pool_blocks"], bs, batch, 40, seed=ag["seed"], shuffle=True)
+    for s, n in enumerate(ctxs):
+        pool.add_sequence(s, n)
+    table = pool.table()
+    rng = np.random.default_rng(3)
+    planes = [rng.integers(0, 255, size=ag["pool_blocks"] * bs * ROW_BYTES, dtype=np.uint8) for _ in range(sample_layers)]
+    rows = rng.integers(0, 255, size=(sample_layers, batch * ROW_BYTES), dtype=np.uint8)
+    slots = np.array([int(table[s, (n - 1) // bs]) * bs + (n - 1) % bs for s, n in enumerate(ctxs)], dtype=np.int32)
+    times = []
+    for rep in range(6):
+        t0 = time.perf_counter()
+        for layer in range(sample_layers):
+            orc.append_rows(planes[layer], bs * ROW_BYTES, ROW_BYTES, bs, rows[layer], ROW_BYTES, ROW_BYTES, slots)
+            orc.gather_rows(planes[layer], bs * ROW_BYTES, ROW_BYTES, bs, table, ctxs, ROW_BYTES)
+        times.append(time.perf_counter() - t0)
+    times = sorted(times[1:])
+    median = times[len(times) // 2]
+    nbytes = sample_layers * (2 * sum(ctxs) * ROW_BYTES + 2 * batch * ROW_BYTES)
+    return {"value": nbytes / median / 1e9, "unit": "GB/s", "cores": 1, "kind": "port",
+            "sample": f"append+gather of {sample_layers} of 43 layers of the same workload (fused 576-element rows), "
+                      f"median of 5 runs after one warm-up, host cores visible: {os.cpu_count()}"}
+
+
+def cpu_attention_baseline(np):
+    import oracle_ffi as orc
+    bs, heads, ctx, batch = 64, 64, 2048, 1
+    rng = np.random.default_rng(4)
+    blocks = ctx // bs
+    latent = orc.bf16_to_f32(np.zeros(1, np.uint16))  # warm the library
+    latent_plane = (rng.standard_normal(blocks * bs * LATENT).astype(np.float32).view(np.uint32) >> 16).astype(np.uint16)
+    rope_plane = (rng.standard_normal(blocks * bs * ROPE).astype(np.float32).view(np.uint32) >> 16).astype(np.uint16)
+    q_lat = (rng.standard_normal((batch, heads, LATENT)).astype(np.float32).view(np.uint32) >> 16).astype(np.uint16)
+    q_rope = (rng.standard_normal((batch, heads, ROPE)).astype(np.float32).view(np.uint32) >> 16).astype(np.uint16)
+    table = np.arange(blocks, dtype=np.int32).reshape(1, blocks)
+    t0 = time.perf_counter()
+    orc.mla_decode(q_lat, q_rope, latent_plane, rope_plane, bs, table, [ctx], 1 / math.sqrt(192.0), accum_f32=True)
+    seconds = time.perf_counter() - t0
+    return {"value": seconds * 32 * 1e6, "unit": "us/step", "cores": 1, "kind": "port",
+            "sample": "1 of 32 sequences (64 heads, ctx 2048, fp32 accumulate), time scaled by 32"}
+
+
+def main():
+    args = parse_args()
+    if args.gpus != 1:
+        sys.stderr.write("bench.py measures one GPU: this path has no multi-GPU leg (sequences shard with no exchange); "
+                         "run with --gpus 1\n")
+        return 2
+    import numpy as np
+    import torch
+
+    import mlakv_ffi as ffi
+    if not torch.cuda.is_available():
+        sys.stderr.write("bench.py needs a GPU: the HIP library has no CPU fallback\n")
+        return 3
+    torch.cuda.set_device(0)
+    # A plain 1 GiB device copy of known size: the reference point that scales rocprofv3's
+    # FETCH_SIZE / WRITE_SIZE readings for the kernels below.
+    calib_src = torch.ones(1 << 30, dtype=torch.uint8, device="cuda")
+    calib_dst = torch.empty_like(calib_src)
+    calib_dst.copy_(calib_src)
+    torch.cuda.synchronize()
+    del calib_src, calib_dst
+    ag = bench_append_gather(args, torch, np, ffi)
+    line = {
+        "metric": "paged-KV append+gather GB/s; MLA decode attn us/step (% HBM roofline)",
+        "value": ag["value"], "unit": "GB/s", "n_gpus": 1, "steps": args.steps, "warmup": args.warmup,
+        "ms_per_step": ag["ms_per_step"], "higher_is_better": True, "scaling": "weak", "vs_baseline": None,
+        "dtype": "bf16", "data": "synthetic",
+        "config": {"workload": "configs[1]: paged append+gather, 43 layers, batch 32, ctx uniform [128,2048] "
+                               f"(mean {ag['mean_ctx']:.0f} in the timed steps), block 64, seeded-shuffled free list, bf16 rows "
+                               "of 576 elements, 1 row appended per sequence per layer then full-context gather into "
+                               + ("separate latent/rope planes" if args.split_out else "contiguous 576-element rows"),
+                   "bytes_per_step": ag["bytes_per_step"], "frac_of_hbm_peak": ag["value"] / HBM_PEAK_GBPS},
+        "roofline": {"bound": "hbm", "achieved": ag["gather_gbps"], "peak": HBM_PEAK_GBPS, "unit": "GB/s",
+                     "frac": ag["gather_gbps"] / HBM_PEAK_GBPS, "traffic": None, "kernel": "GatherBf16Kernel",
+                     "avg_launch_ms": ag["gather_ms"], "algorithmic_bytes_per_launch": ag["gather_bytes_per_launch"]},
+        "append": {"avg_launch_ms": ag["append_ms"], "achieved_gbps": ag["append_gbps"]},
+    }
+    if not args.no_attention:
+        line["attention"] = bench_attention(args, torch, np, ffi)
+        line["attention_fp8"] = bench_attention(args, torch, np, ffi, fp8=True, batch=64, ctx=4352, iters=64)
+    if not args.no_cpu_baseline:
+        line["cpu_baseline"] = cpu_baseline(np, ag)
+        if not args.no_attention:
+            line["attention"]["cpu_baseline"] = cpu_attention_baseline(np)
+    print(json.dumps(line))
+    return 0
+
+
+if __name__ == "__main__":
+    sys.exit(main())
