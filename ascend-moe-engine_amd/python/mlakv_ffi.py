@@ -129,6 +129,13 @@ def load():
     global _lib
     if _lib is not None:
         return _lib
+    # PyTorch ships its own copy of the HIP runtime. A process must hold exactly one, so when
+    # torch is part of the process it has to be loaded first: this library then binds to the
+    # runtime that is already there instead of bringing a second one.
+    try:
+        import torch  # noqa: F401
+    except ImportError:
+        pass
     if not os.path.exists(LIB_PATH):
         raise FileNotFoundError(
             f"{LIB_PATH} is not built: run `make -C {PACKAGE_DIR}` (or __graft_entry__.build()). "

@@ -1,0 +1,229 @@
+"""The drop-in boundary without a GPU: exported symbols, descriptor engine, plan-time contracts
+and IR-index address swaps of the two operators, in the shape the reference engine uses them
+(src/memory/static_arena_manager.cpp:567-588, src/pipeline/pipeline.cpp:226-249, :390-400).
+No compute call is made here."""
+import ctypes as C
+import os
+import re
+import subprocess
+
+import pytest
+
+import acl_ffi as acl
+import mlakv_ffi as ffi
+
+ROOT = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+FAKE = 0x7F0000000000  # plan-time descriptors only carry addresses; nothing is dereferenced
+
+
+def _declared_functions(header):
+    text = open(os.path.join(ROOT, "include", header)).read()
+    text = re.sub(r"/\*.*?\*/", "", text, flags=re.S)
+    return sorted(set(re.findall(r"\b((?:mlakv|acl|aclnn|aclrt)[A-Za-z0-9]+)\s*\(", text)))
+
+
+def test_library_exports_every_declared_symbol():
+    lib = C.CDLL(ffi.LIB_PATH)
+    for header, minimum in (("mlakv.h", 45), ("aclnn_hip.h", 55)):
+        names = _declared_functions(header)
+        assert len(names) >= minimum, (header, len(names))
+        for name in names:
+            assert hasattr(lib, name), f"{name} declared in include/{header} is not exported"
+    assert set(_declared_functions("mlakv.h")) == set(ffi.PROTOTYPES)
+    assert set(_declared_functions("aclnn_hip.h")) == set(acl.PROTOTYPES)
+
+
+def test_signatures_match_the_reference_typedefs(tmp_path):
+    """The same technique as the reference (tests/mock_pipeline_e2e.cpp:59-73): static_assert the
+    exported declarations against the plan / launch function-pointer types the engine casts
+    its dlsym results to (include/moe/core/op_table.hpp:365-372, :438-454, :1022)."""
+    source = tmp_path / "signature_check.cpp"
+    source.write_text(r'''
+#include <type_traits>
+#include "aclnn_hip.h"
+using ScatterPaKvCachePlanFn = int (*)(const aclTensor*, aclTensor*, const aclTensor*, const aclTensor*, aclTensor*,
+                                       const aclTensor*, const aclTensor*, const aclTensor*, char*, char*, const aclIntArray*,
+                                       const aclIntArray*, uint64_t*, aclOpExecutor**);
+using FusedInferAttentionScoreV5PlanFn = int (*)(
+    const aclTensor*, const aclTensorList*, const aclTensorList*, const aclTensor*, const aclTensor*, const aclIntArray*,
+    const aclIntArray*, const aclTensor*, const aclTensor*, const aclTensor*, const aclTensor*, const aclTensor*, const aclTensor*,
+    const aclTensor*, const aclTensor*, const aclTensor*, const aclTensor*, const aclTensor*, const aclTensor*, const aclTensor*,
+    const aclTensor*, const aclTensor*, const aclTensor*, const aclIntArray*, const aclTensor*, const aclTensor*, const aclTensor*,
+    const aclTensor*, const aclTensor*, const aclIntArray*, const aclIntArray*, int64_t, double, int64_t, int64_t, char*, int64_t,
+    int64_t, int64_t, int64_t, int64_t, bool, int64_t, int64_t, int64_t, int64_t, const aclTensor*, const aclTensor*, uint64_t*,
+    aclOpExecutor**);
+using AclnnLaunchFn = int (*)(void*, uint64_t, aclOpExecutor*, void*);
+static_assert(std::is_same_v<decltype(&aclnnScatterPaKvCacheGetWorkspaceSize), ScatterPaKvCachePlanFn>);
+static_assert(std::is_same_v<decltype(&aclnnFusedInferAttentionScoreV5GetWorkspaceSize), FusedInferAttentionScoreV5PlanFn>);
+static_assert(std::is_same_v<decltype(&aclnnScatterPaKvCache), AclnnLaunchFn>);
+static_assert(std::is_same_v<decltype(&aclnnFusedInferAttentionScoreV5), AclnnLaunchFn>);
+int main() { return 0; }
+''')
+    subprocess.run(["g++", "-std=c++17", "-fsyntax-only", "-I", os.path.join(ROOT, "include"), str(source)], check=True)
+
+
+def test_descriptor_round_trip_and_list_ownership():
+    lib = acl.load()
+    keep = acl.Keep()
+    t = keep.tensor([128, 64, 1, 512], acl.ACL_BF16, FAKE)
+    dims, count = C.POINTER(C.c_int64)(), C.c_uint64()
+    assert lib.aclGetViewShape(t, C.byref(dims), C.byref(count)) == 0
+    assert [dims[i] for i in range(count.value)] == [128, 64, 1, 512]
+    assert lib.aclGetViewStrides(t, C.byref(dims), C.byref(count)) == 0
+    assert [dims[i] for i in range(count.value)] == [64 * 512, 512, 512, 1]  # contiguous when strides are omitted
+    dtype, fmt, addr, off = C.c_int32(), C.c_int32(), C.c_void_p(), C.c_int64()
+    assert lib.aclGetDataType(t, C.byref(dtype)) == 0 and dtype.value == acl.ACL_BF16
+    assert lib.aclGetFormat(t, C.byref(fmt)) == 0 and fmt.value == acl.ACL_FORMAT_ND
+    assert lib.aclGetRawTensorAddr(t, C.byref(addr)) == 0 and addr.value == FAKE
+    assert lib.aclGetViewOffset(t, C.byref(off)) == 0 and off.value == 0
+    # a list owns copies of descriptors; destroying it destroys them (reference static_arena.cpp:172-208)
+    copy = keep.tensor([128, 64, 1, 512], acl.ACL_BF16, FAKE)
+    lst = keep.tensor_list([copy])
+    assert lib.aclDestroyTensorList(lst) == 0
+    assert lib.aclGetDataType(copy, C.byref(dtype)) == 161002  # gone with its list
+    assert lib.aclDestroyTensor(copy) == 161002
+    assert lib.aclDestroyTensor(t) == 0
+    assert lib.aclDestroyTensor(t) == 161002
+    assert lib.aclGetDataType(None, C.byref(dtype)) == 161001
+    assert not lib.aclCreateTensorList(None, 0)
+    assert not lib.aclCreateIntArray(None, 0)
+    assert "empty" in acl.last_error()
+
+
+class Engine:
+    """Descriptors as the reference's CreateDescriptors builds them, for one sequence."""
+
+    def __init__(self, block_size=64, max_context=8192, heads=64):
+        self.keep = acl.Keep()
+        k = self.keep
+        self.bs, self.heads = block_size, heads
+        self.blocks = -(-max_context // block_size)
+        self.q_b = FAKE + 0x100000
+        self.q_latent = k.tensor([1, heads, 512], acl.ACL_BF16, self.q_b, strides=[heads * 576, 576, 1])
+        self.q_rope = k.tensor([1, heads, 64], acl.ACL_BF16, self.q_b + 1024, strides=[heads * 576, 576, 1])
+        self.kv_latent_normed = k.tensor([1, 512], acl.ACL_BF16, FAKE + 0x200000)
+        self.k_rope = k.tensor([1, 1, 64], acl.ACL_BF16, FAKE + 0x201000)
+        self.latent_cache = k.tensor([self.blocks, block_size, 1, 512], acl.ACL_BF16, FAKE + 0x1000000)
+        self.rope_cache = k.tensor([self.blocks, block_size, 1, 64], acl.ACL_BF16, FAKE + 0x9000000)
+        self.rope_cache_view = k.tensor([self.blocks, block_size, 1, 64], acl.ACL_BF16, FAKE + 0x9000000)
+        self.key_list = k.tensor_list([k.tensor([self.blocks, block_size, 1, 512], acl.ACL_BF16, FAKE + 0x1000000)])
+        self.value_list = k.tensor_list([k.tensor([self.blocks, block_size, 1, 512], acl.ACL_BF16, FAKE + 0x1000000)])
+        self.block_table = k.tensor([1, self.blocks], acl.ACL_INT32, FAKE + 0x300000)
+        self.slot_mapping = k.tensor([1], acl.ACL_INT32, FAKE + 0x301000)
+        self.seq_q, _ = k.int_array([1])
+        self.seq_kv, self.seq_kv_storage = k.int_array([max_context])
+        self.attn_out = k.tensor([1, heads, 512], acl.ACL_BF16, FAKE + 0x400000)
+        self.lse = k.tensor([1, heads, 1], acl.ACL_FLOAT32, FAKE + 0x500000)
+
+    def plan_attention(self, **kw):
+        args = dict(heads=self.heads, scale=1.0 / 192 ** 0.5, block_size=self.bs)
+        args.update(kw)
+        return acl.plan_attention(self.q_latent, self.key_list, self.value_list, self.seq_q, self.seq_kv, self.block_table,
+                                  self.q_rope, self.rope_cache_view, out=self.attn_out, lse=self.lse, **args)
+
+
+def test_scatter_plan_contract_and_address_swaps():
+    lib = acl.load()
+    e = Engine()
+    status, workspace, executor = acl.plan_scatter(e.kv_latent_normed, e.latent_cache, e.slot_mapping, e.k_rope, e.rope_cache)
+    assert status == 0 and executor and workspace == 0, acl.last_error()
+    assert lib.aclSetAclOpExecutorRepeatable(executor) == 0
+    # per-layer slices: IR indices 1 and 4 (reference pipeline.hpp:176-184)
+    assert lib.aclSetTensorAddr(executor, 1, e.latent_cache, FAKE + 0x2000000) == 0
+    assert lib.aclSetTensorAddr(executor, 4, e.rope_cache, FAKE + 0xA000000) == 0
+    assert lib.aclSetTensorAddr(executor, 5, e.rope_cache, FAKE) == 161002   # bound as null at plan time
+    assert lib.aclSetTensorAddr(executor, 40, e.rope_cache, FAKE) == 161002  # outside the captured arguments
+    assert lib.aclSetTensorAddr(executor, 1, e.rope_cache, FAKE) == 161002   # shape is frozen after the plan
+    assert lib.aclSetTensorAddr(executor, 1, e.latent_cache, None) == 161001
+    assert lib.aclSetDynamicTensorAddr(executor, 1, 0, e.key_list, FAKE) == 161002  # slot 1 is a tensor, not a list
+    assert lib.aclDestroyAclOpExecutor(executor) == 0
+    assert lib.aclSetAclOpExecutorRepeatable(executor) == 161002
+    # refusals
+    k = e.keep
+    assert acl.plan_scatter(None, e.latent_cache, e.slot_mapping, e.k_rope, e.rope_cache)[0] == 161001
+    slots64 = k.tensor([1], acl.ACL_INT64, FAKE)
+    assert acl.plan_scatter(e.kv_latent_normed, e.latent_cache, slots64, e.k_rope, e.rope_cache)[0] == 161002
+    assert acl.plan_scatter(e.kv_latent_normed, e.latent_cache, e.slot_mapping, e.k_rope, e.rope_cache, cache_mode=b"PA_NZ")[0] == 161002
+    assert acl.plan_scatter(e.kv_latent_normed, e.latent_cache, e.slot_mapping, e.k_rope, e.rope_cache, seq_lens=e.slot_mapping)[0] == 161002
+    assert acl.plan_scatter(e.kv_latent_normed, e.rope_cache, e.slot_mapping, e.k_rope, e.rope_cache)[0] == 161002  # key cache width
+    flat = k.tensor([e.blocks * 64 * 512], acl.ACL_BF16, FAKE)
+    assert acl.plan_scatter(e.kv_latent_normed, flat, e.slot_mapping, e.k_rope, e.rope_cache)[0] == 161002       # not paged
+    status, _, executor = acl.plan_scatter(e.kv_latent_normed, e.latent_cache, e.slot_mapping, e.k_rope, e.rope_cache, cache_mode=None)
+    assert status == 0 and lib.aclDestroyAclOpExecutor(executor) == 0
+    assert acl.plan_scatter(123456, e.latent_cache, e.slot_mapping, e.k_rope, e.rope_cache)[0] == 161002          # stale handle
+
+
+def test_attention_plan_contract_workspace_and_ir_indices():
+    lib = acl.load()
+    e = Engine()
+    status, workspace, executor = e.plan_attention()
+    assert status == 0 and executor, acl.last_error()
+    plan = ffi.AttnPlan()
+    ffi.check(ffi.load().mlakvAttnPlanInit(1, 64, 8192, 64, ffi.DTYPE_BF16, C.byref(plan)))
+    assert plan.max_chunks > 1 and workspace >= plan.workspace_bytes + 4  # split-KV partials + the lengths
+    assert lib.aclSetAclOpExecutorRepeatable(executor) == 0
+    layer_latent, layer_rope = FAKE + 0x3000000, FAKE + 0xB000000
+    assert lib.aclSetDynamicTensorAddr(executor, 1, 0, e.key_list, layer_latent) == 0    # kFiaKeyList
+    assert lib.aclSetDynamicTensorAddr(executor, 2, 0, e.value_list, layer_latent) == 0  # kFiaValueList
+    assert lib.aclSetTensorAddr(executor, 25, e.rope_cache_view, layer_rope) == 0         # kFiaKeyRope
+    assert lib.aclSetTensorAddr(executor, 24, e.q_rope, FAKE + 0x600000) == 0
+    assert lib.aclSetTensorAddr(executor, 22, e.rope_cache_view, layer_rope) == 161002    # the mock's index is not the IR index
+    assert lib.aclSetDynamicTensorAddr(executor, 1, 1, e.key_list, layer_latent) == 161002
+    assert lib.aclSetDynamicTensorAddr(executor, 1, 0, e.value_list, layer_latent) == 161002
+    assert lib.aclnnMlaKvBindSeqLens(executor, FAKE) == 0 and lib.aclnnMlaKvBindSeqLens(executor, None) == 0
+    assert lib.aclDestroyAclOpExecutor(executor) == 0
+    # refusals, each naming the contract it breaks
+    assert e.plan_attention(heads=32)[0] == 161002
+    assert e.plan_attention(scale=0.0)[0] == 161002
+    assert e.plan_attention(layout=b"BSND")[0] == 161002
+    assert e.plan_attention(kv_heads=64)[0] == 161002
+    assert e.plan_attention(block_size=128)[0] == 161002
+    assert e.plan_attention(sparse_mode=4)[0] == 161002
+    assert e.plan_attention(extra={4: e.block_table})[0] == 161002   # an attention mask
+    assert e.plan_attention(extra={12: e.lse})[0] == 161002          # antiquant scale
+    k = e.keep
+    two, _ = k.int_array([5, 6])
+    assert acl.plan_attention(e.q_latent, e.key_list, e.value_list, e.seq_q, two, e.block_table, e.q_rope, e.rope_cache_view, 64,
+                              0.07, 64, e.attn_out)[0] == 161002
+    assert acl.plan_attention(e.q_latent, e.key_list, e.value_list, e.seq_q, None, e.block_table, e.q_rope, e.rope_cache_view, 64,
+                              0.07, 64, e.attn_out)[0] == 161001
+    assert acl.plan_attention(e.q_latent, e.key_list, e.value_list, e.seq_q, e.seq_kv, e.block_table, e.q_rope, e.rope_cache_view,
+                              64, 0.07, 64, e.attn_out, lse=None, lse_flag=True)[0] == 161002
+    status, _, executor = e.plan_attention(lse_flag=True)
+    assert status == 0 and lib.aclDestroyAclOpExecutor(executor) == 0
+    # the failed plans returned no executor (the caller's partial-executor cleanup has nothing to do)
+    assert e.plan_attention(heads=32)[2] is None
+
+
+def test_thin_abi_argument_validation_without_a_device():
+    lib = ffi.load()
+    plan = ffi.AttnPlan()
+    assert lib.mlakvAttnPlanInit(32, 64, 2048, 64, ffi.DTYPE_BF16, C.byref(plan)) == 0
+    assert (plan.chunk_tiles, plan.max_chunks) == (4, 8)  # 256 CUs / 32 sequences
+    assert plan.workspace_bytes == 32 * 8 * 64 * 512 * 4 + 32 * 8 * 64 * 4
+    assert lib.mlakvAttnPlanInit(32, 60, 2048, 64, ffi.DTYPE_BF16, C.byref(plan)) == ffi.ERR_PARAM_INVALID
+    assert lib.mlakvAttnPlanInit(32, 64, 2048, 64, 7, C.byref(plan)) == ffi.ERR_PARAM_INVALID
+    assert lib.mlakvAttnPlanInit(32, 64, 2048, 64, ffi.DTYPE_BF16, None) == ffi.ERR_PARAM_NULLPTR
+    view = ffi.CacheView(latent=FAKE, latent_layer_stride=1 << 20, latent_block_stride=65536, latent_row_stride=1024,
+                         rope=FAKE + (1 << 30), rope_layer_stride=1 << 17, rope_block_stride=8192, rope_row_stride=128,
+                         num_layers=2, num_blocks=16, block_size=64, latent_dim=512, rope_dim=64, dtype=ffi.DTYPE_BF16)
+    assert lib.mlakvAppend(None, 0, 1, FAKE, 0, 1024, FAKE, 0, 128, FAKE, 1, None) == ffi.ERR_PARAM_NULLPTR
+    assert lib.mlakvAppend(C.byref(view), 0, 3, FAKE, 0, 1024, FAKE, 0, 128, FAKE, 1, None) == ffi.ERR_PARAM_INVALID   # layers
+    assert lib.mlakvAppend(C.byref(view), 0, 1, FAKE + 2, 0, 1024, FAKE, 0, 128, FAKE, 1, None) == ffi.ERR_PARAM_INVALID  # alignment
+    assert lib.mlakvAppend(C.byref(view), 0, 1, None, 0, 1024, FAKE, 0, 128, FAKE, 1, None) == ffi.ERR_PARAM_NULLPTR
+    assert lib.mlakvAppend(C.byref(view), 0, 1, FAKE, 0, 1024, FAKE, 0, 128, FAKE, 0, None) == 0                       # nothing to do
+    bad = ffi.CacheView.from_buffer_copy(view)
+    bad.latent_dim = 256
+    assert lib.mlakvGather(C.byref(bad), 0, 1, FAKE, 4, FAKE, FAKE, 1, 64, FAKE, 0, 1024, FAKE, 0, 128, None) == ffi.ERR_PARAM_INVALID
+    assert "512" in ffi.last_error()
+    assert lib.mlakvGather(C.byref(view), 0, 1, FAKE, 1, FAKE, FAKE, 1, 4096, FAKE, 0, 1024, FAKE, 0, 128, None) == ffi.ERR_PARAM_INVALID
+    fp8 = ffi.CacheView.from_buffer_copy(view)
+    fp8.dtype = ffi.DTYPE_FP8_E4M3
+    assert lib.mlakvCopyBlocks(C.byref(fp8), 0, 1, FAKE, 1, None) == ffi.ERR_PARAM_NULLPTR  # FP8 without a scale plane
+
+
+@pytest.mark.skipif(ffi.load().mlakvDeviceCount() > 0, reason="checks the no-device behaviour")
+def test_no_device_fails_loudly_instead_of_falling_back():
+    with pytest.raises(ffi.MlakvError) as info:
+        ffi.Arena(ffi.BACKEND_HIP)
+    assert "no HIP device" in str(info.value)
