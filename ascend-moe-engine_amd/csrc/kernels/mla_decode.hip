@@ -7,9 +7,11 @@
 // as both K (with the 64 rope columns appended) and V.
 //
 // Work decomposition
-//   workgroup = (kv chunk, sequence, group of 64 heads); 4 wavefronts, 16 heads each.
-//   A chunk is `chunk_tiles` tiles of 64 tokens. Tiles are staged in LDS (two buffers of
-//   64 x 1152 B) through registers, one tile ahead of the math.
+//   workgroup = (kv chunk, sequence, group of 64 heads); 4 wavefronts, 16 heads each, one
+//   workgroup per CU. A chunk is `chunk_tiles` tiles of 64 tokens. Two tile buffers in LDS;
+//   bf16 tiles are filled by direct global->LDS loads (global_load_lds_dwordx4: no staging
+//   registers, no ds_write), issued one tile ahead of the math; FP8 tiles are dequantised
+//   to bf16 through registers on their way into LDS.
 //
 // MFMA formulation (v_mfma_f32_16x16x32_bf16; A: lane holds row l%16, k = 8*(l/16)..+7;
 // B: lane holds column l%16, same k; D: lane holds rows 4*(l/16)..+3 of column l%16)
@@ -22,11 +24,18 @@
 //   row-major tile with ds_read_b64_tr_b16 (a 4x16 transpose per 16 lanes), B = P.
 //   So P never leaves registers and the online-softmax statistics of a head live in the
 //   four lanes {h, h+16, h+32, h+48}: two wavefront shuffles per reduction.
+//   Each wavefront is alone on its SIMD, so LDS latency is hidden inside the instruction
+//   stream: operand fragments are fetched eight MFMAs ahead into a second register set.
 //
-// LDS layout: row pitch 1152 B (72 chunks of 16 B), chunk index XORed with
-//   f(token & 7) = ((t & 3) << 1) | (t >> 2): eight consecutive tokens hit eight distinct
-//   16-byte bank groups for the K reads and four consecutive tokens hit four distinct
-//   32-byte groups for the transposed V reads.
+// LDS tile: latent region 64 rows x 1024 B, then rope region 64 rows x 128 B; the 16-byte
+//   chunk index inside a row is XORed with f(token & 7) = ((t & 3) << 1) | (t >> 2): eight
+//   consecutive tokens hit eight distinct 16-byte bank groups for the K reads and four
+//   consecutive tokens hit four distinct 32-byte groups for the transposed V reads. With
+//   direct loads the swizzle is applied on the global side: lane L of a row fetches chunk L ^ f.
+//
+// Online softmax keeps a reference maximum per head and only moves it (rescaling O) when a
+// tile's maximum exceeds it by more than 2^8, so exponentials stay below 256 and most
+// tiles skip the rescale.
 //
 // Chunks of one sequence are merged by a second small kernel from fp32 partials
 // (normalised O and log2-domain LSE) held in the caller's workspace.
@@ -45,132 +54,132 @@ typedef __attribute__((ext_vector_type(2))) unsigned int u32x2;
 typedef __attribute__((ext_vector_type(4))) short s16x4;
 
 constexpr int kThreads = 256;
-constexpr int kRowBytes = (kLatentDim + kRopeDim) * 2;  // 1152
-constexpr int kTileBytes = kTileTokens * kRowBytes;     // 73728
-constexpr int kKSteps = (kLatentDim + kRopeDim) / 32;   // 18
-constexpr int kDvTiles = kLatentDim / 16;               // 32
-constexpr int kLdsBytes = 2 * kTileBytes;
+constexpr int kLatRowBytes = kLatentDim * 2;                 // 1024
+constexpr int kRopeRowBytes = kRopeDim * 2;                  // 128
+constexpr int kLatRegion = kTileTokens * kLatRowBytes;       // 65536
+constexpr int kTileBytes = kLatRegion + kTileTokens * kRopeRowBytes;  // 73728
+constexpr int kKSteps = (kLatentDim + kRopeDim) / 32;        // 18
+constexpr int kDvTiles = kLatentDim / 16;                    // 32
+constexpr int kTableEntries = 2048;                          // block-table entries of one chunk staged in LDS
+constexpr int kLdsBytes = 2 * kTileBytes + kTableEntries * 4;
+constexpr float kRescaleThreshold = 8.0f;                    // log2 domain
 
 __device__ __forceinline__ int Uniform(int v) { return __builtin_amdgcn_readfirstlane(v); }
 __device__ __forceinline__ int Swizzle(int token) {
   const int t = token & 7;
   return ((t & 3) << 1) | (t >> 2);
 }
-__device__ __forceinline__ int LdsOffset(int token, int chunk) { return token * kRowBytes + ((chunk ^ Swizzle(token)) << 4); }
+__device__ __forceinline__ int LatOffset(int token, int chunk) { return token * kLatRowBytes + ((chunk ^ Swizzle(token)) << 4); }
+__device__ __forceinline__ int RopeOffset(int token, int chunk) {
+  return kLatRegion + token * kRopeRowBytes + ((chunk ^ Swizzle(token)) << 4);
+}
 
 __device__ __forceinline__ u32x4 GlobalLoad16(const char* p) { return *reinterpret_cast<const u32x4*>(p); }
+__device__ __forceinline__ void DirectLoad16(const char* global, unsigned char* lds_wave_base) {
+  // Lane L's 16 bytes land at lds_wave_base + 16 * L; lds_wave_base is wave-uniform.
+  __builtin_amdgcn_global_load_lds((const __attribute__((address_space(1))) void*)global,
+                                   (__attribute__((address_space(3))) void*)lds_wave_base, 16, 0, 0);
+}
 
-struct Locator {
-  const int32_t* table_row;
-  int block_size;
-  int block_shift;  // log2(block_size) or -1
-  int num_blocks;
-  // Physical block and in-block slot of token position `pos`; false when the table entry is
-  // outside the pool (such a row is read as zeros rather than faulting).
-  __device__ __forceinline__ bool operator()(int pos, int* block, int* slot) const {
-    int logical;
-    if (block_shift >= 0) {
-      logical = pos >> block_shift;
-      *slot = pos & (block_size - 1);
+// Where the rows of one tile live. Block-table entries of the chunk are staged once in LDS
+// (-1 marks an entry outside the pool), so a tile's row addresses need no dependent global
+// load. ALIGNED (block_size a multiple of 64): the whole tile sits in one physical block.
+template <bool ALIGNED>
+struct TileMap {
+  const int* entries;  // LDS
+  int first_block, block_size, seq_len;
+  int tile_block, tile_slot0;  // ALIGNED only
+
+  __device__ __forceinline__ void Begin(int tile) {
+    if (ALIGNED) {
+      const int pos0 = tile * kTileTokens;
+      const int logical = pos0 / block_size;
+      tile_block = entries[logical - first_block];
+      tile_slot0 = pos0 - logical * block_size;
+    }
+  }
+  // Physical block (clamped to a readable one) and slot of row `r` of tile `tile`; returns
+  // whether the row is real (inside the sequence, behind a valid table entry).
+  __device__ __forceinline__ bool Row(int tile, int r, int* block, int* slot) const {
+    const int pos = tile * kTileTokens + r;
+    if (ALIGNED) {
+      *block = tile_block < 0 ? 0 : tile_block;
+      *slot = pos < seq_len ? tile_slot0 + r : 0;
+      return pos < seq_len && tile_block >= 0;
+    }
+    const int clamped = pos < seq_len ? pos : seq_len - 1;
+    const int logical = clamped / block_size;
+    const int entry = entries[logical - first_block];
+    *block = entry < 0 ? 0 : entry;
+    *slot = clamped - logical * block_size;
+    return pos < seq_len && entry >= 0;
+  }
+};
+
+// ---- bf16 tiles: direct global -> LDS ----------------------------------------------------
+
+template <bool ALIGNED>
+__device__ __forceinline__ void IssueTileBf16(const AttnArgs& a, TileMap<ALIGNED>& map, int tile, unsigned char* buf, int tid) {
+  const int lane = tid & 63, wave = Uniform(tid >> 6);
+  map.Begin(tile);
+  int block[16], slot[16];
+  bool real[16];
+#pragma unroll
+  for (int i = 0; i < 16; ++i) real[i] = map.Row(tile, wave + 4 * i, &block[i], &slot[i]);
+#pragma unroll
+  for (int i = 0; i < 16; ++i) {
+    const int row = wave + 4 * i;  // wave-uniform
+    unsigned char* dst = buf + row * kLatRowBytes;
+    if (real[i]) {
+      const char* src = a.latent.base + Uniform(block[i]) * a.latent.block_stride + Uniform(slot[i]) * a.latent.row_stride;
+      DirectLoad16(src + ((lane ^ Swizzle(row)) << 4), dst);
     } else {
-      logical = pos / block_size;
-      *slot = pos - logical * block_size;
+      *reinterpret_cast<u32x4*>(dst + lane * 16) = u32x4{0u, 0u, 0u, 0u};
     }
-    *block = table_row[logical];
-    return static_cast<unsigned>(*block) < static_cast<unsigned>(num_blocks);
   }
-};
-
-// ---- tile staging: global -> registers -> LDS -------------------------------------
-
-// bf16 rows: 16 latent chunks + 2 rope chunks of 16 B per thread.
-struct TileRegsBf16 {
-  u32x4 v[18];
-};
-
-__device__ __forceinline__ void LoadTile(TileRegsBf16& r, const AttnArgs& a, const Locator& locate, int tile, int seq_len,
-                                         int tid) {
-  const int lane = tid & 63, wave = tid >> 6;
-  const int pos0 = tile * kTileTokens;
-#pragma unroll
-  for (int i = 0; i < 16; ++i) {
-    const int token = wave + 4 * i;  // wave-uniform
-    const int pos = pos0 + token;
-    u32x4 v = {0u, 0u, 0u, 0u};
-    int block, slot;
-    if (pos < seq_len && locate(pos, &block, &slot)) {
-      block = Uniform(block);
-      v = GlobalLoad16(a.latent.base + block * a.latent.block_stride + slot * a.latent.row_stride + lane * 16);
-    }
-    r.v[i] = v;
-  }
+  // rope: one wave access covers 8 rows x 128 B
 #pragma unroll
   for (int i = 0; i < 2; ++i) {
-    const int idx = tid + kThreads * i;
-    const int token = idx >> 3, chunk = idx & 7;
-    const int pos = pos0 + token;
-    u32x4 v = {0u, 0u, 0u, 0u};
-    int block, slot;
-    if (pos < seq_len && locate(pos, &block, &slot)) {
-      v = GlobalLoad16(a.rope.base + block * a.rope.block_stride + slot * a.rope.row_stride + chunk * 16);
+    const int group = wave + 4 * i;  // wave-uniform: rows 8*group .. 8*group+7
+    const int row = 8 * group + (lane >> 3);
+    int rblock, rslot;
+    const bool rreal = map.Row(tile, row, &rblock, &rslot);
+    unsigned char* dst = buf + kLatRegion + group * 8 * kRopeRowBytes;
+    if (rreal) {
+      const char* src = a.rope.base + rblock * a.rope.block_stride + rslot * a.rope.row_stride;
+      DirectLoad16(src + (((lane & 7) ^ Swizzle(row)) << 4), dst);
+    } else {
+      *reinterpret_cast<u32x4*>(dst + lane * 16) = u32x4{0u, 0u, 0u, 0u};
     }
-    r.v[16 + i] = v;
   }
 }
 
-__device__ __forceinline__ void StoreTile(const TileRegsBf16& r, unsigned char* buf, int tid) {
-  const int lane = tid & 63, wave = tid >> 6;
-#pragma unroll
-  for (int i = 0; i < 16; ++i) {
-    const int token = wave + 4 * i;
-    *reinterpret_cast<u32x4*>(buf + LdsOffset(token, lane)) = r.v[i];
-  }
-#pragma unroll
-  for (int i = 0; i < 2; ++i) {
-    const int idx = tid + kThreads * i;
-    const int token = idx >> 3, chunk = 64 + (idx & 7);
-    *reinterpret_cast<u32x4*>(buf + LdsOffset(token, chunk)) = r.v[16 + i];
-  }
-}
+// ---- FP8 tiles: global -> registers -> (dequantise) -> LDS ------------------------------------
 
-// FP8 rows: 8 latent chunks + 1 rope chunk of 16 codes per thread, and their row scales.
+// 8 latent chunks + 1 rope chunk of 16 codes per thread, and their row scales (0 for a row
+// that is not real).
 struct TileRegsFp8 {
   u32x4 v[9];
   float scale[9];
 };
 
-__device__ __forceinline__ void LoadTile(TileRegsFp8& r, const AttnArgs& a, const Locator& locate, int tile, int seq_len,
-                                         int tid) {
-  const int pos0 = tile * kTileTokens;
+template <bool ALIGNED>
+__device__ __forceinline__ void LoadTileFp8(TileRegsFp8& r, const AttnArgs& a, TileMap<ALIGNED>& map, int tile, int tid) {
+  map.Begin(tile);
+  int block[9], slot[9];
+  bool real[9];
 #pragma unroll
   for (int i = 0; i < 9; ++i) {
-    int token, chunk;
-    const char* base;
-    int64_t block_stride, row_stride;
-    if (i < 8) {
-      const int idx = tid + kThreads * i;
-      token = idx >> 5;
-      chunk = idx & 31;
-      base = a.latent.base;
-      block_stride = a.latent.block_stride;
-      row_stride = a.latent.row_stride;
-    } else {
-      token = tid >> 2;
-      chunk = tid & 3;
-      base = a.rope.base;
-      block_stride = a.rope.block_stride;
-      row_stride = a.rope.row_stride;
-    }
-    const int pos = pos0 + token;
-    u32x4 v = {0u, 0u, 0u, 0u};
-    float scale = 0.0f;
-    int block, slot;
-    if (pos < seq_len && locate(pos, &block, &slot)) {
-      v = GlobalLoad16(base + block * block_stride + slot * row_stride + chunk * 16);
-      scale = reinterpret_cast<const float*>(a.scale.base + block * a.scale.block_stride)[slot];
-    }
-    r.v[i] = v;
-    r.scale[i] = scale;
+    const int token = i < 8 ? (tid + kThreads * i) >> 5 : tid >> 2;
+    real[i] = map.Row(tile, token, &block[i], &slot[i]);
+  }
+#pragma unroll
+  for (int i = 0; i < 9; ++i) {
+    const int chunk = i < 8 ? (tid + kThreads * i) & 31 : tid & 3;
+    const Plane& plane = i < 8 ? a.latent : a.rope;
+    r.v[i] = GlobalLoad16(plane.base + block[i] * plane.block_stride + slot[i] * plane.row_stride + chunk * 16);
+    const float scale = reinterpret_cast<const float*>(a.scale.base + block[i] * a.scale.block_stride)[slot[i]];
+    r.scale[i] = real[i] ? scale : 0.0f;
   }
 }
 
@@ -187,18 +196,9 @@ __device__ __forceinline__ void Dequant4(unsigned int codes, float scale, unsign
   *hi = PackBf16(b.x * scale, b.y * scale);
 }
 
-__device__ __forceinline__ void StoreTile(const TileRegsFp8& r, unsigned char* buf, int tid) {
+__device__ __forceinline__ void StoreTileFp8(const TileRegsFp8& r, unsigned char* buf, int tid) {
 #pragma unroll
   for (int i = 0; i < 9; ++i) {
-    int token, chunk;  // chunk: index of the first of two 16-byte bf16 chunks
-    if (i < 8) {
-      const int idx = tid + kThreads * i;
-      token = idx >> 5;
-      chunk = 2 * (idx & 31);
-    } else {
-      token = tid >> 2;
-      chunk = 64 + 2 * (tid & 3);
-    }
     u32x4 first, second;
     unsigned int lo, hi;
     Dequant4(r.v[i].x, r.scale[i], &lo, &hi);
@@ -213,23 +213,26 @@ __device__ __forceinline__ void StoreTile(const TileRegsFp8& r, unsigned char* b
     Dequant4(r.v[i].w, r.scale[i], &lo, &hi);
     second.z = lo;
     second.w = hi;
-    *reinterpret_cast<u32x4*>(buf + LdsOffset(token, chunk)) = first;
-    *reinterpret_cast<u32x4*>(buf + LdsOffset(token, chunk + 1)) = second;
+    if (r.scale[i] == 0.0f) {  // not a real row: zeros, whatever the fetched codes were
+      first = u32x4{0u, 0u, 0u, 0u};
+      second = first;
+    }
+    if (i < 8) {
+      const int idx = tid + kThreads * i;
+      const int token = idx >> 5, chunk = 2 * (idx & 31);
+      *reinterpret_cast<u32x4*>(buf + LatOffset(token, chunk)) = first;
+      *reinterpret_cast<u32x4*>(buf + LatOffset(token, chunk + 1)) = second;
+    } else {
+      const int token = tid >> 2, chunk = 2 * (tid & 3);
+      *reinterpret_cast<u32x4*>(buf + RopeOffset(token, chunk)) = first;
+      *reinterpret_cast<u32x4*>(buf + RopeOffset(token, chunk + 1)) = second;
+    }
   }
 }
 
-template <bool FP8>
-struct TileRegsFor {
-  using type = TileRegsBf16;
-};
-template <>
-struct TileRegsFor<true> {
-  using type = TileRegsFp8;
-};
-
 // ---- main kernel -------------------------------------------------------------------
 
-template <bool FP8>
+template <bool FP8, bool ALIGNED>
 __global__ __launch_bounds__(kThreads, 1) void MlaDecodeKernel(AttnArgs a) {
   extern __shared__ __attribute__((aligned(16))) unsigned char lds[];
   const int tid = threadIdx.x;
@@ -255,11 +258,23 @@ __global__ __launch_bounds__(kThreads, 1) void MlaDecodeKernel(AttnArgs a) {
   }
   const int tile_end = min(tile_begin + a.chunk_tiles, num_tiles);
 
-  Locator locate;
-  locate.table_row = a.block_table + static_cast<int64_t>(seq) * a.table_stride;
-  locate.block_size = a.block_size;
-  locate.block_shift = (a.block_size & (a.block_size - 1)) == 0 ? __builtin_ctz(a.block_size) : -1;
-  locate.num_blocks = a.num_blocks;
+  // Stage this chunk's block-table entries in LDS.
+  int* table_lds = reinterpret_cast<int*>(lds + 2 * kTileBytes);
+  TileMap<ALIGNED> map;
+  map.entries = table_lds;
+  map.block_size = a.block_size;
+  map.seq_len = seq_len;
+  {
+    const int first_pos = tile_begin * kTileTokens;
+    const int last_pos = min(tile_end * kTileTokens, seq_len) - 1;
+    map.first_block = first_pos / a.block_size;
+    const int count = last_pos / a.block_size - map.first_block + 1;  // <= kTableEntries, ensured by the plan
+    const int32_t* table_row = a.block_table + static_cast<int64_t>(seq) * a.table_stride + map.first_block;
+    for (int i = tid; i < count; i += kThreads) {
+      const int entry = table_row[i];
+      table_lds[i] = static_cast<unsigned>(entry) < static_cast<unsigned>(a.num_blocks) ? entry : -1;
+    }
+  }
 
   // Q fragments: lane (head i16, k-group g) holds Q[head][32*ks + 8g .. +7].
   bf16x8 q[kKSteps];
@@ -277,51 +292,76 @@ __global__ __launch_bounds__(kThreads, 1) void MlaDecodeKernel(AttnArgs a) {
   f32x4 o[kDvTiles];
 #pragma unroll
   for (int n = 0; n < kDvTiles; ++n) o[n] = f32x4{0.f, 0.f, 0.f, 0.f};
-  float m_run = -__builtin_inff();  // running max, log2 domain (scores * scale * log2 e)
+  float m_ref = -__builtin_inff();  // reference maximum of the exponentials, log2 domain
   float l_run = 0.0f;               // this lane's share of the running denominator
 
   // Lane-constant LDS offsets.
-  const int swk = Swizzle(i16);                  // K reads: token = 16t + i16
-  const int k_lane = i16 * kRowBytes;
+  const int swk = Swizzle(i16);  // K reads: token = 16t + i16
   const int k_e0 = ((g ^ swk) << 4), k_e1 = (((4 + g) ^ swk) << 4);
-  const int v_row = 4 * g + (i16 >> 2);          // V reads: token = 32u + (16) + 4g + i16/4
+  const int k_lat = i16 * kLatRowBytes, k_rope = kLatRegion + i16 * kRopeRowBytes;
+  const int v_row = 4 * g + (i16 >> 2);  // V reads: token = 32u (+16) + 4g + i16/4
   const int swv = Swizzle(v_row);
   const int v_c1 = (i16 & 3) >> 1;
-  const int v_lane = v_row * kRowBytes + (i16 & 1) * 8;
+  const int v_lane = v_row * kLatRowBytes + (i16 & 1) * 8;
   int v_e[4];
 #pragma unroll
   for (int j = 0; j < 4; ++j) v_e[j] = (((2 * j + v_c1) ^ swv) << 4);
 
-  typename TileRegsFor<FP8>::type regs;
-  LoadTile(regs, a, locate, tile_begin, seq_len, tid);
-  StoreTile(regs, lds, tid);
-  if (tile_begin + 1 < tile_end) LoadTile(regs, a, locate, tile_begin + 1, seq_len, tid);
+  __syncthreads();  // table entries visible
+  TileRegsFp8 regs;
+  if (FP8) {
+    LoadTileFp8(regs, a, map, tile_begin, tid);
+    StoreTileFp8(regs, lds, tid);
+    if (tile_begin + 1 < tile_end) LoadTileFp8(regs, a, map, tile_begin + 1, tid);
+  } else {
+    IssueTileBf16(a, map, tile_begin, lds, tid);
+    asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+  }
   __syncthreads();
 
   for (int tile = tile_begin; tile < tile_end; ++tile) {
     unsigned char* cur = lds + ((tile - tile_begin) & 1) * kTileBytes;
     unsigned char* nxt = lds + (((tile - tile_begin) & 1) ^ 1) * kTileBytes;
 
+    // The other buffer was last read before the barrier that ended the previous iteration.
+    if (!FP8 && tile + 1 < tile_end) IssueTileBf16(a, map, tile + 1, nxt, tid);
+
     f32x4 s[4];
     if (active) {
+      // ---- S^T = K Q^T, K fragments fetched eight MFMAs (two k-steps) ahead ----
 #pragma unroll
       for (int t = 0; t < 4; ++t) s[t] = f32x4{0.f, 0.f, 0.f, 0.f};
+      bf16x8 kb[2][8];
+      const auto load_k = [&](bf16x8* dst, int pair) {
 #pragma unroll
-      for (int ks = 0; ks < kKSteps; ++ks) {
-        const int e = (ks & 1) ? k_e1 : k_e0;
+        for (int kk = 0; kk < 2; ++kk) {
+          const int ks = 2 * pair + kk;
+          const int e = kk ? k_e1 : k_e0;  // ks & 1 == kk
+          const int base = ks < 16 ? k_lat + (ks >> 1) * 128 + e : k_rope + e;
+          const int row_pitch = ks < 16 ? kLatRowBytes : kRopeRowBytes;
 #pragma unroll
-        for (int t = 0; t < 4; ++t) {
-          const bf16x8 kf = *reinterpret_cast<const bf16x8*>(cur + k_lane + t * 16 * kRowBytes + (ks >> 1) * 128 + e);
-          s[t] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(kf, q[ks], s[t], 0, 0, 0);
+          for (int t = 0; t < 4; ++t) dst[kk * 4 + t] = *reinterpret_cast<const bf16x8*>(cur + base + t * 16 * row_pitch);
         }
+      };
+      load_k(kb[0], 0);
+#pragma unroll
+      for (int pair = 0; pair < kKSteps / 2; ++pair) {
+        if (pair + 1 < kKSteps / 2) load_k(kb[(pair + 1) & 1], pair + 1);
+        __builtin_amdgcn_sched_barrier(0);
+#pragma unroll
+        for (int kk = 0; kk < 2; ++kk) {
+#pragma unroll
+          for (int t = 0; t < 4; ++t) {
+            s[t] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(kb[pair & 1][kk * 4 + t], q[2 * pair + kk], s[t], 0, 0, 0);
+          }
+        }
+        __builtin_amdgcn_sched_barrier(0);
       }
     }
 
-    // Stage the next tile while the scores are reduced. Its buffer was last read before the
-    // barrier that ended the previous iteration.
-    if (tile + 1 < tile_end) {
-      StoreTile(regs, nxt, tid);
-      if (tile + 2 < tile_end) LoadTile(regs, a, locate, tile + 2, seq_len, tid);
+    if (FP8 && tile + 1 < tile_end) {
+      StoreTileFp8(regs, nxt, tid);
+      if (tile + 2 < tile_end) LoadTileFp8(regs, a, map, tile + 2, tid);
     }
 
     if (active) {
@@ -340,49 +380,56 @@ __global__ __launch_bounds__(kThreads, 1) void MlaDecodeKernel(AttnArgs a) {
       }
       tile_max = fmaxf(tile_max, __shfl_xor(tile_max, 16));
       tile_max = fmaxf(tile_max, __shfl_xor(tile_max, 32));
-      const float m_new = fmaxf(m_run, tile_max);  // finite: token 0 of the tile is valid
-      const float alpha = __builtin_amdgcn_exp2f(m_run - m_new);
+      // Move the reference only when some head's maximum outgrew it by more than the threshold.
+      if (__builtin_amdgcn_ballot_w64(tile_max > m_ref + kRescaleThreshold) != 0) {
+        const float m_new = fmaxf(m_ref, tile_max);  // finite: token 0 of the tile is valid
+        const float alpha = __builtin_amdgcn_exp2f(m_ref - m_new);
+        l_run *= alpha;
+        m_ref = m_new;
+#pragma unroll
+        for (int n = 0; n < kDvTiles; ++n) o[n] *= alpha;
+      }
       float row_sum = 0.0f;
+      bf16x8 p[2];
 #pragma unroll
       for (int t = 0; t < 4; ++t) {
 #pragma unroll
         for (int j = 0; j < 4; ++j) {
-          const float p = __builtin_amdgcn_exp2f(s[t][j] - m_new);
-          s[t][j] = p;
-          row_sum += p;
+          const float e = __builtin_amdgcn_exp2f(s[t][j] - m_ref);
+          row_sum += e;
+          p[t >> 1][(t & 1) * 4 + j] = static_cast<__bf16>(e);
         }
       }
-      l_run = l_run * alpha + row_sum;
-      m_run = m_new;
-      if (__builtin_amdgcn_ballot_w64(alpha != 1.0f) != 0) {
-#pragma unroll
-        for (int n = 0; n < kDvTiles; ++n) o[n] *= alpha;
-      }
+      l_run += row_sum;
 
-      // ---- O^T += V^T P ----
+      // ---- O^T += V^T P, V fragments fetched eight MFMAs ahead ----
+      bf16x8 vb[2][8];
+      const auto load_v = [&](bf16x8* dst, int group) {  // group: u = group / 4, n = 8 * (group % 4) .. +7
+        const unsigned char* vbase = cur + v_lane + (group >> 2) * 32 * kLatRowBytes;
 #pragma unroll
-      for (int u = 0; u < 2; ++u) {
-        bf16x8 p;
-#pragma unroll
-        for (int j = 0; j < 4; ++j) {
-          p[j] = static_cast<__bf16>(s[2 * u][j]);
-          p[4 + j] = static_cast<__bf16>(s[2 * u + 1][j]);
-        }
-        const unsigned char* vbase = cur + v_lane + u * 32 * kRowBytes;
-#pragma unroll
-        for (int n = 0; n < kDvTiles; ++n) {
+        for (int j = 0; j < 8; ++j) {
+          const int n = 8 * (group & 3) + j;
           const unsigned char* addr = vbase + (n >> 2) * 128 + v_e[n & 3];
-          const s16x4 lo = __builtin_amdgcn_ds_read_tr16_b64_v4i16(
-              (__attribute__((address_space(3))) s16x4*)(addr));
+          const s16x4 lo = __builtin_amdgcn_ds_read_tr16_b64_v4i16((__attribute__((address_space(3))) s16x4*)(addr));
           const s16x4 hi = __builtin_amdgcn_ds_read_tr16_b64_v4i16(
-              (__attribute__((address_space(3))) s16x4*)(addr + 16 * kRowBytes));
-          const bf16x4 lo_b = __builtin_bit_cast(bf16x4, lo);
-          const bf16x4 hi_b = __builtin_bit_cast(bf16x4, hi);
-          const bf16x8 vf = __builtin_shufflevector(lo_b, hi_b, 0, 1, 2, 3, 4, 5, 6, 7);
-          o[n] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(vf, p, o[n], 0, 0, 0);
+              (__attribute__((address_space(3))) s16x4*)(addr + 16 * kLatRowBytes));
+          dst[j] = __builtin_shufflevector(__builtin_bit_cast(bf16x4, lo), __builtin_bit_cast(bf16x4, hi), 0, 1, 2, 3, 4, 5, 6, 7);
         }
+      };
+      load_v(vb[0], 0);
+#pragma unroll
+      for (int group = 0; group < 8; ++group) {
+        if (group + 1 < 8) load_v(vb[(group + 1) & 1], group + 1);
+        __builtin_amdgcn_sched_barrier(0);
+#pragma unroll
+        for (int j = 0; j < 8; ++j) {
+          const int n = 8 * (group & 3) + j;
+          o[n] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(vb[group & 1][j], p[group >> 2], o[n], 0, 0, 0);
+        }
+        __builtin_amdgcn_sched_barrier(0);
       }
     }
+    if (!FP8) asm volatile("s_waitcnt vmcnt(0)" ::: "memory");  // the next tile has landed in LDS
     __syncthreads();
   }
 
@@ -390,7 +437,7 @@ __global__ __launch_bounds__(kThreads, 1) void MlaDecodeKernel(AttnArgs a) {
   float l_total = l_run + __shfl_xor(l_run, 16);
   l_total += __shfl_xor(l_total, 32);
   const float inv = 1.0f / l_total;
-  const float lse2 = m_run + __builtin_amdgcn_logf(l_total);  // v_log_f32 is log2
+  const float lse2 = m_ref + __builtin_amdgcn_logf(l_total);  // v_log_f32 is log2
   if (direct) {
     char* out = a.out + seq * a.out_seq_stride + head * a.out_head_stride;
 #pragma unroll
@@ -444,25 +491,27 @@ __global__ __launch_bounds__(128) void MlaCombineKernel(AttnArgs a) {
   if (a.lse != nullptr && tid == 0) a.lse[seq * a.heads + head] = (m + __builtin_amdgcn_logf(denom)) * 0.6931471805599453f;
 }
 
+template <bool FP8, bool ALIGNED>
+hipError_t Launch(const AttnArgs& args, const dim3& grid, hipStream_t stream) {
+  // Dynamic LDS above 64 KB needs the attribute once per kernel and process.
+  static const hipError_t prepared = hipFuncSetAttribute(reinterpret_cast<const void*>(&MlaDecodeKernel<FP8, ALIGNED>),
+                                                         hipFuncAttributeMaxDynamicSharedMemorySize, kLdsBytes);
+  if (prepared != hipSuccess) return prepared;
+  hipLaunchKernelGGL((MlaDecodeKernel<FP8, ALIGNED>), grid, dim3(kThreads), kLdsBytes, stream, args);
+  return hipGetLastError();
+}
+
 }  // namespace
 
-hipError_t PrepareAttnKernels() {
-  hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(&MlaDecodeKernel<false>),
-                                     hipFuncAttributeMaxDynamicSharedMemorySize, kLdsBytes);
-  if (e != hipSuccess) return e;
-  return hipFuncSetAttribute(reinterpret_cast<const void*>(&MlaDecodeKernel<true>),
-                             hipFuncAttributeMaxDynamicSharedMemorySize, kLdsBytes);
-}
+hipError_t PrepareAttnKernels() { return hipSuccess; }
 
 hipError_t LaunchAttnDecode(const AttnArgs& args, hipStream_t stream) {
   if (args.batch <= 0) return hipSuccess;
   const dim3 grid(args.max_chunks, args.batch, (args.heads + 63) / 64);
-  if (args.fp8) {
-    hipLaunchKernelGGL(MlaDecodeKernel<true>, grid, dim3(kThreads), kLdsBytes, stream, args);
-  } else {
-    hipLaunchKernelGGL(MlaDecodeKernel<false>, grid, dim3(kThreads), kLdsBytes, stream, args);
-  }
-  hipError_t e = hipGetLastError();
+  const bool aligned = args.block_size % kTileTokens == 0;
+  hipError_t e;
+  if (args.fp8) e = aligned ? Launch<true, true>(args, grid, stream) : Launch<true, false>(args, grid, stream);
+  else e = aligned ? Launch<false, true>(args, grid, stream) : Launch<false, false>(args, grid, stream);
   if (e != hipSuccess) return e;
   if (args.max_chunks > 1) {
     hipLaunchKernelGGL(MlaCombineKernel, dim3(args.heads, args.batch), dim3(128), 0, stream, args);

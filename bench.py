@@ -40,6 +40,7 @@ def parse_args():
     p.add_argument("--warmup", type=int, default=5)
     p.add_argument("--no-cpu-baseline", action="store_true")
     p.add_argument("--no-attention", action="store_true")
+    p.add_argument("--attention-only", action="store_true", help="development aid: time only the attention configurations")
     p.add_argument("--split-out", action="store_true", help="gather into separate latent/rope planes instead of 576-wide rows")
     return p.parse_args()
 
@@ -292,6 +293,10 @@ def main():
     calib_dst.copy_(calib_src)
     torch.cuda.synchronize()
     del calib_src, calib_dst
+    if args.attention_only:
+        print(json.dumps({"attention": bench_attention(args, torch, np, ffi),
+                          "attention_fp8": bench_attention(args, torch, np, ffi, fp8=True, batch=64, ctx=4352, iters=64)}))
+        return 0
     ag = bench_append_gather(args, torch, np, ffi)
     line = {
         "metric": "paged-KV append+gather GB/s; MLA decode attn us/step (% HBM roofline)",
