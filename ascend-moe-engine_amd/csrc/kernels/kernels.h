@@ -82,6 +82,7 @@ struct AttnArgs {
   int32_t block_size;
   int32_t chunk_tiles;
   int32_t max_chunks;
+  int32_t debug;  // development switches, 0 in production
   bool fp8;
 };
 

@@ -39,6 +39,8 @@
 //
 // Chunks of one sequence are merged by a second small kernel from fp32 partials
 // (normalised O and log2-domain LSE) held in the caller's workspace.
+#include <cstdlib>
+
 #include "kernels.h"
 
 namespace mlakv {
@@ -65,13 +67,16 @@ constexpr int kLdsBytes = 2 * kTileBytes + kTableEntries * 4;
 constexpr float kRescaleThreshold = 8.0f;                    // log2 domain
 
 __device__ __forceinline__ int Uniform(int v) { return __builtin_amdgcn_readfirstlane(v); }
-__device__ __forceinline__ int Swizzle(int token) {
-  const int t = token & 7;
-  return ((t & 3) << 1) | (t >> 2);
-}
-__device__ __forceinline__ int LatOffset(int token, int chunk) { return token * kLatRowBytes + ((chunk ^ Swizzle(token)) << 4); }
+// LDS is 64 banks x 4 B (256 B per clock): a ds_read_b128 serves 16 lanes per clock, a
+// ds_read_b64_tr_b16 32 lanes. Latent rows (1024 B): the chunk index is XORed with a 4-bit
+// function of the token so that 16 consecutive tokens land in 16 distinct 16-byte slots (K
+// reads) and 8 consecutive tokens in 8 distinct 32-byte slots (transposed V reads). Rope rows
+// (128 B, two per 256 B): 3-bit XOR by token/2.
+__device__ __forceinline__ int SwizzleLat(int token) { return ((token & 7) << 1) | ((token >> 3) & 1); }
+__device__ __forceinline__ int SwizzleRope(int token) { return (token >> 1) & 7; }
+__device__ __forceinline__ int LatOffset(int token, int chunk) { return token * kLatRowBytes + ((chunk ^ SwizzleLat(token)) << 4); }
 __device__ __forceinline__ int RopeOffset(int token, int chunk) {
-  return kLatRegion + token * kRopeRowBytes + ((chunk ^ Swizzle(token)) << 4);
+  return kLatRegion + token * kRopeRowBytes + ((chunk ^ SwizzleRope(token)) << 4);
 }
 
 __device__ __forceinline__ u32x4 GlobalLoad16(const char* p) { return *reinterpret_cast<const u32x4*>(p); }
@@ -118,10 +123,34 @@ struct TileMap {
 
 // ---- bf16 tiles: direct global -> LDS ----------------------------------------------------
 
+// Lane-constant byte offsets of the chunk a lane fetches for the rows its wave owns: a wave
+// owns latent rows w, w+4, ... (16 of them; row & 15 takes four values) and rope row groups w, w+4.
+struct IssueLane {
+  int lat[4];   // latent rows with (row >> 2) & 3 == j
+  int rope[2];  // rope groups w and w + 4
+};
+
 template <bool ALIGNED>
-__device__ __forceinline__ void IssueTileBf16(const AttnArgs& a, TileMap<ALIGNED>& map, int tile, unsigned char* buf, int tid) {
+__device__ __forceinline__ void IssueTileBf16(const AttnArgs& a, TileMap<ALIGNED>& map, const IssueLane& il, int tile,
+                                              unsigned char* buf, int tid) {
   const int lane = tid & 63, wave = Uniform(tid >> 6);
   map.Begin(tile);
+  const int rows = map.seq_len - tile * kTileTokens;  // real rows in this tile, >= 1
+  if (ALIGNED && rows >= kTileTokens && map.tile_block >= 0) {
+    // The whole tile is real and sits in one physical block: uniform base + row pitch.
+    const int block = Uniform(map.tile_block), slot0 = Uniform(map.tile_slot0);
+    const char* latent = a.latent.base + block * a.latent.block_stride + (slot0 + wave) * a.latent.row_stride;
+    const int64_t pitch = 4 * a.latent.row_stride;
+#pragma unroll
+    for (int i = 0; i < 16; ++i) DirectLoad16(latent + i * pitch + il.lat[i & 3], buf + (wave + 4 * i) * kLatRowBytes);
+    const char* rope = a.rope.base + block * a.rope.block_stride + (slot0 + (lane >> 3)) * a.rope.row_stride;
+#pragma unroll
+    for (int i = 0; i < 2; ++i) {
+      const int group = wave + 4 * i;
+      DirectLoad16(rope + group * 8 * a.rope.row_stride + il.rope[i], buf + kLatRegion + group * 8 * kRopeRowBytes);
+    }
+    return;
+  }
   int block[16], slot[16];
   bool real[16];
 #pragma unroll
@@ -132,7 +161,7 @@ __device__ __forceinline__ void IssueTileBf16(const AttnArgs& a, TileMap<ALIGNED
     unsigned char* dst = buf + row * kLatRowBytes;
     if (real[i]) {
       const char* src = a.latent.base + Uniform(block[i]) * a.latent.block_stride + Uniform(slot[i]) * a.latent.row_stride;
-      DirectLoad16(src + ((lane ^ Swizzle(row)) << 4), dst);
+      DirectLoad16(src + il.lat[i & 3], dst);
     } else {
       *reinterpret_cast<u32x4*>(dst + lane * 16) = u32x4{0u, 0u, 0u, 0u};
     }
@@ -147,7 +176,7 @@ __device__ __forceinline__ void IssueTileBf16(const AttnArgs& a, TileMap<ALIGNED
     unsigned char* dst = buf + kLatRegion + group * 8 * kRopeRowBytes;
     if (rreal) {
       const char* src = a.rope.base + rblock * a.rope.block_stride + rslot * a.rope.row_stride;
-      DirectLoad16(src + (((lane & 7) ^ Swizzle(row)) << 4), dst);
+      DirectLoad16(src + il.rope[i], dst);
     } else {
       *reinterpret_cast<u32x4*>(dst + lane * 16) = u32x4{0u, 0u, 0u, 0u};
     }
@@ -296,16 +325,28 @@ __global__ __launch_bounds__(kThreads, 1) void MlaDecodeKernel(AttnArgs a) {
   float l_run = 0.0f;               // this lane's share of the running denominator
 
   // Lane-constant LDS offsets.
-  const int swk = Swizzle(i16);  // K reads: token = 16t + i16
-  const int k_e0 = ((g ^ swk) << 4), k_e1 = (((4 + g) ^ swk) << 4);
+  // K reads: token = 16t + i16, chunk = 4 ks + g (latent, ks < 16) or 4 (ks - 16) + g (rope).
   const int k_lat = i16 * kLatRowBytes, k_rope = kLatRegion + i16 * kRopeRowBytes;
-  const int v_row = 4 * g + (i16 >> 2);  // V reads: token = 32u (+16) + 4g + i16/4
-  const int swv = Swizzle(v_row);
-  const int v_c1 = (i16 & 3) >> 1;
-  const int v_lane = v_row * kLatRowBytes + (i16 & 1) * 8;
-  int v_e[4];
+  int k_e[4], kr_e[2];
 #pragma unroll
-  for (int j = 0; j < 4; ++j) v_e[j] = (((2 * j + v_c1) ^ swv) << 4);
+  for (int j = 0; j < 4; ++j) k_e[j] = ((4 * j + g) ^ SwizzleLat(i16)) << 4;
+#pragma unroll
+  for (int j = 0; j < 2; ++j) kr_e[j] = ((4 * j + g) ^ SwizzleRope(i16)) << 4;
+  // V reads: token = 32u (+16) + 4g + i16/4, chunk = 2n + (i16 & 3) / 2, 8-byte half i16 & 1.
+  const int v_row = 4 * g + (i16 >> 2);
+  const int v_lane = v_row * kLatRowBytes + (i16 & 1) * 8;
+  int v_e[8];
+#pragma unroll
+  for (int j = 0; j < 8; ++j) v_e[j] = ((2 * j + ((i16 & 3) >> 1)) ^ SwizzleLat(v_row)) << 4;
+  // Direct loads: lane L of a latent row fetches chunk L ^ swizzle(row); rows of this wave.
+  IssueLane il;
+  {
+    const int w = Uniform(tid >> 6);
+#pragma unroll
+    for (int j = 0; j < 4; ++j) il.lat[j] = (lane ^ SwizzleLat(w + 4 * j)) << 4;
+#pragma unroll
+    for (int j = 0; j < 2; ++j) il.rope[j] = ((lane & 7) ^ SwizzleRope(8 * (w + 4 * j) + (lane >> 3))) << 4;
+  }
 
   __syncthreads();  // table entries visible
   TileRegsFp8 regs;
@@ -314,7 +355,7 @@ __global__ __launch_bounds__(kThreads, 1) void MlaDecodeKernel(AttnArgs a) {
     StoreTileFp8(regs, lds, tid);
     if (tile_begin + 1 < tile_end) LoadTileFp8(regs, a, map, tile_begin + 1, tid);
   } else {
-    IssueTileBf16(a, map, tile_begin, lds, tid);
+    IssueTileBf16(a, map, il, tile_begin, lds, tid);
     asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
   }
   __syncthreads();
@@ -324,10 +365,10 @@ __global__ __launch_bounds__(kThreads, 1) void MlaDecodeKernel(AttnArgs a) {
     unsigned char* nxt = lds + (((tile - tile_begin) & 1) ^ 1) * kTileBytes;
 
     // The other buffer was last read before the barrier that ended the previous iteration.
-    if (!FP8 && tile + 1 < tile_end) IssueTileBf16(a, map, tile + 1, nxt, tid);
+    if (!FP8 && tile + 1 < tile_end && !(a.debug & 8)) IssueTileBf16(a, map, il, tile + 1, nxt, tid);
 
     f32x4 s[4];
-    if (active) {
+    if (active && !(a.debug & 1)) {
       // ---- S^T = K Q^T, K fragments fetched eight MFMAs (two k-steps) ahead ----
 #pragma unroll
       for (int t = 0; t < 4; ++t) s[t] = f32x4{0.f, 0.f, 0.f, 0.f};
@@ -336,8 +377,7 @@ __global__ __launch_bounds__(kThreads, 1) void MlaDecodeKernel(AttnArgs a) {
 #pragma unroll
         for (int kk = 0; kk < 2; ++kk) {
           const int ks = 2 * pair + kk;
-          const int e = kk ? k_e1 : k_e0;  // ks & 1 == kk
-          const int base = ks < 16 ? k_lat + (ks >> 1) * 128 + e : k_rope + e;
+          const int base = ks < 16 ? k_lat + (ks >> 2) * 256 + k_e[ks & 3] : k_rope + kr_e[ks & 1];
           const int row_pitch = ks < 16 ? kLatRowBytes : kRopeRowBytes;
 #pragma unroll
           for (int t = 0; t < 4; ++t) dst[kk * 4 + t] = *reinterpret_cast<const bf16x8*>(cur + base + t * 16 * row_pitch);
@@ -395,7 +435,7 @@ __global__ __launch_bounds__(kThreads, 1) void MlaDecodeKernel(AttnArgs a) {
       for (int t = 0; t < 4; ++t) {
 #pragma unroll
         for (int j = 0; j < 4; ++j) {
-          const float e = __builtin_amdgcn_exp2f(s[t][j] - m_ref);
+          const float e = (a.debug & 2) ? 1.0f : __builtin_amdgcn_exp2f(s[t][j] - m_ref);
           row_sum += e;
           p[t >> 1][(t & 1) * 4 + j] = static_cast<__bf16>(e);
         }
@@ -409,16 +449,16 @@ __global__ __launch_bounds__(kThreads, 1) void MlaDecodeKernel(AttnArgs a) {
 #pragma unroll
         for (int j = 0; j < 8; ++j) {
           const int n = 8 * (group & 3) + j;
-          const unsigned char* addr = vbase + (n >> 2) * 128 + v_e[n & 3];
+          const unsigned char* addr = vbase + (n >> 3) * 256 + v_e[n & 7];
           const s16x4 lo = __builtin_amdgcn_ds_read_tr16_b64_v4i16((__attribute__((address_space(3))) s16x4*)(addr));
           const s16x4 hi = __builtin_amdgcn_ds_read_tr16_b64_v4i16(
               (__attribute__((address_space(3))) s16x4*)(addr + 16 * kLatRowBytes));
           dst[j] = __builtin_shufflevector(__builtin_bit_cast(bf16x4, lo), __builtin_bit_cast(bf16x4, hi), 0, 1, 2, 3, 4, 5, 6, 7);
         }
       };
-      load_v(vb[0], 0);
+      if (!(a.debug & 4)) load_v(vb[0], 0);
 #pragma unroll
-      for (int group = 0; group < 8; ++group) {
+      for (int group = 0; group < 8 && !(a.debug & 4); ++group) {
         if (group + 1 < 8) load_v(vb[(group + 1) & 1], group + 1);
         __builtin_amdgcn_sched_barrier(0);
 #pragma unroll
@@ -505,7 +545,10 @@ hipError_t Launch(const AttnArgs& args, const dim3& grid, hipStream_t stream) {
 
 hipError_t PrepareAttnKernels() { return hipSuccess; }
 
-hipError_t LaunchAttnDecode(const AttnArgs& args, hipStream_t stream) {
+hipError_t LaunchAttnDecode(const AttnArgs& args_in, hipStream_t stream) {
+  AttnArgs args = args_in;
+  static const int debug = std::getenv("MLAKV_ATTN_DEBUG") ? std::atoi(std::getenv("MLAKV_ATTN_DEBUG")) : 0;
+  args.debug = debug;
   if (args.batch <= 0) return hipSuccess;
   const dim3 grid(args.max_chunks, args.batch, (args.heads + 63) / 64);
   const bool aligned = args.block_size % kTileTokens == 0;

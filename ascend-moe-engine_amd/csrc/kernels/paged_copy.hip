@@ -20,6 +20,8 @@ constexpr int kWave = 64;
 constexpr int kWavesPerGroup = 4;
 constexpr int kThreads = kWave * kWavesPerGroup;
 
+// Every byte is touched once: non-temporal on both sides measured 3-8% faster than cached
+// accesses for the gather.
 __device__ __forceinline__ u32x4 Load16(const char* p) {
   return __builtin_nontemporal_load(reinterpret_cast<const u32x4*>(p));
 }
@@ -231,6 +233,65 @@ __global__ __launch_bounds__(kThreads) void GatherBf16Kernel(GatherArgs g, int r
   CopyRows<kRopeDim * 2 / 16>(rope_src, g.rope.row_stride, rope_dst, g.rope_dst.row_stride, item.nrows, lane);
 }
 
+// Fast path for block sizes that are a multiple of WG_ROWS: one workgroup owns WG_ROWS
+// consecutive rows of one physical block. Each wave moves WG_ROWS/4 latent rows (one
+// 1024-byte row per access) and the first WG_ROWS/8 waves move eight 128-byte rope rows
+// each, so full items run without any per-lane predicate. The three table reads are
+// independent and issued together.
+// Measured on MI355X (batch 32, contexts 128..2048, 43 layers): 8 rows per workgroup beats 16
+// and 32 (5.77 vs 5.54 vs 5.43 TB/s), and holding residency to five workgroups per CU with
+// an unused LDS reservation adds another 1.5%: fewer concurrent streams keep DRAM pages open.
+constexpr int kGatherTileRows = 8;
+constexpr int kGatherLdsReserve = 32000;
+
+template <int WG_ROWS>
+__global__ __launch_bounds__(kThreads) void GatherBf16TileKernel(GatherArgs g, int items_per_block) {
+  static_assert(WG_ROWS % 8 == 0 && WG_ROWS <= 32, "rope rows go eight per wave access");
+  constexpr int kLatentRowsPerWave = WG_ROWS / kWavesPerGroup;
+  constexpr int kRopeWaves = WG_ROWS / 8;
+  const int lane = threadIdx.x & (kWave - 1);
+  const int wave = Uniform(threadIdx.x >> 6);
+  const int seq = blockIdx.y;
+  const int layer = blockIdx.z;
+  const int logical_block = blockIdx.x / items_per_block;
+  const int row0 = (blockIdx.x - logical_block * items_per_block) * WG_ROWS;
+  const int seq_len = Uniform(g.seq_lens[seq]);
+  const int64_t out_base = Uniform(g.cu_seq_lens[seq]);
+  const int physical_block = Uniform(g.block_table[static_cast<int64_t>(seq) * g.table_stride + logical_block]);
+  const int position0 = logical_block * g.block_size + row0;
+  if (position0 >= seq_len) return;
+  if (static_cast<unsigned>(physical_block) >= static_cast<unsigned>(g.num_blocks)) return;
+  const int nrows = min(WG_ROWS, seq_len - position0);
+  const int64_t out_row0 = out_base + position0;
+  const char* latent_src = g.latent.base + layer * g.latent.layer_stride + physical_block * g.latent.block_stride +
+                           (row0 + wave * kLatentRowsPerWave) * g.latent.row_stride + lane * 16;
+  char* latent_dst = g.latent_dst.base + layer * g.latent_dst.layer_stride +
+                     (out_row0 + wave * kLatentRowsPerWave) * g.latent_dst.row_stride + lane * 16;
+  const int sub = lane >> 3, chunk = lane & 7;
+  const char* rope_src = g.rope.base + layer * g.rope.layer_stride + physical_block * g.rope.block_stride +
+                         (row0 + wave * 8 + sub) * g.rope.row_stride + chunk * 16;
+  char* rope_dst = g.rope_dst.base + layer * g.rope_dst.layer_stride + (out_row0 + wave * 8 + sub) * g.rope_dst.row_stride +
+                   chunk * 16;
+  if (nrows == WG_ROWS) {
+    u32x4 v[kLatentRowsPerWave];
+    u32x4 r;
+#pragma unroll
+    for (int u = 0; u < kLatentRowsPerWave; ++u) v[u] = Load16(latent_src + u * g.latent.row_stride);
+    if (wave < kRopeWaves) r = Load16(rope_src);
+#pragma unroll
+    for (int u = 0; u < kLatentRowsPerWave; ++u) Store16(latent_dst + u * g.latent_dst.row_stride, v[u]);
+    if (wave < kRopeWaves) Store16(rope_dst, r);
+  } else {
+#pragma unroll
+    for (int u = 0; u < kLatentRowsPerWave; ++u) {
+      if (wave * kLatentRowsPerWave + u < nrows) {
+        Store16(latent_dst + u * g.latent_dst.row_stride, Load16(latent_src + u * g.latent.row_stride));
+      }
+    }
+    if (wave * 8 + sub < nrows) Store16(rope_dst, Load16(rope_src));
+  }
+}
+
 // FP8 rows: each lane decodes 8 codes (8-byte load) to 8 bf16 (16-byte store).
 __global__ __launch_bounds__(kThreads) void GatherFp8Kernel(GatherArgs g, int rows_per_item) {
   const GatherItem item = ResolveGatherItem(g, rows_per_item);
@@ -327,10 +388,17 @@ hipError_t LaunchAppend(const AppendArgs& args, hipStream_t stream) {
 
 hipError_t LaunchGather(const GatherArgs& args, hipStream_t stream) {
   if (args.batch <= 0 || args.num_layers <= 0 || args.max_seq_len <= 0) return hipSuccess;
-  // 16-row items keep more than 8 waves per CU busy even when the batch holds few blocks.
-  const int rows_per_item = RowsPerItem(args.block_size, 16);
-  const int items_per_block = args.block_size / rows_per_item;
   const int blocks = DivUp(args.max_seq_len, args.block_size);
+  if (!args.fp8 && args.block_size % kGatherTileRows == 0) {
+    const int per_block = args.block_size / kGatherTileRows;
+    const dim3 tile_grid(blocks * per_block, args.batch, args.num_layers);
+    hipLaunchKernelGGL(GatherBf16TileKernel<kGatherTileRows>, tile_grid, dim3(kThreads), kGatherLdsReserve, stream, args,
+                       per_block);
+    return hipGetLastError();
+  }
+  // Two-row items measured fastest for the generic kernels as well (more, shorter waves).
+  const int rows_per_item = RowsPerItem(args.block_size, args.fp8 ? 4 : 2);
+  const int items_per_block = args.block_size / rows_per_item;
   const dim3 grid(DivUp(blocks * items_per_block, kWavesPerGroup), args.batch, args.num_layers);
   if (args.fp8) {
     hipLaunchKernelGGL(GatherFp8Kernel, grid, dim3(kThreads), 0, stream, args, rows_per_item);

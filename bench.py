@@ -155,6 +155,7 @@ def bench_append_gather(args, torch, np, ffi):
 def bench_attention(args, torch, np, ffi, fp8=False, batch=32, ctx=2048, heads=64, slices=8, iters=None):
     lib = ffi.load()
     bs = 64
+    slices = int(os.environ.get("MLAKV_BENCH_SLICES", slices))  # development aid: 1 keeps the KV cache-resident
     blocks_per_seq = -(-ctx // bs)
     pool_blocks = batch * blocks_per_seq + 8
     arena = ffi.Arena(ffi.BACKEND_HIP)
@@ -309,7 +310,7 @@ def main():
                                + ("separate latent/rope planes" if args.split_out else "contiguous 576-element rows"),
                    "bytes_per_step": ag["bytes_per_step"], "frac_of_hbm_peak": ag["value"] / HBM_PEAK_GBPS},
         "roofline": {"bound": "hbm", "achieved": ag["gather_gbps"], "peak": HBM_PEAK_GBPS, "unit": "GB/s",
-                     "frac": ag["gather_gbps"] / HBM_PEAK_GBPS, "traffic": None, "kernel": "GatherBf16Kernel",
+                     "frac": ag["gather_gbps"] / HBM_PEAK_GBPS, "traffic": None, "kernel": "GatherBf16TileKernel",
                      "avg_launch_ms": ag["gather_ms"], "algorithmic_bytes_per_launch": ag["gather_bytes_per_launch"]},
         "append": {"avg_launch_ms": ag["append_ms"], "achieved_gbps": ag["append_gbps"]},
     }
