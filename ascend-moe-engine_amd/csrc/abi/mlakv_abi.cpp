@@ -233,11 +233,11 @@ mlakvStatus mlakvAttnPlanInit(int32_t batch, int32_t heads, int32_t max_seq_len,
   }
   const int max_tiles = (max_seq_len + mlakv::kTileTokens - 1) / mlakv::kTileTokens;
   const int head_groups = (heads + 63) / 64;
-  // One workgroup occupies a whole CU (two 72 KB tile buffers), so aim for one chunk per CU.
+  // One workgroup occupies a whole CU (a ring of four 36 KB tile buffers), so aim for one chunk per CU.
   int chunks_wanted = ComputeUnits() / (batch * head_groups);
   if (chunks_wanted < 1) chunks_wanted = 1;
   int chunk_tiles = (max_tiles + chunks_wanted - 1) / chunks_wanted;
-  if (chunk_tiles < 2) chunk_tiles = max_tiles < 2 ? 1 : 2;  // amortise the query load over at least two tiles
+  if (chunk_tiles < 4) chunk_tiles = max_tiles < 4 ? max_tiles : 4;  // amortise the query load over at least 128 tokens
   if (const char* forced = std::getenv("MLAKV_ATTN_CHUNK_TILES")) {
     const int value = std::atoi(forced);
     if (value > 0) chunk_tiles = value;
@@ -255,7 +255,8 @@ mlakvStatus mlakvAttnPlanInit(int32_t batch, int32_t heads, int32_t max_seq_len,
   plan->reserved = 0;
   if (plan->max_chunks > 1) {
     const uint64_t rows = static_cast<uint64_t>(batch) * plan->max_chunks * heads;
-    plan->workspace_bytes = rows * mlakv::kLatentDim * sizeof(float) + ((rows * sizeof(float) + 255) & ~255ull);
+    // bf16 partial outputs, then fp32 partial log-sum-exps
+    plan->workspace_bytes = rows * mlakv::kLatentDim * 2 + ((rows * sizeof(float) + 255) & ~255ull);
   } else {
     plan->workspace_bytes = 0;
   }
@@ -318,8 +319,8 @@ mlakvStatus mlakvAttnDecode(const mlakvAttnPlan* plan, const mlakvCacheView* cac
   args.out_head_stride = out_head_stride;
   args.lse = lse;
   const uint64_t rows = static_cast<uint64_t>(plan->batch) * plan->max_chunks * plan->heads;
-  args.partial_out = static_cast<float*>(workspace);
-  args.partial_lse = workspace == nullptr ? nullptr : static_cast<float*>(workspace) + rows * mlakv::kLatentDim;
+  args.partial_out = static_cast<char*>(workspace);
+  args.partial_lse = workspace == nullptr ? nullptr : reinterpret_cast<float*>(static_cast<char*>(workspace) + rows * mlakv::kLatentDim * 2);
   args.scale_log2 = static_cast<float>(scale * 1.4426950408889634);
   args.batch = plan->batch;
   args.heads = plan->heads;

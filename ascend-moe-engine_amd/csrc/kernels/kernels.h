@@ -73,7 +73,7 @@ struct AttnArgs {
   char* out;
   int64_t out_seq_stride, out_head_stride;
   float* lse;            // optional
-  float* partial_out;    // workspace: [batch][max_chunks][heads][512] fp32
+  char* partial_out;     // workspace: [batch][max_chunks][heads][512] bf16
   float* partial_lse;    // workspace: [batch][max_chunks][heads] fp32, log2 domain
   float scale_log2;      // softmax scale * log2(e)
   int32_t batch;
@@ -82,14 +82,13 @@ struct AttnArgs {
   int32_t block_size;
   int32_t chunk_tiles;
   int32_t max_chunks;
-  int32_t debug;  // development switches, 0 in production
   bool fp8;
 };
 
 // MLA geometry the kernels are specialised for (include/moe/core/config.hpp:78-109 defaults).
 constexpr int kLatentDim = 512;
 constexpr int kRopeDim = 64;
-constexpr int kTileTokens = 64;
+constexpr int kTileTokens = 32;
 
 hipError_t LaunchAppend(const AppendArgs& args, hipStream_t stream);
 hipError_t LaunchGather(const GatherArgs& args, hipStream_t stream);
