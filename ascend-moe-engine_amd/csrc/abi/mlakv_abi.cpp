@@ -243,8 +243,8 @@ mlakvStatus mlakvAttnPlanInit(int32_t batch, int32_t heads, int32_t max_seq_len,
     if (value > 0) chunk_tiles = value;
   }
   if (chunk_tiles > max_tiles) chunk_tiles = max_tiles;
-  // A chunk's block-table entries are staged in LDS (2048 entries).
-  while (chunk_tiles > 1 && (chunk_tiles * mlakv::kTileTokens + block_size - 1) / block_size + 1 > 2048) --chunk_tiles;
+  // A chunk's block-table entries are staged in LDS (1024 entries).
+  while (chunk_tiles > 1 && (chunk_tiles * mlakv::kTileTokens + block_size - 1) / block_size + 1 > 1024) --chunk_tiles;
   plan->batch = batch;
   plan->heads = heads;
   plan->max_seq_len = max_seq_len;

@@ -83,6 +83,9 @@ struct AttnArgs {
   int32_t chunk_tiles;
   int32_t max_chunks;
   bool fp8;
+#ifdef MLAKV_ATTN_TRACE
+  unsigned long long* trace;  // development timeline, see mla_decode.hip
+#endif
 };
 
 // MLA geometry the kernels are specialised for (include/moe/core/config.hpp:78-109 defaults).

@@ -7,12 +7,22 @@
 // as both K (with the 64 rope columns appended) and V.
 //
 // Work decomposition
-//   workgroup = (kv chunk, sequence, group of 64 heads); 4 wavefronts, 16 heads each, one
-//   workgroup per CU. A chunk is `chunk_tiles` tiles of 32 tokens. LDS holds a ring of four
-//   tile buffers: while tile i feeds the second product and tile i+1 the first, tiles i+2 and
-//   i+3 are in flight from HBM. bf16 tiles are filled by direct global->LDS loads
-//   (global_load_lds_dwordx4: no staging registers, no ds_write); FP8 tiles are dequantised
-//   to bf16 through registers on their way into LDS.
+//   workgroup = (kv chunk, sequence, group of 64 heads), one workgroup per CU, 8 wavefronts in
+//   two roles, one of each role per SIMD:
+//     score waves 0..3 (16 heads each) hold the query in registers, compute S^T = K Q^T for a
+//       tile, run the online softmax and publish P (bf16, already in MFMA operand layout)
+//       through LDS, one tile ahead of
+//     output waves 4..7, which hold the O accumulators and compute O^T += V^T P.
+//   A single wave per SIMD is bound by instruction issue (one instruction per four cycles,
+//   every stall exposed); with the two roles the softmax VALU work, the LDS traffic and the
+//   MFMAs of neighbouring tiles overlap in hardware, and neither role has to hold both the
+//   query (72 registers) and O (128 registers).
+//   A chunk is `chunk_tiles` tiles of 32 tokens. LDS holds a ring of four tile buffers: while
+//   tile i feeds the second product and tile i+1 the first, tiles i+2 and i+3 are in flight
+//   from HBM. bf16 tiles are filled by direct global->LDS loads (global_load_lds_dwordx4: no
+//   staging registers, no ds_write) issued by all eight waves; FP8 tiles are dequantised to
+//   bf16 through registers on their way into LDS. One workgroup barrier per tile publishes
+//   tile i+1 and P(i) and retires tile i-1.
 //
 // MFMA formulation (v_mfma_f32_16x16x32_bf16; A: lane holds row l%16, k = 8*(l/16)..+7;
 // B: lane holds column l%16, same k; D: lane holds rows 4*(l/16)..+3 of column l%16)
@@ -23,23 +33,18 @@
 //   kappa = 8g+e <-> token 4g+e, kappa = 8g+4+e <-> token 16+4g+e:
 //   O^T[dv][head] += V^T[dv][token] . P[token][head]   A = V^T fragment, read from the
 //   row-major tile with ds_read_b64_tr_b16 (a 4x16 transpose per 16 lanes), B = P.
-//   So P never leaves registers and the online-softmax statistics of a head live in the
-//   four lanes {h, h+16, h+32, h+48}: two v_permlane swaps per reduction.
-//
-// Software pipeline: each wavefront is alone on its SIMD, so nothing hides latency but the
-// instruction order. The loop body is written out step by step (one MFMA, the LDS read that
-// refills its operand register several steps ahead, and a slice of the softmax of the
-// previous tile) with a scheduling fence after every step: the softmax VALU work of tile i
-// (exponentials, denominator, P) runs in the shadow of the S^T MFMAs of tile i+1, and the score
-// scaling and maximum of tile i+1 in the shadow of the O^T MFMAs of tile i.
+//   So a score lane writes its eight P values as one 16-byte LDS store and the output lane
+//   with the same lane id reads them back as its B operand; the online-softmax statistics of
+//   a head live in the four lanes {h, h+16, h+32, h+48}: two v_permlane swaps per reduction.
+//   Operand fragments are fetched several MFMAs ahead, with a scheduling fence per step.
 //
 // LDS tile: latent region 32 rows x 1024 B, then rope region 32 rows x 128 B; the 16-byte
 //   chunk index inside a row is XORed with a function of the token (see SwizzleLat). With
 //   direct loads the swizzle is applied on the global side: lane L of a row fetches chunk L ^ f.
 //
-// Online softmax keeps a reference maximum per head and only moves it (rescaling O) when a
-// tile's maximum exceeds it by more than 2^8, so exponentials stay below 256 and most
-// tiles skip the rescale.
+// Online softmax keeps a reference maximum per head and only moves it when a tile's maximum
+// exceeds it by more than 2^8, so exponentials stay below 256; when it moves, the score wave
+// hands the factor to its output wave, which rescales O before adding the tile.
 //
 // Chunks of one sequence are merged by a second small kernel from partials (normalised O in
 // bf16, log2-domain LSE in fp32) held in the caller's workspace.
@@ -48,6 +53,22 @@
 #include "kernels.h"
 
 #pragma clang diagnostic ignored "-Winline-asm"
+
+// Development timeline (built only with -DMLAKV_ATTN_TRACE): lane 0 of waves 0 and 4 of every
+// workgroup stamps the 100 MHz wall clock into a caller-provided buffer.
+#ifdef MLAKV_ATTN_TRACE
+#include <cstdlib>
+#define MLAKV_STAMP(slot)                                                                              \
+  do {                                                                                                 \
+    if (a.trace != nullptr && lane == 0 && (wave == 0 || wave == 4) && (slot) < 32) {                     \
+      a.trace[((blockIdx.y * gridDim.x + blockIdx.x) * 2 + (wave >> 2)) * 32 + (slot)] = __builtin_amdgcn_s_memrealtime(); \
+    }                                                                                                  \
+  } while (0)
+#else
+#define MLAKV_STAMP(slot) \
+  do {                    \
+  } while (0)
+#endif
 
 namespace mlakv {
 namespace {
@@ -61,7 +82,9 @@ typedef __attribute__((ext_vector_type(4))) unsigned int u32x4;
 typedef __attribute__((ext_vector_type(2))) unsigned int u32x2;
 typedef __attribute__((ext_vector_type(4))) short s16x4;
 
-constexpr int kThreads = 256;
+constexpr int kThreads = 512;
+constexpr int kWaves = kThreads / 64;
+constexpr int kScoreWaves = 4;
 constexpr int kLatRowBytes = kLatentDim * 2;                 // 1024
 constexpr int kRopeRowBytes = kRopeDim * 2;                  // 128
 constexpr int kLatRegion = kTileTokens * kLatRowBytes;       // 32768
@@ -70,10 +93,16 @@ constexpr int kRing = 4;                                     // tile buffers in 
 constexpr int kKSteps = (kLatentDim + kRopeDim) / 32;        // 18
 constexpr int kQkSteps = 2 * kKSteps;                        // 36 MFMAs: 18 k-steps x 2 token subtiles
 constexpr int kDvTiles = kLatentDim / 16;                    // 32
-constexpr int kTableEntries = 2048;                          // block-table entries of one chunk staged in LDS
-constexpr int kLdsBytes = kRing * kTileBytes + kTableEntries * 4;
-constexpr int kLoadsPerTile = kTileTokens / 4 + 1;           // direct loads one wave issues for a full tile
-constexpr int kUnknownLoads = -1;
+constexpr int kTableEntries = 1024;                          // block-table entries of one chunk staged in LDS
+// LDS map after the ring.
+constexpr int kTableOff = kRing * kTileBytes;                // int[kTableEntries]
+constexpr int kPOff = kTableOff + kTableEntries * 4;         // P[2][4 waves][64 lanes] x 16 B
+constexpr int kAlphaOff = kPOff + 2 * kScoreWaves * 64 * 16; // alpha[2][4][64] fp32
+constexpr int kInvOff = kAlphaOff + 2 * kScoreWaves * 64 * 4;  // 1/denominator[4][64] fp32
+constexpr int kFlagOff = kInvOff + kScoreWaves * 64 * 4;     // rescale flag[2][4] int
+constexpr int kLdsBytes = kFlagOff + 64;
+static_assert(kLdsBytes <= 160 * 1024, "one workgroup owns the LDS of a CU");
+constexpr int kRowsPerWave = kTileTokens / kWaves;           // latent rows one wave fetches per tile
 constexpr float kRescaleThreshold = 8.0f;                    // log2 domain
 constexpr int kKAhead = 8;                                   // K fragments in flight ahead of their MFMA
 constexpr int kVAhead = 4;                                   // V fragments (two transposed reads each)
@@ -93,11 +122,17 @@ __device__ __forceinline__ void StaticFor(F&& f) {
 }
 
 // LDS is 64 banks x 4 B (256 B per clock): a ds_read_b128 serves 16 lanes per clock, a
-// ds_read_b64_tr_b16 32 lanes. Latent rows (1024 B): the chunk index is XORed with a 4-bit
-// function of the token so that 16 consecutive tokens land in 16 distinct 16-byte slots (K
-// reads) and 8 consecutive tokens in 8 distinct 32-byte slots (transposed V reads). Rope rows
-// (128 B, two per 256 B): 3-bit XOR by token/2.
-__device__ __forceinline__ int SwizzleLat(int token) { return ((token & 7) << 1) | ((token >> 3) & 1); }
+// ds_read_b64_tr_b16 32 lanes. Latent rows (1024 B): the 16-byte chunk index is XORed with a
+// 4-bit function of the token, (g32 << 1) | (token >> 3 & 1). g32 picks the 32-byte slot inside
+// a 256-byte window and is distinct over each of the token sets {0..7}, {8..15}, {0..3, 8..11}
+// and {4..7, 12..15}: the transposed V reads of 32 lanes touch eight rows, and the measured
+// conflict count says the hardware pairs lanes 0-15 with 32-47, not with 16-31. The low bit
+// separates the two tokens that share a g32, so the 16 tokens of a K read land in 16 distinct
+// 16-byte slots. Rope rows (128 B, two per 256 B): 3-bit XOR by token/2.
+__device__ __forceinline__ int SwizzleLat(int token) {
+  const int g32 = (token & 3) | ((((token >> 2) ^ (token >> 3)) & 1) << 2);
+  return (g32 << 1) | ((token >> 3) & 1);
+}
 __device__ __forceinline__ int SwizzleRope(int token) { return (token >> 1) & 7; }
 __device__ __forceinline__ int LatOffset(int token, int chunk) { return token * kLatRowBytes + ((chunk ^ SwizzleLat(token)) << 4); }
 __device__ __forceinline__ int RopeOffset(int token, int chunk) {
@@ -122,33 +157,19 @@ __device__ __forceinline__ void DirectLoad16PerLane(const char* lane_pointer, un
                : "v"(lane_pointer), "s"(lds_wave_base)
                : "memory", "m0");
 }
-// Waits until at most `newer` of this wave's vector-memory loads are outstanding (loads
-// complete in issue order). Anything but a whole number of full tiles waits for everything.
-__device__ __forceinline__ void WaitLoads(int newer) {
-  if (newer == 2 * kLoadsPerTile) {
-    asm volatile("s_waitcnt vmcnt(%0)" ::"n"(2 * kLoadsPerTile) : "memory");
-  } else if (newer == kLoadsPerTile) {
-    asm volatile("s_waitcnt vmcnt(%0)" ::"n"(kLoadsPerTile) : "memory");
+// Waits until at most `tiles` later tiles' worth of this wave's loads are outstanding (loads
+// complete in issue order); `per_tile` is 4 or 5 (waves that also fetch rope rows).
+__device__ __forceinline__ void WaitLoads(int tiles, int per_tile) {
+  if (tiles == 2 && per_tile == 4) {
+    asm volatile("s_waitcnt vmcnt(8)" ::: "memory");
+  } else if (tiles == 2 && per_tile == 5) {
+    asm volatile("s_waitcnt vmcnt(10)" ::: "memory");
+  } else if (tiles == 1 && per_tile == 4) {
+    asm volatile("s_waitcnt vmcnt(4)" ::: "memory");
+  } else if (tiles == 1 && per_tile == 5) {
+    asm volatile("s_waitcnt vmcnt(5)" ::: "memory");
   } else {
     asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
-  }
-}
-
-// The O accumulators must stay in accumulation registers for the whole loop (the 256
-// architectural VGPRs are needed for the query, the operand fragments and the scores), so
-// the second product is issued from inline assembly with the accumulator pinned to the AGPR
-// class. The compiler does not see an MFMA there and inserts no wait states around it:
-// FIRST adds the two the hardware wants between a v_accvgpr_write and an MFMA that reads the
-// register as its addend, LAST the (at most 19) it wants before a VALU instruction may read
-// an MFMA result; the MFMAs of one product retire in order, so covering the last covers all.
-template <bool FIRST, bool LAST>
-__device__ __forceinline__ void MfmaPinned(f32x4& acc, const bf16x8& a, const bf16x8& b) {
-  if (FIRST) {
-    asm volatile("s_nop 1\n\tv_mfma_f32_16x16x32_bf16 %0, %1, %2, %0" : "+a"(acc) : "v"(a), "v"(b));
-  } else if (LAST) {
-    asm volatile("v_mfma_f32_16x16x32_bf16 %0, %1, %2, %0\n\ts_nop 15\n\ts_nop 3" : "+a"(acc) : "v"(a), "v"(b));
-  } else {
-    asm volatile("v_mfma_f32_16x16x32_bf16 %0, %1, %2, %0" : "+a"(acc) : "v"(a), "v"(b));
   }
 }
 
@@ -185,14 +206,20 @@ template <bool ALIGNED>
 struct TileMap {
   const int* entries;  // LDS
   int first_block, block_size, seq_len;
-  int tile_block, tile_slot0;  // ALIGNED only
+  int tile_block, tile_slot0;  // ALIGNED only: where the tile of the last Begin() sits
+  int next_entry, next_slot0;  // ALIGNED only: cursor of the next tile (tiles are begun in order)
 
+  // Tiles are begun in increasing order starting with the first tile of the chunk, so the
+  // ALIGNED case walks a cursor instead of dividing.
   __device__ __forceinline__ void Begin(int tile) {
     if (ALIGNED) {
-      const int pos0 = tile * kTileTokens;
-      const int logical = pos0 / block_size;
-      tile_block = entries[logical - first_block];
-      tile_slot0 = pos0 - logical * block_size;
+      tile_block = entries[next_entry];
+      tile_slot0 = next_slot0;
+      next_slot0 += kTileTokens;
+      if (next_slot0 >= block_size) {
+        next_slot0 = 0;
+        ++next_entry;
+      }
     }
   }
   // Physical block (clamped to a readable one) and slot of row `r` of tile `tile`; returns
@@ -215,94 +242,99 @@ struct TileMap {
 
 // ---- bf16 tiles: direct global -> LDS ----------------------------------------------------
 
-// Lane-constant byte offsets of the chunk a lane fetches for the rows its wave owns: a wave
-// owns latent rows w, w+4, ... (8 of them; row & 15 takes four values) and rope rows 8w..8w+7.
+// Lane-constant byte offsets of the chunk a lane fetches for the rows its wave owns: wave w
+// of 8 owns latent rows w, w+8, w+16, w+24 (row & 15 takes two values); waves 4..7 also own
+// the rope rows 8(w-4) .. 8(w-4)+7.
 struct IssueLane {
-  int lat[4];  // latent rows with (row >> 2) & 3 == j
-  int rope;    // this lane's rope row and chunk, relative to rope row 8w
+  int lat[2];      // latent rows w + 8i with i & 1 == j
+  int rope;        // this lane's rope row and chunk, relative to the first rope row of the wave
   int rope_chunk;
 };
 
-// Issues the loads of one tile into the buffer at LDS address `buf`; rows that are not real
-// are zero-filled instead. Returns how many loads this wave issued when that is the same for
-// every tile of this shape (a full tile), kUnknownLoads otherwise.
+__device__ __forceinline__ int LoadsPerTile(int wave) { return kRowsPerWave + (wave >= kScoreWaves ? 1 : 0); }
+
+// Issues this wave's loads of one tile into the buffer at LDS address `buf`; rows that are not
+// real are zero-filled instead. Returns true when the wave issued exactly LoadsPerTile(wave)
+// loads (a full tile), false when the number is not known.
 template <bool ALIGNED>
-__device__ __forceinline__ int IssueTileBf16(const AttnArgs& a, TileMap<ALIGNED>& map, const IssueLane& il, int tile,
-                                             unsigned buf, unsigned char* buf_ptr, int tid) {
+__device__ __forceinline__ bool IssueTileBf16(const AttnArgs& a, TileMap<ALIGNED>& map, const IssueLane& il, int tile,
+                                              unsigned buf, unsigned char* buf_ptr, int tid) {
   const int lane = tid & 63, wave = Uniform(tid >> 6);
+  const bool rope_wave = wave >= kScoreWaves;
+  const int rope_group = wave - kScoreWaves;
   map.Begin(tile);
   const int rows = map.seq_len - tile * kTileTokens;  // real rows in this tile, >= 1
   if (ALIGNED && rows >= kTileTokens && map.tile_block >= 0) {
     // The whole tile is real and sits in one physical block: uniform base + row pitch.
     const int block = Uniform(map.tile_block), slot0 = Uniform(map.tile_slot0);
     const char* latent = a.latent.base + block * a.latent.block_stride + (slot0 + wave) * a.latent.row_stride;
-    const int64_t pitch = 4 * a.latent.row_stride;
+    const int64_t pitch = kWaves * a.latent.row_stride;
 #pragma unroll
-    for (int i = 0; i < kTileTokens / 4; ++i) DirectLoad16(latent + i * pitch, il.lat[i & 3], buf + (wave + 4 * i) * kLatRowBytes);
-    const char* rope = a.rope.base + block * a.rope.block_stride + (slot0 + 8 * wave) * a.rope.row_stride;
-    DirectLoad16(rope, il.rope, buf + kLatRegion + wave * 8 * kRopeRowBytes);
-    return kLoadsPerTile;
+    for (int i = 0; i < kRowsPerWave; ++i) DirectLoad16(latent + i * pitch, il.lat[i & 1], buf + (wave + kWaves * i) * kLatRowBytes);
+    if (rope_wave) {
+      const char* rope = a.rope.base + block * a.rope.block_stride + (slot0 + 8 * rope_group) * a.rope.row_stride;
+      DirectLoad16(rope, il.rope, buf + kLatRegion + rope_group * 8 * kRopeRowBytes);
+    }
+    return true;
   }
-  int block[kTileTokens / 4], slot[kTileTokens / 4];
-  bool real[kTileTokens / 4];
+  // Rare path (last tile of a sequence, unaligned block sizes, bad table entries): one row at a
+  // time, kept as a loop so that it costs little code.
   bool all_real = true;
-#pragma unroll
-  for (int i = 0; i < kTileTokens / 4; ++i) {
-    real[i] = map.Row(tile, wave + 4 * i, &block[i], &slot[i]);
-    all_real = all_real && real[i];
-  }
-  int rblock, rslot;
-  const bool rreal = map.Row(tile, 8 * wave + (lane >> 3), &rblock, &rslot);
-  all_real = all_real && (__builtin_amdgcn_ballot_w64(!rreal) == 0);
-#pragma unroll
-  for (int i = 0; i < kTileTokens / 4; ++i) {
-    const int row = wave + 4 * i;  // wave-uniform
-    if (real[i]) {
-      const char* src = a.latent.base + Uniform(block[i]) * a.latent.block_stride + Uniform(slot[i]) * a.latent.row_stride;
-      DirectLoad16(src, il.lat[i & 3], buf + row * kLatRowBytes);
+#pragma nounroll
+  for (int i = 0; i < kRowsPerWave; ++i) {
+    const int row = wave + kWaves * i;  // wave-uniform
+    int block, slot;
+    const bool real = map.Row(tile, row, &block, &slot);
+    all_real = all_real && real;
+    if (real) {
+      const char* src = a.latent.base + Uniform(block) * a.latent.block_stride + Uniform(slot) * a.latent.row_stride;
+      DirectLoad16(src, (lane ^ SwizzleLat(row)) << 4, buf + row * kLatRowBytes);
     } else {
       *reinterpret_cast<u32x4*>(buf_ptr + row * kLatRowBytes + lane * 16) = u32x4{0u, 0u, 0u, 0u};
     }
   }
+  if (!rope_wave) return all_real;
   // rope: one wave access covers 8 rows x 128 B, each lane resolving its own row
-  if (all_real) {
-    DirectLoad16PerLane(a.rope.base + rblock * a.rope.block_stride + rslot * a.rope.row_stride + il.rope_chunk,
-                        buf + kLatRegion + wave * 8 * kRopeRowBytes);
-    return kLoadsPerTile;
+  int rblock, rslot;
+  const bool rreal = map.Row(tile, 8 * rope_group + (lane >> 3), &rblock, &rslot);
+  const char* rsrc = a.rope.base + rblock * a.rope.block_stride + rslot * a.rope.row_stride + il.rope_chunk;
+  const unsigned rdst = buf + kLatRegion + rope_group * 8 * kRopeRowBytes;
+  if (__builtin_amdgcn_ballot_w64(!rreal) == 0) {
+    DirectLoad16PerLane(rsrc, rdst);
+    return all_real;
   }
   if (rreal) {
-    DirectLoad16PerLane(a.rope.base + rblock * a.rope.block_stride + rslot * a.rope.row_stride + il.rope_chunk,
-                        buf + kLatRegion + wave * 8 * kRopeRowBytes);
+    DirectLoad16PerLane(rsrc, rdst);
   } else {
-    *reinterpret_cast<u32x4*>(buf_ptr + kLatRegion + wave * 8 * kRopeRowBytes + lane * 16) = u32x4{0u, 0u, 0u, 0u};
+    *reinterpret_cast<u32x4*>(buf_ptr + kLatRegion + rope_group * 8 * kRopeRowBytes + lane * 16) = u32x4{0u, 0u, 0u, 0u};
   }
-  return kUnknownLoads;
+  return false;
 }
 
 // ---- FP8 tiles: global -> registers -> (dequantise) -> LDS ------------------------------------
 
-// 4 latent chunks + (first two waves) 1 rope chunk of 16 codes per thread, and their row
+// 2 latent chunks + (first two waves) 1 rope chunk of 16 codes per thread, and their row
 // scales (0 for a row that is not real).
 struct TileRegsFp8 {
-  u32x4 v[5];
-  float scale[5];
+  u32x4 v[3];
+  float scale[3];
 };
 
 template <bool ALIGNED>
 __device__ __forceinline__ void LoadTileFp8(TileRegsFp8& r, const AttnArgs& a, TileMap<ALIGNED>& map, int tile, int tid) {
   map.Begin(tile);
-  int block[5], slot[5];
-  bool real[5];
+  int block[3], slot[3];
+  bool real[3];
 #pragma unroll
-  for (int i = 0; i < 5; ++i) {
-    const int token = i < 4 ? (tid + kThreads * i) >> 5 : (tid & 127) >> 2;
+  for (int i = 0; i < 3; ++i) {
+    const int token = i < 2 ? (tid + kThreads * i) >> 5 : (tid & 127) >> 2;
     real[i] = map.Row(tile, token, &block[i], &slot[i]);
   }
 #pragma unroll
-  for (int i = 0; i < 5; ++i) {
-    if (i == 4 && tid >= 128) break;  // wave-uniform: 32 rope rows x 4 chunks
-    const int chunk = i < 4 ? (tid + kThreads * i) & 31 : tid & 3;
-    const Plane& plane = i < 4 ? a.latent : a.rope;
+  for (int i = 0; i < 3; ++i) {
+    if (i == 2 && tid >= 128) break;  // wave-uniform: 32 rope rows x 4 chunks
+    const int chunk = i < 2 ? (tid + kThreads * i) & 31 : tid & 3;
+    const Plane& plane = i < 2 ? a.latent : a.rope;
     r.v[i] = GlobalLoad16(plane.base + block[i] * plane.block_stride + slot[i] * plane.row_stride + chunk * 16);
     const float scale = reinterpret_cast<const float*>(a.scale.base + block[i] * a.scale.block_stride)[slot[i]];
     r.scale[i] = real[i] ? scale : 0.0f;
@@ -324,8 +356,8 @@ __device__ __forceinline__ void Dequant4(unsigned int codes, float scale, unsign
 
 __device__ __forceinline__ void StoreTileFp8(const TileRegsFp8& r, unsigned char* buf, int tid) {
 #pragma unroll
-  for (int i = 0; i < 5; ++i) {
-    if (i == 4 && tid >= 128) break;
+  for (int i = 0; i < 3; ++i) {
+    if (i == 2 && tid >= 128) break;
     u32x4 first, second;
     unsigned int lo, hi;
     Dequant4(r.v[i].x, r.scale[i], &lo, &hi);
@@ -344,7 +376,7 @@ __device__ __forceinline__ void StoreTileFp8(const TileRegsFp8& r, unsigned char
       first = u32x4{0u, 0u, 0u, 0u};
       second = first;
     }
-    if (i < 4) {
+    if (i < 2) {
       const int idx = tid + kThreads * i;
       const int token = idx >> 5, chunk = 2 * (idx & 31);
       *reinterpret_cast<u32x4*>(buf + LatOffset(token, chunk)) = first;
@@ -359,33 +391,28 @@ __device__ __forceinline__ void StoreTileFp8(const TileRegsFp8& r, unsigned char
 
 // ---- main kernel -------------------------------------------------------------------
 
-// Online-softmax state of one wave: lane (head i16, token group g).
-struct Softmax {
-  float m_ref;   // reference maximum of the exponentials, log2 domain
-  float l_run;   // this lane's share of the running denominator
-  float x[8];    // scaled scores, then exponentials, of tokens 4g+j (x[0..3]) and 16+4g+j (x[4..7])
-  float tile_max;
-  bf16x8 p;
-};
-
 template <bool FP8, bool ALIGNED>
-__global__ __launch_bounds__(kThreads, 1) void MlaDecodeKernel(AttnArgs a) {
+__global__ __launch_bounds__(kThreads) void MlaDecodeKernel(AttnArgs a) {
   extern __shared__ __attribute__((aligned(16))) unsigned char lds[];
   const unsigned lds_base = static_cast<unsigned>(reinterpret_cast<size_t>((__attribute__((address_space(3))) unsigned char*)lds));
   const int tid = threadIdx.x;
-  const int lane = tid & 63, wave = tid >> 6;
+  const int lane = tid & 63, wave = Uniform(tid >> 6);
+  const bool score_wave = wave < kScoreWaves;   // wave-uniform role
+  const int hw = wave & (kScoreWaves - 1);      // which 16 heads of the 64
   const int g = lane >> 4, i16 = lane & 15;
   const int chunk_index = blockIdx.x;
   const int seq = blockIdx.y;
-  const int head_base = blockIdx.z * 64 + wave * 16;
+  const int head_base = blockIdx.z * 64 + hw * 16;
   const bool active = head_base < a.heads;  // wave-uniform
   const int head = head_base + i16;
   const bool direct = a.max_chunks == 1;  // single chunk: write the final output here
+  const int per_tile = LoadsPerTile(wave);
+  MLAKV_STAMP(0);
 
-  // Q fragments: lane (head i16, k-group g) holds Q[head][32*ks + 8g .. +7]. Issued first so
-  // that they travel while the lengths and the block table are fetched.
+  // Q fragments (score waves): lane (head i16, k-group g) holds Q[head][32*ks + 8g .. +7].
+  // Issued first so that they travel while the lengths and the block table are fetched.
   bf16x8 q[kKSteps];
-  if (active) {
+  if (score_wave && active) {
     const char* q_latent = a.q_latent + seq * a.q_latent_seq_stride + head * a.q_latent_head_stride;
     const char* q_rope = a.q_rope + seq * a.q_rope_seq_stride + head * a.q_rope_head_stride;
 #pragma unroll
@@ -400,7 +427,7 @@ __global__ __launch_bounds__(kThreads, 1) void MlaDecodeKernel(AttnArgs a) {
   // table row, not by the sequence length, so it does not wait for the length to arrive;
   // entries past the sequence are never used.
   const int tile_begin = chunk_index * a.chunk_tiles;
-  int* table_lds = reinterpret_cast<int*>(lds + kRing * kTileBytes);
+  int* table_lds = reinterpret_cast<int*>(lds + kTableOff);
   TileMap<ALIGNED> map;
   map.entries = table_lds;
   map.block_size = a.block_size;
@@ -408,6 +435,8 @@ __global__ __launch_bounds__(kThreads, 1) void MlaDecodeKernel(AttnArgs a) {
     const int first_pos = tile_begin * kTileTokens;
     const int last_pos = first_pos + a.chunk_tiles * kTileTokens - 1;
     map.first_block = first_pos / a.block_size;
+    map.next_entry = 0;
+    map.next_slot0 = first_pos - map.first_block * a.block_size;
     int count = last_pos / a.block_size - map.first_block + 1;  // <= kTableEntries, ensured by the plan
     count = min(count, a.table_stride - map.first_block);
     const int32_t* table_row = a.block_table + static_cast<int64_t>(seq) * a.table_stride + map.first_block;
@@ -424,173 +453,38 @@ __global__ __launch_bounds__(kThreads, 1) void MlaDecodeKernel(AttnArgs a) {
   const int num_tiles = (seq_len + kTileTokens - 1) / kTileTokens;
   if (tile_begin >= num_tiles) {
     if (direct && active) {  // empty sequence: zeros, lse = -inf
-      char* out = a.out + seq * a.out_seq_stride + head * a.out_head_stride;
-      for (int n = g; n < kLatentDim / 8; n += 4) *reinterpret_cast<u32x4*>(out + n * 16) = u32x4{0u, 0u, 0u, 0u};
-      if (a.lse != nullptr && g == 0) a.lse[seq * a.heads + head] = -__builtin_inff();
+      if (score_wave) {
+        if (a.lse != nullptr && g == 0) a.lse[seq * a.heads + head] = -__builtin_inff();
+      } else {
+        char* out = a.out + seq * a.out_seq_stride + head * a.out_head_stride;
+        for (int n = g; n < kLatentDim / 8; n += 4) *reinterpret_cast<u32x4*>(out + n * 16) = u32x4{0u, 0u, 0u, 0u};
+      }
     }
     return;
   }
   const int ntiles = min(a.chunk_tiles, num_tiles - tile_begin);  // tiles of this chunk, >= 1
 
-  f32x4 o[kDvTiles];
-#pragma unroll
-  for (int n = 0; n < kDvTiles; ++n) o[n] = f32x4{0.f, 0.f, 0.f, 0.f};
-  Softmax sm;
-  sm.m_ref = 0.0f;
-  sm.l_run = 0.0f;
-
-  // Lane-constant LDS offsets.
-  // K reads: token = 16t + i16, chunk = 4 ks + g (latent, ks < 16) or 4 (ks - 16) + g (rope).
-  const int k_lat = i16 * kLatRowBytes, k_rope = kLatRegion + i16 * kRopeRowBytes;
-  int k_e[4], kr_e[2];
-#pragma unroll
-  for (int j = 0; j < 4; ++j) k_e[j] = ((4 * j + g) ^ SwizzleLat(i16)) << 4;
-#pragma unroll
-  for (int j = 0; j < 2; ++j) kr_e[j] = ((4 * j + g) ^ SwizzleRope(i16)) << 4;
-  // V reads: token = (16 +) 4g + i16/4, chunk = 2n + (i16 & 3) / 2, 8-byte half i16 & 1.
-  const int v_row = 4 * g + (i16 >> 2);
-  const int v_lane = v_row * kLatRowBytes + (i16 & 1) * 8;
-  int v_e[8];
-#pragma unroll
-  for (int j = 0; j < 8; ++j) v_e[j] = ((2 * j + ((i16 & 3) >> 1)) ^ SwizzleLat(v_row)) << 4;
   // Direct loads: lane L of a latent row fetches chunk L ^ swizzle(row); rows of this wave.
   IssueLane il;
-  {
-    const int w = Uniform(tid >> 6);
 #pragma unroll
-    for (int j = 0; j < 4; ++j) il.lat[j] = (lane ^ SwizzleLat(w + 4 * j)) << 4;
-    il.rope_chunk = ((lane & 7) ^ SwizzleRope(8 * w + (lane >> 3))) << 4;
-    il.rope = (lane >> 3) * static_cast<int>(a.rope.row_stride) + il.rope_chunk;
-  }
+  for (int j = 0; j < 2; ++j) il.lat[j] = (lane ^ SwizzleLat(wave + kWaves * j)) << 4;
+  il.rope_chunk = ((lane & 7) ^ SwizzleRope(8 * (wave - kScoreWaves) + (lane >> 3))) << 4;
+  il.rope = (lane >> 3) * static_cast<int>(a.rope.row_stride) + il.rope_chunk;
 
   const auto ring = [&](int i) __attribute__((always_inline)) { return (i & (kRing - 1)) * kTileBytes; };
 
-  // K fragment of pipeline step `step` (k-step step/2, token subtile step&1) of the tile at `buf`.
-  const auto k_frag = [&](const unsigned char* buf, int step) __attribute__((always_inline)) {
-    const int ks = step >> 1, t = step & 1;
-    const int offset = ks < 16 ? k_lat + (ks >> 2) * 256 + k_e[ks & 3] + t * 16 * kLatRowBytes
-                               : k_rope + kr_e[ks & 1] + t * 16 * kRopeRowBytes;
-    return *reinterpret_cast<const bf16x8*>(buf + offset);
-  };
-  // V^T fragment of output tile n (dv 16n..16n+15) over the 32 tokens of the tile at `buf`.
-  const auto v_frag = [&](const unsigned char* buf, int n) __attribute__((always_inline)) {
-    const unsigned char* addr = buf + v_lane + (n >> 3) * 256 + v_e[n & 7];
-    const s16x4 lo = __builtin_amdgcn_ds_read_tr16_b64_v4i16((__attribute__((address_space(3))) s16x4*)(addr));
-    const s16x4 hi = __builtin_amdgcn_ds_read_tr16_b64_v4i16((__attribute__((address_space(3))) s16x4*)(addr + 16 * kLatRowBytes));
-    return __builtin_shufflevector(__builtin_bit_cast(bf16x4, lo), __builtin_bit_cast(bf16x4, hi), 0, 1, 2, 3, 4, 5, 6, 7);
-  };
-
-  // The softmax of a tile is cut in two halves that hide behind different MFMA phases.
-  // ScoreStep (behind the second product of the previous tile): scale, mask and the tile
-  // maximum of fresh scores. ExpStep (behind the first product of the next tile): exponentials
-  // against the reference maximum, denominator, bf16 P operand. Between the two, outside any
-  // pipelined region, the reference maximum moves if it has to (rare; rescales O).
-  const auto score_step = [&](auto step_c, const f32x4* s, int tile_rel) __attribute__((always_inline)) {
-    constexpr int step = decltype(step_c)::value;
-    if constexpr (step == 0) {
-#pragma unroll
-      for (int j = 0; j < 4; ++j) sm.x[j] = s[0][j] * a.scale_log2;
-    } else if constexpr (step == 2) {
-#pragma unroll
-      for (int j = 0; j < 4; ++j) sm.x[4 + j] = s[1][j] * a.scale_log2;
-    } else if constexpr (step == 3) {
-      const int valid = seq_len - (tile_begin + tile_rel) * kTileTokens;  // >= 1
-      if (valid < kTileTokens) {  // wave-uniform: only the last tile of a sequence
-#pragma unroll
-        for (int j = 0; j < 8; ++j) {
-          if (16 * (j >> 2) + 4 * g + (j & 3) >= valid) sm.x[j] = -__builtin_inff();
-        }
-      }
-    } else if constexpr (step == 4) {
-      sm.tile_max = fmaxf(fmaxf(fmaxf(sm.x[0], sm.x[1]), fmaxf(sm.x[2], sm.x[3])),
-                          fmaxf(fmaxf(sm.x[4], sm.x[5]), fmaxf(sm.x[6], sm.x[7])));
-    } else if constexpr (step == 6) {
-      sm.tile_max = MaxAcrossRows16(sm.tile_max);
-    } else if constexpr (step == 8) {
-      sm.tile_max = MaxAcrossHalves(sm.tile_max);
-    }
-  };
-  constexpr int kScoreSteps = 9;
-  const auto exp_step = [&](auto step_c) __attribute__((always_inline)) {
-    constexpr int step = decltype(step_c)::value;
-    if constexpr (step <= 6 && (step & 1) == 0) {
-      sm.x[step] = __builtin_amdgcn_exp2f(sm.x[step] - sm.m_ref);
-      sm.x[step + 1] = __builtin_amdgcn_exp2f(sm.x[step + 1] - sm.m_ref);
-    } else if constexpr (step == 8) {
-      sm.l_run += ((sm.x[0] + sm.x[1]) + (sm.x[2] + sm.x[3])) + ((sm.x[4] + sm.x[5]) + (sm.x[6] + sm.x[7]));
-    } else if constexpr (step == 10) {
-#pragma unroll
-      for (int j = 0; j < 8; ++j) sm.p[j] = static_cast<__bf16>(sm.x[j]);
-    }
-  };
-  constexpr int kExpSteps = 11;
-  // Moves the reference maximum when some head's tile maximum outgrew it by more than the
-  // threshold; O and the denominator are rescaled to the new reference.
-  const auto move_reference = [&]() __attribute__((always_inline)) {
-    if (__builtin_amdgcn_ballot_w64(sm.tile_max > sm.m_ref + kRescaleThreshold) != 0) {
-      const float m_new = fmaxf(sm.m_ref, sm.tile_max);  // finite: token 0 of the tile is valid
-      const float alpha = __builtin_amdgcn_exp2f(sm.m_ref - m_new);
-      sm.l_run *= alpha;
-      sm.m_ref = m_new;
-#pragma unroll
-      for (int n = 0; n < kDvTiles; ++n) o[n] *= alpha;
-    }
-  };
-
-  // S^T of the tile at `buf` into s_out. With OVERLAP the exponentials of the previous tile
-  // are spread over the steps and the first V fragments of `vbuf` are fetched at the tail.
-  bf16x8 vf[kVAhead];
-  const auto qk = [&](const unsigned char* buf, f32x4* s_out, auto overlap_c, const unsigned char* vbuf)
-                      __attribute__((always_inline)) {
-    constexpr bool overlap = decltype(overlap_c)::value;
-    f32x4 acc[4];
-#pragma unroll
-    for (int j = 0; j < 4; ++j) acc[j] = f32x4{0.f, 0.f, 0.f, 0.f};
-    bf16x8 kf[kKAhead];
-#pragma unroll
-    for (int d = 0; d < kKAhead; ++d) kf[d] = k_frag(buf, d);
-    __builtin_amdgcn_sched_barrier(0);
-    StaticFor<kQkSteps>([&](auto step_c) __attribute__((always_inline)) {
-      constexpr int step = decltype(step_c)::value;
-      constexpr int slot = (step & 1) * 2 + ((step >> 1) & 1);  // two accumulators per token subtile
-      acc[slot] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(kf[step % kKAhead], q[step >> 1], acc[slot], 0, 0, 0);
-      if constexpr (step + kKAhead < kQkSteps) {
-        kf[step % kKAhead] = k_frag(buf, step + kKAhead);
-      } else if constexpr (overlap && step + kKAhead - kQkSteps < kVAhead) {
-        vf[step + kKAhead - kQkSteps] = v_frag(vbuf, step + kKAhead - kQkSteps);
-      }
-      if constexpr (overlap && step < kExpSteps) exp_step(step_c);
-      __builtin_amdgcn_sched_barrier(0);
-    });
-    s_out[0] = acc[0] + acc[1];
-    s_out[1] = acc[2] + acc[3];
-  };
-
-  // O^T += V^T P over the tile at `buf`; the first kVAhead fragments are already in vf. With
-  // OVERLAP the scores `s_new` of tile `tile_rel` are scaled, masked and reduced to their maximum.
-  const auto pv = [&](const unsigned char* buf, auto overlap_c, const f32x4* s_new, int tile_rel)
-                      __attribute__((always_inline)) {
-    constexpr bool overlap = decltype(overlap_c)::value;
-    StaticFor<kDvTiles>([&](auto n_c) __attribute__((always_inline)) {
-      constexpr int n = decltype(n_c)::value;
-      o[n] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(vf[n % kVAhead], sm.p, o[n], 0, 0, 0);
-      if constexpr (n + kVAhead < kDvTiles) vf[n % kVAhead] = v_frag(buf, n + kVAhead);
-      if constexpr (overlap && n < kScoreSteps) score_step(n_c, s_new, tile_rel);
-      __builtin_amdgcn_sched_barrier(0);
-    });
-  };
-
   // The query must have arrived before the tile loads are issued: the compiler's own wait for
   // it would otherwise also wait for every tile load issued in between.
-  if (active) {
+  if (score_wave && active) {
 #pragma unroll
     for (int ks = 0; ks < kKSteps; ++ks) asm volatile("" ::"v"(q[ks]));
   }
+  MLAKV_STAMP(1);
   __syncthreads();  // table entries visible
 
-  // Prologue: tiles 0..2 on their way, tile 0 landed, S^T of tile 0.
+  // Prologue: tiles 0..2 on their way, tile 0 landed and published.
   TileRegsFp8 regs;
-  int newest_loads = kUnknownLoads;  // loads this wave issued for the newest tile in flight
+  bool newest_known = false;  // the newest tile in flight took exactly per_tile loads of this wave
   if (FP8) {
     LoadTileFp8(regs, a, map, tile_begin, tid);
     StoreTileFp8(regs, lds + ring(0), tid);
@@ -600,72 +494,202 @@ __global__ __launch_bounds__(kThreads, 1) void MlaDecodeKernel(AttnArgs a) {
     }
     if (2 < ntiles) LoadTileFp8(regs, a, map, tile_begin + 2, tid);
   } else {
-    int in_flight = 0;  // loads of tiles 1 and 2, when known
+    int in_flight = 0;  // tiles 1 and 2
     bool known = true;
     IssueTileBf16(a, map, il, tile_begin, lds_base + ring(0), lds + ring(0), tid);
     for (int i = 1; i < 3 && i < ntiles; ++i) {
-      newest_loads = IssueTileBf16(a, map, il, tile_begin + i, lds_base + ring(i), lds + ring(i), tid);
-      known = known && newest_loads == kLoadsPerTile;
-      in_flight += kLoadsPerTile;
+      newest_known = IssueTileBf16(a, map, il, tile_begin + i, lds_base + ring(i), lds + ring(i), tid);
+      known = known && newest_known;
+      ++in_flight;
     }
-    WaitLoads(known ? in_flight : 0);
+    MLAKV_STAMP(2);
+    WaitLoads(known ? in_flight : 0, per_tile);
   }
   __syncthreads();
-  if (active) {
-    // S^T of tile 0 and its maximum, which becomes the first reference (O is still zero).
-    f32x4 s_first[2];
-    qk(lds + ring(0), s_first, std::false_type{}, nullptr);
-    StaticFor<kScoreSteps>([&](auto step_c) __attribute__((always_inline)) { score_step(step_c, s_first, 0); });
-    sm.m_ref = sm.tile_max;
-  }
+  MLAKV_STAMP(3);
 
-  for (int i = 0; i < ntiles; ++i) {
-    // Tile i+1 must have landed; tile i+2 may still be in flight. The barrier also retires
-    // every wave's reads of tile i-1, whose buffer tile i+3 reuses.
-    if (i + 1 < ntiles) {
-      if (!FP8) WaitLoads(i + 2 < ntiles && newest_loads == kLoadsPerTile ? kLoadsPerTile : 0);
-      __syncthreads();
-    }
+  // Top of iteration i, both roles: tile i+1 must have landed (tile i+2 may still be in
+  // flight); the barrier publishes it together with P(i) and retires every wave's reads of
+  // tile i-1, whose ring slot tile i+3 then reuses.
+  const auto advance = [&](int i) __attribute__((always_inline)) {
+    MLAKV_STAMP(4 + 2 * i);
+    if (!FP8 && i + 1 < ntiles) WaitLoads(i + 2 < ntiles && newest_known ? 1 : 0, per_tile);
+    __syncthreads();
+    MLAKV_STAMP(5 + 2 * i);
     if (FP8) {
       if (i + 2 < ntiles) StoreTileFp8(regs, lds + ring(i + 2), tid);
       if (i + 3 < ntiles) LoadTileFp8(regs, a, map, tile_begin + i + 3, tid);
     } else if (i + 3 < ntiles) {
-      newest_loads = IssueTileBf16(a, map, il, tile_begin + i + 3, lds_base + ring(i + 3), lds + ring(i + 3), tid);
+      newest_known = IssueTileBf16(a, map, il, tile_begin + i + 3, lds_base + ring(i + 3), lds + ring(i + 3), tid);
+    }
+  };
+
+  unsigned char* p_lds = lds + kPOff + (hw * 64 + lane) * 16;           // + parity * kScoreWaves * 64 * 16
+  float* alpha_lds = reinterpret_cast<float*>(lds + kAlphaOff) + hw * 64 + lane;  // + parity * kScoreWaves * 64
+  float* inv_lds = reinterpret_cast<float*>(lds + kInvOff) + hw * 64 + lane;
+  int* flag_lds = reinterpret_cast<int*>(lds + kFlagOff) + hw;          // + parity * kScoreWaves
+
+  if (score_wave) {
+    // ---------------------------------------------------------------- score waves
+    // K reads: token = 16t + i16, chunk = 4 ks + g (latent, ks < 16) or 4 (ks - 16) + g (rope).
+    const int k_lat = i16 * kLatRowBytes, k_rope = kLatRegion + i16 * kRopeRowBytes;
+    int k_e[4], kr_e[2];
+#pragma unroll
+    for (int j = 0; j < 4; ++j) k_e[j] = ((4 * j + g) ^ SwizzleLat(i16)) << 4;
+#pragma unroll
+    for (int j = 0; j < 2; ++j) kr_e[j] = ((4 * j + g) ^ SwizzleRope(i16)) << 4;
+    // K fragment of pipeline step `step` (k-step step/2, token subtile step&1) of the tile at `buf`.
+    const auto k_frag = [&](const unsigned char* buf, int step) __attribute__((always_inline)) {
+      const int ks = step >> 1, t = step & 1;
+      const int offset = ks < 16 ? k_lat + (ks >> 2) * 256 + k_e[ks & 3] + t * 16 * kLatRowBytes
+                                 : k_rope + kr_e[ks & 1] + t * 16 * kRopeRowBytes;
+      return *reinterpret_cast<const bf16x8*>(buf + offset);
+    };
+
+    float m_ref = -__builtin_inff();  // reference maximum of the exponentials, log2 domain
+    float l_run = 0.0f;               // this lane's share of the running denominator
+
+    // S^T of tile `tile_rel`, its softmax against the running reference, P and the rescale
+    // request into the LDS slots of the tile's parity.
+    const auto score_tile = [&](int tile_rel) __attribute__((always_inline)) {
+      const unsigned char* buf = lds + ring(tile_rel);
+      f32x4 acc[4];
+#pragma unroll
+      for (int j = 0; j < 4; ++j) acc[j] = f32x4{0.f, 0.f, 0.f, 0.f};
+      bf16x8 kf[kKAhead];
+#pragma unroll
+      for (int d = 0; d < kKAhead; ++d) kf[d] = k_frag(buf, d);
+      __builtin_amdgcn_sched_barrier(0);
+      StaticFor<kQkSteps>([&](auto step_c) __attribute__((always_inline)) {
+        constexpr int step = decltype(step_c)::value;
+        constexpr int slot = (step & 1) * 2 + ((step >> 1) & 1);  // two accumulators per token subtile
+        acc[slot] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(kf[step % kKAhead], q[step >> 1], acc[slot], 0, 0, 0);
+        if constexpr (step + kKAhead < kQkSteps) kf[step % kKAhead] = k_frag(buf, step + kKAhead);
+        __builtin_amdgcn_sched_barrier(0);
+      });
+      // lane holds tokens 4g+j (x[0..3]) and 16+4g+j (x[4..7]) of head i16
+      float x[8];
+#pragma unroll
+      for (int j = 0; j < 4; ++j) {
+        x[j] = (acc[0][j] + acc[1][j]) * a.scale_log2;
+        x[4 + j] = (acc[2][j] + acc[3][j]) * a.scale_log2;
+      }
+      const int valid = seq_len - (tile_begin + tile_rel) * kTileTokens;  // >= 1
+      if (valid < kTileTokens) {  // wave-uniform: only the last tile of a sequence
+#pragma unroll
+        for (int j = 0; j < 8; ++j) {
+          if (16 * (j >> 2) + 4 * g + (j & 3) >= valid) x[j] = -__builtin_inff();
+        }
+      }
+      float tile_max = fmaxf(fmaxf(fmaxf(x[0], x[1]), fmaxf(x[2], x[3])), fmaxf(fmaxf(x[4], x[5]), fmaxf(x[6], x[7])));
+      tile_max = MaxAcrossHalves(MaxAcrossRows16(tile_max));
+      const int parity = tile_rel & 1;
+      // Move the reference only when some head's maximum outgrew it by more than the threshold.
+      const bool moved = __builtin_amdgcn_ballot_w64(tile_max > m_ref + kRescaleThreshold) != 0;
+      if (moved) {
+        const float m_new = fmaxf(m_ref, tile_max);  // finite: token 0 of the tile is valid
+        const float alpha = __builtin_amdgcn_exp2f(m_ref - m_new);
+        l_run *= alpha;
+        m_ref = m_new;
+        alpha_lds[parity * kScoreWaves * 64] = alpha;
+      }
+      if (lane == 0) flag_lds[parity * kScoreWaves] = moved && tile_rel != 0 ? 1 : 0;  // O is still zero on the first tile
+      bf16x8 p;
+      float sum = 0.0f;
+#pragma unroll
+      for (int j = 0; j < 8; ++j) {
+        const float e = __builtin_amdgcn_exp2f(x[j] - m_ref);
+        sum += e;
+        p[j] = static_cast<__bf16>(e);
+      }
+      l_run += sum;
+      *reinterpret_cast<bf16x8*>(p_lds + parity * kScoreWaves * 64 * 16) = p;
+    };
+
+    if (active) score_tile(0);
+    for (int i = 0; i < ntiles; ++i) {
+      advance(i);
+      if (active && i + 1 < ntiles) score_tile(i + 1);
     }
     if (active) {
-      const unsigned char* cur = lds + ring(i);
-      f32x4 s_next[2] = {f32x4{0.f, 0.f, 0.f, 0.f}, f32x4{0.f, 0.f, 0.f, 0.f}};
-      if (i + 1 < ntiles) {
-        qk(lds + ring(i + 1), s_next, std::true_type{}, cur);  // + exponentials of tile i
-      } else {
-        StaticFor<kExpSteps>([&](auto step_c) __attribute__((always_inline)) { exp_step(step_c); });
-#pragma unroll
-        for (int d = 0; d < kVAhead; ++d) vf[d] = v_frag(cur, d);
+      const float l_total = SumAcrossHeadLanes(l_run);
+      *inv_lds = 1.0f / l_total;
+      const float lse2 = m_ref + __builtin_amdgcn_logf(l_total);  // v_log_f32 is log2
+      if (g == 0) {
+        if (direct) {
+          if (a.lse != nullptr) a.lse[seq * a.heads + head] = lse2 * 0.6931471805599453f;
+        } else {
+          a.partial_lse[(static_cast<int64_t>(seq) * a.max_chunks + chunk_index) * a.heads + head] = lse2;
+        }
       }
-      pv(cur, std::true_type{}, s_next, i + 1);  // + scores of tile i+1 (unused after the last tile)
-      if (i + 1 < ntiles) move_reference();
     }
-  }
-
-  if (!active) return;
-  const float l_total = SumAcrossHeadLanes(sm.l_run);
-  const float inv = 1.0f / l_total;
-  const float lse2 = sm.m_ref + __builtin_amdgcn_logf(l_total);  // v_log_f32 is log2
-  char* out_row;
-  if (direct) {
-    out_row = a.out + seq * a.out_seq_stride + head * a.out_head_stride;
-    if (a.lse != nullptr && g == 0) a.lse[seq * a.heads + head] = lse2 * 0.6931471805599453f;
+    MLAKV_STAMP(4 + 2 * ntiles);
+    __syncthreads();  // 1/denominator visible to the output waves
+    MLAKV_STAMP(5 + 2 * ntiles);
   } else {
-    const int64_t row = (static_cast<int64_t>(seq) * a.max_chunks + chunk_index) * a.heads + head;
-    out_row = a.partial_out + row * (kLatentDim * 2);
-    if (g == 0) a.partial_lse[row] = lse2;
-  }
+    // ---------------------------------------------------------------- output waves
+    // V reads: token = (16 +) 4g + i16/4, chunk = 2n + (i16 & 3) / 2, 8-byte half i16 & 1.
+    const int v_row = 4 * g + (i16 >> 2);
+    const int v_lane = v_row * kLatRowBytes + (i16 & 1) * 8;
+    int v_e[8];
 #pragma unroll
-  for (int n = 0; n < kDvTiles; ++n) {
-    u32x2 packed;
-    packed.x = PackBf16(o[n][0] * inv, o[n][1] * inv);
-    packed.y = PackBf16(o[n][2] * inv, o[n][3] * inv);
-    *reinterpret_cast<u32x2*>(out_row + (16 * n + 4 * g) * 2) = packed;
+    for (int j = 0; j < 8; ++j) v_e[j] = ((2 * j + ((i16 & 3) >> 1)) ^ SwizzleLat(v_row)) << 4;
+    // V^T fragment of output tile n (dv 16n..16n+15) over the 32 tokens of the tile at `buf`.
+    const auto v_frag = [&](const unsigned char* buf, int n) __attribute__((always_inline)) {
+      const unsigned char* addr = buf + v_lane + (n >> 3) * 256 + v_e[n & 7];
+      const s16x4 lo = __builtin_amdgcn_ds_read_tr16_b64_v4i16((__attribute__((address_space(3))) s16x4*)(addr));
+      const s16x4 hi = __builtin_amdgcn_ds_read_tr16_b64_v4i16((__attribute__((address_space(3))) s16x4*)(addr + 16 * kLatRowBytes));
+      return __builtin_shufflevector(__builtin_bit_cast(bf16x4, lo), __builtin_bit_cast(bf16x4, hi), 0, 1, 2, 3, 4, 5, 6, 7);
+    };
+
+    f32x4 o[kDvTiles];
+#pragma unroll
+    for (int n = 0; n < kDvTiles; ++n) o[n] = f32x4{0.f, 0.f, 0.f, 0.f};
+
+    for (int i = 0; i < ntiles; ++i) {
+      advance(i);
+      if (active) {
+        const unsigned char* buf = lds + ring(i);
+        const int parity = i & 1;
+        bf16x8 vf[kVAhead];
+#pragma unroll
+        for (int d = 0; d < kVAhead; ++d) vf[d] = v_frag(buf, d);
+        const bf16x8 p = *reinterpret_cast<const bf16x8*>(p_lds + parity * kScoreWaves * 64 * 16);
+        if (Uniform(flag_lds[parity * kScoreWaves]) != 0) {  // the reference maximum moved: rescale O first
+          const float alpha = alpha_lds[parity * kScoreWaves * 64];
+#pragma unroll
+          for (int n = 0; n < kDvTiles; ++n) o[n] *= alpha;
+        }
+        __builtin_amdgcn_sched_barrier(0);
+        StaticFor<kDvTiles>([&](auto n_c) __attribute__((always_inline)) {
+          constexpr int n = decltype(n_c)::value;
+          o[n] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(vf[n % kVAhead], p, o[n], 0, 0, 0);
+          if constexpr (n + kVAhead < kDvTiles) vf[n % kVAhead] = v_frag(buf, n + kVAhead);
+          __builtin_amdgcn_sched_barrier(0);
+        });
+      }
+    }
+    MLAKV_STAMP(4 + 2 * ntiles);
+    __syncthreads();  // 1/denominator from the score waves
+    MLAKV_STAMP(5 + 2 * ntiles);
+    if (active) {
+      const float inv = *inv_lds;
+      char* out_row;
+      if (direct) {
+        out_row = a.out + seq * a.out_seq_stride + head * a.out_head_stride;
+      } else {
+        const int64_t row = (static_cast<int64_t>(seq) * a.max_chunks + chunk_index) * a.heads + head;
+        out_row = a.partial_out + row * (kLatentDim * 2);
+      }
+#pragma unroll
+      for (int n = 0; n < kDvTiles; ++n) {
+        u32x2 packed;
+        packed.x = PackBf16(o[n][0] * inv, o[n][1] * inv);
+        packed.y = PackBf16(o[n][2] * inv, o[n][3] * inv);
+        __builtin_nontemporal_store(packed, reinterpret_cast<u32x2*>(out_row + (16 * n + 4 * g) * 2));
+      }
+    }
+    MLAKV_STAMP(6 + 2 * ntiles);
   }
 }
 
@@ -746,7 +770,11 @@ hipError_t Launch(const AttnArgs& args, const dim3& grid, hipStream_t stream) {
 
 hipError_t PrepareAttnKernels() { return hipSuccess; }
 
-hipError_t LaunchAttnDecode(const AttnArgs& args, hipStream_t stream) {
+hipError_t LaunchAttnDecode(const AttnArgs& args_in, hipStream_t stream) {
+  AttnArgs args = args_in;
+#ifdef MLAKV_ATTN_TRACE
+  args.trace = std::getenv("MLAKV_ATTN_TRACE_PTR") ? reinterpret_cast<unsigned long long*>(std::strtoull(std::getenv("MLAKV_ATTN_TRACE_PTR"), nullptr, 0)) : nullptr;
+#endif
   if (args.batch <= 0) return hipSuccess;
   const dim3 grid(args.max_chunks, args.batch, (args.heads + 63) / 64);
   const bool aligned = args.block_size % kTileTokens == 0;
