@@ -60,7 +60,7 @@
 #include <cstdlib>
 #define MLAKV_STAMP(slot)                                                                              \
   do {                                                                                                 \
-    if (a.trace != nullptr && lane == 0 && (wave == 0 || wave == 4) && (slot) < 32) {                     \
+    if (a.trace != nullptr && lane == 0 && (wave == 0 || wave == 4) && (slot) >= 0 && (slot) < 32) {                     \
       a.trace[((blockIdx.y * gridDim.x + blockIdx.x) * 2 + (wave >> 2)) * 32 + (slot)] = __builtin_amdgcn_s_memrealtime(); \
     }                                                                                                  \
   } while (0)
@@ -146,15 +146,21 @@ __device__ __forceinline__ u32x4 GlobalLoad16(const char* p) { return *reinterpr
 // compiler does not serialise every later LDS read behind them; the kernel waits for them
 // itself with WaitLoads() before the workgroup barrier that publishes a tile.
 __device__ __forceinline__ void DirectLoad16(const char* uniform_base, int lane_offset, unsigned lds_wave_base) {
+  // The base and the LDS address must sit in scalar registers whatever the compiler concluded
+  // about their uniformity.
+  const unsigned long long bits = reinterpret_cast<unsigned long long>(uniform_base);
+  const unsigned lo = __builtin_amdgcn_readfirstlane(static_cast<unsigned>(bits));
+  const unsigned hi = __builtin_amdgcn_readfirstlane(static_cast<unsigned>(bits >> 32));
+  const unsigned long long base = (static_cast<unsigned long long>(hi) << 32) | lo;
   asm volatile("s_mov_b32 m0, %2\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %0, %1"
                :
-               : "v"(lane_offset), "s"(uniform_base), "s"(lds_wave_base)
+               : "v"(lane_offset), "s"(base), "s"(__builtin_amdgcn_readfirstlane(lds_wave_base))
                : "memory", "m0");
 }
 __device__ __forceinline__ void DirectLoad16PerLane(const char* lane_pointer, unsigned lds_wave_base) {
   asm volatile("s_mov_b32 m0, %1\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %0, off"
                :
-               : "v"(lane_pointer), "s"(lds_wave_base)
+               : "v"(lane_pointer), "s"(__builtin_amdgcn_readfirstlane(lds_wave_base))
                : "memory", "m0");
 }
 // Waits until at most `tiles` later tiles' worth of this wave's loads are outstanding (loads
@@ -254,7 +260,7 @@ struct IssueLane {
 __device__ __forceinline__ int LoadsPerTile(int wave) { return kRowsPerWave + (wave >= kScoreWaves ? 1 : 0); }
 
 // Issues this wave's loads of one tile into the buffer at LDS address `buf`; rows that are not
-// real are zero-filled instead. Returns true when the wave issued exactly LoadsPerTile(wave)
+// real are zero-filled instead. Returns true when the wave issues exactly LoadsPerTile(wave)
 // loads (a full tile), false when the number is not known.
 template <bool ALIGNED>
 __device__ __forceinline__ bool IssueTileBf16(const AttnArgs& a, TileMap<ALIGNED>& map, const IssueLane& il, int tile,
@@ -269,12 +275,10 @@ __device__ __forceinline__ bool IssueTileBf16(const AttnArgs& a, TileMap<ALIGNED
     const int block = Uniform(map.tile_block), slot0 = Uniform(map.tile_slot0);
     const char* latent = a.latent.base + block * a.latent.block_stride + (slot0 + wave) * a.latent.row_stride;
     const int64_t pitch = kWaves * a.latent.row_stride;
+    const char* rope = a.rope.base + block * a.rope.block_stride + (slot0 + 8 * rope_group) * a.rope.row_stride;
 #pragma unroll
     for (int i = 0; i < kRowsPerWave; ++i) DirectLoad16(latent + i * pitch, il.lat[i & 1], buf + (wave + kWaves * i) * kLatRowBytes);
-    if (rope_wave) {
-      const char* rope = a.rope.base + block * a.rope.block_stride + (slot0 + 8 * rope_group) * a.rope.row_stride;
-      DirectLoad16(rope, il.rope, buf + kLatRegion + rope_group * 8 * kRopeRowBytes);
-    }
+    if (rope_wave) DirectLoad16(rope, il.rope, buf + kLatRegion + rope_group * 8 * kRopeRowBytes);
     return true;
   }
   // Rare path (last tile of a sequence, unaligned block sizes, bad table entries): one row at a
@@ -512,16 +516,17 @@ __global__ __launch_bounds__(kThreads) void MlaDecodeKernel(AttnArgs a) {
   // flight); the barrier publishes it together with P(i) and retires every wave's reads of
   // tile i-1, whose ring slot tile i+3 then reuses.
   const auto advance = [&](int i) __attribute__((always_inline)) {
-    MLAKV_STAMP(4 + 2 * i);
+    MLAKV_STAMP(4 + 6 * i);
     if (!FP8 && i + 1 < ntiles) WaitLoads(i + 2 < ntiles && newest_known ? 1 : 0, per_tile);
     __syncthreads();
-    MLAKV_STAMP(5 + 2 * i);
+    MLAKV_STAMP(5 + 6 * i);
     if (FP8) {
       if (i + 2 < ntiles) StoreTileFp8(regs, lds + ring(i + 2), tid);
       if (i + 3 < ntiles) LoadTileFp8(regs, a, map, tile_begin + i + 3, tid);
     } else if (i + 3 < ntiles) {
       newest_known = IssueTileBf16(a, map, il, tile_begin + i + 3, lds_base + ring(i + 3), lds + ring(i + 3), tid);
     }
+    MLAKV_STAMP(6 + 6 * i);
   };
 
   unsigned char* p_lds = lds + kPOff + (hw * 64 + lane) * 16;           // + parity * kScoreWaves * 64 * 16
@@ -567,6 +572,7 @@ __global__ __launch_bounds__(kThreads) void MlaDecodeKernel(AttnArgs a) {
         if constexpr (step + kKAhead < kQkSteps) kf[step % kKAhead] = k_frag(buf, step + kKAhead);
         __builtin_amdgcn_sched_barrier(0);
       });
+      MLAKV_STAMP(7 + 6 * (tile_rel - 1));
       // lane holds tokens 4g+j (x[0..3]) and 16+4g+j (x[4..7]) of head i16
       float x[8];
 #pragma unroll
@@ -604,6 +610,7 @@ __global__ __launch_bounds__(kThreads) void MlaDecodeKernel(AttnArgs a) {
       }
       l_run += sum;
       *reinterpret_cast<bf16x8*>(p_lds + parity * kScoreWaves * 64 * 16) = p;
+      MLAKV_STAMP(8 + 6 * (tile_rel - 1));
     };
 
     if (active) score_tile(0);
@@ -623,9 +630,9 @@ __global__ __launch_bounds__(kThreads) void MlaDecodeKernel(AttnArgs a) {
         }
       }
     }
-    MLAKV_STAMP(4 + 2 * ntiles);
+    MLAKV_STAMP(29);
     __syncthreads();  // 1/denominator visible to the output waves
-    MLAKV_STAMP(5 + 2 * ntiles);
+    MLAKV_STAMP(30);
   } else {
     // ---------------------------------------------------------------- output waves
     // V reads: token = (16 +) 4g + i16/4, chunk = 2n + (i16 & 3) / 2, 8-byte half i16 & 1.
@@ -667,11 +674,12 @@ __global__ __launch_bounds__(kThreads) void MlaDecodeKernel(AttnArgs a) {
           if constexpr (n + kVAhead < kDvTiles) vf[n % kVAhead] = v_frag(buf, n + kVAhead);
           __builtin_amdgcn_sched_barrier(0);
         });
+        MLAKV_STAMP(7 + 6 * i);
       }
     }
-    MLAKV_STAMP(4 + 2 * ntiles);
+    MLAKV_STAMP(29);
     __syncthreads();  // 1/denominator from the score waves
-    MLAKV_STAMP(5 + 2 * ntiles);
+    MLAKV_STAMP(30);
     if (active) {
       const float inv = *inv_lds;
       char* out_row;
@@ -689,7 +697,7 @@ __global__ __launch_bounds__(kThreads) void MlaDecodeKernel(AttnArgs a) {
         __builtin_nontemporal_store(packed, reinterpret_cast<u32x2*>(out_row + (16 * n + 4 * g) * 2));
       }
     }
-    MLAKV_STAMP(6 + 2 * ntiles);
+    MLAKV_STAMP(31);
   }
 }
 
