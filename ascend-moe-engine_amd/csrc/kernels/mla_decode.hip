@@ -456,13 +456,15 @@ __global__ __launch_bounds__(kThreads) void MlaDecodeKernel(AttnArgs a) {
   map.seq_len = seq_len;
   const int num_tiles = (seq_len + kTileTokens - 1) / kTileTokens;
   if (tile_begin >= num_tiles) {
-    if (direct && active) {  // empty sequence: zeros, lse = -inf
+    if (active && direct) {  // empty sequence: zeros, lse = -inf
       if (score_wave) {
         if (a.lse != nullptr && g == 0) a.lse[seq * a.heads + head] = -__builtin_inff();
       } else {
         char* out = a.out + seq * a.out_seq_stride + head * a.out_head_stride;
         for (int n = g; n < kLatentDim / 8; n += 4) *reinterpret_cast<u32x4*>(out + n * 16) = u32x4{0u, 0u, 0u, 0u};
       }
+    } else if (active && score_wave && g == 0) {  // empty chunk: the merge reads every chunk's LSE
+      a.partial_lse[(static_cast<int64_t>(seq) * a.max_chunks + chunk_index) * a.heads + head] = -__builtin_inff();
     }
     return;
   }
@@ -702,24 +704,17 @@ __global__ __launch_bounds__(kThreads) void MlaDecodeKernel(AttnArgs a) {
 }
 
 // Merges the chunks of one (sequence, head): out = sum_c w_c O_c / sum_c w_c with
-// w_c = 2^(lse2_c - max lse2). 256 threads = 4 heads x 64 lanes, 8 output columns per lane;
-// the loads of up to eight chunks are issued before the first is used.
+// w_c = 2^(lse2_c - max lse2). 256 threads = 4 heads x 64 lanes, 8 output columns per lane.
+// Every chunk slot carries an LSE (-inf for a chunk past the end of its sequence, whose O slot
+// was never written), so all loads of a group of eight chunks are issued at once, with no
+// dependence on the sequence length.
 constexpr int kCombineHeads = 4;
 __global__ __launch_bounds__(256) void MlaCombineKernel(AttnArgs a) {
   const int head = blockIdx.x * kCombineHeads + (threadIdx.x >> 6), seq = blockIdx.y;
   const int lane = threadIdx.x & 63;
   if (head >= a.heads) return;
-  const int seq_len = static_cast<int>(
-      min(static_cast<int64_t>(a.seq_lens[seq]), static_cast<int64_t>(a.table_stride) * a.block_size));  // as in the main kernel
-  const int num_tiles = (seq_len + kTileTokens - 1) / kTileTokens;
-  const int chunks = min((num_tiles + a.chunk_tiles - 1) / a.chunk_tiles, a.max_chunks);
-  char* out = a.out + seq * a.out_seq_stride + head * a.out_head_stride + lane * 16;
-  if (chunks == 0) {
-    *reinterpret_cast<u32x4*>(out) = u32x4{0u, 0u, 0u, 0u};
-    if (a.lse != nullptr && lane == 0) a.lse[seq * a.heads + head] = -__builtin_inff();
-    return;
-  }
-  const int64_t row0 = static_cast<int64_t>(seq) * a.max_chunks * a.heads + head;
+  const int chunks = a.max_chunks;
+  const int64_t row0 = static_cast<int64_t>(seq) * chunks * a.heads + head;
   float acc[8];
 #pragma unroll
   for (int j = 0; j < 8; ++j) acc[j] = 0.0f;
@@ -732,11 +727,12 @@ __global__ __launch_bounds__(256) void MlaCombineKernel(AttnArgs a) {
       const int c = min(c0 + u, chunks - 1);
       const int64_t row = row0 + static_cast<int64_t>(c) * a.heads;
       l[u] = c0 + u < chunks ? a.partial_lse[row] : -__builtin_inff();
-      v[u] = GlobalLoad16(a.partial_out + row * (kLatentDim * 2) + lane * 16);
+      v[u] = __builtin_nontemporal_load(reinterpret_cast<const u32x4*>(a.partial_out + row * (kLatentDim * 2) + lane * 16));
     }
     float group_max = m;
 #pragma unroll
     for (int u = 0; u < 8; ++u) group_max = fmaxf(group_max, l[u]);
+    if (group_max == -__builtin_inff()) continue;  // nothing but empty chunks so far
     const float rescale = __builtin_amdgcn_exp2f(m - group_max);  // 0 on the first group
     m = group_max;
     denom *= rescale;
@@ -744,7 +740,8 @@ __global__ __launch_bounds__(256) void MlaCombineKernel(AttnArgs a) {
     for (int j = 0; j < 8; ++j) acc[j] *= rescale;
 #pragma unroll
     for (int u = 0; u < 8; ++u) {
-      const float w = __builtin_amdgcn_exp2f(l[u] - m);  // 0 for the padding slots
+      if (l[u] == -__builtin_inff()) continue;  // empty or padding slot: its O bytes are not data
+      const float w = __builtin_amdgcn_exp2f(l[u] - m);
       denom += w;
       const unsigned words[4] = {v[u].x, v[u].y, v[u].z, v[u].w};
 #pragma unroll
@@ -753,6 +750,12 @@ __global__ __launch_bounds__(256) void MlaCombineKernel(AttnArgs a) {
         acc[2 * j + 1] += w * __builtin_bit_cast(float, words[j] & 0xffff0000u);
       }
     }
+  }
+  char* out = a.out + seq * a.out_seq_stride + head * a.out_head_stride + lane * 16;
+  if (denom == 0.0f) {  // empty sequence
+    *reinterpret_cast<u32x4*>(out) = u32x4{0u, 0u, 0u, 0u};
+    if (a.lse != nullptr && lane == 0) a.lse[seq * a.heads + head] = -__builtin_inff();
+    return;
   }
   const float inv = 1.0f / denom;
   u32x4 packed;

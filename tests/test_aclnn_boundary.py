@@ -199,8 +199,8 @@ def test_thin_abi_argument_validation_without_a_device():
     lib = ffi.load()
     plan = ffi.AttnPlan()
     assert lib.mlakvAttnPlanInit(32, 64, 2048, 64, ffi.DTYPE_BF16, C.byref(plan)) == 0
-    assert (plan.chunk_tiles, plan.max_chunks) == (4, 8)  # 256 CUs / 32 sequences
-    assert plan.workspace_bytes == 32 * 8 * 64 * 512 * 4 + 32 * 8 * 64 * 4
+    assert (plan.chunk_tiles, plan.max_chunks) == (8, 8)  # 32-token tiles; 256 CUs / 32 sequences
+    assert plan.workspace_bytes == 32 * 8 * 64 * 512 * 2 + 32 * 8 * 64 * 4  # bf16 partial outputs + fp32 partial LSEs
     assert lib.mlakvAttnPlanInit(32, 60, 2048, 64, ffi.DTYPE_BF16, C.byref(plan)) == ffi.ERR_PARAM_INVALID
     assert lib.mlakvAttnPlanInit(32, 64, 2048, 64, 7, C.byref(plan)) == ffi.ERR_PARAM_INVALID
     assert lib.mlakvAttnPlanInit(32, 64, 2048, 64, ffi.DTYPE_BF16, None) == ffi.ERR_PARAM_NULLPTR
