@@ -27,6 +27,10 @@ ROOT = os.path.dirname(os.path.abspath(__file__))
 sys.path.insert(0, os.path.join(ROOT, "ascend-moe-engine_amd", "python"))
 sys.path.insert(0, os.path.join(ROOT, "oracle"))
 
+# HBM bytes per algorithmic byte of the gather kernel, from two rocprofv3 --pmc runs of this file
+# (FETCH_SIZE scaled by 2.000, WRITE_SIZE by 1.000, the factors a plain 1 GiB copy gives):
+# (1956.8 + 1956.7) MB measured per dispatch against 3912.4 MB algorithmic.
+GATHER_TRAFFIC_PER_ALGORITHMIC_BYTE = 1.0003
 HBM_PEAK_GBPS = 8000.0      # MI355X HBM3E, published
 MFMA_BF16_PEAK_TFLOPS = 2500.0
 LATENT, ROPE, ROW = 512, 64, 576
@@ -310,7 +314,11 @@ def main():
                                + ("separate latent/rope planes" if args.split_out else "contiguous 576-element rows"),
                    "bytes_per_step": ag["bytes_per_step"], "frac_of_hbm_peak": ag["value"] / HBM_PEAK_GBPS},
         "roofline": {"bound": "hbm", "achieved": ag["gather_gbps"], "peak": HBM_PEAK_GBPS, "unit": "GB/s",
-                     "frac": ag["gather_gbps"] / HBM_PEAK_GBPS, "traffic": None, "kernel": "GatherBf16TileKernel",
+                     "frac": ag["gather_gbps"] / HBM_PEAK_GBPS,
+                     "traffic": ag["gather_bytes_per_launch"] * GATHER_TRAFFIC_PER_ALGORITHMIC_BYTE,
+                     "traffic_source": "rocprofv3 --pmc FETCH_SIZE x2.000 + WRITE_SIZE x1.000 per gather dispatch of this "
+                                       "command, applied as a ratio to the algorithmic bytes of the timed launches",
+                     "kernel": "GatherBf16TileKernel",
                      "avg_launch_ms": ag["gather_ms"], "algorithmic_bytes_per_launch": ag["gather_bytes_per_launch"]},
         "append": {"avg_launch_ms": ag["append_ms"], "achieved_gbps": ag["append_gbps"]},
     }
