@@ -4,6 +4,7 @@ there is no Python implementation of anything behind it, and loading fails loudl
 library has not been built.
 """
 import ctypes as C
+import weakref
 import os
 
 _HERE = os.path.dirname(os.path.abspath(__file__))
@@ -168,9 +169,14 @@ class Arena:
         handle = _vp()
         check(self.lib.mlakvArenaCreate(backend, C.byref(handle)))
         self.handle = handle
+        self._caches = weakref.WeakSet()  # KvCache objects built on this arena
 
     def close(self):
+        """Destroys the caches built on this arena first: they hold pinned staging buffers that
+        are released through the arena's backend, whatever order the garbage collector picks."""
         if self.handle:
+            for cache in list(self._caches):
+                cache.close()
             self.lib.mlakvArenaDestroy(self.handle)
             self.handle = None
 
@@ -265,6 +271,7 @@ class KvCache:
         handle = _vp()
         check(self.lib.mlakvKvCacheCreate(arena.handle, C.byref(cfg), C.byref(handle)))
         self.handle = handle
+        arena._caches.add(self)
 
     def close(self):
         if self.handle:

@@ -156,7 +156,7 @@ def bench_append_gather(args, torch, np, ffi):
     return result
 
 
-def bench_attention(args, torch, np, ffi, fp8=False, batch=32, ctx=2048, heads=64, slices=8, iters=None):
+def bench_attention(args, torch, np, ffi, fp8=False, batch=32, ctx=2048, heads=64, slices=8, iters=None, label=None):
     lib = ffi.load()
     bs = 64
     slices = int(os.environ.get("MLAKV_BENCH_SLICES", slices))  # development aid: 1 keeps the KV cache-resident
@@ -214,7 +214,7 @@ def bench_attention(args, torch, np, ffi, fp8=False, batch=32, ctx=2048, heads=6
     flops = 2.0 * batch * heads * ctx * (ROW + LATENT)
     result = {
         "us_per_step": us,
-        "workload": f"configs[{3 if fp8 else 2}]-shape: 1 layer per launch, batch {batch}, {heads} heads, ctx {ctx}, block 64, "
+        "workload": f"{label or ('configs[3]-shape' if fp8 else 'configs[2]-shape')}: 1 layer per launch, batch {batch}, {heads} heads, ctx {ctx}, block 64, "
                     f"{'fp8 e4m3 + fp32 row scale' if fp8 else 'bf16'} KV, shuffled table, {slices} rotating layer slices",
         "roofline": {"bound": "hbm", "achieved": algorithmic / (us * 1e-6) / 1e9, "peak": HBM_PEAK_GBPS, "unit": "GB/s",
                      "frac": algorithmic / (us * 1e-6) / 1e9 / HBM_PEAK_GBPS, "traffic": None},
@@ -300,7 +300,9 @@ def main():
     del calib_src, calib_dst
     if args.attention_only:
         print(json.dumps({"attention": bench_attention(args, torch, np, ffi),
-                          "attention_fp8": bench_attention(args, torch, np, ffi, fp8=True, batch=64, ctx=4352, iters=64)}))
+                          "attention_fp8": bench_attention(args, torch, np, ffi, fp8=True, batch=64, ctx=4352, iters=64),
+                          "attention_long": bench_attention(args, torch, np, ffi, batch=128, ctx=8192, slices=2, iters=16,
+                                                            label="configs[4]-scale decode shape (one workgroup per sequence)")}))
         return 0
     ag = bench_append_gather(args, torch, np, ffi)
     line = {
@@ -325,6 +327,8 @@ def main():
     if not args.no_attention:
         line["attention"] = bench_attention(args, torch, np, ffi)
         line["attention_fp8"] = bench_attention(args, torch, np, ffi, fp8=True, batch=64, ctx=4352, iters=64)
+        line["attention_long"] = bench_attention(args, torch, np, ffi, batch=128, ctx=8192, slices=2, iters=16,
+                                                 label="configs[4]-scale decode shape (one workgroup per sequence)")
     if not args.no_cpu_baseline:
         line["cpu_baseline"] = cpu_baseline(np, ag)
         if not args.no_attention:
