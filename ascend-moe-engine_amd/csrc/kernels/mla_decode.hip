@@ -81,32 +81,44 @@ typedef __attribute__((ext_vector_type(2))) float f32x2;
 typedef __attribute__((ext_vector_type(4))) unsigned int u32x4;
 typedef __attribute__((ext_vector_type(2))) unsigned int u32x2;
 typedef __attribute__((ext_vector_type(4))) short s16x4;
+typedef __attribute__((ext_vector_type(8))) short s16x8;
+typedef __attribute__((ext_vector_type(2))) int i32x2;
 
 constexpr int kThreads = 512;
 constexpr int kWaves = kThreads / 64;
 constexpr int kScoreWaves = 4;
-constexpr int kLatRowBytes = kLatentDim * 2;                 // 1024
-constexpr int kRopeRowBytes = kRopeDim * 2;                  // 128
-constexpr int kLatRegion = kTileTokens * kLatRowBytes;       // 32768
-constexpr int kTileBytes = kLatRegion + kTileTokens * kRopeRowBytes;  // 36864
-constexpr int kRing = 4;                                     // tile buffers in LDS
 constexpr int kKSteps = (kLatentDim + kRopeDim) / 32;        // 18
 constexpr int kQkSteps = 2 * kKSteps;                        // 36 MFMAs: 18 k-steps x 2 token subtiles
 constexpr int kDvTiles = kLatentDim / 16;                    // 32
 constexpr int kTableEntries = 1024;                          // block-table entries of one chunk staged in LDS
-// LDS map after the ring.
-constexpr int kTableOff = kRing * kTileBytes;                // int[kTableEntries]
-constexpr int kPOff = kTableOff + kTableEntries * 4;         // P[2][4 waves][64 lanes] x 16 B
-constexpr int kAlphaOff = kPOff + 2 * kScoreWaves * 64 * 16; // alpha[2][4][64] fp32
-constexpr int kInvOff = kAlphaOff + 2 * kScoreWaves * 64 * 4;  // 1/denominator[4][64] fp32
-constexpr int kFlagOff = kInvOff + kScoreWaves * 64 * 4;     // rescale flag[2][4] int
-constexpr int kLdsBytes = kFlagOff + 64;
-static_assert(kLdsBytes <= 160 * 1024, "one workgroup owns the LDS of a CU");
-constexpr int kRowsPerWave = kTileTokens / kWaves;           // latent rows one wave fetches per tile
-constexpr float kRescaleThreshold = 8.0f;                    // log2 domain
-constexpr int kKAhead = 8;                                   // K fragments in flight ahead of their MFMA
-constexpr int kVAhead = 4;                                   // V fragments (two transposed reads each)
 static_assert(kTileTokens == 32, "the fragment maps below are written for 32-token tiles");
+
+// LDS geometry. A bf16 tile is 32 latent rows of 1024 B followed by 32 rope rows of 128 B. An
+// FP8 tile keeps the E4M3 codes as they are in the cache (32 x 512 B, 32 x 64 B) followed by the
+// 32 fp32 row scales, padded to a multiple of 512 B so that the XOR-swizzled part of an address
+// can be formed before the tile base is added. The ring is as deep as the 160 KB allow.
+template <bool FP8>
+struct Geom {
+  static constexpr int kLatRow = FP8 ? kLatentDim : kLatentDim * 2;
+  static constexpr int kRopeRow = FP8 ? kRopeDim : kRopeDim * 2;
+  static constexpr int kLatRegion = kTileTokens * kLatRow;
+  static constexpr int kScaleOff = kLatRegion + kTileTokens * kRopeRow;  // FP8 only
+  static constexpr int kTileBytes = FP8 ? ((kScaleOff + kTileTokens * 4 + 511) / 512) * 512 : kScaleOff;
+  static constexpr int kRing = FP8 ? 7 : 4;
+  static constexpr int kTableOff = kRing * kTileBytes;                 // int[kTableEntries]
+  static constexpr int kPOff = kTableOff + kTableEntries * 4;          // P[2][4 waves][64 lanes] x 16 B
+  static constexpr int kAlphaOff = kPOff + 2 * kScoreWaves * 64 * 16;  // alpha[2][4][64] fp32
+  static constexpr int kInvOff = kAlphaOff + 2 * kScoreWaves * 64 * 4; // 1/denominator[4][64] fp32
+  static constexpr int kFlagOff = kInvOff + kScoreWaves * 64 * 4;      // rescale flag[2][4] int
+  static constexpr int kLdsBytes = kFlagOff + 64;
+  static_assert(kLdsBytes <= 160 * 1024, "one workgroup owns the LDS of a CU");
+  __device__ static __forceinline__ int Slot(int i) { return (kRing == 4 ? (i & 3) : (i % kRing)) * kTileBytes; }
+};
+constexpr int kRowsPerWave = kTileTokens / kWaves;           // bf16: latent rows one wave fetches per tile
+constexpr float kRescaleThreshold = 8.0f;                    // log2 domain
+constexpr int kKAhead = 8;                                   // bf16 K fragments in flight ahead of their MFMA
+constexpr int kKAhead8 = 4;                                  // FP8 K reads (two fragments each) in flight
+constexpr int kVAhead = 4;                                   // V fragments in flight
 
 __device__ __forceinline__ int Uniform(int v) { return __builtin_amdgcn_readfirstlane(v); }
 
@@ -134,10 +146,11 @@ __device__ __forceinline__ int SwizzleLat(int token) {
   return (g32 << 1) | ((token >> 3) & 1);
 }
 __device__ __forceinline__ int SwizzleRope(int token) { return (token >> 1) & 7; }
-__device__ __forceinline__ int LatOffset(int token, int chunk) { return token * kLatRowBytes + ((chunk ^ SwizzleLat(token)) << 4); }
-__device__ __forceinline__ int RopeOffset(int token, int chunk) {
-  return kLatRegion + token * kRopeRowBytes + ((chunk ^ SwizzleRope(token)) << 4);
-}
+// FP8 rows (512 B of codes): 4-bit XOR that is distinct over 16 consecutive tokens (K reads) and
+// over the token sets {0..3, 8..11, 16..19, 24..27} and {4..7, 12..15, 20..23, 28..31} (the rows
+// 32 lanes of a transposed 8-bit V read touch). Rope rows (64 B, four per 256 B): XOR by token/4.
+__device__ __forceinline__ int SwizzleLat8(int token) { return (token & 15) ^ ((token >> 4) << 2); }
+__device__ __forceinline__ int SwizzleRope8(int token) { return (token >> 2) & 3; }
 
 __device__ __forceinline__ u32x4 GlobalLoad16(const char* p) { return *reinterpret_cast<const u32x4*>(p); }
 
@@ -163,19 +176,19 @@ __device__ __forceinline__ void DirectLoad16PerLane(const char* lane_pointer, un
                : "v"(lane_pointer), "s"(__builtin_amdgcn_readfirstlane(lds_wave_base))
                : "memory", "m0");
 }
-// Waits until at most `tiles` later tiles' worth of this wave's loads are outstanding (loads
-// complete in issue order); `per_tile` is 4 or 5 (waves that also fetch rope rows).
-__device__ __forceinline__ void WaitLoads(int tiles, int per_tile) {
-  if (tiles == 2 && per_tile == 4) {
-    asm volatile("s_waitcnt vmcnt(8)" ::: "memory");
-  } else if (tiles == 2 && per_tile == 5) {
-    asm volatile("s_waitcnt vmcnt(10)" ::: "memory");
-  } else if (tiles == 1 && per_tile == 4) {
-    asm volatile("s_waitcnt vmcnt(4)" ::: "memory");
-  } else if (tiles == 1 && per_tile == 5) {
-    asm volatile("s_waitcnt vmcnt(5)" ::: "memory");
-  } else {
-    asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+// Waits until at most `newer` of this wave's vector-memory loads are outstanding (loads complete
+// in issue order; the count is an immediate of s_waitcnt, hence the switch).
+__device__ __forceinline__ void WaitLoads(int newer) {
+  switch (newer) {
+#define MLAKV_WAIT_CASE(n) \
+  case n:                  \
+    asm volatile("s_waitcnt vmcnt(" #n ")" ::: "memory"); \
+    break;
+    MLAKV_WAIT_CASE(2) MLAKV_WAIT_CASE(3) MLAKV_WAIT_CASE(4) MLAKV_WAIT_CASE(5) MLAKV_WAIT_CASE(6) MLAKV_WAIT_CASE(8)
+    MLAKV_WAIT_CASE(9) MLAKV_WAIT_CASE(10) MLAKV_WAIT_CASE(12) MLAKV_WAIT_CASE(15)
+#undef MLAKV_WAIT_CASE
+    default:
+      asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
   }
 }
 
@@ -265,6 +278,7 @@ __device__ __forceinline__ int LoadsPerTile(int wave) { return kRowsPerWave + (w
 template <bool ALIGNED>
 __device__ __forceinline__ bool IssueTileBf16(const AttnArgs& a, TileMap<ALIGNED>& map, const IssueLane& il, int tile,
                                               unsigned buf, unsigned char* buf_ptr, int tid) {
+  using G = Geom<false>;
   const int lane = tid & 63, wave = Uniform(tid >> 6);
   const bool rope_wave = wave >= kScoreWaves;
   const int rope_group = wave - kScoreWaves;
@@ -277,8 +291,8 @@ __device__ __forceinline__ bool IssueTileBf16(const AttnArgs& a, TileMap<ALIGNED
     const int64_t pitch = kWaves * a.latent.row_stride;
     const char* rope = a.rope.base + block * a.rope.block_stride + (slot0 + 8 * rope_group) * a.rope.row_stride;
 #pragma unroll
-    for (int i = 0; i < kRowsPerWave; ++i) DirectLoad16(latent + i * pitch, il.lat[i & 1], buf + (wave + kWaves * i) * kLatRowBytes);
-    if (rope_wave) DirectLoad16(rope, il.rope, buf + kLatRegion + rope_group * 8 * kRopeRowBytes);
+    for (int i = 0; i < kRowsPerWave; ++i) DirectLoad16(latent + i * pitch, il.lat[i & 1], buf + (wave + kWaves * i) * G::kLatRow);
+    if (rope_wave) DirectLoad16(rope, il.rope, buf + G::kLatRegion + rope_group * 8 * G::kRopeRow);
     return true;
   }
   // Rare path (last tile of a sequence, unaligned block sizes, bad table entries): one row at a
@@ -292,9 +306,9 @@ __device__ __forceinline__ bool IssueTileBf16(const AttnArgs& a, TileMap<ALIGNED
     all_real = all_real && real;
     if (real) {
       const char* src = a.latent.base + Uniform(block) * a.latent.block_stride + Uniform(slot) * a.latent.row_stride;
-      DirectLoad16(src, (lane ^ SwizzleLat(row)) << 4, buf + row * kLatRowBytes);
+      DirectLoad16(src, (lane ^ SwizzleLat(row)) << 4, buf + row * G::kLatRow);
     } else {
-      *reinterpret_cast<u32x4*>(buf_ptr + row * kLatRowBytes + lane * 16) = u32x4{0u, 0u, 0u, 0u};
+      *reinterpret_cast<u32x4*>(buf_ptr + row * G::kLatRow + lane * 16) = u32x4{0u, 0u, 0u, 0u};
     }
   }
   if (!rope_wave) return all_real;
@@ -302,7 +316,7 @@ __device__ __forceinline__ bool IssueTileBf16(const AttnArgs& a, TileMap<ALIGNED
   int rblock, rslot;
   const bool rreal = map.Row(tile, 8 * rope_group + (lane >> 3), &rblock, &rslot);
   const char* rsrc = a.rope.base + rblock * a.rope.block_stride + rslot * a.rope.row_stride + il.rope_chunk;
-  const unsigned rdst = buf + kLatRegion + rope_group * 8 * kRopeRowBytes;
+  const unsigned rdst = buf + G::kLatRegion + rope_group * 8 * G::kRopeRow;
   if (__builtin_amdgcn_ballot_w64(!rreal) == 0) {
     DirectLoad16PerLane(rsrc, rdst);
     return all_real;
@@ -310,39 +324,71 @@ __device__ __forceinline__ bool IssueTileBf16(const AttnArgs& a, TileMap<ALIGNED
   if (rreal) {
     DirectLoad16PerLane(rsrc, rdst);
   } else {
-    *reinterpret_cast<u32x4*>(buf_ptr + kLatRegion + rope_group * 8 * kRopeRowBytes + lane * 16) = u32x4{0u, 0u, 0u, 0u};
+    *reinterpret_cast<u32x4*>(buf_ptr + G::kLatRegion + rope_group * 8 * G::kRopeRow + lane * 16) = u32x4{0u, 0u, 0u, 0u};
   }
   return false;
 }
 
-// ---- FP8 tiles: global -> registers -> (dequantise) -> LDS ------------------------------------
+// ---- FP8 tiles: direct global -> LDS, codes and row scales as they are in the cache -------------
 
-// 2 latent chunks + (first two waves) 1 rope chunk of 16 codes per thread, and their row
-// scales (0 for a row that is not real).
-struct TileRegsFp8 {
-  u32x4 v[3];
-  float scale[3];
+// Wave w of 8 owns the latent row pairs {2w, 2w+1} and {16+2w, 17+2w} (a 512-byte row is half a
+// wave access); waves 4 and 5 also own the rope rows 16(w-4) .. +15 (64 B each), wave 6 the 32
+// row scales (128 B, eight lanes).
+struct IssueLane8 {
+  int lat[2];  // byte offset of this lane's chunk from the first row of pair i
+  int rope;
 };
 
+__device__ __forceinline__ int LoadsPerTile8(int wave) { return 2 + (wave >= 4 && wave <= 6 ? 1 : 0); }
+
+// FP8 counterpart of IssueTileBf16. The rare path stages through registers; rows that are not
+// real get zero codes and a zero scale.
 template <bool ALIGNED>
-__device__ __forceinline__ void LoadTileFp8(TileRegsFp8& r, const AttnArgs& a, TileMap<ALIGNED>& map, int tile, int tid) {
+__device__ __forceinline__ bool IssueTileFp8(const AttnArgs& a, TileMap<ALIGNED>& map, const IssueLane8& il, int tile,
+                                             unsigned buf, unsigned char* buf_ptr, int tid) {
+  using G = Geom<true>;
+  const int lane = tid & 63, wave = Uniform(tid >> 6);
   map.Begin(tile);
-  int block[3], slot[3];
-  bool real[3];
+  const int rows = map.seq_len - tile * kTileTokens;  // real rows in this tile, >= 1
+  if (ALIGNED && rows >= kTileTokens && map.tile_block >= 0) {
+    const int block = Uniform(map.tile_block), slot0 = Uniform(map.tile_slot0);
+    const char* latent = a.latent.base + block * a.latent.block_stride + (slot0 + 2 * wave) * a.latent.row_stride;
+    const int64_t pitch = 16 * a.latent.row_stride;
 #pragma unroll
-  for (int i = 0; i < 3; ++i) {
-    const int token = i < 2 ? (tid + kThreads * i) >> 5 : (tid & 127) >> 2;
-    real[i] = map.Row(tile, token, &block[i], &slot[i]);
+    for (int i = 0; i < 2; ++i) DirectLoad16(latent + i * pitch, il.lat[i], buf + (2 * wave + 16 * i) * G::kLatRow);
+    if (wave == 4 || wave == 5) {
+      const int h = wave - 4;
+      const char* rope = a.rope.base + block * a.rope.block_stride + (slot0 + 16 * h) * a.rope.row_stride;
+      DirectLoad16(rope, il.rope, buf + G::kLatRegion + 16 * h * G::kRopeRow);
+    } else if (wave == 6) {
+      const char* scale = a.scale.base + block * a.scale.block_stride + slot0 * 4;
+      if (lane < kTileTokens * 4 / 16) DirectLoad16(scale, lane * 16, buf + G::kScaleOff);
+    }
+    return true;
   }
-#pragma unroll
-  for (int i = 0; i < 3; ++i) {
-    if (i == 2 && tid >= 128) break;  // wave-uniform: 32 rope rows x 4 chunks
-    const int chunk = i < 2 ? (tid + kThreads * i) & 31 : tid & 3;
-    const Plane& plane = i < 2 ? a.latent : a.rope;
-    r.v[i] = GlobalLoad16(plane.base + block[i] * plane.block_stride + slot[i] * plane.row_stride + chunk * 16);
-    const float scale = reinterpret_cast<const float*>(a.scale.base + block[i] * a.scale.block_stride)[slot[i]];
-    r.scale[i] = real[i] ? scale : 0.0f;
+#pragma nounroll
+  for (int i = 0; i < 2; ++i) {
+    const int row = 2 * wave + 16 * i + (lane >> 5);
+    int block, slot;
+    const bool real = map.Row(tile, row, &block, &slot);
+    u32x4 codes = GlobalLoad16(a.latent.base + block * a.latent.block_stride + slot * a.latent.row_stride + (lane & 31) * 16);
+    if (!real) codes = u32x4{0u, 0u, 0u, 0u};
+    *reinterpret_cast<u32x4*>(buf_ptr + row * G::kLatRow + (((lane & 31) ^ SwizzleLat8(row)) << 4)) = codes;
   }
+  if (wave == 4 || wave == 5) {
+    const int row = 16 * (wave - 4) + (lane >> 2);
+    int block, slot;
+    const bool real = map.Row(tile, row, &block, &slot);
+    u32x4 codes = GlobalLoad16(a.rope.base + block * a.rope.block_stride + slot * a.rope.row_stride + (lane & 3) * 16);
+    if (!real) codes = u32x4{0u, 0u, 0u, 0u};
+    *reinterpret_cast<u32x4*>(buf_ptr + G::kLatRegion + row * G::kRopeRow + (((lane & 3) ^ SwizzleRope8(row)) << 4)) = codes;
+  } else if (wave == 6 && lane < kTileTokens) {
+    int block, slot;
+    const bool real = map.Row(tile, lane, &block, &slot);
+    const float scale = reinterpret_cast<const float*>(a.scale.base + block * a.scale.block_stride)[slot];
+    reinterpret_cast<float*>(buf_ptr + G::kScaleOff)[lane] = real ? scale : 0.0f;
+  }
+  return false;
 }
 
 __device__ __forceinline__ unsigned int PackBf16(float lo, float hi) {
@@ -350,53 +396,21 @@ __device__ __forceinline__ unsigned int PackBf16(float lo, float hi) {
   return __builtin_bit_cast(unsigned int, packed);
 }
 
-// Four E4M3 codes of one dword -> four bf16 (two dwords), scaled.
-__device__ __forceinline__ void Dequant4(unsigned int codes, float scale, unsigned int* lo, unsigned int* hi) {
-  const f32x2 a = __builtin_amdgcn_cvt_pk_f32_fp8(static_cast<int>(codes), false);
-  const f32x2 b = __builtin_amdgcn_cvt_pk_f32_fp8(static_cast<int>(codes), true);
-  *lo = PackBf16(a.x * scale, a.y * scale);
-  *hi = PackBf16(b.x * scale, b.y * scale);
-}
-
-__device__ __forceinline__ void StoreTileFp8(const TileRegsFp8& r, unsigned char* buf, int tid) {
-#pragma unroll
-  for (int i = 0; i < 3; ++i) {
-    if (i == 2 && tid >= 128) break;
-    u32x4 first, second;
-    unsigned int lo, hi;
-    Dequant4(r.v[i].x, r.scale[i], &lo, &hi);
-    first.x = lo;
-    first.y = hi;
-    Dequant4(r.v[i].y, r.scale[i], &lo, &hi);
-    first.z = lo;
-    first.w = hi;
-    Dequant4(r.v[i].z, r.scale[i], &lo, &hi);
-    second.x = lo;
-    second.y = hi;
-    Dequant4(r.v[i].w, r.scale[i], &lo, &hi);
-    second.z = lo;
-    second.w = hi;
-    if (r.scale[i] == 0.0f) {  // not a real row: zeros, whatever the fetched codes were
-      first = u32x4{0u, 0u, 0u, 0u};
-      second = first;
-    }
-    if (i < 2) {
-      const int idx = tid + kThreads * i;
-      const int token = idx >> 5, chunk = 2 * (idx & 31);
-      *reinterpret_cast<u32x4*>(buf + LatOffset(token, chunk)) = first;
-      *reinterpret_cast<u32x4*>(buf + LatOffset(token, chunk + 1)) = second;
-    } else {
-      const int token = tid >> 2, chunk = 2 * (tid & 3);
-      *reinterpret_cast<u32x4*>(buf + RopeOffset(token, chunk)) = first;
-      *reinterpret_cast<u32x4*>(buf + RopeOffset(token, chunk + 1)) = second;
-    }
-  }
+// Eight E4M3 codes (two dwords) -> eight bf16, exactly (unit scale; the row scale is applied to
+// the scores and to P instead, in fp32).
+__device__ __forceinline__ bf16x8 CodesToBf16(unsigned lo, unsigned hi) {
+  const bf16x2 a = __builtin_amdgcn_cvt_scalef32_pk_bf16_fp8(lo, 1.0f, false);
+  const bf16x2 b = __builtin_amdgcn_cvt_scalef32_pk_bf16_fp8(lo, 1.0f, true);
+  const bf16x2 c = __builtin_amdgcn_cvt_scalef32_pk_bf16_fp8(hi, 1.0f, false);
+  const bf16x2 d = __builtin_amdgcn_cvt_scalef32_pk_bf16_fp8(hi, 1.0f, true);
+  return bf16x8{a.x, a.y, b.x, b.y, c.x, c.y, d.x, d.y};
 }
 
 // ---- main kernel -------------------------------------------------------------------
 
 template <bool FP8, bool ALIGNED>
 __global__ __launch_bounds__(kThreads) void MlaDecodeKernel(AttnArgs a) {
+  using G = Geom<FP8>;
   extern __shared__ __attribute__((aligned(16))) unsigned char lds[];
   const unsigned lds_base = static_cast<unsigned>(reinterpret_cast<size_t>((__attribute__((address_space(3))) unsigned char*)lds));
   const int tid = threadIdx.x;
@@ -410,18 +424,21 @@ __global__ __launch_bounds__(kThreads) void MlaDecodeKernel(AttnArgs a) {
   const bool active = head_base < a.heads;  // wave-uniform
   const int head = head_base + i16;
   const bool direct = a.max_chunks == 1;  // single chunk: write the final output here
-  const int per_tile = LoadsPerTile(wave);
+  const int per_tile = FP8 ? LoadsPerTile8(wave) : LoadsPerTile(wave);
   MLAKV_STAMP(0);
 
-  // Q fragments (score waves): lane (head i16, k-group g) holds Q[head][32*ks + 8g .. +7].
-  // Issued first so that they travel while the lengths and the block table are fetched.
+  // Q fragments (score waves): lane (head i16, k-group g) holds, for k-step ks, the eight query
+  // elements that meet the lane's K fragment of that step: Q[head][32 ks + 8g .. +7] for bf16
+  // tiles; for FP8 tiles one 16-byte K read feeds two k-steps, so the order inside each 64-wide
+  // window is Q[head][64 (ks/2) + 16g + 8 (ks&1) .. +7]. Issued first so that they travel while
+  // the lengths and the block table are fetched.
   bf16x8 q[kKSteps];
   if (score_wave && active) {
     const char* q_latent = a.q_latent + seq * a.q_latent_seq_stride + head * a.q_latent_head_stride;
     const char* q_rope = a.q_rope + seq * a.q_rope_seq_stride + head * a.q_rope_head_stride;
 #pragma unroll
     for (int ks = 0; ks < kKSteps; ++ks) {
-      const int d0 = 32 * ks + 8 * g;
+      const int d0 = FP8 ? 64 * (ks >> 1) + 16 * g + 8 * (ks & 1) : 32 * ks + 8 * g;
       const char* p = d0 < kLatentDim ? q_latent + d0 * 2 : q_rope + (d0 - kLatentDim) * 2;
       q[ks] = __builtin_bit_cast(bf16x8, GlobalLoad16(p));
     }
@@ -431,7 +448,7 @@ __global__ __launch_bounds__(kThreads) void MlaDecodeKernel(AttnArgs a) {
   // table row, not by the sequence length, so it does not wait for the length to arrive;
   // entries past the sequence are never used.
   const int tile_begin = chunk_index * a.chunk_tiles;
-  int* table_lds = reinterpret_cast<int*>(lds + kTableOff);
+  int* table_lds = reinterpret_cast<int*>(lds + G::kTableOff);
   TileMap<ALIGNED> map;
   map.entries = table_lds;
   map.block_size = a.block_size;
@@ -472,12 +489,31 @@ __global__ __launch_bounds__(kThreads) void MlaDecodeKernel(AttnArgs a) {
 
   // Direct loads: lane L of a latent row fetches chunk L ^ swizzle(row); rows of this wave.
   IssueLane il;
+  IssueLane8 il8;
+  if (FP8) {
 #pragma unroll
-  for (int j = 0; j < 2; ++j) il.lat[j] = (lane ^ SwizzleLat(wave + kWaves * j)) << 4;
-  il.rope_chunk = ((lane & 7) ^ SwizzleRope(8 * (wave - kScoreWaves) + (lane >> 3))) << 4;
-  il.rope = (lane >> 3) * static_cast<int>(a.rope.row_stride) + il.rope_chunk;
+    for (int j = 0; j < 2; ++j) {
+      const int row = 2 * wave + 16 * j + (lane >> 5);
+      il8.lat[j] = (lane >> 5) * static_cast<int>(a.latent.row_stride) + (((lane & 31) ^ SwizzleLat8(row)) << 4);
+    }
+    const int rope_row = 16 * (wave & 1) + (lane >> 2);
+    il8.rope = (lane >> 2) * static_cast<int>(a.rope.row_stride) + (((lane & 3) ^ SwizzleRope8(rope_row)) << 4);
+  } else {
+#pragma unroll
+    for (int j = 0; j < 2; ++j) il.lat[j] = (lane ^ SwizzleLat(wave + kWaves * j)) << 4;
+    il.rope_chunk = ((lane & 7) ^ SwizzleRope(8 * (wave - kScoreWaves) + (lane >> 3))) << 4;
+    il.rope = (lane >> 3) * static_cast<int>(a.rope.row_stride) + il.rope_chunk;
+  }
 
-  const auto ring = [&](int i) __attribute__((always_inline)) { return (i & (kRing - 1)) * kTileBytes; };
+  const auto ring = [&](int i) __attribute__((always_inline)) { return G::Slot(i); };
+  // Issues this wave's loads of chunk-relative tile t; returns whether their number is known.
+  const auto issue = [&](int t) __attribute__((always_inline)) {
+    if constexpr (FP8) {
+      return IssueTileFp8(a, map, il8, tile_begin + t, lds_base + ring(t), lds + ring(t), tid);
+    } else {
+      return IssueTileBf16(a, map, il, tile_begin + t, lds_base + ring(t), lds + ring(t), tid);
+    }
+  };
 
   // The query must have arrived before the tile loads are issued: the compiler's own wait for
   // it would otherwise also wait for every tile load issued in between.
@@ -488,58 +524,48 @@ __global__ __launch_bounds__(kThreads) void MlaDecodeKernel(AttnArgs a) {
   MLAKV_STAMP(1);
   __syncthreads();  // table entries visible
 
-  // Prologue: tiles 0..2 on their way, tile 0 landed and published.
-  TileRegsFp8 regs;
-  bool newest_known = false;  // the newest tile in flight took exactly per_tile loads of this wave
-  if (FP8) {
-    LoadTileFp8(regs, a, map, tile_begin, tid);
-    StoreTileFp8(regs, lds + ring(0), tid);
-    if (1 < ntiles) {
-      LoadTileFp8(regs, a, map, tile_begin + 1, tid);
-      StoreTileFp8(regs, lds + ring(1), tid);
-    }
-    if (2 < ntiles) LoadTileFp8(regs, a, map, tile_begin + 2, tid);
-  } else {
-    int in_flight = 0;  // tiles 1 and 2
-    bool known = true;
-    IssueTileBf16(a, map, il, tile_begin, lds_base + ring(0), lds + ring(0), tid);
-    for (int i = 1; i < 3 && i < ntiles; ++i) {
-      newest_known = IssueTileBf16(a, map, il, tile_begin + i, lds_base + ring(i), lds + ring(i), tid);
-      known = known && newest_known;
-      ++in_flight;
-    }
-    MLAKV_STAMP(2);
-    WaitLoads(known ? in_flight : 0, per_tile);
+  // Prologue: tiles 0 .. kRing-2 on their way, tile 0 landed and published. A tile whose load
+  // count is not known (rare path) makes every wait up to and including its own a full one.
+  int last_unknown = -1;  // newest tile issued with an unknown number of loads
+  int issued = 0;         // tiles issued so far
+  for (; issued < G::kRing - 1 && issued < ntiles; ++issued) {
+    if (!issue(issued)) last_unknown = issued;
   }
+  MLAKV_STAMP(2);
+  WaitLoads(last_unknown >= 0 ? 0 : (issued - 1) * per_tile);
   __syncthreads();
   MLAKV_STAMP(3);
 
-  // Top of iteration i, both roles: tile i+1 must have landed (tile i+2 may still be in
+  // Top of iteration i, both roles: tile i+1 must have landed (later tiles may still be in
   // flight); the barrier publishes it together with P(i) and retires every wave's reads of
-  // tile i-1, whose ring slot tile i+3 then reuses.
-  const auto advance = [&](int i) __attribute__((always_inline)) {
+  // tile i-1, whose ring slot the next tile to be issued reuses.
+  const auto publish = [&](int i) __attribute__((always_inline)) {
     MLAKV_STAMP(4 + 6 * i);
-    if (!FP8 && i + 1 < ntiles) WaitLoads(i + 2 < ntiles && newest_known ? 1 : 0, per_tile);
+    if (i + 1 < ntiles) WaitLoads(last_unknown >= i + 1 ? 0 : (issued - (i + 2)) * per_tile);
     __syncthreads();
     MLAKV_STAMP(5 + 6 * i);
-    if (FP8) {
-      if (i + 2 < ntiles) StoreTileFp8(regs, lds + ring(i + 2), tid);
-      if (i + 3 < ntiles) LoadTileFp8(regs, a, map, tile_begin + i + 3, tid);
-    } else if (i + 3 < ntiles) {
-      newest_known = IssueTileBf16(a, map, il, tile_begin + i + 3, lds_base + ring(i + 3), lds + ring(i + 3), tid);
+  };
+  // Issues the next tile of the ring (tile i + kRing - 1 during iteration i), right after
+  // publish(i): the memory-bound shapes want every load in flight as early as possible (issuing
+  // after the score waves' MFMA phase, to skew the two MFMA phases of a SIMD, gained 6 % where
+  // the kernel is compute-bound and lost 4 % where it is not).
+  const auto issue_next = [&](int i) __attribute__((always_inline)) {
+    if (issued < ntiles) {
+      if (!issue(issued)) last_unknown = issued;
+      ++issued;
     }
     MLAKV_STAMP(6 + 6 * i);
   };
 
-  unsigned char* p_lds = lds + kPOff + (hw * 64 + lane) * 16;           // + parity * kScoreWaves * 64 * 16
-  float* alpha_lds = reinterpret_cast<float*>(lds + kAlphaOff) + hw * 64 + lane;  // + parity * kScoreWaves * 64
-  float* inv_lds = reinterpret_cast<float*>(lds + kInvOff) + hw * 64 + lane;
-  int* flag_lds = reinterpret_cast<int*>(lds + kFlagOff) + hw;          // + parity * kScoreWaves
+  unsigned char* p_lds = lds + G::kPOff + (hw * 64 + lane) * 16;           // + parity * kScoreWaves * 64 * 16
+  float* alpha_lds = reinterpret_cast<float*>(lds + G::kAlphaOff) + hw * 64 + lane;  // + parity * kScoreWaves * 64
+  float* inv_lds = reinterpret_cast<float*>(lds + G::kInvOff) + hw * 64 + lane;
+  int* flag_lds = reinterpret_cast<int*>(lds + G::kFlagOff) + hw;          // + parity * kScoreWaves
 
   if (score_wave) {
     // ---------------------------------------------------------------- score waves
-    // K reads: token = 16t + i16, chunk = 4 ks + g (latent, ks < 16) or 4 (ks - 16) + g (rope).
-    const int k_lat = i16 * kLatRowBytes, k_rope = kLatRegion + i16 * kRopeRowBytes;
+    // bf16 K reads: token = 16t + i16, chunk = 4 ks + g (latent, ks < 16) or 4 (ks - 16) + g (rope).
+    const int k_lat = i16 * Geom<false>::kLatRow, k_rope = Geom<false>::kLatRegion + i16 * Geom<false>::kRopeRow;
     int k_e[4], kr_e[2];
 #pragma unroll
     for (int j = 0; j < 4; ++j) k_e[j] = ((4 * j + g) ^ SwizzleLat(i16)) << 4;
@@ -548,9 +574,22 @@ __global__ __launch_bounds__(kThreads) void MlaDecodeKernel(AttnArgs a) {
     // K fragment of pipeline step `step` (k-step step/2, token subtile step&1) of the tile at `buf`.
     const auto k_frag = [&](const unsigned char* buf, int step) __attribute__((always_inline)) {
       const int ks = step >> 1, t = step & 1;
-      const int offset = ks < 16 ? k_lat + (ks >> 2) * 256 + k_e[ks & 3] + t * 16 * kLatRowBytes
-                                 : k_rope + kr_e[ks & 1] + t * 16 * kRopeRowBytes;
+      const int offset = ks < 16 ? k_lat + (ks >> 2) * 256 + k_e[ks & 3] + t * 16 * Geom<false>::kLatRow
+                                 : k_rope + kr_e[ks & 1] + t * 16 * Geom<false>::kRopeRow;
       return *reinterpret_cast<const bf16x8*>(buf + offset);
+    };
+    // FP8 K reads: read u = 2 kp + t fetches the 16 codes k = 64 kp + 16 g .. +15 of token 16t + i16
+    // (k-steps 2kp and 2kp+1): chunk (4 kp + g) ^ swizzle(token) of the 512-byte row; kp = 8 is the
+    // rope row (chunk g ^ swizzle). The tile base is a multiple of 512, so the XOR with kp << 6 is
+    // applied to the lane-constant part.
+    int k8_lat[2];
+#pragma unroll
+    for (int t = 0; t < 2; ++t) k8_lat[t] = (16 * t + i16) * Geom<true>::kLatRow + ((g ^ SwizzleLat8(16 * t + i16)) << 4);
+    const int k8_rope = Geom<true>::kLatRegion + i16 * Geom<true>::kRopeRow + ((g ^ SwizzleRope8(i16)) << 4);
+    const auto k8_read = [&](const unsigned char* buf, int u) __attribute__((always_inline)) {
+      const int kp = u >> 1, t = u & 1;
+      const int offset = kp < 8 ? (k8_lat[t] ^ (kp << 6)) : k8_rope + t * 16 * Geom<true>::kRopeRow;
+      return *reinterpret_cast<const u32x4*>(buf + offset);
     };
 
     float m_ref = -__builtin_inff();  // reference maximum of the exponentials, log2 domain
@@ -563,17 +602,37 @@ __global__ __launch_bounds__(kThreads) void MlaDecodeKernel(AttnArgs a) {
       f32x4 acc[4];
 #pragma unroll
       for (int j = 0; j < 4; ++j) acc[j] = f32x4{0.f, 0.f, 0.f, 0.f};
-      bf16x8 kf[kKAhead];
+      f32x4 row_scale[2];  // FP8: scales of tokens 4g+j and 16+4g+j
+      if constexpr (FP8) {
+        const float* scales = reinterpret_cast<const float*>(buf + G::kScaleOff);
+        row_scale[0] = *reinterpret_cast<const f32x4*>(scales + 4 * g);
+        row_scale[1] = *reinterpret_cast<const f32x4*>(scales + 16 + 4 * g);
+        u32x4 kr[kKAhead8];
 #pragma unroll
-      for (int d = 0; d < kKAhead; ++d) kf[d] = k_frag(buf, d);
-      __builtin_amdgcn_sched_barrier(0);
-      StaticFor<kQkSteps>([&](auto step_c) __attribute__((always_inline)) {
-        constexpr int step = decltype(step_c)::value;
-        constexpr int slot = (step & 1) * 2 + ((step >> 1) & 1);  // two accumulators per token subtile
-        acc[slot] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(kf[step % kKAhead], q[step >> 1], acc[slot], 0, 0, 0);
-        if constexpr (step + kKAhead < kQkSteps) kf[step % kKAhead] = k_frag(buf, step + kKAhead);
+        for (int d = 0; d < kKAhead8; ++d) kr[d] = k8_read(buf, d);
         __builtin_amdgcn_sched_barrier(0);
-      });
+        StaticFor<kKSteps>([&](auto u_c) __attribute__((always_inline)) {
+          constexpr int u = decltype(u_c)::value;  // kp = u / 2, token subtile t = u & 1
+          const u32x4 codes = kr[u % kKAhead8];
+          if constexpr (u + kKAhead8 < kKSteps) kr[u % kKAhead8] = k8_read(buf, u + kKAhead8);
+          constexpr int t = u & 1, kp = u >> 1;
+          acc[2 * t] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(CodesToBf16(codes.x, codes.y), q[2 * kp], acc[2 * t], 0, 0, 0);
+          acc[2 * t + 1] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(CodesToBf16(codes.z, codes.w), q[2 * kp + 1], acc[2 * t + 1], 0, 0, 0);
+          __builtin_amdgcn_sched_barrier(0);
+        });
+      } else {
+        bf16x8 kf[kKAhead];
+#pragma unroll
+        for (int d = 0; d < kKAhead; ++d) kf[d] = k_frag(buf, d);
+        __builtin_amdgcn_sched_barrier(0);
+        StaticFor<kQkSteps>([&](auto step_c) __attribute__((always_inline)) {
+          constexpr int step = decltype(step_c)::value;
+          constexpr int slot = (step & 1) * 2 + ((step >> 1) & 1);  // two accumulators per token subtile
+          acc[slot] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(kf[step % kKAhead], q[step >> 1], acc[slot], 0, 0, 0);
+          if constexpr (step + kKAhead < kQkSteps) kf[step % kKAhead] = k_frag(buf, step + kKAhead);
+          __builtin_amdgcn_sched_barrier(0);
+        });
+      }
       MLAKV_STAMP(7 + 6 * (tile_rel - 1));
       // lane holds tokens 4g+j (x[0..3]) and 16+4g+j (x[4..7]) of head i16
       float x[8];
@@ -581,6 +640,10 @@ __global__ __launch_bounds__(kThreads) void MlaDecodeKernel(AttnArgs a) {
       for (int j = 0; j < 4; ++j) {
         x[j] = (acc[0][j] + acc[1][j]) * a.scale_log2;
         x[4 + j] = (acc[2][j] + acc[3][j]) * a.scale_log2;
+        if constexpr (FP8) {  // the codes were multiplied unscaled
+          x[j] *= row_scale[0][j];
+          x[4 + j] *= row_scale[1][j];
+        }
       }
       const int valid = seq_len - (tile_begin + tile_rel) * kTileTokens;  // >= 1
       if (valid < kTileTokens) {  // wave-uniform: only the last tile of a sequence
@@ -608,7 +671,7 @@ __global__ __launch_bounds__(kThreads) void MlaDecodeKernel(AttnArgs a) {
       for (int j = 0; j < 8; ++j) {
         const float e = __builtin_amdgcn_exp2f(x[j] - m_ref);
         sum += e;
-        p[j] = static_cast<__bf16>(e);
+        p[j] = static_cast<__bf16>(FP8 ? e * row_scale[j >> 2][j & 3] : e);  // FP8: V is multiplied unscaled as well
       }
       l_run += sum;
       *reinterpret_cast<bf16x8*>(p_lds + parity * kScoreWaves * 64 * 16) = p;
@@ -617,7 +680,8 @@ __global__ __launch_bounds__(kThreads) void MlaDecodeKernel(AttnArgs a) {
 
     if (active) score_tile(0);
     for (int i = 0; i < ntiles; ++i) {
-      advance(i);
+      publish(i);
+      issue_next(i);
       if (active && i + 1 < ntiles) score_tile(i + 1);
     }
     if (active) {
@@ -637,18 +701,36 @@ __global__ __launch_bounds__(kThreads) void MlaDecodeKernel(AttnArgs a) {
     MLAKV_STAMP(30);
   } else {
     // ---------------------------------------------------------------- output waves
-    // V reads: token = (16 +) 4g + i16/4, chunk = 2n + (i16 & 3) / 2, 8-byte half i16 & 1.
+    // bf16 V reads: token = (16 +) 4g + i16/4, chunk = 2n + (i16 & 3) / 2, 8-byte half i16 & 1.
     const int v_row = 4 * g + (i16 >> 2);
-    const int v_lane = v_row * kLatRowBytes + (i16 & 1) * 8;
+    const int v_lane = v_row * Geom<false>::kLatRow + (i16 & 1) * 8;
     int v_e[8];
 #pragma unroll
     for (int j = 0; j < 8; ++j) v_e[j] = ((2 * j + ((i16 & 3) >> 1)) ^ SwizzleLat(v_row)) << 4;
-    // V^T fragment of output tile n (dv 16n..16n+15) over the 32 tokens of the tile at `buf`.
-    const auto v_frag = [&](const unsigned char* buf, int n) __attribute__((always_inline)) {
-      const unsigned char* addr = buf + v_lane + (n >> 3) * 256 + v_e[n & 7];
-      const s16x4 lo = __builtin_amdgcn_ds_read_tr16_b64_v4i16((__attribute__((address_space(3))) s16x4*)(addr));
-      const s16x4 hi = __builtin_amdgcn_ds_read_tr16_b64_v4i16((__attribute__((address_space(3))) s16x4*)(addr + 16 * kLatRowBytes));
-      return __builtin_shufflevector(__builtin_bit_cast(bf16x4, lo), __builtin_bit_cast(bf16x4, hi), 0, 1, 2, 3, 4, 5, 6, 7);
+    // FP8 V reads (ds_read_b64_tr_b8: output lane i of a 16-lane group, element e <- byte i & 7 of
+    // the 8 bytes addressed by lane 2e + (i >> 3)): as a source, lane j addresses bytes
+    // 16n + 8 (j & 1) .. +7 of the row of token kappa = j >> 1 (tokens 4g + kappa, 16 + 4g + kappa - 4).
+    const int v8_token = 4 * g + ((i16 >> 1) & 3) + 16 * (i16 >> 3);
+    const int v8_base = v8_token * Geom<true>::kLatRow + (SwizzleLat8(v8_token) << 4) + 8 * (i16 & 1);
+    // Raw V^T fragment of output tile n (dv 16n..16n+15) over the 32 tokens of the tile at `buf`:
+    // eight bf16 for bf16 tiles, eight codes in the low two dwords for FP8 tiles.
+    const auto v_fetch = [&](const unsigned char* buf, int n) __attribute__((always_inline)) {
+      if constexpr (FP8) {
+        const i32x2 codes = __builtin_amdgcn_ds_read_tr8_b64_v2i32((__attribute__((address_space(3))) i32x2*)(buf + (v8_base ^ (n << 4))));
+        return u32x4{static_cast<unsigned>(codes.x), static_cast<unsigned>(codes.y), 0u, 0u};
+      } else {
+        const unsigned char* addr = buf + v_lane + (n >> 3) * 256 + v_e[n & 7];
+        const s16x4 lo = __builtin_amdgcn_ds_read_tr16_b64_v4i16((__attribute__((address_space(3))) s16x4*)(addr));
+        const s16x4 hi = __builtin_amdgcn_ds_read_tr16_b64_v4i16((__attribute__((address_space(3))) s16x4*)(addr + 16 * Geom<false>::kLatRow));
+        return __builtin_bit_cast(u32x4, __builtin_shufflevector(lo, hi, 0, 1, 2, 3, 4, 5, 6, 7));
+      }
+    };
+    const auto v_operand = [&](const u32x4& raw) __attribute__((always_inline)) {
+      if constexpr (FP8) {
+        return CodesToBf16(raw.x, raw.y);
+      } else {
+        return __builtin_bit_cast(bf16x8, raw);
+      }
     };
 
     f32x4 o[kDvTiles];
@@ -656,13 +738,14 @@ __global__ __launch_bounds__(kThreads) void MlaDecodeKernel(AttnArgs a) {
     for (int n = 0; n < kDvTiles; ++n) o[n] = f32x4{0.f, 0.f, 0.f, 0.f};
 
     for (int i = 0; i < ntiles; ++i) {
-      advance(i);
+      publish(i);
+      issue_next(i);
       if (active) {
         const unsigned char* buf = lds + ring(i);
         const int parity = i & 1;
-        bf16x8 vf[kVAhead];
+        u32x4 vf[kVAhead];
 #pragma unroll
-        for (int d = 0; d < kVAhead; ++d) vf[d] = v_frag(buf, d);
+        for (int d = 0; d < kVAhead; ++d) vf[d] = v_fetch(buf, d);
         const bf16x8 p = *reinterpret_cast<const bf16x8*>(p_lds + parity * kScoreWaves * 64 * 16);
         if (Uniform(flag_lds[parity * kScoreWaves]) != 0) {  // the reference maximum moved: rescale O first
           const float alpha = alpha_lds[parity * kScoreWaves * 64];
@@ -672,8 +755,8 @@ __global__ __launch_bounds__(kThreads) void MlaDecodeKernel(AttnArgs a) {
         __builtin_amdgcn_sched_barrier(0);
         StaticFor<kDvTiles>([&](auto n_c) __attribute__((always_inline)) {
           constexpr int n = decltype(n_c)::value;
-          o[n] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(vf[n % kVAhead], p, o[n], 0, 0, 0);
-          if constexpr (n + kVAhead < kDvTiles) vf[n % kVAhead] = v_frag(buf, n + kVAhead);
+          o[n] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(v_operand(vf[n % kVAhead]), p, o[n], 0, 0, 0);
+          if constexpr (n + kVAhead < kDvTiles) vf[n % kVAhead] = v_fetch(buf, n + kVAhead);
           __builtin_amdgcn_sched_barrier(0);
         });
         MLAKV_STAMP(7 + 6 * i);
@@ -771,9 +854,9 @@ template <bool FP8, bool ALIGNED>
 hipError_t Launch(const AttnArgs& args, const dim3& grid, hipStream_t stream) {
   // Dynamic LDS above 64 KB needs the attribute once per kernel and process.
   static const hipError_t prepared = hipFuncSetAttribute(reinterpret_cast<const void*>(&MlaDecodeKernel<FP8, ALIGNED>),
-                                                         hipFuncAttributeMaxDynamicSharedMemorySize, kLdsBytes);
+                                                         hipFuncAttributeMaxDynamicSharedMemorySize, Geom<FP8>::kLdsBytes);
   if (prepared != hipSuccess) return prepared;
-  hipLaunchKernelGGL((MlaDecodeKernel<FP8, ALIGNED>), grid, dim3(kThreads), kLdsBytes, stream, args);
+  hipLaunchKernelGGL((MlaDecodeKernel<FP8, ALIGNED>), grid, dim3(kThreads), Geom<FP8>::kLdsBytes, stream, args);
   return hipGetLastError();
 }
 
