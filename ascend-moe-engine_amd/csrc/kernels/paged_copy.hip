@@ -81,22 +81,6 @@ __device__ __forceinline__ unsigned int F32ToBf16(float v) {
   return bits >> 16;
 }
 
-// OCP E4M3FN encode: round to nearest even, saturate to +-448, subnormal grid 2^-9 below 2^-6.
-__device__ __forceinline__ unsigned int E4m3Encode(float v) {
-  const unsigned int bits = __builtin_bit_cast(unsigned int, v);
-  const unsigned int sign = (bits >> 24) & 0x80u;
-  const unsigned int mag_bits = bits & 0x7fffffffu;
-  if (mag_bits > 0x7f800000u) return sign | 0x7fu;
-  const float mag = __builtin_bit_cast(float, mag_bits);
-  if (mag >= 448.0f) return sign | 0x7eu;
-  if (mag < 0.015625f) return sign | static_cast<unsigned int>(static_cast<int>(__builtin_rintf(mag * 512.0f)));
-  const unsigned int rounded = mag_bits + 0x7ffffu + ((mag_bits >> 20) & 1u);
-  const int exponent = static_cast<int>(rounded >> 23) - 120;
-  const unsigned int mantissa = (rounded >> 20) & 7u;
-  if (exponent > 15 || (exponent == 15 && mantissa == 7u)) return sign | 0x7eu;
-  return sign | (static_cast<unsigned int>(exponent) << 3) | mantissa;
-}
-
 // Eight E4M3 codes -> eight bf16, each decoded value times `scale`, rounded to nearest even.
 __device__ __forceinline__ u32x4 Dequant8(u32x2 codes, float scale) {
   const f32x2 a = __builtin_amdgcn_cvt_pk_f32_fp8(static_cast<int>(codes.x), false);
@@ -137,10 +121,21 @@ __global__ __launch_bounds__(kThreads) void AppendBf16Kernel(AppendArgs a) {
   if (lane < kRopeDim * 2 / 16) Store16(rope_dst + lane * 16, r);
 }
 
+// Two quotients -> two E4M3 codes in the low half of a dword. v_cvt_pk_fp8_f32 rounds to nearest
+// even onto the OCP E4M3FN grid (subnormal grid 2^-9 below 2^-6 included): checked against a
+// software encoder over every float bit pattern below 464; beyond that it returns NaN, so the
+// clamp to +-448 provides the saturation for every finite input.
+__device__ __forceinline__ unsigned int E4m3EncodePair(float a, float b) {
+  a = fminf(fmaxf(a, -448.0f), 448.0f);
+  b = fminf(fmaxf(b, -448.0f), 448.0f);
+  return static_cast<unsigned int>(__builtin_amdgcn_cvt_pk_fp8_f32(a, b, 0, false)) & 0xffffu;
+}
+
 // Quantize-on-append: per-row absmax over latent+rope by wave shuffles, scale = absmax/448,
-// code = e4m3(x / scale). Each lane quantizes the 8 latent values it loaded (8-byte store);
-// lanes 0..7 also the rope values.
+// code = e4m3(x / scale) with the correctly rounded quotient. Each lane quantizes the 8 latent
+// values it loaded (8-byte store) and one of the 64 rope values (1-byte store).
 __global__ __launch_bounds__(kThreads) void AppendFp8Kernel(AppendArgs a) {
+  static_assert(kRopeDim == kWave, "one rope element per lane");
   const int lane = threadIdx.x & (kWave - 1);
   const int token = blockIdx.x * kWavesPerGroup + (threadIdx.x >> 6);
   const int layer = blockIdx.y;
@@ -152,37 +147,29 @@ __global__ __launch_bounds__(kThreads) void AppendFp8Kernel(AppendArgs a) {
   if (block >= a.num_blocks) return;
   const char* latent_src = a.latent_src.base + layer * a.latent_src.layer_stride + token * a.latent_src.row_stride;
   const char* rope_src = a.rope_src.base + layer * a.rope_src.layer_stride + token * a.rope_src.row_stride;
-  const bool has_rope = lane < kRopeDim * 2 / 16;
   const u32x4 lv = Load16(latent_src + lane * 16);
-  u32x4 rv = {0u, 0u, 0u, 0u};
-  if (has_rope) rv = Load16(rope_src + lane * 16);
-  float x[8], y[8];
+  const float y = Bf16ToF32(*reinterpret_cast<const unsigned short*>(rope_src + lane * 2));
+  float x[8];
 #pragma unroll
   for (int i = 0; i < 4; ++i) {
     x[2 * i] = Bf16ToF32(lv[i] & 0xffffu);
     x[2 * i + 1] = Bf16ToF32(lv[i] >> 16);
-    y[2 * i] = Bf16ToF32(rv[i] & 0xffffu);
-    y[2 * i + 1] = Bf16ToF32(rv[i] >> 16);
   }
-  float absmax = 0.0f;
+  float absmax = fabsf(y);
 #pragma unroll
-  for (int i = 0; i < 8; ++i) absmax = fmaxf(absmax, fmaxf(fabsf(x[i]), fabsf(y[i])));
+  for (int i = 0; i < 8; ++i) absmax = fmaxf(absmax, fabsf(x[i]));
 #pragma unroll
   for (int offset = 32; offset >= 1; offset >>= 1) absmax = fmaxf(absmax, __shfl_xor(absmax, offset));
   const float scale = absmax == 0.0f ? 1.0f : absmax / 448.0f;
-  u32x2 lq = {0u, 0u}, rq = {0u, 0u};
-#pragma unroll
-  for (int i = 0; i < 4; ++i) {
-    lq.x |= E4m3Encode(x[i] / scale) << (8 * i);
-    lq.y |= E4m3Encode(x[4 + i] / scale) << (8 * i);
-    rq.x |= E4m3Encode(y[i] / scale) << (8 * i);
-    rq.y |= E4m3Encode(y[4 + i] / scale) << (8 * i);
-  }
+  u32x2 lq;
+  lq.x = E4m3EncodePair(x[0] / scale, x[1] / scale) | (E4m3EncodePair(x[2] / scale, x[3] / scale) << 16);
+  lq.y = E4m3EncodePair(x[4] / scale, x[5] / scale) | (E4m3EncodePair(x[6] / scale, x[7] / scale) << 16);
+  const unsigned int rq = E4m3EncodePair(y / scale, 0.0f) & 0xffu;
   char* latent_dst = a.latent.base + layer * a.latent.layer_stride + block * a.latent.block_stride +
                      in_block * a.latent.row_stride;
   char* rope_dst = a.rope.base + layer * a.rope.layer_stride + block * a.rope.block_stride + in_block * a.rope.row_stride;
   Store8(latent_dst + lane * 8, lq);
-  if (has_rope) Store8(rope_dst + lane * 8, rq);
+  reinterpret_cast<unsigned char*>(rope_dst)[lane] = static_cast<unsigned char>(rq);
   if (lane == 0) {
     float* scale_dst = reinterpret_cast<float*>(a.scale.base + layer * a.scale.layer_stride + block * a.scale.block_stride) + in_block;
     *scale_dst = scale;
@@ -410,7 +397,8 @@ hipError_t LaunchGather(const GatherArgs& args, hipStream_t stream) {
 
 hipError_t LaunchCopyBlocks(const CopyBlocksArgs& args, hipStream_t stream) {
   if (args.num_moves <= 0 || args.num_layers <= 0) return hipSuccess;
-  const int rows_per_item = RowsPerItem(args.block_size, 16);
+  // Two-row items: measured 6.0 TB/s against 5.4 TB/s with 16-row items (1196 blocks x 8 layers).
+  const int rows_per_item = RowsPerItem(args.block_size, 2);
   const int items_per_block = args.block_size / rows_per_item;
   const dim3 grid(DivUp(args.num_moves * items_per_block, kWavesPerGroup), args.num_layers);
   if (args.latent_row_bytes == kLatentDim * 2 && args.rope_row_bytes == kRopeDim * 2) {

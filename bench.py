@@ -44,6 +44,7 @@ def parse_args():
     p.add_argument("--warmup", type=int, default=5)
     p.add_argument("--no-cpu-baseline", action="store_true")
     p.add_argument("--no-attention", action="store_true")
+    p.add_argument("--side-only", action="store_true", help="development aid: time only the FP8 append/gather and compaction kernels")
     p.add_argument("--attention-only", action="store_true", help="development aid: time only the attention configurations")
     p.add_argument("--split-out", action="store_true", help="gather into separate latent/rope planes instead of 576-wide rows")
     return p.parse_args()
@@ -229,6 +230,93 @@ def bench_attention(args, torch, np, ffi, fp8=False, batch=32, ctx=2048, heads=6
     return result
 
 
+def bench_side_kernels(args, torch, np, ffi):
+    """The other data-movement kernels of the path at configs[3]/[4]-like sizes (8 layers to bound
+    memory): FP8 quantize-on-append, FP8 dequantising gather, bf16 compaction copy. HIP-event
+    time per launch against algorithmic bytes."""
+    lib = ffi.load()
+    bs, layers, batch, max_ctx = 64, 8, 64, 8192
+    rng = np.random.default_rng(11)
+    ctxs = [int(v) for v in rng.integers(512, 8193, size=batch)]
+    total = sum(ctxs)
+    blocks = sum(-(-c // bs) for c in ctxs)
+    out = {}
+
+    def timed(fn, reps=5):
+        fn()
+        torch.cuda.synchronize()
+        start, stop = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+        start.record()
+        for _ in range(reps):
+            fn()
+        stop.record()
+        torch.cuda.synchronize()
+        return start.elapsed_time(stop) / reps
+
+    gen = torch.Generator(device="cuda").manual_seed(5)
+    lat = torch.randn(layers, total, LATENT, generator=gen, device="cuda").to(torch.bfloat16)
+    rop = torch.randn(layers, total, ROPE, generator=gen, device="cuda").to(torch.bfloat16)
+    for fp8 in (True, False):
+        arena = ffi.Arena(ffi.BACKEND_HIP)
+        cache = ffi.KvCache(arena, num_layers=layers, block_size=bs, max_context_len=max_ctx, max_batch=batch,
+                            pool_blocks=blocks + 16, seed=3, shuffle=1, dtype=ffi.DTYPE_FP8_E4M3 if fp8 else ffi.DTYPE_BF16)
+        arena.commit()
+        cache.bind()
+        arena.seal()
+        view = cache.view()
+        for s, n in enumerate(ctxs):
+            cache.add_sequence(s, n)
+        cache.upload_step(stream_ptr(torch))
+        table = cache.host_block_table()
+        slots = torch.as_tensor(np.concatenate([table[s, np.arange(n) // bs].astype(np.int64) * bs + np.arange(n) % bs
+                                                for s, n in enumerate(ctxs)]).astype(np.int32), device="cuda")
+
+        def append():
+            ffi.check(lib.mlakvAppend(C.byref(view), 0, layers, lat.data_ptr(), total * LATENT * 2, LATENT * 2, rop.data_ptr(),
+                                      total * ROPE * 2, ROPE * 2, slots.data_ptr(), total, stream_ptr(torch)))
+        ms = timed(append)
+        if fp8:
+            nbytes = layers * (total * (ROW_BYTES + 580) + 4 * total)
+            out["append_fp8"] = {"ms": ms, "gbps": nbytes / (ms * 1e-3) / 1e9, "frac": nbytes / (ms * 1e-3) / 1e9 / HBM_PEAK_GBPS,
+                                 "rows": total, "layers": layers}
+            dst = torch.empty(layers, total, ROW, dtype=torch.bfloat16, device="cuda")
+
+            def gather():
+                ffi.check(lib.mlakvGather(C.byref(view), 0, layers, cache.device_block_table, cache.num_blocks,
+                                          cache.device_seq_lens, cache.device_cu_seq_lens, batch, max_ctx, dst.data_ptr(),
+                                          total * ROW_BYTES, ROW_BYTES, dst.data_ptr() + LATENT * 2, total * ROW_BYTES, ROW_BYTES,
+                                          stream_ptr(torch)))
+            ms = timed(gather)
+            nbytes = layers * (total * (580 + ROW_BYTES) + 4 * blocks)
+            out["gather_fp8"] = {"ms": ms, "gbps": nbytes / (ms * 1e-3) / 1e9, "frac": nbytes / (ms * 1e-3) / 1e9 / HBM_PEAK_GBPS,
+                                 "rows": total, "layers": layers}
+            del dst
+        else:
+            # free every other sequence, then compact: the device copies each moved block in every layer
+            for s in range(0, batch, 2):
+                cache.free_sequence(s)
+            torch.cuda.synchronize()
+            start, stop = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+            start.record()
+            moves = cache.compact(stream_ptr(torch))
+            stop.record()
+            torch.cuda.synchronize()
+            whole_ms = start.elapsed_time(stop)
+            # the copy kernel alone, replaying the same move list from device memory
+            moves_dev = torch.as_tensor(np.asarray(moves, dtype=np.int32).reshape(-1), device="cuda")
+
+            def copy():
+                ffi.check(lib.mlakvCopyBlocks(C.byref(view), 0, layers, moves_dev.data_ptr(), len(moves), stream_ptr(torch)))
+            ms = timed(copy)
+            nbytes = 2 * len(moves) * bs * ROW_BYTES * layers
+            out["compaction_bf16"] = {"ms": ms, "gbps": nbytes / (ms * 1e-3) / 1e9, "frac": nbytes / (ms * 1e-3) / 1e9 / HBM_PEAK_GBPS,
+                                      "moved_blocks": len(moves), "layers": layers,
+                                      "ms_with_host_plan_and_upload": whole_ms}
+        cache.close()
+        arena.close()
+    return out
+
+
 def cpu_baseline(np, ag):
     """The CPU oracle (a port: the reference has no CPU numerics for this path) on one core, on a
     bounded sample of the same workload: the append+gather step of 4 of the 43 layers."""
@@ -298,6 +386,9 @@ def main():
     calib_dst.copy_(calib_src)
     torch.cuda.synchronize()
     del calib_src, calib_dst
+    if args.side_only:
+        print(json.dumps({"side_kernels": bench_side_kernels(args, torch, np, ffi)}))
+        return 0
     if args.attention_only:
         print(json.dumps({"attention": bench_attention(args, torch, np, ffi),
                           "attention_fp8": bench_attention(args, torch, np, ffi, fp8=True, batch=64, ctx=4352, iters=64),
@@ -329,6 +420,7 @@ def main():
         line["attention_fp8"] = bench_attention(args, torch, np, ffi, fp8=True, batch=64, ctx=4352, iters=64)
         line["attention_long"] = bench_attention(args, torch, np, ffi, batch=128, ctx=8192, slices=2, iters=16,
                                                  label="configs[4]-scale decode shape (one workgroup per sequence)")
+        line["side_kernels"] = bench_side_kernels(args, torch, np, ffi)
     if not args.no_cpu_baseline:
         line["cpu_baseline"] = cpu_baseline(np, ag)
         if not args.no_attention:

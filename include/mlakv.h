@@ -114,7 +114,7 @@ typedef struct mlakvAttnPlan {
   int32_t block_size;
   int32_t dtype;           /* cache dtype */
   int32_t chunk_tiles;     /* 32-token tiles per workgroup; chosen by the plan */
-  int32_t max_chunks;      /* ceil(ceil(max_seq_len / 64) / chunk_tiles) */
+  int32_t max_chunks;      /* ceil(ceil(max_seq_len / 32) / chunk_tiles) */
   int32_t reserved;
   uint64_t workspace_bytes;
 } mlakvAttnPlan;
