@@ -169,3 +169,43 @@ def test_config3_full_size_against_oracle_sample_and_torch():
     sample = [0, 7, 19, 31]
     expected, _ = kt.oracle_attention(cache, 0, q[sample], table[sample], [ctx] * len(sample), SCALE)
     _assert_close(out[sample], expected, TOL_BF16)
+
+
+@pytest.mark.parametrize("fp8", [False, True])
+def test_maximum_context_single_sequence_many_chunks(fp8):
+    """BASELINE's largest context (32768 tokens) for one sequence: the plan splits it into hundreds
+    of chunks, so the merge runs over many groups of partials. The whole sequence is checked
+    against a float32 torch evaluation on the GPU (library routine), 16 heads of it against the
+    float64 oracle; a second, short sequence in the same batch leaves most chunks empty."""
+    heads, bs = 64, 128
+    ctxs = [32768, 200]
+    blocks = sum(-(-c // bs) for c in ctxs) + 8
+    pool = kt.build_tables(ctxs, bs, blocks, seed=5)
+    table = pool.table()
+    cache = kt.PagedCache(1, blocks, bs, fp8=fp8)
+    gen = torch.Generator(device="cuda").manual_seed(9)
+    total = sum(ctxs)
+    latent_src = torch.randn(1, total, LATENT, generator=gen, device="cuda").to(torch.bfloat16)
+    rope_src = torch.randn(1, total, ROPE, generator=gen, device="cuda").to(torch.bfloat16)
+    kt.append(cache, latent_src, rope_src, kt.dev_i32(kt.slots_for(table, ctxs, bs)))
+    q = torch.randn(len(ctxs), heads, LATENT + ROPE, generator=gen, device="cuda").to(torch.bfloat16)
+    out, lse, plan = kt.attention(cache, 0, q, kt.dev_i32(table), kt.dev_i32(ctxs), SCALE)
+    assert plan.max_chunks >= 64
+    tol = TOL_FP8 if fp8 else TOL_BF16
+    if fp8:  # compare against the values the cache really holds
+        lat_rows, rope_rows = kt.gather(cache, kt.dev_i32(table), kt.dev_i32(ctxs))
+        lat_rows, rope_rows = lat_rows[0].float(), rope_rows[0].float()
+    else:
+        lat_rows, rope_rows = latent_src[0].float(), rope_src[0].float()
+    start = 0
+    for b, n in enumerate(ctxs):
+        k = torch.cat([lat_rows[start:start + n], rope_rows[start:start + n]], dim=-1)
+        scores = (q[b].float() @ k.T) * SCALE
+        ref = torch.softmax(scores, dim=-1) @ lat_rows[start:start + n]
+        peak = ref.abs().max().item()
+        assert (out[b].float() - ref).abs().max().item() <= tol * peak, (b, n)
+        assert (lse[b] - torch.logsumexp(scores, dim=-1)).abs().max().item() <= 2e-2
+        start += n
+    if not fp8:
+        expected, _ = kt.oracle_attention(cache, 0, q[:1, :16].contiguous(), table[:1], ctxs[:1], SCALE)
+        _assert_close(out[:1, :16], expected, TOL_BF16)
