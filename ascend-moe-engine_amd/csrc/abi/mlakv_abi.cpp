@@ -159,6 +159,78 @@ mlakvStatus mlakvAppend(const mlakvCacheView* cache, int32_t layer_begin, int32_
   return status == hipSuccess ? MLAKV_SUCCESS : HipFail(status, "mlakvAppend");
 }
 
+mlakvStatus mlakvNormRopeAppend(const mlakvCacheView* cache, int32_t layer, const void* kv_a, int64_t kv_a_row_stride,
+                                const void* gamma, double epsilon, const void* rope_cos, const void* rope_sin,
+                                int64_t rope_table_row_stride, const int32_t* positions, const int32_t* slot_mapping,
+                                int32_t num_tokens, void* latent_normed_out, int64_t latent_normed_row_stride,
+                                void* rope_out, int64_t rope_out_row_stride, void* q_rope, int64_t q_rope_token_stride,
+                                int64_t q_rope_head_stride, int32_t num_heads, void* stream) {
+  const char* who = "mlakvNormRopeAppend";
+  if (mlakvStatus s = CheckView(cache, who)) return s;
+  if (mlakvStatus s = CheckLayers(cache, layer, 1, who)) return s;
+  if (num_tokens < 0) return Fail(MLAKV_ERR_PARAM_INVALID, "%s: negative token count", who);
+  if (num_tokens == 0) return MLAKV_SUCCESS;
+  if (kv_a == nullptr || gamma == nullptr || rope_cos == nullptr || rope_sin == nullptr || positions == nullptr ||
+      slot_mapping == nullptr) {
+    return Fail(MLAKV_ERR_PARAM_NULLPTR, "%s: rows, gamma, rope tables, positions and slot mapping are required", who);
+  }
+  if (!(epsilon > 0.0) || !std::isfinite(epsilon)) return Fail(MLAKV_ERR_PARAM_INVALID, "%s: a positive epsilon is required", who);
+  if (!Aligned16(kv_a) || kv_a_row_stride % 16 != 0 || !Aligned16(gamma)) {
+    return Fail(MLAKV_ERR_PARAM_INVALID, "%s: kv_a rows and gamma must be 16-byte aligned, the row stride a multiple of 16", who);
+  }
+  if (kv_a_row_stride < (cache->latent_dim + cache->rope_dim) * 2) {
+    return Fail(MLAKV_ERR_PARAM_INVALID, "%s: a kv_a row holds latent and rope, %d bytes", who, (cache->latent_dim + cache->rope_dim) * 2);
+  }
+  if (rope_table_row_stride % 2 != 0 || rope_table_row_stride < cache->rope_dim * 2 ||
+      reinterpret_cast<uintptr_t>(rope_cos) % 2 != 0 || reinterpret_cast<uintptr_t>(rope_sin) % 2 != 0) {
+    return Fail(MLAKV_ERR_PARAM_INVALID, "%s: rope table rows hold %d bf16 values", who, cache->rope_dim);
+  }
+  if ((latent_normed_out != nullptr && (!Aligned16(latent_normed_out) || latent_normed_row_stride % 16 != 0)) ||
+      (rope_out != nullptr && (reinterpret_cast<uintptr_t>(rope_out) % 2 != 0 || rope_out_row_stride % 2 != 0))) {
+    return Fail(MLAKV_ERR_PARAM_INVALID, "%s: optional outputs must be aligned to their element groups (16 / 2 bytes)", who);
+  }
+  if (q_rope != nullptr) {
+    if (num_heads <= 0 || num_heads > 4096) return Fail(MLAKV_ERR_PARAM_INVALID, "%s: query rope needs a head count in [1, 4096]", who);
+    if (!Aligned16(q_rope) || q_rope_token_stride % 16 != 0 || q_rope_head_stride % 16 != 0 ||
+        q_rope_head_stride < cache->rope_dim * 2 || q_rope_token_stride < q_rope_head_stride * num_heads) {
+      return Fail(MLAKV_ERR_PARAM_INVALID,
+                  "%s: query rope slices must be 16-byte aligned with strides that are multiples of 16 and do not overlap", who);
+    }
+    if (!Aligned16(rope_cos) || !Aligned16(rope_sin) || rope_table_row_stride % 16 != 0) {
+      return Fail(MLAKV_ERR_PARAM_INVALID, "%s: with query rope the table rows must be 16-byte aligned", who);
+    }
+    if (static_cast<int64_t>(num_tokens) * (1 + (num_heads + 7) / 8) > (int64_t{1} << 30)) {
+      return Fail(MLAKV_ERR_PARAM_INVALID, "%s: too many (token, head group) items for one launch", who);
+    }
+  }
+  mlakv::NormRopeAppendArgs args{};
+  FillPlanes(cache, layer, &args.append.latent, &args.append.rope, &args.append.scale);
+  args.append.slots = slot_mapping;
+  args.append.num_tokens = num_tokens;
+  args.append.num_layers = 1;
+  args.append.num_blocks = cache->num_blocks;
+  args.append.block_size = cache->block_size;
+  args.append.fp8 = cache->dtype == MLAKV_DTYPE_FP8_E4M3;
+  args.kv_a = static_cast<const char*>(kv_a);
+  args.kv_a_row_stride = kv_a_row_stride;
+  args.gamma = static_cast<const char*>(gamma);
+  args.epsilon = static_cast<float>(epsilon);
+  args.rope_cos = static_cast<const char*>(rope_cos);
+  args.rope_sin = static_cast<const char*>(rope_sin);
+  args.rope_table_row_stride = rope_table_row_stride;
+  args.positions = positions;
+  args.latent_out = static_cast<char*>(latent_normed_out);
+  args.latent_out_row_stride = latent_normed_row_stride;
+  args.rope_out = static_cast<char*>(rope_out);
+  args.rope_out_row_stride = rope_out_row_stride;
+  args.q_rope = static_cast<char*>(q_rope);
+  args.q_rope_token_stride = q_rope_token_stride;
+  args.q_rope_head_stride = q_rope_head_stride;
+  args.num_heads = q_rope != nullptr ? num_heads : 0;
+  const hipError_t status = mlakv::LaunchNormRopeAppend(args, static_cast<hipStream_t>(stream));
+  return status == hipSuccess ? MLAKV_SUCCESS : HipFail(status, who);
+}
+
 mlakvStatus mlakvGather(const mlakvCacheView* cache, int32_t layer_begin, int32_t layer_count, const int32_t* block_table,
                         int32_t table_stride, const int32_t* seq_lens, const int32_t* cu_seq_lens, int32_t batch,
                         int32_t max_seq_len, void* latent_dst, int64_t latent_dst_layer_stride,

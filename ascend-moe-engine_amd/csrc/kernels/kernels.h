@@ -34,6 +34,29 @@ struct AppendArgs {
   bool fp8;
 };
 
+// Fused latent RMSNorm + key RoPE + append of one layer: `append` carries the cache planes
+// (already offset to the layer) and the slot mapping; its source fields are unused.
+struct NormRopeAppendArgs {
+  AppendArgs append;
+  const char* kv_a;          // bf16 rows [latent 512 | rope 64]
+  int64_t kv_a_row_stride;   // bytes
+  const char* gamma;         // bf16 [512]
+  float epsilon;
+  const char* rope_cos;      // bf16 [positions][64]
+  const char* rope_sin;
+  int64_t rope_table_row_stride;  // bytes
+  const int32_t* positions;
+  char* latent_out;          // optional bf16 [tokens][512]
+  int64_t latent_out_row_stride;
+  char* rope_out;            // optional bf16 [tokens][64]
+  int64_t rope_out_row_stride;
+  char* q_rope;              // optional bf16 [tokens][heads][64], rotated in place
+  int64_t q_rope_token_stride;
+  int64_t q_rope_head_stride;
+  int num_heads;
+  int items_per_token;       // set by the launcher: 1 + groups of eight query heads
+};
+
 struct GatherArgs {
   Plane latent, rope, scale;
   Rows latent_dst, rope_dst;  // bf16 destinations
@@ -94,6 +117,7 @@ constexpr int kRopeDim = 64;
 constexpr int kTileTokens = 32;
 
 hipError_t LaunchAppend(const AppendArgs& args, hipStream_t stream);
+hipError_t LaunchNormRopeAppend(const NormRopeAppendArgs& args, hipStream_t stream);
 hipError_t LaunchGather(const GatherArgs& args, hipStream_t stream);
 hipError_t LaunchCopyBlocks(const CopyBlocksArgs& args, hipStream_t stream);
 hipError_t LaunchAttnDecode(const AttnArgs& args, hipStream_t stream);

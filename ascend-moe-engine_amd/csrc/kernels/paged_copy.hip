@@ -131,6 +131,32 @@ __device__ __forceinline__ unsigned int E4m3EncodePair(float a, float b) {
   return static_cast<unsigned int>(__builtin_amdgcn_cvt_pk_fp8_f32(a, b, 0, false)) & 0xffffu;
 }
 
+// Quantises one row held by a wave (lane: 8 latent values, 1 rope value) and stores codes and
+// scale: per-row absmax by wave shuffles, scale = absmax/448, code = e4m3(x / scale) with the
+// correctly rounded quotient.
+__device__ __forceinline__ void QuantizeRowAndStore(const AppendArgs& a, int layer, int block, int in_block, int lane,
+                                                    const float (&x)[8], float y) {
+  float absmax = fabsf(y);
+#pragma unroll
+  for (int i = 0; i < 8; ++i) absmax = fmaxf(absmax, fabsf(x[i]));
+#pragma unroll
+  for (int offset = 32; offset >= 1; offset >>= 1) absmax = fmaxf(absmax, __shfl_xor(absmax, offset));
+  const float scale = absmax == 0.0f ? 1.0f : absmax / 448.0f;
+  u32x2 lq;
+  lq.x = E4m3EncodePair(x[0] / scale, x[1] / scale) | (E4m3EncodePair(x[2] / scale, x[3] / scale) << 16);
+  lq.y = E4m3EncodePair(x[4] / scale, x[5] / scale) | (E4m3EncodePair(x[6] / scale, x[7] / scale) << 16);
+  const unsigned int rq = E4m3EncodePair(y / scale, 0.0f) & 0xffu;
+  char* latent_dst = a.latent.base + layer * a.latent.layer_stride + block * a.latent.block_stride +
+                     in_block * a.latent.row_stride;
+  char* rope_dst = a.rope.base + layer * a.rope.layer_stride + block * a.rope.block_stride + in_block * a.rope.row_stride;
+  Store8(latent_dst + lane * 8, lq);
+  reinterpret_cast<unsigned char*>(rope_dst)[lane] = static_cast<unsigned char>(rq);
+  if (lane == 0) {
+    float* scale_dst = reinterpret_cast<float*>(a.scale.base + layer * a.scale.layer_stride + block * a.scale.block_stride) + in_block;
+    *scale_dst = scale;
+  }
+}
+
 // Quantize-on-append: per-row absmax over latent+rope by wave shuffles, scale = absmax/448,
 // code = e4m3(x / scale) with the correctly rounded quotient. Each lane quantizes the 8 latent
 // values it loaded (8-byte store) and one of the 64 rope values (1-byte store).
@@ -155,24 +181,104 @@ __global__ __launch_bounds__(kThreads) void AppendFp8Kernel(AppendArgs a) {
     x[2 * i] = Bf16ToF32(lv[i] & 0xffffu);
     x[2 * i + 1] = Bf16ToF32(lv[i] >> 16);
   }
-  float absmax = fabsf(y);
+  QuantizeRowAndStore(a, layer, block, in_block, lane, x, y);
+}
+
+// ---- latent RMSNorm + key RoPE + append ---------------------------------------------------
+
+// One wavefront per token of one layer: lane l holds latent elements 8l..8l+7 and rope element l.
+//   y = x * gamma / sqrt(mean(x^2) + eps)   (fp32; sum of squares by wave shuffles)
+//   r'[i] = r[i] cos[i] - r[i+32] sin[i],  r'[i+32] = r[i+32] cos[i+32] + r[i] sin[i+32]  ("half" rotation)
+// both rounded to bf16 (nearest even) and written to the cache row of slot[t] (quantised first for
+// an FP8 cache, from the bf16 values, as the unfused stages would) and to the optional outputs.
+// Query rope slices, rotated in place: a wavefront takes eight heads of one token, eight lanes per
+// head, 16 bytes (8 values) per lane. The partner half of a head sits four lanes away.
+constexpr int kQueryHeadsPerItem = 8;
+
+__device__ __forceinline__ void RotateQueryHeads(const NormRopeAppendArgs& n, int token, int head0, int lane) {
+  static_assert(kRopeDim == 64, "eight lanes of eight values cover a head's rope slice");
+  const int head = head0 + (lane >> 3);
+  const int part = lane & 7;
+  if (head >= n.num_heads) return;
+  const int position = Uniform(n.positions[token]);
+  char* q = n.q_rope + token * n.q_rope_token_stride + head * n.q_rope_head_stride + part * 16;
+  const u32x4 qv = Load16(q);
+  const u32x4 cv = *reinterpret_cast<const u32x4*>(n.rope_cos + position * n.rope_table_row_stride + part * 16);
+  const u32x4 sv = *reinterpret_cast<const u32x4*>(n.rope_sin + position * n.rope_table_row_stride + part * 16);
+  u32x4 out;
 #pragma unroll
-  for (int i = 0; i < 8; ++i) absmax = fmaxf(absmax, fabsf(x[i]));
+  for (int i = 0; i < 4; ++i) {
+    const unsigned pv = __shfl_xor(qv[i], 4);
+    unsigned packed = 0;
 #pragma unroll
-  for (int offset = 32; offset >= 1; offset >>= 1) absmax = fmaxf(absmax, __shfl_xor(absmax, offset));
-  const float scale = absmax == 0.0f ? 1.0f : absmax / 448.0f;
-  u32x2 lq;
-  lq.x = E4m3EncodePair(x[0] / scale, x[1] / scale) | (E4m3EncodePair(x[2] / scale, x[3] / scale) << 16);
-  lq.y = E4m3EncodePair(x[4] / scale, x[5] / scale) | (E4m3EncodePair(x[6] / scale, x[7] / scale) << 16);
-  const unsigned int rq = E4m3EncodePair(y / scale, 0.0f) & 0xffu;
-  char* latent_dst = a.latent.base + layer * a.latent.layer_stride + block * a.latent.block_stride +
-                     in_block * a.latent.row_stride;
-  char* rope_dst = a.rope.base + layer * a.rope.layer_stride + block * a.rope.block_stride + in_block * a.rope.row_stride;
-  Store8(latent_dst + lane * 8, lq);
-  reinterpret_cast<unsigned char*>(rope_dst)[lane] = static_cast<unsigned char>(rq);
-  if (lane == 0) {
-    float* scale_dst = reinterpret_cast<float*>(a.scale.base + layer * a.scale.layer_stride + block * a.scale.block_stride) + in_block;
-    *scale_dst = scale;
+    for (int h = 0; h < 2; ++h) {
+      const float x = Bf16ToF32((qv[i] >> (16 * h)) & 0xffffu), partner = Bf16ToF32((pv >> (16 * h)) & 0xffffu);
+      const float c = Bf16ToF32((cv[i] >> (16 * h)) & 0xffffu), s = Bf16ToF32((sv[i] >> (16 * h)) & 0xffffu);
+      packed |= F32ToBf16(part < 4 ? x * c - partner * s : x * c + partner * s) << (16 * h);
+    }
+    out[i] = packed;
+  }
+  Store16(q, out);
+}
+
+template <bool FP8>
+__global__ __launch_bounds__(kThreads) void NormRopeAppendKernel(NormRopeAppendArgs n) {
+  static_assert(kRopeDim == kWave && kLatentDim == 8 * kWave, "lane = 8 latent + 1 rope element");
+  const AppendArgs& a = n.append;
+  const int lane = threadIdx.x & (kWave - 1);
+  const int wave_item = blockIdx.x * kWavesPerGroup + (threadIdx.x >> 6);
+  const int token = wave_item / n.items_per_token;
+  const int sub_item = wave_item - token * n.items_per_token;
+  if (token >= a.num_tokens) return;
+  if (sub_item > 0) {
+    RotateQueryHeads(n, token, (sub_item - 1) * kQueryHeadsPerItem, lane);
+    return;
+  }
+  const char* row = n.kv_a + token * n.kv_a_row_stride;
+  const u32x4 lv = Load16(row + lane * 16);
+  const u32x4 gv = *reinterpret_cast<const u32x4*>(n.gamma + lane * 16);
+  const float r = Bf16ToF32(*reinterpret_cast<const unsigned short*>(row + kLatentDim * 2 + lane * 2));
+  const int position = Uniform(n.positions[token]);
+  const float c = Bf16ToF32(*reinterpret_cast<const unsigned short*>(n.rope_cos + position * n.rope_table_row_stride + lane * 2));
+  const float s = Bf16ToF32(*reinterpret_cast<const unsigned short*>(n.rope_sin + position * n.rope_table_row_stride + lane * 2));
+  float x[8], g[8];
+#pragma unroll
+  for (int i = 0; i < 4; ++i) {
+    x[2 * i] = Bf16ToF32(lv[i] & 0xffffu);
+    x[2 * i + 1] = Bf16ToF32(lv[i] >> 16);
+    g[2 * i] = Bf16ToF32(gv[i] & 0xffffu);
+    g[2 * i + 1] = Bf16ToF32(gv[i] >> 16);
+  }
+  float sum_squares = 0.0f;
+#pragma unroll
+  for (int i = 0; i < 8; ++i) sum_squares += x[i] * x[i];
+#pragma unroll
+  for (int offset = 32; offset >= 1; offset >>= 1) sum_squares += __shfl_xor(sum_squares, offset);
+  const float rstd = 1.0f / __builtin_sqrtf(sum_squares * (1.0f / kLatentDim) + n.epsilon);
+  u32x4 yv;
+#pragma unroll
+  for (int i = 0; i < 4; ++i) {
+    const unsigned lo = F32ToBf16(x[2 * i] * rstd * g[2 * i]), hi = F32ToBf16(x[2 * i + 1] * rstd * g[2 * i + 1]);
+    yv[i] = lo | (hi << 16);
+    x[2 * i] = Bf16ToF32(lo);
+    x[2 * i + 1] = Bf16ToF32(hi);
+  }
+  const float partner = __shfl_xor(r, 32);
+  const unsigned rotated = F32ToBf16(lane < 32 ? r * c - partner * s : r * c + partner * s);
+  if (n.latent_out != nullptr) Store16(n.latent_out + token * n.latent_out_row_stride + lane * 16, yv);
+  if (n.rope_out != nullptr) *reinterpret_cast<unsigned short*>(n.rope_out + token * n.rope_out_row_stride + lane * 2) = static_cast<unsigned short>(rotated);
+  const int slot = Uniform(a.slots[token]);
+  if (slot < 0) return;
+  const int block = slot / a.block_size;
+  const int in_block = slot - block * a.block_size;
+  if (block >= a.num_blocks) return;
+  if (FP8) {
+    QuantizeRowAndStore(a, 0, block, in_block, lane, x, Bf16ToF32(rotated));
+  } else {
+    char* latent_dst = a.latent.base + block * a.latent.block_stride + in_block * a.latent.row_stride;
+    char* rope_dst = a.rope.base + block * a.rope.block_stride + in_block * a.rope.row_stride;
+    Store16(latent_dst + lane * 16, yv);
+    *reinterpret_cast<unsigned short*>(rope_dst + lane * 2) = static_cast<unsigned short>(rotated);
   }
 }
 
@@ -369,6 +475,21 @@ hipError_t LaunchAppend(const AppendArgs& args, hipStream_t stream) {
     hipLaunchKernelGGL(AppendFp8Kernel, grid, dim3(kThreads), 0, stream, args);
   } else {
     hipLaunchKernelGGL(AppendBf16Kernel, grid, dim3(kThreads), 0, stream, args);
+  }
+  return hipGetLastError();
+}
+
+hipError_t LaunchNormRopeAppend(const NormRopeAppendArgs& args, hipStream_t stream) {
+  if (args.append.num_tokens <= 0) return hipSuccess;
+  NormRopeAppendArgs launch = args;
+  launch.items_per_token = 1 + (args.q_rope != nullptr ? DivUp(args.num_heads, kQueryHeadsPerItem) : 0);
+  const int64_t items = static_cast<int64_t>(args.append.num_tokens) * launch.items_per_token;
+  if (items > 0x7fffffff - kWavesPerGroup) return hipErrorInvalidValue;  // the kernel indexes work items in 32 bits
+  const dim3 grid(DivUp(static_cast<int>(items), kWavesPerGroup));
+  if (args.append.fp8) {
+    hipLaunchKernelGGL(NormRopeAppendKernel<true>, grid, dim3(kThreads), 0, stream, launch);
+  } else {
+    hipLaunchKernelGGL(NormRopeAppendKernel<false>, grid, dim3(kThreads), 0, stream, launch);
   }
   return hipGetLastError();
 }

@@ -72,6 +72,8 @@ PROTOTYPES = {
     "mlakvGetLastError": (C.c_char_p, []),
     "mlakvDeviceCount": (_i32, []),
     "mlakvAppend": (_i32, [_P(CacheView), _i32, _i32, _vp, _i64, _i64, _vp, _i64, _i64, _vp, _i32, _vp]),
+    "mlakvNormRopeAppend": (_i32, [_P(CacheView), _i32, _vp, _i64, _vp, C.c_double, _vp, _vp, _i64, _vp, _vp, _i32, _vp, _i64,
+                                   _vp, _i64, _vp, _i64, _i64, _i32, _vp]),
     "mlakvGather": (_i32, [_P(CacheView), _i32, _i32, _vp, _i32, _vp, _vp, _i32, _i32, _vp, _i64, _i64, _vp, _i64, _i64, _vp]),
     "mlakvCopyBlocks": (_i32, [_P(CacheView), _i32, _i32, _vp, _i32, _vp]),
     "mlakvAttnPlanInit": (_i32, [_i32, _i32, _i32, _i32, _i32, _P(AttnPlan)]),

@@ -292,6 +292,39 @@ def bench_side_kernels(args, torch, np, ffi):
                                  "rows": total, "layers": layers}
             del dst
         else:
+            # fused latent RMSNorm + key RoPE + append of one layer over every row (prefill-sized launch)
+            kv_a = torch.cat([lat[0], rop[0]], dim=1).contiguous()
+            gamma = torch.ones(LATENT, dtype=torch.bfloat16, device="cuda")
+            ang = torch.outer(torch.arange(max_ctx, dtype=torch.float32, device="cuda"),
+                              10000.0 ** (-torch.arange(0, ROPE // 2, dtype=torch.float32, device="cuda") * 2 / ROPE))
+            cos = torch.cat([ang.cos(), ang.cos()], dim=1).to(torch.bfloat16)
+            sin = torch.cat([ang.sin(), ang.sin()], dim=1).to(torch.bfloat16)
+            positions = torch.as_tensor(np.concatenate([np.arange(n) for n in ctxs]).astype(np.int32), device="cuda")
+
+            def fused():
+                ffi.check(lib.mlakvNormRopeAppend(C.byref(view), 0, kv_a.data_ptr(), ROW_BYTES, gamma.data_ptr(), 1e-6, cos.data_ptr(),
+                                                  sin.data_ptr(), ROPE * 2, positions.data_ptr(), slots.data_ptr(), total, None, 0,
+                                                  None, 0, None, 0, 0, 0, stream_ptr(torch)))
+            ms = timed(fused)
+            nbytes = total * (2 * ROW_BYTES + 8)
+            out["norm_rope_append_bf16"] = {"ms": ms, "gbps": nbytes / (ms * 1e-3) / 1e9,
+                                            "frac": nbytes / (ms * 1e-3) / 1e9 / HBM_PEAK_GBPS, "rows": total, "layers": 1}
+            # the same with the query's rope slices (64 heads, 128 of every 1152 bytes) rotated in place
+            q_tokens, heads = min(total, 32768), 64
+            q = torch.randn(q_tokens, heads, ROW, device="cuda").to(torch.bfloat16)
+
+            def fused_with_query():
+                ffi.check(lib.mlakvNormRopeAppend(C.byref(view), 0, kv_a.data_ptr(), ROW_BYTES, gamma.data_ptr(), 1e-6, cos.data_ptr(),
+                                                  sin.data_ptr(), ROPE * 2, positions.data_ptr(), slots.data_ptr(), q_tokens, None, 0,
+                                                  None, 0, q.data_ptr() + LATENT * 2, heads * ROW_BYTES, ROW_BYTES, heads,
+                                                  stream_ptr(torch)))
+            ms = timed(fused_with_query)
+            nbytes = q_tokens * (2 * ROW_BYTES + 8 + heads * 2 * ROPE * 2)
+            out["norm_rope_append_query_rope_bf16"] = {"ms": ms, "gbps": nbytes / (ms * 1e-3) / 1e9,
+                                                       "frac": nbytes / (ms * 1e-3) / 1e9 / HBM_PEAK_GBPS, "rows": q_tokens,
+                                                       "heads": heads, "layers": 1}
+            del q
+            del kv_a
             # free every other sequence, then compact: the device copies each moved block in every layer
             for s in range(0, batch, 2):
                 cache.free_sequence(s)

@@ -80,6 +80,34 @@ mlakvStatus mlakvAppend(const mlakvCacheView* cache, int32_t layer_begin, int32_
                         const void* rope_src, int64_t rope_src_layer_stride, int64_t rope_src_row_stride,
                         const int32_t* slot_mapping, int32_t num_tokens, void* stream);
 
+/* Fused latent RMSNorm + RoPE (key and, optionally, query slices) + append of one layer: the
+ * stages `kv_a_norm`, `rope` and `kv_cache_write` that the reference launches back to back
+ * (src/pipeline/pipeline.cpp:213-234; operator contracts include/moe/core/op_table.hpp:151-170
+ * aclnnRmsNorm "y = x * gamma / sqrt(mean(x*x) + epsilon)", :315-337 aclnnApplyRotaryPosEmbV2 with
+ * "half" rotation, :339-372 aclnnScatterPaKvCache; epsilon = kRmsNormEpsilon, config.hpp:56).
+ * kv_a holds bf16 rows [latent 512 | rope 64] as the reference lays out act.kv_a
+ * (src/memory/static_arena_manager.cpp:488-490); gamma is the layer's bf16 [512] weight;
+ * rope_cos / rope_sin are bf16 tables [position][64] (row = position, pipeline.cpp:403-406);
+ * positions and slot_mapping are device int32 [num_tokens]. For token t with p = positions[t]:
+ *   y[d]    = bf16(x[d] * gamma[d] / sqrt(mean(x^2) + epsilon))
+ *   r'[i]   = bf16(r[i] cos[p][i] - r[i+32] sin[p][i]),  r'[i+32] = bf16(r[i+32] cos[p][i+32] + r[i] sin[p][i+32])
+ *   cache[layer][slot_mapping[t]] = (y, r')        (skipped when slot_mapping[t] < 0)
+ * Arithmetic in fp32, one rounding to bf16; an FP8 cache quantizes the bf16 values as mlakvAppend
+ * does. latent_normed_out (bf16 [num_tokens][512]) and rope_out (bf16 [num_tokens][64]) are
+ * optional copies of y and r' (the reference's act.kv_latent_normed and the rotated k_rope;
+ * rope_out may be the rope columns of kv_a itself, which is the reference's in-place rotation).
+ * q_rope, when not null, is the query's rope slices bf16 [num_tokens][num_heads][64] at the given
+ * byte strides (the reference's view into q_b, static_arena_manager.cpp:481-485: head stride
+ * 576 * 2); they are rotated in place with the same table row, as the reference's one
+ * aclnnApplyRotaryPosEmbV2 call rotates q_rope and k_rope together (pipeline.cpp:219-225). With
+ * q_rope the table rows must be 16-byte aligned. */
+mlakvStatus mlakvNormRopeAppend(const mlakvCacheView* cache, int32_t layer, const void* kv_a, int64_t kv_a_row_stride,
+                                const void* gamma, double epsilon, const void* rope_cos, const void* rope_sin,
+                                int64_t rope_table_row_stride, const int32_t* positions, const int32_t* slot_mapping,
+                                int32_t num_tokens, void* latent_normed_out, int64_t latent_normed_row_stride,
+                                void* rope_out, int64_t rope_out_row_stride, void* q_rope, int64_t q_rope_token_stride,
+                                int64_t q_rope_head_stride, int32_t num_heads, void* stream);
+
 /* Gather: the paged read that the reference leaves implicit inside its attention
  * operator (addressing as in third_party/ops_transformer/attention/quant_lightning_indexer/
  * op_kernel/arch35/quant_lightning_indexer_service_cube.h:243-270):

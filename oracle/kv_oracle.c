@@ -402,6 +402,63 @@ void kvo_gather_rows_fp8(const uint8_t* latent_plane, int64_t latent_block_strid
 }
 
 /* ------------------------------------------------------------------------- */
+/* latent RMSNorm + key RoPE (the stages in front of the cache write)          */
+/* ------------------------------------------------------------------------- */
+
+/* One rounding, nearest even, straight from double: going through float first would round twice
+ * when the double lies just off a bf16 midpoint (which a float represents exactly). */
+static uint16_t bf16_from_double(double v) {
+  float f = (float)v;
+  uint32_t bits;
+  memcpy(&bits, &f, sizeof bits);
+  if ((bits & 0xffffu) == 0x8000u && (double)f != v) {
+    bits += fabs(v) > fabs((double)f) ? 1u : 0xffffffffu;  /* off the midpoint, on the side v is on */
+    memcpy(&f, &bits, sizeof f);
+  }
+  return kvo_bf16_from_f32(f);
+}
+
+void kvo_rope_rows(const uint16_t* rows, int64_t row_stride, const uint16_t* rope_cos, const uint16_t* rope_sin,
+                   int64_t rope_table_row_stride, const int32_t* positions, int64_t rows_per_position, int64_t num_rows,
+                   int64_t rope_dim, uint16_t* out, int64_t out_row_stride) {
+  const int64_t half = rope_dim / 2;
+  for (int64_t t = 0; t < num_rows; ++t) {
+    const uint16_t* r = rows + t * row_stride;
+    const int64_t position = positions[t / rows_per_position];
+    const uint16_t* c = rope_cos + position * rope_table_row_stride;
+    const uint16_t* s = rope_sin + position * rope_table_row_stride;
+    for (int64_t i = 0; i < half; ++i) {
+      const double lo = (double)kvo_bf16_to_f32(r[i]), hi = (double)kvo_bf16_to_f32(r[i + half]);
+      out[t * out_row_stride + i] = bf16_from_double(lo * (double)kvo_bf16_to_f32(c[i]) - hi * (double)kvo_bf16_to_f32(s[i]));
+      out[t * out_row_stride + i + half] =
+          bf16_from_double(hi * (double)kvo_bf16_to_f32(c[i + half]) + lo * (double)kvo_bf16_to_f32(s[i + half]));
+    }
+  }
+}
+
+void kvo_norm_rope_rows(const uint16_t* kv_a, int64_t kv_a_row_stride, const uint16_t* gamma, double epsilon,
+                        const uint16_t* rope_cos, const uint16_t* rope_sin, int64_t rope_table_row_stride,
+                        const int32_t* positions, int64_t num_tokens, int64_t latent_dim, int64_t rope_dim,
+                        uint16_t* latent_out, int64_t latent_out_row_stride, uint16_t* rope_out,
+                        int64_t rope_out_row_stride) {
+  for (int64_t t = 0; t < num_tokens; ++t) {
+    const uint16_t* x = kv_a + t * kv_a_row_stride;
+    double sum_squares = 0.0;
+    for (int64_t d = 0; d < latent_dim; ++d) {
+      const double v = (double)kvo_bf16_to_f32(x[d]);
+      sum_squares += v * v;
+    }
+    const double rstd = 1.0 / sqrt(sum_squares / (double)latent_dim + epsilon);
+    for (int64_t d = 0; d < latent_dim; ++d) {
+      latent_out[t * latent_out_row_stride + d] =
+          bf16_from_double((double)kvo_bf16_to_f32(x[d]) * rstd * (double)kvo_bf16_to_f32(gamma[d]));
+    }
+  }
+  kvo_rope_rows(kv_a + latent_dim, kv_a_row_stride, rope_cos, rope_sin, rope_table_row_stride, positions, 1, num_tokens,
+                rope_dim, rope_out, rope_out_row_stride);
+}
+
+/* ------------------------------------------------------------------------- */
 /* absorbed-MLA decode attention                                              */
 /* ------------------------------------------------------------------------- */
 

@@ -139,6 +139,30 @@ float kvo_e4m3_to_f32(uint8_t code);
 float kvo_fp8_row_scale(const uint16_t* latent_bf16, int64_t latent_dim, const uint16_t* rope_bf16,
                         int64_t rope_dim);
 
+/* Latent RMSNorm and key RoPE of the two stages in front of the cache write
+ * (reference src/pipeline/pipeline.cpp:213-225; operator contracts include/moe/core/op_table.hpp:151-170
+ * "y = x * gamma / sqrt(mean(x*x) + epsilon)" and :315-337 "half rotation"; rope table row = position
+ * (pipeline.cpp:403-406)). Evaluated in double, rounded once to bf16 (nearest even):
+ *   latent_out[t][d] = bf16(x[t][d] * gamma[d] / sqrt(mean_d x[t][d]^2 + epsilon))
+ *   rope_out[t][i]        = bf16(r[t][i] cos[p][i] - r[t][i+h] sin[p][i])          i < h = rope_dim / 2
+ *   rope_out[t][i+h]      = bf16(r[t][i+h] cos[p][i+h] + r[t][i] sin[p][i+h])
+ * kv_a rows hold [latent | rope] bf16 (reference static_arena_manager.cpp:488-490).
+ * Parity with CANN's rounding is unpinned (no reference numerics); pinned by closed forms in
+ * tests/test_oracle_norm_rope.py. */
+void kvo_norm_rope_rows(const uint16_t* kv_a, int64_t kv_a_row_stride, const uint16_t* gamma, double epsilon,
+                        const uint16_t* rope_cos, const uint16_t* rope_sin, int64_t rope_table_row_stride,
+                        const int32_t* positions, int64_t num_tokens, int64_t latent_dim, int64_t rope_dim,
+                        uint16_t* latent_out, int64_t latent_out_row_stride, uint16_t* rope_out,
+                        int64_t rope_out_row_stride);
+
+/* The rotation alone, for rows that share a position in groups of rows_per_position consecutive
+ * rows (the query's rope slices: one row per head, reference q_rope view
+ * static_arena_manager.cpp:481-485, rotated by the same aclnnApplyRotaryPosEmbV2 call as k_rope,
+ * pipeline.cpp:219-225): row t uses table row positions[t / rows_per_position]. */
+void kvo_rope_rows(const uint16_t* rows, int64_t row_stride, const uint16_t* rope_cos, const uint16_t* rope_sin,
+                   int64_t rope_table_row_stride, const int32_t* positions, int64_t rows_per_position, int64_t num_rows,
+                   int64_t rope_dim, uint16_t* out, int64_t out_row_stride);
+
 /* Quantize-on-append: one fp32 scale per token row over latent+rope, code = e4m3(x / scale). */
 void kvo_append_rows_fp8(uint8_t* latent_plane, int64_t latent_block_stride, int64_t latent_row_stride,
                          uint8_t* rope_plane, int64_t rope_block_stride, int64_t rope_row_stride,

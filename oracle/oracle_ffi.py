@@ -73,6 +73,8 @@ _PROTOTYPES = {
                                    _vp, _i64]),
     "kvo_gather_rows_fp8": (None, [_vp, _i64, _i64, _vp, _i64, _i64, _vp, _i64, _i64, _vp, _i64, _vp, _i64, _vp, _i64,
                                    _vp, _i64, _i64, _i64]),
+    "kvo_norm_rope_rows": (None, [_vp, _i64, _vp, C.c_double, _vp, _vp, _i64, _vp, _i64, _i64, _i64, _vp, _i64, _vp, _i64]),
+    "kvo_rope_rows": (None, [_vp, _i64, _vp, _vp, _i64, _vp, _i64, _i64, _i64, _vp, _i64]),
     "kvo_mla_decode": (None, [_vp, _i64, _i64, _vp, _i64, _i64, _P(CacheView), _vp, _i64, _vp, _i64, _i64, C.c_double,
                               _vp, _vp, C.c_int]),
     "kvo_splitmix64": (_u64, [_P(_u64)]),
@@ -216,6 +218,35 @@ def append_rows_fp8(latent_plane, rope_plane, scale_plane, block_size, latent_sr
                                rope_row_stride * block_size, rope_row_stride, _ptr(scale_plane), block_size, block_size,
                                _ptr(latent_src), latent_src.shape[1], _ptr(rope_src), rope_src.shape[1], latent_dim,
                                rope_dim, _ptr(slots), len(slots))
+
+
+def norm_rope_rows(kv_a, gamma, epsilon, rope_cos, rope_sin, positions, latent_dim=512, rope_dim=64):
+    """kv_a uint16 [T, latent+rope] bf16 bits; gamma uint16 [latent]; rope_cos/sin uint16 [P, rope];
+    positions int32 [T]. Returns (latent uint16 [T, latent], rope uint16 [T, rope])."""
+    kv_a = np.ascontiguousarray(kv_a, dtype=np.uint16)
+    gamma = np.ascontiguousarray(gamma, dtype=np.uint16)
+    rope_cos = np.ascontiguousarray(rope_cos, dtype=np.uint16)
+    rope_sin = np.ascontiguousarray(rope_sin, dtype=np.uint16)
+    positions = np.ascontiguousarray(positions, dtype=np.int32)
+    n = kv_a.shape[0]
+    latent = np.zeros((n, latent_dim), dtype=np.uint16)
+    rope = np.zeros((n, rope_dim), dtype=np.uint16)
+    load().kvo_norm_rope_rows(_ptr(kv_a), kv_a.shape[1], _ptr(gamma), float(epsilon), _ptr(rope_cos), _ptr(rope_sin), rope_cos.shape[1],
+                              _ptr(positions), n, latent_dim, rope_dim, _ptr(latent), latent_dim, _ptr(rope), rope_dim)
+    return latent, rope
+
+
+def rope_rows(rows, rope_cos, rope_sin, positions, rows_per_position=1):
+    """rows uint16 [N, rope] bf16 bits (N = len(positions) * rows_per_position). Returns the rotated rows."""
+    rows = np.ascontiguousarray(rows, dtype=np.uint16)
+    rope_cos = np.ascontiguousarray(rope_cos, dtype=np.uint16)
+    rope_sin = np.ascontiguousarray(rope_sin, dtype=np.uint16)
+    positions = np.ascontiguousarray(positions, dtype=np.int32)
+    assert rows.shape[0] == len(positions) * rows_per_position
+    out = np.zeros_like(rows)
+    load().kvo_rope_rows(_ptr(rows), rows.shape[1], _ptr(rope_cos), _ptr(rope_sin), rope_cos.shape[1], _ptr(positions),
+                         rows_per_position, rows.shape[0], rows.shape[1], _ptr(out), rows.shape[1])
+    return out
 
 
 def gather_rows_fp8(latent_plane, rope_plane, scale_plane, block_size, table, seq_lens, latent_dim=512, rope_dim=64):
