@@ -335,45 +335,61 @@ mlakvStatus mlakvAttnPlanInit(int32_t batch, int32_t heads, int32_t max_seq_len,
   return MLAKV_SUCCESS;
 }
 
-mlakvStatus mlakvAttnDecode(const mlakvAttnPlan* plan, const mlakvCacheView* cache, int32_t layer, const void* q_latent,
-                            int64_t q_latent_seq_stride, int64_t q_latent_head_stride, const void* q_rope,
-                            int64_t q_rope_seq_stride, int64_t q_rope_head_stride, const int32_t* block_table,
-                            int32_t table_stride, const int32_t* seq_lens, double scale, void* out, int64_t out_seq_stride,
-                            int64_t out_head_stride, float* lse, void* workspace, uint64_t workspace_bytes, void* stream) {
-  if (plan == nullptr) return Fail(MLAKV_ERR_PARAM_NULLPTR, "mlakvAttnDecode: plan is null");
-  if (mlakvStatus s = CheckView(cache, "mlakvAttnDecode")) return s;
-  if (mlakvStatus s = CheckLayers(cache, layer, 1, "mlakvAttnDecode")) return s;
-  if (q_latent == nullptr || q_rope == nullptr || block_table == nullptr || seq_lens == nullptr || out == nullptr) {
-    return Fail(MLAKV_ERR_PARAM_NULLPTR, "mlakvAttnDecode: query, block table, lengths and output are required");
+}  // extern "C"
+
+namespace {
+mlakvStatus AttnDecodeImpl(const char* who, const mlakvAttnPlan* plan, const mlakvCacheView* cache, int32_t layer,
+                           const void* q_latent, int64_t q_latent_seq_stride, int64_t q_latent_head_stride, const void* q_rope,
+                           int64_t q_rope_seq_stride, int64_t q_rope_head_stride, const int32_t* block_table,
+                           int32_t table_stride, const int32_t* seq_lens, double scale, void* out, int64_t out_seq_stride,
+                           int64_t out_head_stride, const mlakvMxQuantOut* quant, float* lse, void* workspace,
+                           uint64_t workspace_bytes, void* stream) {
+  if (plan == nullptr) return Fail(MLAKV_ERR_PARAM_NULLPTR, "%s: plan is null", who);
+  if (mlakvStatus s = CheckView(cache, who)) return s;
+  if (mlakvStatus s = CheckLayers(cache, layer, 1, who)) return s;
+  if (q_latent == nullptr || q_rope == nullptr || block_table == nullptr || seq_lens == nullptr) {
+    return Fail(MLAKV_ERR_PARAM_NULLPTR, "%s: query, block table and lengths are required", who);
+  }
+  if (out == nullptr && quant == nullptr) return Fail(MLAKV_ERR_PARAM_NULLPTR, "%s: an output is required", who);
+  if (quant != nullptr) {
+    if (quant->codes == nullptr || quant->scales == nullptr) {
+      return Fail(MLAKV_ERR_PARAM_NULLPTR, "%s: the quantised output needs codes and scales", who);
+    }
+    if (!Aligned16(quant->codes) || quant->codes_seq_stride % 16 != 0 || quant->codes_head_stride % 16 != 0 ||
+        quant->codes_head_stride < mlakv::kLatentDim || !Aligned16(quant->scales) || quant->scales_seq_stride % 16 != 0 ||
+        quant->scales_head_stride % 16 != 0 || quant->scales_head_stride < mlakv::kLatentDim / 32) {
+      return Fail(MLAKV_ERR_PARAM_INVALID,
+                  "%s: codes (512 per head) and scales (16 per head) must be 16-byte aligned with 16-byte-multiple strides", who);
+    }
   }
   if (plan->dtype != cache->dtype || plan->block_size != cache->block_size) {
-    return Fail(MLAKV_ERR_PARAM_INVALID, "mlakvAttnDecode: the plan was made for dtype %d / block %d, the cache has %d / %d",
+    return Fail(MLAKV_ERR_PARAM_INVALID, "%s: the plan was made for dtype %d / block %d, the cache has %d / %d", who,
                 plan->dtype, plan->block_size, cache->dtype, cache->block_size);
   }
-  if (!(scale > 0.0) || !std::isfinite(scale)) return Fail(MLAKV_ERR_PARAM_INVALID, "mlakvAttnDecode: a positive softmax scale is required");
+  if (!(scale > 0.0) || !std::isfinite(scale)) return Fail(MLAKV_ERR_PARAM_INVALID, "%s: a positive softmax scale is required", who);
   if (static_cast<int64_t>(table_stride) * cache->block_size < plan->max_seq_len) {
-    return Fail(MLAKV_ERR_PARAM_INVALID, "mlakvAttnDecode: a table row of %d blocks cannot address %d tokens", table_stride,
+    return Fail(MLAKV_ERR_PARAM_INVALID, "%s: a table row of %d blocks cannot address %d tokens", who, table_stride,
                 plan->max_seq_len);
   }
   if (!Aligned16(q_latent) || !Aligned16(q_rope) || q_latent_seq_stride % 16 != 0 || q_latent_head_stride % 16 != 0 ||
       q_rope_seq_stride % 16 != 0 || q_rope_head_stride % 16 != 0) {
-    return Fail(MLAKV_ERR_PARAM_INVALID, "mlakvAttnDecode: query rows must be 16-byte aligned with 16-byte-multiple strides");
+    return Fail(MLAKV_ERR_PARAM_INVALID, "%s: query rows must be 16-byte aligned with 16-byte-multiple strides", who);
   }
-  if (!Aligned16(out) || out_seq_stride % 16 != 0 || out_head_stride % 16 != 0) {
-    return Fail(MLAKV_ERR_PARAM_INVALID, "mlakvAttnDecode: output rows must be 16-byte aligned with 16-byte-multiple strides");
+  if (out != nullptr && (!Aligned16(out) || out_seq_stride % 16 != 0 || out_head_stride % 16 != 0)) {
+    return Fail(MLAKV_ERR_PARAM_INVALID, "%s: output rows must be 16-byte aligned with 16-byte-multiple strides", who);
   }
   if (plan->workspace_bytes > 0) {
-    if (workspace == nullptr) return Fail(MLAKV_ERR_PARAM_NULLPTR, "mlakvAttnDecode: the plan needs %llu workspace bytes",
+    if (workspace == nullptr) return Fail(MLAKV_ERR_PARAM_NULLPTR, "%s: the plan needs %llu workspace bytes", who,
                                           static_cast<unsigned long long>(plan->workspace_bytes));
     if (workspace_bytes < plan->workspace_bytes || !Aligned16(workspace)) {
-      return Fail(MLAKV_ERR_PARAM_INVALID, "mlakvAttnDecode: workspace of %llu bytes (16-byte aligned) needed, %llu given",
+      return Fail(MLAKV_ERR_PARAM_INVALID, "%s: workspace of %llu bytes (16-byte aligned) needed, %llu given", who,
                   static_cast<unsigned long long>(plan->workspace_bytes), static_cast<unsigned long long>(workspace_bytes));
     }
   }
   static std::once_flag prepared;
   static hipError_t prepare_status = hipSuccess;
   std::call_once(prepared, [] { prepare_status = mlakv::PrepareAttnKernels(); });
-  if (prepare_status != hipSuccess) return HipFail(prepare_status, "mlakvAttnDecode (kernel attributes)");
+  if (prepare_status != hipSuccess) return HipFail(prepare_status, who);
 
   mlakv::AttnArgs args{};
   FillPlanes(cache, layer, &args.latent, &args.rope, &args.scale);
@@ -390,6 +406,14 @@ mlakvStatus mlakvAttnDecode(const mlakvAttnPlan* plan, const mlakvCacheView* cac
   args.out_seq_stride = out_seq_stride;
   args.out_head_stride = out_head_stride;
   args.lse = lse;
+  if (quant != nullptr) {
+    args.out_codes = static_cast<char*>(quant->codes);
+    args.out_codes_seq_stride = quant->codes_seq_stride;
+    args.out_codes_head_stride = quant->codes_head_stride;
+    args.out_scales = static_cast<char*>(quant->scales);
+    args.out_scales_seq_stride = quant->scales_seq_stride;
+    args.out_scales_head_stride = quant->scales_head_stride;
+  }
   const uint64_t rows = static_cast<uint64_t>(plan->batch) * plan->max_chunks * plan->heads;
   args.partial_out = static_cast<char*>(workspace);
   args.partial_lse = workspace == nullptr ? nullptr : reinterpret_cast<float*>(static_cast<char*>(workspace) + rows * mlakv::kLatentDim * 2);
@@ -402,7 +426,61 @@ mlakvStatus mlakvAttnDecode(const mlakvAttnPlan* plan, const mlakvCacheView* cac
   args.max_chunks = plan->max_chunks;
   args.fp8 = cache->dtype == MLAKV_DTYPE_FP8_E4M3;
   const hipError_t status = mlakv::LaunchAttnDecode(args, static_cast<hipStream_t>(stream));
-  return status == hipSuccess ? MLAKV_SUCCESS : HipFail(status, "mlakvAttnDecode");
+  return status == hipSuccess ? MLAKV_SUCCESS : HipFail(status, who);
+}
+
+}  // namespace
+
+extern "C" {
+
+mlakvStatus mlakvAttnDecode(const mlakvAttnPlan* plan, const mlakvCacheView* cache, int32_t layer, const void* q_latent,
+                            int64_t q_latent_seq_stride, int64_t q_latent_head_stride, const void* q_rope,
+                            int64_t q_rope_seq_stride, int64_t q_rope_head_stride, const int32_t* block_table,
+                            int32_t table_stride, const int32_t* seq_lens, double scale, void* out, int64_t out_seq_stride,
+                            int64_t out_head_stride, float* lse, void* workspace, uint64_t workspace_bytes, void* stream) {
+  if (out == nullptr) return Fail(MLAKV_ERR_PARAM_NULLPTR, "mlakvAttnDecode: the output is required");
+  return AttnDecodeImpl("mlakvAttnDecode", plan, cache, layer, q_latent, q_latent_seq_stride, q_latent_head_stride, q_rope,
+                        q_rope_seq_stride, q_rope_head_stride, block_table, table_stride, seq_lens, scale, out, out_seq_stride,
+                        out_head_stride, nullptr, lse, workspace, workspace_bytes, stream);
+}
+
+mlakvStatus mlakvAttnDecodeMxQuant(const mlakvAttnPlan* plan, const mlakvCacheView* cache, int32_t layer, const void* q_latent,
+                                   int64_t q_latent_seq_stride, int64_t q_latent_head_stride, const void* q_rope,
+                                   int64_t q_rope_seq_stride, int64_t q_rope_head_stride, const int32_t* block_table,
+                                   int32_t table_stride, const int32_t* seq_lens, double scale, void* out, int64_t out_seq_stride,
+                                   int64_t out_head_stride, const mlakvMxQuantOut* quant, float* lse, void* workspace,
+                                   uint64_t workspace_bytes, void* stream) {
+  if (quant == nullptr) return Fail(MLAKV_ERR_PARAM_NULLPTR, "mlakvAttnDecodeMxQuant: the quantised output is required");
+  return AttnDecodeImpl("mlakvAttnDecodeMxQuant", plan, cache, layer, q_latent, q_latent_seq_stride, q_latent_head_stride, q_rope,
+                        q_rope_seq_stride, q_rope_head_stride, block_table, table_stride, seq_lens, scale, out, out_seq_stride,
+                        out_head_stride, quant, lse, workspace, workspace_bytes, stream);
+}
+
+mlakvStatus mlakvDynamicMxQuant(const void* x, int64_t x_row_stride, int64_t rows, int32_t cols, void* codes,
+                                int64_t codes_row_stride, void* scales, int64_t scales_row_stride, void* stream) {
+  const char* who = "mlakvDynamicMxQuant";
+  if (rows < 0 || cols < 0) return Fail(MLAKV_ERR_PARAM_INVALID, "%s: negative shape", who);
+  if (rows == 0 || cols == 0) return MLAKV_SUCCESS;
+  if (x == nullptr || codes == nullptr || scales == nullptr) return Fail(MLAKV_ERR_PARAM_NULLPTR, "%s: input, codes and scales are required", who);
+  if (cols % 32 != 0) return Fail(MLAKV_ERR_PARAM_INVALID, "%s: %d columns are not a whole number of blocks of 32", who, cols);
+  if (!Aligned16(x) || x_row_stride % 16 != 0 || x_row_stride < static_cast<int64_t>(cols) * 2) {
+    return Fail(MLAKV_ERR_PARAM_INVALID, "%s: input rows must be 16-byte aligned and hold %d bf16 values", who, cols);
+  }
+  if (reinterpret_cast<uintptr_t>(codes) % 8 != 0 || codes_row_stride % 8 != 0 || codes_row_stride < cols ||
+      scales_row_stride < cols / 32) {
+    return Fail(MLAKV_ERR_PARAM_INVALID, "%s: code rows must be 8-byte aligned and hold %d bytes, scale rows %d", who, cols, cols / 32);
+  }
+  mlakv::MxQuantArgs args{};
+  args.x = static_cast<const char*>(x);
+  args.x_row_stride = x_row_stride;
+  args.codes = static_cast<char*>(codes);
+  args.codes_row_stride = codes_row_stride;
+  args.scales = static_cast<char*>(scales);
+  args.scales_row_stride = scales_row_stride;
+  args.rows = rows;
+  args.cols = cols;
+  const hipError_t status = mlakv::LaunchMxQuant(args, static_cast<hipStream_t>(stream));
+  return status == hipSuccess ? MLAKV_SUCCESS : HipFail(status, who);
 }
 
 }  // extern "C"

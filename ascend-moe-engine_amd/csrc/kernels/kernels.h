@@ -96,6 +96,12 @@ struct AttnArgs {
   char* out;
   int64_t out_seq_stride, out_head_stride;
   float* lse;            // optional
+  // Optional block-32 MX quantisation of the output (E4M3 codes [batch][heads][512], E8M0 scales
+  // [batch][heads][16]); `out` may then be null.
+  char* out_codes;
+  int64_t out_codes_seq_stride, out_codes_head_stride;
+  char* out_scales;
+  int64_t out_scales_seq_stride, out_scales_head_stride;
   char* partial_out;     // workspace: [batch][max_chunks][heads][512] bf16
   float* partial_lse;    // workspace: [batch][max_chunks][heads] fp32, log2 domain
   float scale_log2;      // softmax scale * log2(e)
@@ -111,6 +117,17 @@ struct AttnArgs {
 #endif
 };
 
+struct MxQuantArgs {
+  const char* x;   // bf16 [rows][cols], cols a multiple of 32, rows 16-byte aligned
+  int64_t x_row_stride;
+  char* codes;     // E4M3 [rows][cols], rows 8-byte aligned
+  int64_t codes_row_stride;
+  char* scales;    // E8M0 [rows][cols / 32]
+  int64_t scales_row_stride;
+  int64_t rows;
+  int32_t cols;
+};
+
 // MLA geometry the kernels are specialised for (include/moe/core/config.hpp:78-109 defaults).
 constexpr int kLatentDim = 512;
 constexpr int kRopeDim = 64;
@@ -121,6 +138,7 @@ hipError_t LaunchNormRopeAppend(const NormRopeAppendArgs& args, hipStream_t stre
 hipError_t LaunchGather(const GatherArgs& args, hipStream_t stream);
 hipError_t LaunchCopyBlocks(const CopyBlocksArgs& args, hipStream_t stream);
 hipError_t LaunchAttnDecode(const AttnArgs& args, hipStream_t stream);
+hipError_t LaunchMxQuant(const MxQuantArgs& args, hipStream_t stream);
 // One-time per-process kernel attribute setup (dynamic LDS above 64 KB).
 hipError_t PrepareAttnKernels();
 

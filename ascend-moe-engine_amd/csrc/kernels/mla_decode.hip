@@ -51,6 +51,7 @@
 #include <utility>
 
 #include "kernels.h"
+#include "mx_quant_device.h"
 
 #pragma clang diagnostic ignored "-Winline-asm"
 
@@ -205,6 +206,15 @@ __device__ __forceinline__ float MaxAcrossHalves(float x) {
   const u32x2 swapped = __builtin_amdgcn_permlane32_swap(bits, bits, false, false);
   const unsigned a = swapped.x, b = swapped.y;
   return fmaxf(__builtin_bit_cast(float, a), __builtin_bit_cast(float, b));
+}
+__device__ __forceinline__ unsigned UMaxAcrossHeadLanes(unsigned bits) {
+  u32x2 swapped = __builtin_amdgcn_permlane16_swap(bits, bits, false, false);
+  unsigned a = swapped.x, b = swapped.y;
+  bits = max(a, b);
+  swapped = __builtin_amdgcn_permlane32_swap(bits, bits, false, false);
+  a = swapped.x;
+  b = swapped.y;
+  return max(a, b);
 }
 __device__ __forceinline__ float SumAcrossHeadLanes(float x) {
   unsigned bits = __builtin_bit_cast(unsigned, x);
@@ -408,7 +418,9 @@ __device__ __forceinline__ bf16x8 CodesToBf16(unsigned lo, unsigned hi) {
 
 // ---- main kernel -------------------------------------------------------------------
 
-template <bool FP8, bool ALIGNED>
+// MXQ: the single-chunk launch also quantises its output (and its bf16 output is optional). Kept
+// out of the common instantiation, whose register allocation has no room to spare.
+template <bool FP8, bool ALIGNED, bool MXQ>
 __global__ __launch_bounds__(kThreads) void MlaDecodeKernel(AttnArgs a) {
   using G = Geom<FP8>;
   extern __shared__ __attribute__((aligned(16))) unsigned char lds[];
@@ -477,8 +489,15 @@ __global__ __launch_bounds__(kThreads) void MlaDecodeKernel(AttnArgs a) {
       if (score_wave) {
         if (a.lse != nullptr && g == 0) a.lse[seq * a.heads + head] = -__builtin_inff();
       } else {
-        char* out = a.out + seq * a.out_seq_stride + head * a.out_head_stride;
-        for (int n = g; n < kLatentDim / 8; n += 4) *reinterpret_cast<u32x4*>(out + n * 16) = u32x4{0u, 0u, 0u, 0u};
+        if (!MXQ || a.out != nullptr) {
+          char* out = a.out + seq * a.out_seq_stride + head * a.out_head_stride;
+          for (int n = g; n < kLatentDim / 8; n += 4) *reinterpret_cast<u32x4*>(out + n * 16) = u32x4{0u, 0u, 0u, 0u};
+        }
+        if constexpr (MXQ) {  // zeros quantise to zero codes under the smallest scale
+          char* codes = a.out_codes + seq * a.out_codes_seq_stride + head * a.out_codes_head_stride;
+          for (int n = g; n < kLatentDim / 16; n += 4) *reinterpret_cast<u32x4*>(codes + n * 16) = u32x4{0u, 0u, 0u, 0u};
+          if (g == 0) *reinterpret_cast<u32x4*>(a.out_scales + seq * a.out_scales_seq_stride + head * a.out_scales_head_stride) = u32x4{0u, 0u, 0u, 0u};
+        }
       }
     } else if (active && score_wave && g == 0) {  // empty chunk: the merge reads every chunk's LSE
       a.partial_lse[(static_cast<int64_t>(seq) * a.max_chunks + chunk_index) * a.heads + head] = -__builtin_inff();
@@ -769,17 +788,49 @@ __global__ __launch_bounds__(kThreads) void MlaDecodeKernel(AttnArgs a) {
       const float inv = *inv_lds;
       char* out_row;
       if (direct) {
-        out_row = a.out + seq * a.out_seq_stride + head * a.out_head_stride;
+        out_row = MXQ && a.out == nullptr ? nullptr : a.out + seq * a.out_seq_stride + head * a.out_head_stride;
       } else {
         const int64_t row = (static_cast<int64_t>(seq) * a.max_chunks + chunk_index) * a.heads + head;
         out_row = a.partial_out + row * (kLatentDim * 2);
       }
+      if (MXQ && direct) {
+        // Quantising epilogue of the single-chunk case: a block of 32 columns is the tile pair
+        // (2k, 2k+1) over the four lanes that share this head.
+        char* codes_row = a.out_codes + seq * a.out_codes_seq_stride + head * a.out_codes_head_stride;
+        unsigned scale_codes[4] = {0u, 0u, 0u, 0u};
 #pragma unroll
-      for (int n = 0; n < kDvTiles; ++n) {
-        u32x2 packed;
-        packed.x = PackBf16(o[n][0] * inv, o[n][1] * inv);
-        packed.y = PackBf16(o[n][2] * inv, o[n][3] * inv);
-        __builtin_nontemporal_store(packed, reinterpret_cast<u32x2*>(out_row + (16 * n + 4 * g) * 2));
+        for (int k = 0; k < kDvTiles / 2; ++k) {
+          u32x2 packed[2];
+          unsigned magnitude = 0u;
+#pragma unroll
+          for (int h = 0; h < 2; ++h) {
+            const int n = 2 * k + h;
+            packed[h].x = PackBf16(o[n][0] * inv, o[n][1] * inv);
+            packed[h].y = PackBf16(o[n][2] * inv, o[n][3] * inv);
+            magnitude = MxMagnitudeMax(packed[h].y, MxMagnitudeMax(packed[h].x, magnitude));
+            if (out_row != nullptr) __builtin_nontemporal_store(packed[h], reinterpret_cast<u32x2*>(out_row + (16 * n + 4 * g) * 2));
+          }
+          magnitude = UMaxAcrossHeadLanes(magnitude);
+          const MxScale s = MxScaleFromMaxBits(magnitude);
+#pragma unroll
+          for (int h = 0; h < 2; ++h) {
+            const unsigned four = MxEncodeWord(packed[h].x, s) | (MxEncodeWord(packed[h].y, s) << 16);
+            __builtin_nontemporal_store(four, reinterpret_cast<unsigned*>(codes_row + 16 * (2 * k + h) + 4 * g));
+          }
+          scale_codes[k >> 2] |= s.code << (8 * (k & 3));
+        }
+        if (g == 0) {
+          *reinterpret_cast<u32x4*>(a.out_scales + seq * a.out_scales_seq_stride + head * a.out_scales_head_stride) =
+              u32x4{scale_codes[0], scale_codes[1], scale_codes[2], scale_codes[3]};
+        }
+      } else {
+#pragma unroll
+        for (int n = 0; n < kDvTiles; ++n) {
+          u32x2 packed;
+          packed.x = PackBf16(o[n][0] * inv, o[n][1] * inv);
+          packed.y = PackBf16(o[n][2] * inv, o[n][3] * inv);
+          __builtin_nontemporal_store(packed, reinterpret_cast<u32x2*>(out_row + (16 * n + 4 * g) * 2));
+        }
       }
     }
     MLAKV_STAMP(31);
@@ -834,30 +885,53 @@ __global__ __launch_bounds__(256) void MlaCombineKernel(AttnArgs a) {
       }
     }
   }
-  char* out = a.out + seq * a.out_seq_stride + head * a.out_head_stride + lane * 16;
-  if (denom == 0.0f) {  // empty sequence
-    *reinterpret_cast<u32x4*>(out) = u32x4{0u, 0u, 0u, 0u};
-    if (a.lse != nullptr && lane == 0) a.lse[seq * a.heads + head] = -__builtin_inff();
-    return;
-  }
-  const float inv = 1.0f / denom;
+  // An empty sequence (no live chunk) yields zeros and lse = -inf.
+  const float inv = denom == 0.0f ? 0.0f : 1.0f / denom;
   u32x4 packed;
   packed.x = PackBf16(acc[0] * inv, acc[1] * inv);
   packed.y = PackBf16(acc[2] * inv, acc[3] * inv);
   packed.z = PackBf16(acc[4] * inv, acc[5] * inv);
   packed.w = PackBf16(acc[6] * inv, acc[7] * inv);
-  *reinterpret_cast<u32x4*>(out) = packed;
-  if (a.lse != nullptr && lane == 0) a.lse[seq * a.heads + head] = (m + __builtin_amdgcn_logf(denom)) * 0.6931471805599453f;
+  if (a.out != nullptr) *reinterpret_cast<u32x4*>(a.out + seq * a.out_seq_stride + head * a.out_head_stride + lane * 16) = packed;
+  if (a.out_codes != nullptr) {
+    // Quantising epilogue (the reference's stage behind the attention): the four lanes of a
+    // block of 32 columns are neighbours; the codes come from the bf16-rounded values, as they
+    // would from the bf16 tensor.
+    unsigned magnitude = 0u;
+#pragma unroll
+    for (int i = 0; i < 4; ++i) magnitude = MxMagnitudeMax(packed[i], magnitude);
+    magnitude = max(magnitude, static_cast<unsigned>(__shfl_xor(static_cast<int>(magnitude), 1)));
+    magnitude = max(magnitude, static_cast<unsigned>(__shfl_xor(static_cast<int>(magnitude), 2)));
+    const MxScale s = MxScaleFromMaxBits(magnitude);
+    u32x2 codes;
+    codes.x = MxEncodeWord(packed.x, s) | (MxEncodeWord(packed.y, s) << 16);
+    codes.y = MxEncodeWord(packed.z, s) | (MxEncodeWord(packed.w, s) << 16);
+    *reinterpret_cast<u32x2*>(a.out_codes + seq * a.out_codes_seq_stride + head * a.out_codes_head_stride + lane * 8) = codes;
+    if ((lane & 3) == 0) {
+      reinterpret_cast<unsigned char*>(a.out_scales + seq * a.out_scales_seq_stride + head * a.out_scales_head_stride)[lane >> 2] =
+          static_cast<unsigned char>(s.code);
+    }
+  }
+  if (a.lse != nullptr && lane == 0) {
+    a.lse[seq * a.heads + head] = denom == 0.0f ? -__builtin_inff() : (m + __builtin_amdgcn_logf(denom)) * 0.6931471805599453f;
+  }
 }
 
-template <bool FP8, bool ALIGNED>
+template <bool FP8, bool ALIGNED, bool MXQ>
 hipError_t Launch(const AttnArgs& args, const dim3& grid, hipStream_t stream) {
   // Dynamic LDS above 64 KB needs the attribute once per kernel and process.
-  static const hipError_t prepared = hipFuncSetAttribute(reinterpret_cast<const void*>(&MlaDecodeKernel<FP8, ALIGNED>),
+  static const hipError_t prepared = hipFuncSetAttribute(reinterpret_cast<const void*>(&MlaDecodeKernel<FP8, ALIGNED, MXQ>),
                                                          hipFuncAttributeMaxDynamicSharedMemorySize, Geom<FP8>::kLdsBytes);
   if (prepared != hipSuccess) return prepared;
-  hipLaunchKernelGGL((MlaDecodeKernel<FP8, ALIGNED>), grid, dim3(kThreads), Geom<FP8>::kLdsBytes, stream, args);
+  hipLaunchKernelGGL((MlaDecodeKernel<FP8, ALIGNED, MXQ>), grid, dim3(kThreads), Geom<FP8>::kLdsBytes, stream, args);
   return hipGetLastError();
+}
+
+template <bool MXQ>
+hipError_t LaunchByCache(const AttnArgs& args, const dim3& grid, hipStream_t stream) {
+  const bool aligned = args.block_size % kTileTokens == 0;
+  if (args.fp8) return aligned ? Launch<true, true, MXQ>(args, grid, stream) : Launch<true, false, MXQ>(args, grid, stream);
+  return aligned ? Launch<false, true, MXQ>(args, grid, stream) : Launch<false, false, MXQ>(args, grid, stream);
 }
 
 }  // namespace
@@ -871,10 +945,9 @@ hipError_t LaunchAttnDecode(const AttnArgs& args_in, hipStream_t stream) {
 #endif
   if (args.batch <= 0) return hipSuccess;
   const dim3 grid(args.max_chunks, args.batch, (args.heads + 63) / 64);
-  const bool aligned = args.block_size % kTileTokens == 0;
-  hipError_t e;
-  if (args.fp8) e = aligned ? Launch<true, true>(args, grid, stream) : Launch<true, false>(args, grid, stream);
-  else e = aligned ? Launch<false, true>(args, grid, stream) : Launch<false, false>(args, grid, stream);
+  // With several chunks the merge kernel owns the final output and the optional quantisation.
+  const bool quantise_here = args.max_chunks == 1 && args.out_codes != nullptr;
+  hipError_t e = quantise_here ? LaunchByCache<true>(args, grid, stream) : LaunchByCache<false>(args, grid, stream);
   if (e != hipSuccess) return e;
   if (args.max_chunks > 1) {
     hipLaunchKernelGGL(MlaCombineKernel, dim3((args.heads + kCombineHeads - 1) / kCombineHeads, args.batch), dim3(256), 0,

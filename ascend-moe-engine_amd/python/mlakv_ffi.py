@@ -40,6 +40,11 @@ class CacheView(C.Structure):
     ]
 
 
+class MxQuantOut(C.Structure):
+    _fields_ = [("codes", C.c_void_p), ("codes_seq_stride", C.c_int64), ("codes_head_stride", C.c_int64),
+                ("scales", C.c_void_p), ("scales_seq_stride", C.c_int64), ("scales_head_stride", C.c_int64)]
+
+
 class AttnPlan(C.Structure):
     _fields_ = [
         ("batch", C.c_int32), ("heads", C.c_int32), ("max_seq_len", C.c_int32), ("block_size", C.c_int32),
@@ -79,6 +84,9 @@ PROTOTYPES = {
     "mlakvAttnPlanInit": (_i32, [_i32, _i32, _i32, _i32, _i32, _P(AttnPlan)]),
     "mlakvAttnDecode": (_i32, [_P(AttnPlan), _P(CacheView), _i32, _vp, _i64, _i64, _vp, _i64, _i64, _vp, _i32, _vp,
                                C.c_double, _vp, _i64, _i64, _vp, _vp, _u64, _vp]),
+    "mlakvAttnDecodeMxQuant": (_i32, [_P(AttnPlan), _P(CacheView), _i32, _vp, _i64, _i64, _vp, _i64, _i64, _vp, _i32, _vp,
+                                      C.c_double, _vp, _i64, _i64, _P(MxQuantOut), _vp, _vp, _u64, _vp]),
+    "mlakvDynamicMxQuant": (_i32, [_vp, _i64, _i64, _i32, _vp, _i64, _vp, _i64, _vp]),
     "mlakvArenaCreate": (_i32, [_i32, _P(_vp)]),
     "mlakvArenaDestroy": (None, [_vp]),
     "mlakvArenaReserve": (_i32, [_vp, C.c_char_p, _sz, _sz, _P(_sz)]),

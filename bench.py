@@ -157,7 +157,8 @@ def bench_append_gather(args, torch, np, ffi):
     return result
 
 
-def bench_attention(args, torch, np, ffi, fp8=False, batch=32, ctx=2048, heads=64, slices=8, iters=None, label=None):
+def bench_attention(args, torch, np, ffi, fp8=False, batch=32, ctx=2048, heads=64, slices=8, iters=None, label=None,
+                    mx_quant=False):
     lib = ffi.load()
     bs = 64
     slices = int(os.environ.get("MLAKV_BENCH_SLICES", slices))  # development aid: 1 keeps the KV cache-resident
@@ -200,16 +201,44 @@ def bench_attention(args, torch, np, ffi, fp8=False, batch=32, ctx=2048, heads=6
                                       arena.workspace, arena.workspace_bytes, stream_ptr(torch)))
 
     iters = iters or max(args.steps * 8, 64)
-    for i in range(16):
-        launch(i)
-    torch.cuda.synchronize()
-    start, stop = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
-    start.record()
-    for i in range(iters):
-        launch(i)
-    stop.record()
-    torch.cuda.synchronize()
-    us = start.elapsed_time(stop) * 1e3 / iters
+
+    def timed_us(fn):
+        for i in range(16):
+            fn(i)
+        torch.cuda.synchronize()
+        start, stop = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+        start.record()
+        for i in range(iters):
+            fn(i)
+        stop.record()
+        torch.cuda.synchronize()
+        return start.elapsed_time(stop) * 1e3 / iters
+
+    us = timed_us(launch)
+    mx = None
+    if mx_quant:
+        # the reference's next stage, block-32 MX quantisation of the output: fused into the
+        # attention epilogue, against attention followed by the standalone operator
+        codes = torch.empty(slices, batch, heads, LATENT, dtype=torch.uint8, device="cuda")
+        scales = torch.empty(slices, batch, heads, LATENT // 32, dtype=torch.uint8, device="cuda")
+        targets = [ffi.MxQuantOut(codes[k].data_ptr(), heads * LATENT, LATENT, scales[k].data_ptr(), heads * (LATENT // 32),
+                                  LATENT // 32) for k in range(slices)]
+
+        def fused(i):
+            k = i % slices
+            ffi.check(lib.mlakvAttnDecodeMxQuant(C.byref(plan), C.byref(view), k, q[k].data_ptr(), heads * ROW_BYTES, ROW_BYTES,
+                                                 q[k].data_ptr() + LATENT * 2, heads * ROW_BYTES, ROW_BYTES,
+                                                 cache.device_block_table, cache.num_blocks, cache.device_seq_lens,
+                                                 1.0 / math.sqrt(192.0), None, 0, 0, C.byref(targets[k]), None,
+                                                 arena.workspace, arena.workspace_bytes, stream_ptr(torch)))
+
+        def unfused(i):
+            k = i % slices
+            launch(i)
+            ffi.check(lib.mlakvDynamicMxQuant(out[k].data_ptr(), LATENT * 2, batch * heads, LATENT, codes[k].data_ptr(), LATENT,
+                                              scales[k].data_ptr(), LATENT // 32, stream_ptr(torch)))
+
+        mx = {"us_fused_epilogue": timed_us(fused), "us_attention_then_quant": timed_us(unfused)}
     kv_row = 580 if fp8 else ROW_BYTES
     algorithmic = batch * ctx * kv_row + batch * heads * ROW * 2 + batch * heads * LATENT * 2 + 4 * batch * blocks_per_seq
     flops = 2.0 * batch * heads * ctx * (ROW + LATENT)
@@ -225,6 +254,8 @@ def bench_attention(args, torch, np, ffi, fp8=False, batch=32, ctx=2048, heads=6
         "chunk_tiles": int(plan.chunk_tiles), "max_chunks": int(plan.max_chunks),
         "workspace_bytes": int(plan.workspace_bytes), "launches_timed": iters,
     }
+    if mx is not None:
+        result["mx_quant_output"] = mx
     cache.close()
     arena.close()
     return result
@@ -426,7 +457,7 @@ def main():
         print(json.dumps({"side_kernels": bench_side_kernels(args, torch, np, ffi)}))
         return 0
     if args.attention_only:
-        print(json.dumps({"attention": bench_attention(args, torch, np, ffi),
+        print(json.dumps({"attention": bench_attention(args, torch, np, ffi, mx_quant=True),
                           "attention_fp8": bench_attention(args, torch, np, ffi, fp8=True, batch=64, ctx=4352, iters=64),
                           "attention_long": bench_attention(args, torch, np, ffi, batch=128, ctx=8192, slices=2, iters=16,
                                                             label="configs[4]-scale decode shape (one workgroup per sequence)")}))
@@ -452,7 +483,7 @@ def main():
         "append": {"avg_launch_ms": ag["append_ms"], "achieved_gbps": ag["append_gbps"]},
     }
     if not args.no_attention:
-        line["attention"] = bench_attention(args, torch, np, ffi)
+        line["attention"] = bench_attention(args, torch, np, ffi, mx_quant=True)
         line["attention_fp8"] = bench_attention(args, torch, np, ffi, fp8=True, batch=64, ctx=4352, iters=64)
         line["attention_long"] = bench_attention(args, torch, np, ffi, batch=128, ctx=8192, slices=2, iters=16,
                                                  label="configs[4]-scale decode shape (one workgroup per sequence)")

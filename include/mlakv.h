@@ -160,6 +160,41 @@ mlakvStatus mlakvAttnDecode(const mlakvAttnPlan* plan, const mlakvCacheView* cac
                             void* out, int64_t out_seq_stride, int64_t out_head_stride, float* lse, void* workspace,
                             uint64_t workspace_bytes, void* stream);
 
+/* Block-32 MX quantization of bf16 rows along the last axis: replaces the plan + launch of
+ * aclnnDynamicMxQuant (contract include/moe/core/op_table.hpp:205-233; the reference's stages
+ * `attn_quant` src/pipeline/pipeline.cpp:251-258 and `shared_act_quant`), with the reference's
+ * fixed attributes: axis -1, round mode rint, dst E4M3, blocksize 32, OCP scale algorithm
+ * (OCP Microscaling Formats v1.0, 6.3):
+ *   shared_exp = floor(log2(max |v|)) - 8 clamped to [-127, 127], scale byte = shared_exp + 127 (E8M0)
+ *   code       = e4m3(v * 2^-shared_exp), nearest even, saturating at +-448
+ * A block of zeros gets scale byte 0 and zero codes; a block holding Inf/NaN gets scale 0xff and
+ * NaN codes. x is bf16 [rows][cols] (cols a multiple of 32), codes E4M3 [rows][cols], scales
+ * E8M0 [rows][cols / 32]; strides in bytes. */
+mlakvStatus mlakvDynamicMxQuant(const void* x, int64_t x_row_stride, int64_t rows, int32_t cols, void* codes,
+                                int64_t codes_row_stride, void* scales, int64_t scales_row_stride, void* stream);
+
+/* Where the quantized attention output goes: codes E4M3 [batch][heads][512] and scales E8M0
+ * [batch][heads][16] at byte strides (the reference's act.attn_fp8 [tokens][heads * 512] and
+ * act.attn_mx_scale [tokens][heads * 16], src/memory/static_arena_manager.cpp:493-496). */
+typedef struct mlakvMxQuantOut {
+  void* codes;
+  int64_t codes_seq_stride, codes_head_stride;
+  void* scales;
+  int64_t scales_seq_stride, scales_head_stride;
+} mlakvMxQuantOut;
+
+/* Decode attention with the quantization of its output fused into the epilogue: the stages
+ * `attention` and `attn_quant` that the reference launches back to back
+ * (src/pipeline/pipeline.cpp:235-258, :416-417) in one call. The codes and scales are those
+ * mlakvDynamicMxQuant gives on the bf16 output of mlakvAttnDecode, bit for bit; `out` (bf16) is
+ * optional here and, when given, receives that output as well. */
+mlakvStatus mlakvAttnDecodeMxQuant(const mlakvAttnPlan* plan, const mlakvCacheView* cache, int32_t layer,
+                                   const void* q_latent, int64_t q_latent_seq_stride, int64_t q_latent_head_stride,
+                                   const void* q_rope, int64_t q_rope_seq_stride, int64_t q_rope_head_stride,
+                                   const int32_t* block_table, int32_t table_stride, const int32_t* seq_lens, double scale,
+                                   void* out, int64_t out_seq_stride, int64_t out_head_stride, const mlakvMxQuantOut* quant,
+                                   float* lse, void* workspace, uint64_t workspace_bytes, void* stream);
+
 /* ------------------------------------------------------------------------- */
 /* Static arena (host)                                                        */
 /* ------------------------------------------------------------------------- */

@@ -459,6 +459,51 @@ void kvo_norm_rope_rows(const uint16_t* kv_a, int64_t kv_a_row_stride, const uin
 }
 
 /* ------------------------------------------------------------------------- */
+/* OCP microscaling (MX) quantization of the attention output                 */
+/* ------------------------------------------------------------------------- */
+
+void kvo_mx_quant_rows(const uint16_t* x, int64_t x_row_stride, int64_t rows, int64_t cols, uint8_t* codes,
+                       int64_t codes_row_stride, uint8_t* scales, int64_t scales_row_stride) {
+  const int64_t block = 32;
+  const int element_emax = 8; /* E4M3: largest power of two is 2^8 (448 = 1.75 * 2^8) */
+  for (int64_t r = 0; r < rows; ++r) {
+    for (int64_t b0 = 0; b0 < cols; b0 += block) {
+      const int64_t n = cols - b0 < block ? cols - b0 : block;
+      const uint16_t* v = x + r * x_row_stride + b0;
+      float absmax = 0.0f;
+      int special = 0;
+      for (int64_t i = 0; i < n; ++i) {
+        const float f = kvo_bf16_to_f32(v[i]);
+        if (isnan(f) || isinf(f)) special = 1;
+        else if (fabsf(f) > absmax) absmax = fabsf(f);
+      }
+      uint8_t* out = codes + r * codes_row_stride + b0;
+      uint8_t* scale_code = scales + r * scales_row_stride + b0 / block;
+      if (special) { /* the shared scale is NaN and so is every element */
+        *scale_code = 0xffu;
+        for (int64_t i = 0; i < n; ++i) out[i] = (uint8_t)((v[i] >> 8 & 0x80u) | 0x7fu);
+        continue;
+      }
+      int shared_exp = -127;
+      if (absmax > 0.0f) {
+        int e;
+        (void)frexpf(absmax, &e); /* absmax = m * 2^e, m in [0.5, 1): floor(log2 absmax) = e - 1 */
+        shared_exp = e - 1 - element_emax;
+        if (shared_exp < -127) shared_exp = -127;
+        if (shared_exp > 127) shared_exp = 127;
+      }
+      *scale_code = (uint8_t)(shared_exp + 127);
+      for (int64_t i = 0; i < n; ++i) {
+        /* v * 2^-shared_exp in double is exact; the float cast is exact too unless the value is
+         * far below the element grid, where it rounds to zero either way. */
+        const double scaled = ldexp((double)kvo_bf16_to_f32(v[i]), -shared_exp);
+        out[i] = kvo_e4m3_from_f32((float)scaled);
+      }
+    }
+  }
+}
+
+/* ------------------------------------------------------------------------- */
 /* absorbed-MLA decode attention                                              */
 /* ------------------------------------------------------------------------- */
 

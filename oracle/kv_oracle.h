@@ -163,6 +163,20 @@ void kvo_rope_rows(const uint16_t* rows, int64_t row_stride, const uint16_t* rop
                    int64_t rope_table_row_stride, const int32_t* positions, int64_t rows_per_position, int64_t num_rows,
                    int64_t rope_dim, uint16_t* out, int64_t out_row_stride);
 
+/* Block-32 MX quantization of bf16 rows along the last axis: the stage `attn_quant` behind the
+ * attention (reference src/pipeline/pipeline.cpp:251-258: aclnnDynamicMxQuant, axis -1, round mode
+ * rint, dst E4M3, blocksize kRoutedScaleBlock = 32, scale algorithm OCP; contract
+ * include/moe/core/op_table.hpp:205-233). The operator's kernel is closed (CANN); this restates the
+ * published algorithm it names, OCP Microscaling Formats (MX) v1.0 section 6.3:
+ *   shared_exp = floor(log2(max_i |v_i|)) - 8          (8 = emax of E4M3), clamped to [-127, 127]
+ *   scale code = shared_exp + 127                        (E8M0; 0xff = NaN)
+ *   code_i     = e4m3(v_i / 2^shared_exp)                (round to nearest even, saturating at +-448)
+ * A block of zeros takes the smallest scale (code 0) and zero elements; a block holding an Inf or
+ * NaN takes the NaN scale and NaN elements. A trailing block shorter than 32 is quantized over
+ * the elements it has. Parity with CANN on the zero and non-finite blocks is unpinned. */
+void kvo_mx_quant_rows(const uint16_t* x, int64_t x_row_stride, int64_t rows, int64_t cols, uint8_t* codes,
+                       int64_t codes_row_stride, uint8_t* scales, int64_t scales_row_stride);
+
 /* Quantize-on-append: one fp32 scale per token row over latent+rope, code = e4m3(x / scale). */
 void kvo_append_rows_fp8(uint8_t* latent_plane, int64_t latent_block_stride, int64_t latent_row_stride,
                          uint8_t* rope_plane, int64_t rope_block_stride, int64_t rope_row_stride,

@@ -75,6 +75,7 @@ _PROTOTYPES = {
                                    _vp, _i64, _i64, _i64]),
     "kvo_norm_rope_rows": (None, [_vp, _i64, _vp, C.c_double, _vp, _vp, _i64, _vp, _i64, _i64, _i64, _vp, _i64, _vp, _i64]),
     "kvo_rope_rows": (None, [_vp, _i64, _vp, _vp, _i64, _vp, _i64, _i64, _i64, _vp, _i64]),
+    "kvo_mx_quant_rows": (None, [_vp, _i64, _i64, _i64, _vp, _i64, _vp, _i64]),
     "kvo_mla_decode": (None, [_vp, _i64, _i64, _vp, _i64, _i64, _P(CacheView), _vp, _i64, _vp, _i64, _i64, C.c_double,
                               _vp, _vp, C.c_int]),
     "kvo_splitmix64": (_u64, [_P(_u64)]),
@@ -247,6 +248,16 @@ def rope_rows(rows, rope_cos, rope_sin, positions, rows_per_position=1):
     load().kvo_rope_rows(_ptr(rows), rows.shape[1], _ptr(rope_cos), _ptr(rope_sin), rope_cos.shape[1], _ptr(positions),
                          rows_per_position, rows.shape[0], rows.shape[1], _ptr(out), rows.shape[1])
     return out
+
+
+def mx_quant_rows(x):
+    """x uint16 [rows, cols] bf16 bits. Returns (codes uint8 [rows, cols], scales uint8 [rows, ceil(cols/32)])."""
+    x = np.ascontiguousarray(x, dtype=np.uint16)
+    rows, cols = x.shape
+    codes = np.zeros((rows, cols), dtype=np.uint8)
+    scales = np.zeros((rows, -(-cols // 32)), dtype=np.uint8)
+    load().kvo_mx_quant_rows(_ptr(x), cols, rows, cols, _ptr(codes), cols, _ptr(scales), scales.shape[1])
+    return codes, scales
 
 
 def gather_rows_fp8(latent_plane, rope_plane, scale_plane, block_size, table, seq_lens, latent_dim=512, rope_dim=64):

@@ -120,8 +120,10 @@ def gather(cache, table, seq_lens, fused_out=False, layer_begin=0, layer_count=N
     return latent_out[:, :total], rope_out[:, :total]
 
 
-def attention(cache, layer, q, table, seq_lens, scale, max_seq_len=None, want_lse=True):
-    """q [B, H, 576] bf16 cuda (latent | rope per head). Returns (out [B,H,512] bf16, lse [B,H] f32, plan)."""
+def attention(cache, layer, q, table, seq_lens, scale, max_seq_len=None, want_lse=True, quant=False, want_out=True):
+    """q [B, H, 576] bf16 cuda (latent | rope per head). Returns (out [B,H,512] bf16, lse [B,H] f32, plan);
+    with quant=True through the fused entry point, returning (out or None, lse, plan, codes [B,H,512] u8,
+    scales [B,H,16] u8)."""
     lib = ffi.load()
     batch, heads = q.shape[0], q.shape[1]
     lens = seq_lens.cpu().numpy()
@@ -130,16 +132,23 @@ def attention(cache, layer, q, table, seq_lens, scale, max_seq_len=None, want_ls
     ffi.check(lib.mlakvAttnPlanInit(batch, heads, max_seq_len, cache.block_size,
                                     ffi.DTYPE_FP8_E4M3 if cache.fp8 else ffi.DTYPE_BF16, C.byref(plan)))
     workspace = torch.empty(max(int(plan.workspace_bytes), 16), dtype=torch.uint8, device="cuda")
-    out = torch.full((batch, heads, LATENT), float("nan"), dtype=torch.bfloat16, device="cuda")
+    out = torch.full((batch, heads, LATENT), float("nan"), dtype=torch.bfloat16, device="cuda") if want_out else None
     lse = torch.full((batch, heads), float("nan"), dtype=torch.float32, device="cuda") if want_lse else None
     row = (LATENT + ROPE) * 2
-    ffi.check(lib.mlakvAttnDecode(C.byref(plan), C.byref(cache.view), layer, q.data_ptr(), heads * row, row,
-                                  q.data_ptr() + LATENT * 2, heads * row, row, table.data_ptr(), table.shape[1],
-                                  seq_lens.data_ptr(), float(scale), out.data_ptr(), heads * LATENT * 2, LATENT * 2,
-                                  lse.data_ptr() if want_lse else None, workspace.data_ptr(), int(plan.workspace_bytes),
-                                  stream_ptr()))
+    head_args = (C.byref(plan), C.byref(cache.view), layer, q.data_ptr(), heads * row, row,
+                 q.data_ptr() + LATENT * 2, heads * row, row, table.data_ptr(), table.shape[1],
+                 seq_lens.data_ptr(), float(scale), out.data_ptr() if want_out else None, heads * LATENT * 2, LATENT * 2)
+    tail_args = (lse.data_ptr() if want_lse else None, workspace.data_ptr(), int(plan.workspace_bytes), stream_ptr())
+    if not quant:
+        ffi.check(lib.mlakvAttnDecode(*head_args, *tail_args))
+        torch.cuda.synchronize()
+        return out, lse, plan
+    codes = torch.full((batch, heads, LATENT), 0xAA, dtype=torch.uint8, device="cuda")
+    scales = torch.full((batch, heads, LATENT // 32), 0xAA, dtype=torch.uint8, device="cuda")
+    target = ffi.MxQuantOut(codes.data_ptr(), heads * LATENT, LATENT, scales.data_ptr(), heads * (LATENT // 32), LATENT // 32)
+    ffi.check(lib.mlakvAttnDecodeMxQuant(*head_args, C.byref(target), *tail_args))
     torch.cuda.synchronize()
-    return out, lse, plan
+    return out, lse, plan, codes, scales
 
 
 def oracle_attention(cache, layer, q, table_np, lens_np, scale, accum_f32=False):
