@@ -735,6 +735,32 @@ mlakvStatus mlakvKvCacheGetStats(const mlakvKvCache* cache, mlakvKvStats* stats)
   return MLAKV_SUCCESS;
 }
 
+int64_t mlakvKvStatsFormatJson(const mlakvKvStats* stats, char* buffer, size_t capacity) {
+  if (stats == nullptr) return -1;
+  // %.12g is what an ostream at precision 12 in the classic locale prints for a double; a
+  // non-finite utilisation is written as null.
+  char utilization[40];
+  if (std::isfinite(stats->kv_cache_utilization)) {
+    std::snprintf(utilization, sizeof utilization, "%.12g", stats->kv_cache_utilization);
+    for (char* c = utilization; *c != 0; ++c) {
+      if (*c == ',') *c = '.';  // a process-wide locale with a decimal comma must not leak into JSON
+    }
+  } else {
+    std::snprintf(utilization, sizeof utilization, "null");
+  }
+  const int needed = std::snprintf(buffer, buffer == nullptr ? 0 : capacity,
+                                   "  \"paged_attention\": {\n"
+                                   "    \"total_blocks_allocated\": %llu,\n"
+                                   "    \"active_context_tokens\": %llu,\n"
+                                   "    \"block_size\": %llu,\n"
+                                   "    \"kv_cache_utilization\": %s\n"
+                                   "  }",
+                                   static_cast<unsigned long long>(stats->total_blocks_allocated),
+                                   static_cast<unsigned long long>(stats->active_context_tokens),
+                                   static_cast<unsigned long long>(stats->block_size), utilization);
+  return needed;
+}
+
 const int32_t* mlakvKvCacheHostBlockTable(const mlakvKvCache* cache) { return cache ? cache->manager->host_block_table() : nullptr; }
 const int32_t* mlakvKvCacheHostSlotMapping(const mlakvKvCache* cache) { return cache ? cache->manager->host_slot_mapping() : nullptr; }
 const int32_t* mlakvKvCacheHostSeqLens(const mlakvKvCache* cache) { return cache ? cache->manager->host_seq_lens() : nullptr; }

@@ -119,6 +119,7 @@ PROTOTYPES = {
     "mlakvKvCacheCompact": (_i32, [_vp, _P(_i32), _P(_i64), _vp]),
     "mlakvKvCacheUploadStep": (_i32, [_vp, _vp]),
     "mlakvKvCacheGetStats": (_i32, [_vp, _P(KvStats)]),
+    "mlakvKvStatsFormatJson": (_i64, [_P(KvStats), C.c_char_p, _sz]),
     "mlakvKvCacheHostBlockTable": (_P(_i32), [_vp]),
     "mlakvKvCacheHostSlotMapping": (_P(_i32), [_vp]),
     "mlakvKvCacheHostSeqLens": (_P(_i32), [_vp]),

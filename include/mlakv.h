@@ -290,6 +290,13 @@ mlakvStatus mlakvKvCacheCompact(mlakvKvCache* cache, int32_t* moves, int64_t* nu
  * slot mailbox copy (src/pipeline/pipeline.cpp:515-519). On the host backend it is a memcpy. */
 mlakvStatus mlakvKvCacheUploadStep(mlakvKvCache* cache, void* stream);
 mlakvStatus mlakvKvCacheGetStats(const mlakvKvCache* cache, mlakvKvStats* stats);
+/* The "paged_attention" member of the reference's --diag-json file, byte for byte as
+ * InferenceDiagnostics::DumpJson writes it (src/diagnostics/inference_stats.cpp:42-47: two-space
+ * member indent, numbers at 12 significant digits, null for a non-finite utilization; sample
+ * docs/examples/inference_diagnostics_dry_run.json), without a trailing comma or newline, for a
+ * harness that assembles that file. Returns the length needed excluding the terminator (call with
+ * buffer NULL to size it), or -1 for a null stats pointer; writes at most `capacity` bytes. */
+int64_t mlakvKvStatsFormatJson(const mlakvKvStats* stats, char* buffer, size_t capacity);
 /* Host mirrors (valid until the cache is destroyed). */
 const int32_t* mlakvKvCacheHostBlockTable(const mlakvKvCache* cache);  /* [max_batch][num_blocks] */
 const int32_t* mlakvKvCacheHostSlotMapping(const mlakvKvCache* cache); /* [max_batch], -1 = no token this step */

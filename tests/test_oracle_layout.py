@@ -268,3 +268,60 @@ def test_kv_diagnostics_goldens(oracle, goldens):
     assert utilisations[(128, 256, 1)] == 2.0 / 256.0            # tests/mock_pipeline_e2e.cpp:663-666
     assert utilisations[(64, 8192, 128)] == 0.0157470703125      # docs/preflight-verification.md:42-45
     assert utilisations[(64, 8192, 127)] == 0.015625
+
+
+# The "paged_attention" member of the reference's sample diagnostics file, as it stands there
+# (docs/examples/inference_diagnostics_dry_run.json:19-24: 43 layers, block 128, context 8192,
+# nothing decoded yet).
+_DRY_RUN_PAGED_ATTENTION = (
+    '  "paged_attention": {\n'
+    '    "total_blocks_allocated": 2752,\n'
+    '    "active_context_tokens": 0,\n'
+    '    "block_size": 128,\n'
+    '    "kv_cache_utilization": 0\n'
+    '  }'
+)
+
+
+def test_diag_json_paged_attention_block_matches_the_reference_sample_byte_for_byte():
+    lib = ffi.load()
+    arena = ffi.Arena(ffi.BACKEND_HOST)
+    cache = ffi.KvCache(arena, num_layers=43, block_size=128, max_context_len=8192, max_batch=1)
+    stats = cache.stats()
+    needed = lib.mlakvKvStatsFormatJson(C.byref(stats), None, 0)
+    assert needed == len(_DRY_RUN_PAGED_ATTENTION)
+    buffer = C.create_string_buffer(needed + 1)
+    assert lib.mlakvKvStatsFormatJson(C.byref(stats), buffer, needed + 1) == needed
+    assert buffer.value.decode() == _DRY_RUN_PAGED_ATTENTION
+    # spliced into a document it parses, and a truncating buffer is never overrun
+    import json
+    assert json.loads("{\n" + buffer.value.decode() + "\n}")["paged_attention"]["total_blocks_allocated"] == 2752
+    small = C.create_string_buffer(b"\xff" * 16, 16)
+    assert lib.mlakvKvStatsFormatJson(C.byref(stats), small, 8) == needed
+    assert small.raw[7:8] == b"\x00" and small.raw[8:] == b"\xff" * 8
+    # 12 significant digits as an ostream at precision 12 prints them (docs/preflight-verification.md:42-45
+    # quotes 0.0157470703125 for 129 tokens of 8192), and null for a non-finite value
+    cache.add_sequence(0, 0)
+    for _ in range(129):
+        cache.append_token(0)
+    cache.close()
+    arena.close()
+    arena = ffi.Arena(ffi.BACKEND_HOST)
+    cache = ffi.KvCache(arena, num_layers=43, block_size=64, max_context_len=8192, max_batch=1)
+    cache.add_sequence(0, 0)
+    for _ in range(129):
+        cache.append_token(0)
+    stats = cache.stats()
+    buffer = C.create_string_buffer(256)
+    lib.mlakvKvStatsFormatJson(C.byref(stats), buffer, 256)
+    assert '"kv_cache_utilization": 0.0157470703125\n' in buffer.value.decode()
+    assert '"active_context_tokens": 129,' in buffer.value.decode()
+    stats.kv_cache_utilization = float("nan")
+    lib.mlakvKvStatsFormatJson(C.byref(stats), buffer, 256)
+    assert '"kv_cache_utilization": null\n' in buffer.value.decode()
+    stats.kv_cache_utilization = 1.0 / 3.0
+    lib.mlakvKvStatsFormatJson(C.byref(stats), buffer, 256)
+    assert '"kv_cache_utilization": 0.333333333333\n' in buffer.value.decode()
+    assert lib.mlakvKvStatsFormatJson(None, buffer, 256) == -1
+    cache.close()
+    arena.close()
