@@ -61,8 +61,8 @@
 #include <cstdlib>
 #define MLAKV_STAMP(slot)                                                                              \
   do {                                                                                                 \
-    if (a.trace != nullptr && lane == 0 && (wave == 0 || wave == 4) && (slot) >= 0 && (slot) < 32) {                     \
-      a.trace[((blockIdx.y * gridDim.x + blockIdx.x) * 2 + (wave >> 2)) * 32 + (slot)] = __builtin_amdgcn_s_memrealtime(); \
+    if (a.trace != nullptr && lane == 0 && (wave == 0 || wave == 4) && (slot) >= 0 && (slot) < 40) {                     \
+      a.trace[((blockIdx.y * gridDim.x + blockIdx.x) * 2 + (wave >> 2)) * 40 + (slot)] = __builtin_amdgcn_s_memrealtime(); \
     }                                                                                                  \
   } while (0)
 #else
@@ -73,6 +73,8 @@
 
 namespace mlakv {
 namespace {
+
+constexpr int kXcds = 8;
 
 typedef __attribute__((ext_vector_type(8))) __bf16 bf16x8;
 typedef __attribute__((ext_vector_type(4))) __bf16 bf16x4;
@@ -430,8 +432,20 @@ __global__ __launch_bounds__(kThreads) void MlaDecodeKernel(AttnArgs a) {
   const bool score_wave = wave < kScoreWaves;   // wave-uniform role
   const int hw = wave & (kScoreWaves - 1);      // which 16 heads of the 64
   const int g = lane >> 4, i16 = lane & 15;
-  const int chunk_index = blockIdx.x;
-  const int seq = blockIdx.y;
+  // Workgroups are handed to the eight XCDs round-robin by linear id, and each XCD has its own
+  // L2. The chunks of one sequence all read the same 72 KB of Q, so they are placed on one XCD:
+  // XCD x takes the contiguous range of (sequence, chunk) pairs [x, x+1) * pairs / 8.
+  int chunk_index = blockIdx.x;
+  int seq = blockIdx.y;
+  {
+    const int pairs = gridDim.x * gridDim.y;
+    if ((pairs & (kXcds - 1)) == 0) {
+      const int linear = blockIdx.y * gridDim.x + blockIdx.x;
+      const int pair = (linear & (kXcds - 1)) * (pairs / kXcds) + linear / kXcds;
+      seq = pair / static_cast<int>(gridDim.x);
+      chunk_index = pair - seq * static_cast<int>(gridDim.x);
+    }
+  }
   const int head_base = blockIdx.z * 64 + hw * 16;
   const bool active = head_base < a.heads;  // wave-uniform
   const int head = head_base + i16;
@@ -445,7 +459,7 @@ __global__ __launch_bounds__(kThreads) void MlaDecodeKernel(AttnArgs a) {
   // window is Q[head][64 (ks/2) + 16g + 8 (ks&1) .. +7]. Issued first so that they travel while
   // the lengths and the block table are fetched.
   bf16x8 q[kKSteps];
-  if (score_wave && active) {
+  const auto load_q = [&]() __attribute__((always_inline)) {
     const char* q_latent = a.q_latent + seq * a.q_latent_seq_stride + head * a.q_latent_head_stride;
     const char* q_rope = a.q_rope + seq * a.q_rope_seq_stride + head * a.q_rope_head_stride;
 #pragma unroll
@@ -454,7 +468,9 @@ __global__ __launch_bounds__(kThreads) void MlaDecodeKernel(AttnArgs a) {
       const char* p = d0 < kLatentDim ? q_latent + d0 * 2 : q_rope + (d0 - kLatentDim) * 2;
       q[ks] = __builtin_bit_cast(bf16x8, GlobalLoad16(p));
     }
-  }
+  };
+  if (score_wave && active) load_q();
+  MLAKV_STAMP(32);
 
   // Stage this chunk's block-table entries in LDS. The range is bounded by the chunk and the
   // table row, not by the sequence length, so it does not wait for the length to arrive;
@@ -478,11 +494,13 @@ __global__ __launch_bounds__(kThreads) void MlaDecodeKernel(AttnArgs a) {
       table_lds[i] = static_cast<unsigned>(entry) < static_cast<unsigned>(a.num_blocks) ? entry : -1;
     }
   }
+  MLAKV_STAMP(34);
   // A length beyond what the table row can address is clamped: every position below it has a
   // staged entry.
   const int seq_len = static_cast<int>(
       min(static_cast<int64_t>(Uniform(a.seq_lens[seq])), static_cast<int64_t>(a.table_stride) * a.block_size));
   map.seq_len = seq_len;
+  MLAKV_STAMP(33);
   const int num_tiles = (seq_len + kTileTokens - 1) / kTileTokens;
   if (tile_begin >= num_tiles) {
     if (active && direct) {  // empty sequence: zeros, lse = -inf
@@ -536,6 +554,7 @@ __global__ __launch_bounds__(kThreads) void MlaDecodeKernel(AttnArgs a) {
 
   // The query must have arrived before the tile loads are issued: the compiler's own wait for
   // it would otherwise also wait for every tile load issued in between.
+  MLAKV_STAMP(35);
   if (score_wave && active) {
 #pragma unroll
     for (int ks = 0; ks < kKSteps; ++ks) asm volatile("" ::"v"(q[ks]));
@@ -559,10 +578,10 @@ __global__ __launch_bounds__(kThreads) void MlaDecodeKernel(AttnArgs a) {
   // flight); the barrier publishes it together with P(i) and retires every wave's reads of
   // tile i-1, whose ring slot the next tile to be issued reuses.
   const auto publish = [&](int i) __attribute__((always_inline)) {
-    MLAKV_STAMP(4 + 6 * i);
+    MLAKV_STAMP((i) < 4 ? 4 + 6 * (i) : -1);
     if (i + 1 < ntiles) WaitLoads(last_unknown >= i + 1 ? 0 : (issued - (i + 2)) * per_tile);
     __syncthreads();
-    MLAKV_STAMP(5 + 6 * i);
+    MLAKV_STAMP((i) < 4 ? 5 + 6 * (i) : -1);
   };
   // Issues the next tile of the ring (tile i + kRing - 1 during iteration i), right after
   // publish(i): the memory-bound shapes want every load in flight as early as possible (issuing
@@ -573,7 +592,7 @@ __global__ __launch_bounds__(kThreads) void MlaDecodeKernel(AttnArgs a) {
       if (!issue(issued)) last_unknown = issued;
       ++issued;
     }
-    MLAKV_STAMP(6 + 6 * i);
+    MLAKV_STAMP((i) < 4 ? 6 + 6 * (i) : -1);
   };
 
   unsigned char* p_lds = lds + G::kPOff + (hw * 64 + lane) * 16;           // + parity * kScoreWaves * 64 * 16
@@ -652,7 +671,7 @@ __global__ __launch_bounds__(kThreads) void MlaDecodeKernel(AttnArgs a) {
           __builtin_amdgcn_sched_barrier(0);
         });
       }
-      MLAKV_STAMP(7 + 6 * (tile_rel - 1));
+      MLAKV_STAMP(tile_rel >= 1 && tile_rel <= 4 ? 7 + 6 * (tile_rel - 1) : -1);
       // lane holds tokens 4g+j (x[0..3]) and 16+4g+j (x[4..7]) of head i16
       float x[8];
 #pragma unroll
@@ -694,7 +713,7 @@ __global__ __launch_bounds__(kThreads) void MlaDecodeKernel(AttnArgs a) {
       }
       l_run += sum;
       *reinterpret_cast<bf16x8*>(p_lds + parity * kScoreWaves * 64 * 16) = p;
-      MLAKV_STAMP(8 + 6 * (tile_rel - 1));
+      MLAKV_STAMP(tile_rel >= 1 && tile_rel <= 4 ? 8 + 6 * (tile_rel - 1) : -1);
     };
 
     if (active) score_tile(0);
@@ -778,7 +797,7 @@ __global__ __launch_bounds__(kThreads) void MlaDecodeKernel(AttnArgs a) {
           if constexpr (n + kVAhead < kDvTiles) vf[n % kVAhead] = v_fetch(buf, n + kVAhead);
           __builtin_amdgcn_sched_barrier(0);
         });
-        MLAKV_STAMP(7 + 6 * i);
+        MLAKV_STAMP((i) < 4 ? 7 + 6 * (i) : -1);
       }
     }
     MLAKV_STAMP(29);
@@ -824,12 +843,29 @@ __global__ __launch_bounds__(kThreads) void MlaDecodeKernel(AttnArgs a) {
               u32x4{scale_codes[0], scale_codes[1], scale_codes[2], scale_codes[3]};
         }
       } else {
+        // The accumulators hold O^T (lane = head i16, four columns per 16-column tile), which
+        // stored as it is would write 32-byte pieces of sixteen different rows per instruction.
+        // The tile ring is dead after the last barrier: each output wave transposes its sixteen
+        // rows through its own part of it and writes whole 1-KB rows, 16 bytes per lane. A row
+        // stride of 1040 bytes (= 4 banks mod 64) spreads the 8-byte writes of a half-wave over
+        // all banks.
+        constexpr int kStageRow = kLatentDim * 2 + 16;
+        static_assert((kWaves - kScoreWaves) * 16 * kStageRow <= G::kRing * G::kTileBytes, "the staging rows fit in the ring");
+        unsigned char* stage = lds + G::Slot(0) + hw * (16 * kStageRow);
 #pragma unroll
         for (int n = 0; n < kDvTiles; ++n) {
           u32x2 packed;
           packed.x = PackBf16(o[n][0] * inv, o[n][1] * inv);
           packed.y = PackBf16(o[n][2] * inv, o[n][3] * inv);
-          __builtin_nontemporal_store(packed, reinterpret_cast<u32x2*>(out_row + (16 * n + 4 * g) * 2));
+          *reinterpret_cast<u32x2*>(stage + i16 * kStageRow + (16 * n + 4 * g) * 2) = packed;
+        }
+        // Same wave wrote and reads: the LDS queue is in order, no barrier needed.
+        const int64_t row_stride = direct ? a.out_head_stride : kLatentDim * 2;
+        char* first_row = out_row - i16 * row_stride;  // row of this wave's head 0
+#pragma unroll
+        for (int r = 0; r < 16; ++r) {
+          const u32x4 v = *reinterpret_cast<const u32x4*>(stage + r * kStageRow + lane * 16);
+          __builtin_nontemporal_store(v, reinterpret_cast<u32x4*>(first_row + r * row_stride + lane * 16));
         }
       }
     }
