@@ -102,6 +102,11 @@ struct AttnArgs {
   int64_t out_codes_seq_stride, out_codes_head_stride;
   char* out_scales;
   int64_t out_scales_seq_stride, out_scales_head_stride;
+  // Optional selection: int32 [batch][sparse_count] token positions, valid entries first, -1
+  // after them; when set the sequence attends to those tokens only.
+  const int32_t* sparse_indices;
+  int64_t sparse_seq_stride;  // elements
+  int32_t sparse_count;
   char* partial_out;     // workspace: [batch][max_chunks][heads][512] bf16
   float* partial_lse;    // workspace: [batch][max_chunks][heads] fp32, log2 domain
   float scale_log2;      // softmax scale * log2(e)

@@ -237,6 +237,11 @@ template <bool ALIGNED>
 struct TileMap {
   const int* entries;  // LDS
   int first_block, block_size, seq_len;
+  // Selected-token mode (never ALIGNED): `entries` holds, for each of the chunk's selected tokens
+  // from position `first_pos` of the selection on, the linear pool slot of that token (-1: behind
+  // a bad table entry), and `seq_len` is the number of selected tokens.
+  bool sparse;
+  int first_pos;
   int tile_block, tile_slot0;  // ALIGNED only: where the tile of the last Begin() sits
   int next_entry, next_slot0;  // ALIGNED only: cursor of the next tile (tiles are begun in order)
 
@@ -261,6 +266,13 @@ struct TileMap {
       *block = tile_block < 0 ? 0 : tile_block;
       *slot = pos < seq_len ? tile_slot0 + r : 0;
       return pos < seq_len && tile_block >= 0;
+    }
+    if (sparse) {
+      const int linear = pos < seq_len ? entries[pos - first_pos] : -1;
+      const int usable = linear < 0 ? 0 : linear;
+      *block = usable / block_size;
+      *slot = usable - *block * block_size;
+      return linear >= 0;
     }
     const int clamped = pos < seq_len ? pos : seq_len - 1;
     const int logical = clamped / block_size;
@@ -422,8 +434,11 @@ __device__ __forceinline__ bf16x8 CodesToBf16(unsigned lo, unsigned hi) {
 
 // MXQ: the single-chunk launch also quantises its output (and its bf16 output is optional). Kept
 // out of the common instantiation, whose register allocation has no room to spare.
-template <bool FP8, bool ALIGNED, bool MXQ>
+// SPARSE: the sequence attends to the tokens listed in a.sparse_indices instead of to its whole
+// context (never ALIGNED: every row is located on its own).
+template <bool FP8, bool ALIGNED, bool MXQ, bool SPARSE>
 __global__ __launch_bounds__(kThreads) void MlaDecodeKernel(AttnArgs a) {
+  static_assert(!(SPARSE && (ALIGNED || MXQ)), "selected-token attention uses the row-at-a-time path");
   using G = Geom<FP8>;
   extern __shared__ __attribute__((aligned(16))) unsigned char lds[];
   const unsigned lds_base = static_cast<unsigned>(reinterpret_cast<size_t>((__attribute__((address_space(3))) unsigned char*)lds));
@@ -480,7 +495,9 @@ __global__ __launch_bounds__(kThreads) void MlaDecodeKernel(AttnArgs a) {
   TileMap<ALIGNED> map;
   map.entries = table_lds;
   map.block_size = a.block_size;
-  {
+  map.sparse = SPARSE;
+  map.first_pos = tile_begin * kTileTokens;
+  if constexpr (!SPARSE) {
     const int first_pos = tile_begin * kTileTokens;
     const int last_pos = first_pos + a.chunk_tiles * kTileTokens - 1;
     map.first_block = first_pos / a.block_size;
@@ -497,8 +514,33 @@ __global__ __launch_bounds__(kThreads) void MlaDecodeKernel(AttnArgs a) {
   MLAKV_STAMP(34);
   // A length beyond what the table row can address is clamped: every position below it has a
   // staged entry.
-  const int seq_len = static_cast<int>(
+  int seq_len = static_cast<int>(
       min(static_cast<int64_t>(Uniform(a.seq_lens[seq])), static_cast<int64_t>(a.table_stride) * a.block_size));
+  if constexpr (SPARSE) {
+    // The selection ends at its first entry that is negative or not inside the context. Then
+    // this chunk's part of it is resolved to pool slots through the block table.
+    const int context = seq_len;
+    const int32_t* selection = a.sparse_indices + static_cast<int64_t>(seq) * a.sparse_seq_stride;
+    int* count_lds = reinterpret_cast<int*>(lds + G::kFlagOff) + 2 * kScoreWaves;
+    if (tid == 0) *count_lds = a.sparse_count;
+    __syncthreads();
+    for (int i = tid; i < a.sparse_count; i += kThreads) {
+      const int index = selection[i];
+      if (index < 0 || index >= context) atomicMin(count_lds, i);
+    }
+    __syncthreads();
+    seq_len = Uniform(*count_lds);
+    const int32_t* table_row = a.block_table + static_cast<int64_t>(seq) * a.table_stride;
+    const int chunk_tokens = min(a.chunk_tiles * kTileTokens, seq_len - map.first_pos);  // <= kTableEntries, ensured by the plan
+    for (int i = tid; i < chunk_tokens; i += kThreads) {
+      const int index = selection[map.first_pos + i];  // inside [0, context): before the end of the selection
+      const int logical = index / a.block_size;
+      const int entry = table_row[logical];
+      table_lds[i] = static_cast<unsigned>(entry) < static_cast<unsigned>(a.num_blocks)
+                         ? entry * a.block_size + (index - logical * a.block_size)
+                         : -1;
+    }
+  }
   map.seq_len = seq_len;
   MLAKV_STAMP(33);
   const int num_tiles = (seq_len + kTileTokens - 1) / kTileTokens;
@@ -953,21 +995,21 @@ __global__ __launch_bounds__(256) void MlaCombineKernel(AttnArgs a) {
   }
 }
 
-template <bool FP8, bool ALIGNED, bool MXQ>
+template <bool FP8, bool ALIGNED, bool MXQ, bool SPARSE>
 hipError_t Launch(const AttnArgs& args, const dim3& grid, hipStream_t stream) {
   // Dynamic LDS above 64 KB needs the attribute once per kernel and process.
-  static const hipError_t prepared = hipFuncSetAttribute(reinterpret_cast<const void*>(&MlaDecodeKernel<FP8, ALIGNED, MXQ>),
+  static const hipError_t prepared = hipFuncSetAttribute(reinterpret_cast<const void*>(&MlaDecodeKernel<FP8, ALIGNED, MXQ, SPARSE>),
                                                          hipFuncAttributeMaxDynamicSharedMemorySize, Geom<FP8>::kLdsBytes);
   if (prepared != hipSuccess) return prepared;
-  hipLaunchKernelGGL((MlaDecodeKernel<FP8, ALIGNED, MXQ>), grid, dim3(kThreads), Geom<FP8>::kLdsBytes, stream, args);
+  hipLaunchKernelGGL((MlaDecodeKernel<FP8, ALIGNED, MXQ, SPARSE>), grid, dim3(kThreads), Geom<FP8>::kLdsBytes, stream, args);
   return hipGetLastError();
 }
 
 template <bool MXQ>
 hipError_t LaunchByCache(const AttnArgs& args, const dim3& grid, hipStream_t stream) {
   const bool aligned = args.block_size % kTileTokens == 0;
-  if (args.fp8) return aligned ? Launch<true, true, MXQ>(args, grid, stream) : Launch<true, false, MXQ>(args, grid, stream);
-  return aligned ? Launch<false, true, MXQ>(args, grid, stream) : Launch<false, false, MXQ>(args, grid, stream);
+  if (args.fp8) return aligned ? Launch<true, true, MXQ, false>(args, grid, stream) : Launch<true, false, MXQ, false>(args, grid, stream);
+  return aligned ? Launch<false, true, MXQ, false>(args, grid, stream) : Launch<false, false, MXQ, false>(args, grid, stream);
 }
 
 }  // namespace
@@ -983,7 +1025,12 @@ hipError_t LaunchAttnDecode(const AttnArgs& args_in, hipStream_t stream) {
   const dim3 grid(args.max_chunks, args.batch, (args.heads + 63) / 64);
   // With several chunks the merge kernel owns the final output and the optional quantisation.
   const bool quantise_here = args.max_chunks == 1 && args.out_codes != nullptr;
-  hipError_t e = quantise_here ? LaunchByCache<true>(args, grid, stream) : LaunchByCache<false>(args, grid, stream);
+  hipError_t e;
+  if (args.sparse_indices != nullptr) {
+    e = args.fp8 ? Launch<true, false, false, true>(args, grid, stream) : Launch<false, false, false, true>(args, grid, stream);
+  } else {
+    e = quantise_here ? LaunchByCache<true>(args, grid, stream) : LaunchByCache<false>(args, grid, stream);
+  }
   if (e != hipSuccess) return e;
   if (args.max_chunks > 1) {
     hipLaunchKernelGGL(MlaCombineKernel, dim3((args.heads + kCombineHeads - 1) / kCombineHeads, args.batch), dim3(256), 0,

@@ -86,6 +86,9 @@ PROTOTYPES = {
                                C.c_double, _vp, _i64, _i64, _vp, _vp, _u64, _vp]),
     "mlakvAttnDecodeMxQuant": (_i32, [_P(AttnPlan), _P(CacheView), _i32, _vp, _i64, _i64, _vp, _i64, _i64, _vp, _i32, _vp,
                                       C.c_double, _vp, _i64, _i64, _P(MxQuantOut), _vp, _vp, _u64, _vp]),
+    "mlakvAttnSparsePlanInit": (_i32, [_i32, _i32, _i32, _i32, _i32, _P(AttnPlan)]),
+    "mlakvAttnDecodeSparse": (_i32, [_P(AttnPlan), _P(CacheView), _i32, _vp, _i64, _i64, _vp, _i64, _i64, _vp, _i32, _vp, _vp, _i64,
+                                     C.c_double, _vp, _i64, _i64, _vp, _vp, _u64, _vp]),
     "mlakvDynamicMxQuant": (_i32, [_vp, _i64, _i64, _i32, _vp, _i64, _vp, _i64, _vp]),
     "mlakvArenaCreate": (_i32, [_i32, _P(_vp)]),
     "mlakvArenaDestroy": (None, [_vp]),

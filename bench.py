@@ -158,7 +158,7 @@ def bench_append_gather(args, torch, np, ffi):
 
 
 def bench_attention(args, torch, np, ffi, fp8=False, batch=32, ctx=2048, heads=64, slices=8, iters=None, label=None,
-                    mx_quant=False):
+                    mx_quant=False, sparse_k=None):
     lib = ffi.load()
     bs = 64
     slices = int(os.environ.get("MLAKV_BENCH_SLICES", slices))  # development aid: 1 keeps the KV cache-resident
@@ -168,7 +168,10 @@ def bench_attention(args, torch, np, ffi, fp8=False, batch=32, ctx=2048, heads=6
     cache = ffi.KvCache(arena, num_layers=slices, block_size=bs, max_context_len=ctx, max_batch=batch,
                         pool_blocks=pool_blocks, seed=7, shuffle=1, dtype=ffi.DTYPE_FP8_E4M3 if fp8 else ffi.DTYPE_BF16)
     plan = ffi.AttnPlan()
-    ffi.check(lib.mlakvAttnPlanInit(batch, heads, ctx, bs, cache.config.dtype, C.byref(plan)))
+    if sparse_k:
+        ffi.check(lib.mlakvAttnSparsePlanInit(batch, heads, sparse_k, bs, cache.config.dtype, C.byref(plan)))
+    else:
+        ffi.check(lib.mlakvAttnPlanInit(batch, heads, ctx, bs, cache.config.dtype, C.byref(plan)))
     arena.note_workspace(int(plan.workspace_bytes))
     arena.commit()
     arena.commit_workspace()
@@ -192,7 +195,26 @@ def bench_attention(args, torch, np, ffi, fp8=False, batch=32, ctx=2048, heads=6
     q = torch.randn(slices, batch, heads, ROW, generator=gen, device="cuda").to(torch.bfloat16)
     out = torch.empty(slices, batch, heads, LATENT, dtype=torch.bfloat16, device="cuda")
 
+    selection = None
+    if sparse_k:
+        # every sequence attends to sparse_k distinct random positions of its context (what a
+        # top-k selection looks like to the memory system), a fresh draw per layer slice
+        rng = np.random.default_rng(5)
+        selection = torch.as_tensor(np.stack([np.stack([rng.permutation(ctx)[:sparse_k] for _ in range(batch)])
+                                              for _ in range(slices)]).astype(np.int32), device="cuda")
+
+    def launch_sparse(i):
+        k = i % slices
+        ffi.check(lib.mlakvAttnDecodeSparse(C.byref(plan), C.byref(view), k, q[k].data_ptr(), heads * ROW_BYTES, ROW_BYTES,
+                                            q[k].data_ptr() + LATENT * 2, heads * ROW_BYTES, ROW_BYTES,
+                                            cache.device_block_table, cache.num_blocks, cache.device_seq_lens,
+                                            selection[k].data_ptr(), sparse_k, 1.0 / math.sqrt(192.0), out[k].data_ptr(),
+                                            heads * LATENT * 2, LATENT * 2, None, arena.workspace, arena.workspace_bytes,
+                                            stream_ptr(torch)))
+
     def launch(i):
+        if sparse_k:
+            return launch_sparse(i)
         k = i % slices
         ffi.check(lib.mlakvAttnDecode(C.byref(plan), C.byref(view), k, q[k].data_ptr(), heads * ROW_BYTES, ROW_BYTES,
                                       q[k].data_ptr() + LATENT * 2, heads * ROW_BYTES, ROW_BYTES,
@@ -240,12 +262,16 @@ def bench_attention(args, torch, np, ffi, fp8=False, batch=32, ctx=2048, heads=6
 
         mx = {"us_fused_epilogue": timed_us(fused), "us_attention_then_quant": timed_us(unfused)}
     kv_row = 580 if fp8 else ROW_BYTES
-    algorithmic = batch * ctx * kv_row + batch * heads * ROW * 2 + batch * heads * LATENT * 2 + 4 * batch * blocks_per_seq
-    flops = 2.0 * batch * heads * ctx * (ROW + LATENT)
+    attended = sparse_k or ctx
+    algorithmic = batch * attended * kv_row + batch * heads * ROW * 2 + batch * heads * LATENT * 2 + 4 * batch * blocks_per_seq
+    if sparse_k:
+        algorithmic += 4 * batch * sparse_k
+    flops = 2.0 * batch * heads * attended * (ROW + LATENT)
     result = {
         "us_per_step": us,
         "workload": f"{label or ('configs[3]-shape' if fp8 else 'configs[2]-shape')}: 1 layer per launch, batch {batch}, {heads} heads, ctx {ctx}, block 64, "
-                    f"{'fp8 e4m3 + fp32 row scale' if fp8 else 'bf16'} KV, shuffled table, {slices} rotating layer slices",
+                    f"{'fp8 e4m3 + fp32 row scale' if fp8 else 'bf16'} KV, shuffled table, {slices} rotating layer slices"
+                    + (f", {sparse_k} selected tokens per sequence" if sparse_k else ""),
         "roofline": {"bound": "hbm", "achieved": algorithmic / (us * 1e-6) / 1e9, "peak": HBM_PEAK_GBPS, "unit": "GB/s",
                      "frac": algorithmic / (us * 1e-6) / 1e9 / HBM_PEAK_GBPS, "traffic": None},
         "algorithmic_bytes": algorithmic,
@@ -460,7 +486,9 @@ def main():
         print(json.dumps({"attention": bench_attention(args, torch, np, ffi, mx_quant=True),
                           "attention_fp8": bench_attention(args, torch, np, ffi, fp8=True, batch=64, ctx=4352, iters=64),
                           "attention_long": bench_attention(args, torch, np, ffi, batch=128, ctx=8192, slices=2, iters=16,
-                                                            label="configs[4]-scale decode shape (one workgroup per sequence)")}))
+                                                            label="configs[4]-scale decode shape (one workgroup per sequence)"),
+                          "attention_sparse": bench_attention(args, torch, np, ffi, batch=32, ctx=8192, slices=4, sparse_k=512,
+                                                              label="selected-token decode (index_topk 512 of 8192)")}))
         return 0
     ag = bench_append_gather(args, torch, np, ffi)
     line = {
@@ -487,6 +515,8 @@ def main():
         line["attention_fp8"] = bench_attention(args, torch, np, ffi, fp8=True, batch=64, ctx=4352, iters=64)
         line["attention_long"] = bench_attention(args, torch, np, ffi, batch=128, ctx=8192, slices=2, iters=16,
                                                  label="configs[4]-scale decode shape (one workgroup per sequence)")
+        line["attention_sparse"] = bench_attention(args, torch, np, ffi, batch=32, ctx=8192, slices=4, sparse_k=512,
+                                                   label="selected-token decode (index_topk 512 of 8192)")
         line["side_kernels"] = bench_side_kernels(args, torch, np, ffi)
     if not args.no_cpu_baseline:
         line["cpu_baseline"] = cpu_baseline(np, ag)

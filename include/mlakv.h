@@ -143,7 +143,7 @@ typedef struct mlakvAttnPlan {
   int32_t dtype;           /* cache dtype */
   int32_t chunk_tiles;     /* 32-token tiles per workgroup; chosen by the plan */
   int32_t max_chunks;      /* ceil(ceil(max_seq_len / 32) / chunk_tiles) */
-  int32_t reserved;
+  int32_t reserved;        /* 1: made by mlakvAttnSparsePlanInit (max_seq_len holds sparse_count) */
   uint64_t workspace_bytes;
 } mlakvAttnPlan;
 
@@ -194,6 +194,31 @@ mlakvStatus mlakvAttnDecodeMxQuant(const mlakvAttnPlan* plan, const mlakvCacheVi
                                    const int32_t* block_table, int32_t table_stride, const int32_t* seq_lens, double scale,
                                    void* out, int64_t out_seq_stride, int64_t out_head_stride, const mlakvMxQuantOut* quant,
                                    float* lse, void* workspace, uint64_t workspace_bytes, void* stream);
+
+/* Selected-token decode attention: the consumer of the Lightning Indexer's output, i.e. the same
+ * attention over the k best tokens of each sequence instead of its whole context (the model's
+ * long-context mechanism: index_topk = kIndexTopK = 512, include/moe/core/config.hpp:49-51;
+ * selection contract aclnnQuantLightningIndexer, include/moe/core/op_table.hpp:964-1006: INT32
+ * indices [B, S1, N2, k], sparse_count in [1, 2048]; the vendored kernel writes the valid indices
+ * first and fills the rest with -1, third_party/ops_transformer/attention/quant_lightning_indexer/
+ * op_kernel/arch35/quant_lightning_indexer_service_vector.h:446-541). The reference's pipeline does
+ * not launch a sparse attention yet (src/pipeline/pipeline.cpp:576-578 reports it as not
+ * applied), so this entry has no stage to replace; it reads the same paged pool through the same
+ * block table.
+ *   sparse_indices: device int32 [batch][sparse_count] at `sparse_indices_seq_stride` elements per
+ *   sequence; sequence b attends to the cached rows at positions sparse_indices[b][0 .. n-1], where
+ *   n is the number of entries before the first one that is negative or >= seq_lens[b]
+ *   (n = 0: zeros, lse = -inf). Order does not matter; repeated positions count repeatedly.
+ * The plan comes from mlakvAttnSparsePlanInit (sparse_count takes the place of max_seq_len). */
+mlakvStatus mlakvAttnSparsePlanInit(int32_t batch, int32_t heads, int32_t sparse_count, int32_t block_size, int32_t dtype,
+                                    mlakvAttnPlan* plan);
+mlakvStatus mlakvAttnDecodeSparse(const mlakvAttnPlan* plan, const mlakvCacheView* cache, int32_t layer,
+                                  const void* q_latent, int64_t q_latent_seq_stride, int64_t q_latent_head_stride,
+                                  const void* q_rope, int64_t q_rope_seq_stride, int64_t q_rope_head_stride,
+                                  const int32_t* block_table, int32_t table_stride, const int32_t* seq_lens,
+                                  const int32_t* sparse_indices, int64_t sparse_indices_seq_stride, double scale,
+                                  void* out, int64_t out_seq_stride, int64_t out_head_stride, float* lse, void* workspace,
+                                  uint64_t workspace_bytes, void* stream);
 
 /* ------------------------------------------------------------------------- */
 /* Static arena (host)                                                        */

@@ -525,14 +525,24 @@ static void load_row_f32(const kvo_cache_view_t* cache, int64_t slot, float* lat
   }
 }
 
-void kvo_mla_decode(const uint16_t* q_latent, int64_t q_latent_seq_stride, int64_t q_latent_head_stride,
-                    const uint16_t* q_rope, int64_t q_rope_seq_stride, int64_t q_rope_head_stride,
-                    const kvo_cache_view_t* cache, const int32_t* table, int64_t table_stride,
-                    const int32_t* seq_lens, int64_t batch, int64_t heads, double scale, float* out, float* lse,
-                    int accum_f32) {
+/* Dense (sparse_indices == NULL: positions 0 .. seq_lens[b]-1) or selected-token attention
+ * (positions sparse_indices[b][0 .. n-1], n = the number of entries before the first one that is
+ * negative or not below seq_lens[b], at most sparse_count). */
+static void mla_decode_rows(const uint16_t* q_latent, int64_t q_latent_seq_stride, int64_t q_latent_head_stride,
+                            const uint16_t* q_rope, int64_t q_rope_seq_stride, int64_t q_rope_head_stride,
+                            const kvo_cache_view_t* cache, const int32_t* table, int64_t table_stride,
+                            const int32_t* seq_lens, const int32_t* sparse_indices, int64_t sparse_count,
+                            int64_t sparse_stride, int64_t batch, int64_t heads, double scale, float* out, float* lse,
+                            int accum_f32) {
   const int64_t dl = cache->latent_dim, dr = cache->rope_dim;
   for (int64_t b = 0; b < batch; ++b) {
-    const int64_t n = seq_lens[b];
+    int64_t n = seq_lens[b];
+    const int32_t* selected = sparse_indices ? sparse_indices + b * sparse_stride : NULL;
+    if (selected) {
+      int64_t count = 0;
+      while (count < sparse_count && selected[count] >= 0 && selected[count] < seq_lens[b]) ++count;
+      n = count;
+    }
     float* out_b = out + b * heads * dl;
     if (n <= 0) {
       memset(out_b, 0, (size_t)(heads * dl) * sizeof(float));
@@ -544,7 +554,10 @@ void kvo_mla_decode(const uint16_t* q_latent, int64_t q_latent_seq_stride, int64
     float* rope = (float*)malloc((size_t)(n * dr) * sizeof(float));
     double* scores = (double*)malloc((size_t)n * sizeof(double));
     const int32_t* row_table = table + b * table_stride;
-    for (int64_t i = 0; i < n; ++i) load_row_f32(cache, kvo_slot(row_table, i, cache->block_size), latent + i * dl, rope + i * dr);
+    for (int64_t i = 0; i < n; ++i) {
+      const int64_t position = selected ? selected[i] : i;
+      load_row_f32(cache, kvo_slot(row_table, position, cache->block_size), latent + i * dl, rope + i * dr);
+    }
     for (int64_t h = 0; h < heads; ++h) {
       const uint16_t* ql = q_latent + b * q_latent_seq_stride + h * q_latent_head_stride;
       const uint16_t* qr = q_rope + b * q_rope_seq_stride + h * q_rope_head_stride;
@@ -590,6 +603,24 @@ void kvo_mla_decode(const uint16_t* q_latent, int64_t q_latent_seq_stride, int64
     free(rope);
     free(scores);
   }
+}
+
+void kvo_mla_decode(const uint16_t* q_latent, int64_t q_latent_seq_stride, int64_t q_latent_head_stride,
+                    const uint16_t* q_rope, int64_t q_rope_seq_stride, int64_t q_rope_head_stride,
+                    const kvo_cache_view_t* cache, const int32_t* table, int64_t table_stride,
+                    const int32_t* seq_lens, int64_t batch, int64_t heads, double scale, float* out, float* lse,
+                    int accum_f32) {
+  mla_decode_rows(q_latent, q_latent_seq_stride, q_latent_head_stride, q_rope, q_rope_seq_stride, q_rope_head_stride, cache,
+                  table, table_stride, seq_lens, NULL, 0, 0, batch, heads, scale, out, lse, accum_f32);
+}
+
+void kvo_mla_decode_sparse(const uint16_t* q_latent, int64_t q_latent_seq_stride, int64_t q_latent_head_stride,
+                           const uint16_t* q_rope, int64_t q_rope_seq_stride, int64_t q_rope_head_stride,
+                           const kvo_cache_view_t* cache, const int32_t* table, int64_t table_stride,
+                           const int32_t* seq_lens, const int32_t* sparse_indices, int64_t sparse_count,
+                           int64_t sparse_stride, int64_t batch, int64_t heads, double scale, float* out, float* lse) {
+  mla_decode_rows(q_latent, q_latent_seq_stride, q_latent_head_stride, q_rope, q_rope_seq_stride, q_rope_head_stride, cache,
+                  table, table_stride, seq_lens, sparse_indices, sparse_count, sparse_stride, batch, heads, scale, out, lse, 0);
 }
 
 /* ------------------------------------------------------------------------- */

@@ -220,6 +220,23 @@ void kvo_mla_decode(const uint16_t* q_latent, int64_t q_latent_seq_stride, int64
                     const int32_t* seq_lens, int64_t batch, int64_t heads, double scale, float* out, float* lse,
                     int accum_f32);
 
+/* The same attention over selected tokens only: the consumer of the Lightning Indexer's output
+ * (reference include/moe/core/op_table.hpp:964-1006: INT32 indices [B, S1, N2, k] of the k best
+ * tokens, k = kIndexTopK = 512, include/moe/core/config.hpp:49; the vendored kernel writes the
+ * valid indices first and fills the rest with -1,
+ * third_party/ops_transformer/attention/quant_lightning_indexer/op_kernel/arch35/
+ * quant_lightning_indexer_service_vector.h:446-541). Sequence b attends to the cached rows at
+ * positions sparse_indices[b][0 .. n-1], n = number of entries before the first that is negative
+ * or >= seq_lens[b]; softmax and output as in kvo_mla_decode (double accumulation). The
+ * reference's pipeline does not launch a sparse attention yet (src/pipeline/pipeline.cpp:576-578
+ * says so); pinned by reduction to the dense routine: indices 0..n-1 give the dense result bit
+ * for bit, and any selection equals the dense routine on a cache holding just those rows. */
+void kvo_mla_decode_sparse(const uint16_t* q_latent, int64_t q_latent_seq_stride, int64_t q_latent_head_stride,
+                           const uint16_t* q_rope, int64_t q_rope_seq_stride, int64_t q_rope_head_stride,
+                           const kvo_cache_view_t* cache, const int32_t* table, int64_t table_stride,
+                           const int32_t* seq_lens, const int32_t* sparse_indices, int64_t sparse_count,
+                           int64_t sparse_stride, int64_t batch, int64_t heads, double scale, float* out, float* lse);
+
 /* ---- block pool: free list, block tables, recycling, compaction ---------- */
 /* No reference counterpart (the reference is one sequence with identity paging and
  * never writes its block table, src/memory/static_arena_manager.cpp:298). Semantics:

@@ -78,6 +78,8 @@ _PROTOTYPES = {
     "kvo_mx_quant_rows": (None, [_vp, _i64, _i64, _i64, _vp, _i64, _vp, _i64]),
     "kvo_mla_decode": (None, [_vp, _i64, _i64, _vp, _i64, _i64, _P(CacheView), _vp, _i64, _vp, _i64, _i64, C.c_double,
                               _vp, _vp, C.c_int]),
+    "kvo_mla_decode_sparse": (None, [_vp, _i64, _i64, _vp, _i64, _i64, _P(CacheView), _vp, _i64, _vp, _vp, _i64, _i64, _i64, _i64,
+                                     C.c_double, _vp, _vp]),
     "kvo_splitmix64": (_u64, [_P(_u64)]),
     "kvo_pool_new": (_vp, [_i64, _i64, _i64, _i64, _u64, C.c_int]),
     "kvo_pool_delete": (None, [_vp]),
@@ -274,7 +276,7 @@ def gather_rows_fp8(latent_plane, rope_plane, scale_plane, block_size, table, se
 
 
 def mla_decode(q_latent, q_rope, latent_plane, rope_plane, block_size, table, seq_lens, scale, scale_plane=None,
-               accum_f32=False, latent_row_stride=None, rope_row_stride=None):
+               accum_f32=False, latent_row_stride=None, rope_row_stride=None, sparse_indices=None):
     """q_latent [B,H,512], q_rope [B,H,64]: uint16 bf16 bits, contiguous. Planes for ONE layer:
     bf16 -> uint16 arrays, fp8 -> uint8 arrays with scale_plane float32 [blocks*bs].
     Returns (out float32 [B,H,512], lse float32 [B,H])."""
@@ -296,6 +298,15 @@ def mla_decode(q_latent, q_rope, latent_plane, rope_plane, block_size, table, se
     batch, heads = q_latent.shape[0], q_latent.shape[1]
     out = np.zeros((batch, heads, latent_dim), dtype=np.float32)
     lse = np.zeros((batch, heads), dtype=np.float32)
+    if sparse_indices is not None:
+        # int32 [B, k]: the positions each sequence attends to, valid entries first, -1 after them
+        sparse_indices = np.ascontiguousarray(sparse_indices, dtype=np.int32)
+        assert sparse_indices.shape[0] == batch and not accum_f32
+        lib.kvo_mla_decode_sparse(_ptr(q_latent), heads * latent_dim, latent_dim, _ptr(q_rope), heads * rope_dim, rope_dim,
+                                  C.byref(view), _ptr(table), table.shape[1], _ptr(seq_lens), _ptr(sparse_indices),
+                                  sparse_indices.shape[1], sparse_indices.shape[1], batch, heads, float(scale), _ptr(out),
+                                  _ptr(lse))
+        return out, lse
     lib.kvo_mla_decode(_ptr(q_latent), heads * latent_dim, latent_dim, _ptr(q_rope), heads * rope_dim, rope_dim,
                        C.byref(view), _ptr(table), table.shape[1], _ptr(seq_lens), batch, heads, float(scale), _ptr(out),
                        _ptr(lse), int(accum_f32))

@@ -151,12 +151,33 @@ def attention(cache, layer, q, table, seq_lens, scale, max_seq_len=None, want_ls
     return out, lse, plan, codes, scales
 
 
-def oracle_attention(cache, layer, q, table_np, lens_np, scale, accum_f32=False):
+def sparse_attention(cache, layer, q, table, seq_lens, selection, scale, want_lse=True):
+    """Selected-token attention: `selection` int32 cuda [B, k]. Returns (out, lse, plan)."""
+    lib = ffi.load()
+    batch, heads = q.shape[0], q.shape[1]
+    plan = ffi.AttnPlan()
+    ffi.check(lib.mlakvAttnSparsePlanInit(batch, heads, selection.shape[1], cache.block_size,
+                                          ffi.DTYPE_FP8_E4M3 if cache.fp8 else ffi.DTYPE_BF16, C.byref(plan)))
+    workspace = torch.empty(max(int(plan.workspace_bytes), 16), dtype=torch.uint8, device="cuda")
+    out = torch.full((batch, heads, LATENT), float("nan"), dtype=torch.bfloat16, device="cuda")
+    lse = torch.full((batch, heads), float("nan"), dtype=torch.float32, device="cuda") if want_lse else None
+    row = (LATENT + ROPE) * 2
+    ffi.check(lib.mlakvAttnDecodeSparse(C.byref(plan), C.byref(cache.view), layer, q.data_ptr(), heads * row, row,
+                                        q.data_ptr() + LATENT * 2, heads * row, row, table.data_ptr(), table.shape[1],
+                                        seq_lens.data_ptr(), selection.data_ptr(), selection.stride(0), float(scale),
+                                        out.data_ptr(), heads * LATENT * 2, LATENT * 2, lse.data_ptr() if want_lse else None,
+                                        workspace.data_ptr(), int(plan.workspace_bytes), stream_ptr()))
+    torch.cuda.synchronize()
+    return out, lse, plan
+
+
+def oracle_attention(cache, layer, q, table_np, lens_np, scale, accum_f32=False, sparse_indices=None):
     qb = bits16(q)
     q_lat = np.ascontiguousarray(qb[..., :LATENT])
     q_rope = np.ascontiguousarray(qb[..., LATENT:])
     return orc.mla_decode(q_lat, q_rope, cache.latent_np(layer), cache.rope_np(layer), cache.block_size, table_np,
-                          lens_np, scale, scale_plane=cache.scale_np(layer) if cache.fp8 else None, accum_f32=accum_f32)
+                          lens_np, scale, scale_plane=cache.scale_np(layer) if cache.fp8 else None, accum_f32=accum_f32,
+                          sparse_indices=sparse_indices)
 
 
 def build_tables(ctxs, block_size, pool_blocks, seed, shuffle=True, max_blocks=None):

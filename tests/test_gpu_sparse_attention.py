@@ -1,0 +1,139 @@
+"""GPU parity: selected-token decode attention (mlakvAttnDecodeSparse) through the C ABI against
+the CPU oracle (2e-2 of the peak for bf16 KV, 6e-2 for FP8 KV, as for the dense attention), and
+through what the definition fixes: selecting every token reproduces the dense entry point,
+permuting the selection changes nothing beyond rounding, the selection ends at its first invalid
+entry, an empty selection gives zeros."""
+import ctypes as C
+import math
+
+import numpy as np
+import pytest
+import torch
+
+import kv_testing as kt
+import mlakv_ffi as ffi
+
+pytestmark = pytest.mark.gpu
+
+LATENT, ROPE = kt.LATENT, kt.ROPE
+SCALE = 1.0 / math.sqrt(192.0)
+
+
+def _setup(ctxs, bs, fp8, seed):
+    blocks = sum(-(-c // bs) for c in ctxs) + 3
+    pool = kt.build_tables(ctxs, bs, blocks, seed=seed)
+    table = pool.table()
+    cache = kt.PagedCache(1, blocks, bs, fp8=fp8)
+    total = sum(ctxs)
+    latent = kt.randn_bf16((1, total, LATENT), seed=seed + 1, outlier_fraction=0.01).cuda()
+    rope = kt.randn_bf16((1, total, ROPE), seed=seed + 2).cuda()
+    kt.append(cache, latent, rope, kt.dev_i32(kt.slots_for(table, ctxs, bs)))
+    torch.cuda.synchronize()
+    return cache, table
+
+
+def _close(got_bf16, expected, tol):
+    got = got_bf16.float().cpu().numpy()
+    assert np.isfinite(got).all()
+    peak = max(np.abs(expected).max(), 1e-30)
+    assert np.abs(got - expected).max() <= tol * peak, np.abs(got - expected).max() / peak
+
+
+@pytest.mark.parametrize("fp8", [False, True])
+@pytest.mark.parametrize("bs,k", [(64, 512), (16, 100), (128, 2048)])
+def test_selected_tokens_match_oracle(fp8, bs, k, monkeypatch):
+    heads = 64
+    ctxs = [3000, 700, 1, 0, 2049, 130]
+    cache, table = _setup(ctxs, bs, fp8, seed=80)
+    rng = np.random.default_rng(81)
+    selection = np.full((len(ctxs), k), -1, dtype=np.int32)
+    for s, n in enumerate(ctxs):
+        take = min(n, k)
+        if s == 1:
+            take = min(n, k) // 2          # fewer than k although the context is long enough
+        selection[s, :take] = rng.permutation(n)[:take]
+    q = kt.randn_bf16((len(ctxs), heads, LATENT + ROPE), seed=82).cuda()
+    expected, expected_lse = kt.oracle_attention(cache, 0, q, table, ctxs, SCALE, sparse_indices=selection)
+    table_d, lens_d, sel_d = kt.dev_i32(table), kt.dev_i32(ctxs), kt.dev_i32(selection)
+    for chunk_tiles in (None, 1, 100):
+        if chunk_tiles is None:
+            monkeypatch.delenv("MLAKV_ATTN_CHUNK_TILES", raising=False)
+        else:
+            monkeypatch.setenv("MLAKV_ATTN_CHUNK_TILES", str(chunk_tiles))
+        out, lse, plan = kt.sparse_attention(cache, 0, q, table_d, lens_d, sel_d, SCALE)
+        assert plan.chunk_tiles * 32 <= 1024
+        _close(out, expected, 6e-2 if fp8 else 2e-2)
+        live = np.array([min(n, k) > 0 for n in ctxs])
+        assert np.abs(lse.cpu().numpy()[live] - expected_lse[live]).max() <= (6e-2 if fp8 else 2e-2)
+        assert not out[3].any() and torch.isneginf(lse[3]).all()
+
+
+def test_full_selection_equals_dense_and_order_does_not_matter():
+    bs, heads, k = 64, 64, 512
+    ctxs = [512, 300, 77]
+    cache, table = _setup(ctxs, bs, False, seed=90)
+    q = kt.randn_bf16((len(ctxs), heads, LATENT + ROPE), seed=91).cuda()
+    table_d, lens_d = kt.dev_i32(table), kt.dev_i32(ctxs)
+    dense, dense_lse, _ = kt.attention(cache, 0, q, table_d, lens_d, SCALE)
+    identity = np.full((len(ctxs), k), -1, dtype=np.int32)
+    shuffled = identity.copy()
+    rng = np.random.default_rng(92)
+    for s, n in enumerate(ctxs):
+        identity[s, :n] = np.arange(n)
+        shuffled[s, :n] = rng.permutation(n)
+    out, lse, _ = kt.sparse_attention(cache, 0, q, table_d, lens_d, kt.dev_i32(identity), SCALE)
+    peak = dense.float().abs().max().item()
+    # same tokens in the same tiles: only the chunking may differ
+    assert (out.float() - dense.float()).abs().max().item() <= 2 ** -7 * peak
+    assert (lse - dense_lse).abs().max().item() <= 1e-3
+    out2, lse2, _ = kt.sparse_attention(cache, 0, q, table_d, lens_d, kt.dev_i32(shuffled), SCALE)
+    assert (out2.float() - dense.float()).abs().max().item() <= 2e-2 * peak
+    assert (lse2 - dense_lse).abs().max().item() <= 1e-3
+
+
+def test_selection_ends_at_first_invalid_entry_and_argument_checks():
+    bs, heads, k = 64, 16, 64
+    ctxs = [200, 200]
+    cache, table = _setup(ctxs, bs, False, seed=95)
+    q = kt.randn_bf16((2, heads, LATENT + ROPE), seed=96).cuda()
+    table_d, lens_d = kt.dev_i32(table), kt.dev_i32(ctxs)
+    selection = np.full((2, k), -1, dtype=np.int32)
+    selection[0, :10] = np.arange(10) * 7
+    selection[1, :10] = np.arange(10) * 7
+    selection[1, 10] = 200       # not inside the context: ends the list
+    selection[1, 11:20] = 5      # never looked at
+    out, lse, plan = kt.sparse_attention(cache, 0, q, table_d, lens_d, kt.dev_i32(selection), SCALE)
+    q_same = q.clone()
+    q_same[1] = q[0]
+    cache2, table2 = cache, table
+    # both sequences hold different rows, so compare each with the oracle instead of with each other
+    expected, _ = kt.oracle_attention(cache, 0, q, table, ctxs, SCALE, sparse_indices=selection)
+    _close(out, expected, 2e-2)
+    lib = ffi.load()
+    row = (LATENT + ROPE) * 2
+    sel_d = kt.dev_i32(selection)
+    dense_plan = ffi.AttnPlan()
+    ffi.check(lib.mlakvAttnPlanInit(2, heads, 200, bs, ffi.DTYPE_BF16, C.byref(dense_plan)))
+    workspace = torch.zeros(max(int(plan.workspace_bytes), int(dense_plan.workspace_bytes), 16), dtype=torch.uint8, device="cuda")
+    out_t = torch.zeros(2, heads, LATENT, dtype=torch.bfloat16, device="cuda")
+
+    def sparse_call(p, sel=sel_d.data_ptr(), stride=k, out_ptr=out_t.data_ptr()):
+        return lib.mlakvAttnDecodeSparse(C.byref(p), C.byref(cache.view), 0, q.data_ptr(), heads * row, row, q.data_ptr() + LATENT * 2,
+                                         heads * row, row, table_d.data_ptr(), table_d.shape[1], lens_d.data_ptr(), sel, stride,
+                                         SCALE, out_ptr, heads * LATENT * 2, LATENT * 2, None, workspace.data_ptr(),
+                                         workspace.numel(), kt.stream_ptr())
+
+    assert sparse_call(plan) == 0
+    assert sparse_call(dense_plan) == ffi.ERR_PARAM_INVALID            # a whole-context plan
+    assert sparse_call(plan, sel=None) == ffi.ERR_PARAM_NULLPTR
+    assert sparse_call(plan, stride=k - 1) == ffi.ERR_PARAM_INVALID
+    assert sparse_call(plan, out_ptr=None) == ffi.ERR_PARAM_NULLPTR
+    dense_with_sparse_plan = lib.mlakvAttnDecode(C.byref(plan), C.byref(cache.view), 0, q.data_ptr(), heads * row, row,
+                                                 q.data_ptr() + LATENT * 2, heads * row, row, table_d.data_ptr(), table_d.shape[1],
+                                                 lens_d.data_ptr(), SCALE, out_t.data_ptr(), heads * LATENT * 2, LATENT * 2, None,
+                                                 workspace.data_ptr(), workspace.numel(), kt.stream_ptr())
+    assert dense_with_sparse_plan == ffi.ERR_PARAM_INVALID
+    bad = ffi.AttnPlan()
+    assert lib.mlakvAttnSparsePlanInit(2, heads, 0, bs, ffi.DTYPE_BF16, C.byref(bad)) == ffi.ERR_PARAM_INVALID
+    assert lib.mlakvAttnSparsePlanInit(2, heads, 2049, bs, ffi.DTYPE_BF16, C.byref(bad)) == ffi.ERR_PARAM_INVALID
+    torch.cuda.synchronize()

@@ -131,3 +131,46 @@ def test_fp8_cache_matches_torch_on_dequantized_rows():
                             scale_plane=scale_plane)
     ref, _ = _torch_reference(q, deq, SCALE)
     assert np.abs(out - ref).max() <= 1e-5
+
+
+def test_sparse_selection_reduces_to_the_dense_routine_and_to_torch():
+    """The selected-token variant: (a) indices 0..n-1 reproduce the dense result bit for bit;
+    (b) any selection equals torch's float64 softmax over exactly the selected rows, in the order
+    given; (c) the list ends at the first negative entry or entry beyond the sequence; (d) an
+    empty selection gives zeros and lse = -inf; (e) the result does not depend on the order of
+    the selection beyond float64 rounding."""
+    bs, heads = 16, 3
+    ctxs = [40, 7, 65, 33]
+    q, latent, rope, table, rows = _case(5, ctxs, bs, heads=heads, blocks=14)
+    args = (_bits(q[..., :LATENT]), _bits(q[..., LATENT:]), _bits(latent).reshape(-1), _bits(rope).reshape(-1), bs, table, ctxs, SCALE)
+    dense, dense_lse = orc.mla_decode(*args)
+    k = 48
+    identity = np.full((len(ctxs), k), -1, dtype=np.int32)
+    for s, n in enumerate(ctxs):
+        identity[s, :min(n, k)] = np.arange(min(n, k))
+    out, lse = orc.mla_decode(*args, sparse_indices=identity)
+    for s, n in enumerate(ctxs):
+        if n <= k:  # the whole sequence is selected
+            assert np.array_equal(out[s], dense[s]) and np.array_equal(lse[s], dense_lse[s])
+    rng = np.random.default_rng(6)
+    picks = np.full((len(ctxs), k), -1, dtype=np.int32)
+    counts = [25, 0, 48, 10]
+    for s, n in enumerate(ctxs):
+        picks[s, :counts[s]] = rng.permutation(n)[:counts[s]]
+    picks[3, 10] = 33          # == seq_len: ends the list like a negative entry
+    picks[3, 11] = 2           # after the end: ignored
+    out, lse = orc.mla_decode(*args, sparse_indices=picks)
+    for s in range(len(ctxs)):
+        chosen = picks[s, :counts[s]]
+        if counts[s] == 0:
+            assert not out[s].any() and np.isneginf(lse[s]).all()
+            continue
+        l, r = rows[s]
+        sub = [(l[chosen], r[chosen])]
+        want, want_lse = _torch_reference(q[s:s + 1], sub, SCALE)
+        assert np.abs(out[s] - want[0]).max() <= 1e-6 * max(1.0, np.abs(want).max())
+        assert np.abs(lse[s] - want_lse[0]).max() <= 1e-5
+    shuffled = picks.copy()
+    shuffled[0, :25] = picks[0, :25][::-1]
+    out2, lse2 = orc.mla_decode(*args, sparse_indices=shuffled)
+    assert np.abs(out2[0] - out[0]).max() <= 1e-6 and np.abs(lse2[0] - lse[0]).max() <= 1e-6
