@@ -187,8 +187,10 @@ __device__ __forceinline__ void WaitLoads(int newer) {
   case n:                  \
     asm volatile("s_waitcnt vmcnt(" #n ")" ::: "memory"); \
     break;
-    MLAKV_WAIT_CASE(2) MLAKV_WAIT_CASE(3) MLAKV_WAIT_CASE(4) MLAKV_WAIT_CASE(5) MLAKV_WAIT_CASE(6) MLAKV_WAIT_CASE(8)
-    MLAKV_WAIT_CASE(9) MLAKV_WAIT_CASE(10) MLAKV_WAIT_CASE(12) MLAKV_WAIT_CASE(15)
+    MLAKV_WAIT_CASE(1) MLAKV_WAIT_CASE(2) MLAKV_WAIT_CASE(3) MLAKV_WAIT_CASE(4) MLAKV_WAIT_CASE(5) MLAKV_WAIT_CASE(6)
+    MLAKV_WAIT_CASE(7) MLAKV_WAIT_CASE(8) MLAKV_WAIT_CASE(9) MLAKV_WAIT_CASE(10) MLAKV_WAIT_CASE(11) MLAKV_WAIT_CASE(12)
+    MLAKV_WAIT_CASE(13) MLAKV_WAIT_CASE(14) MLAKV_WAIT_CASE(15) MLAKV_WAIT_CASE(16) MLAKV_WAIT_CASE(17) MLAKV_WAIT_CASE(18)
+    MLAKV_WAIT_CASE(19) MLAKV_WAIT_CASE(20) MLAKV_WAIT_CASE(21) MLAKV_WAIT_CASE(22) MLAKV_WAIT_CASE(23) MLAKV_WAIT_CASE(24)
 #undef MLAKV_WAIT_CASE
     default:
       asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
@@ -290,6 +292,7 @@ struct TileMap {
 // the rope rows 8(w-4) .. 8(w-4)+7.
 struct IssueLane {
   int lat[2];      // latent rows w + 8i with i & 1 == j
+  int partner_lat[2];  // the same for the rows of wave w - 4 (output waves only)
   int rope;        // this lane's rope row and chunk, relative to the first rope row of the wave
   int rope_chunk;
 };
@@ -299,7 +302,9 @@ __device__ __forceinline__ int LoadsPerTile(int wave) { return kRowsPerWave + (w
 // Issues this wave's loads of one tile into the buffer at LDS address `buf`; rows that are not
 // real are zero-filled instead. Returns true when the wave issues exactly LoadsPerTile(wave)
 // loads (a full tile), false when the number is not known.
-template <bool ALIGNED>
+// WITH_PARTNER: an output wave also fetches the latent rows of the score wave it is paired with
+// (wave - kScoreWaves), for the tiles that the output waves issue alone.
+template <bool ALIGNED, bool WITH_PARTNER = false>
 __device__ __forceinline__ bool IssueTileBf16(const AttnArgs& a, TileMap<ALIGNED>& map, const IssueLane& il, int tile,
                                               unsigned buf, unsigned char* buf_ptr, int tid) {
   using G = Geom<false>;
@@ -316,6 +321,13 @@ __device__ __forceinline__ bool IssueTileBf16(const AttnArgs& a, TileMap<ALIGNED
     const char* rope = a.rope.base + block * a.rope.block_stride + (slot0 + 8 * rope_group) * a.rope.row_stride;
 #pragma unroll
     for (int i = 0; i < kRowsPerWave; ++i) DirectLoad16(latent + i * pitch, il.lat[i & 1], buf + (wave + kWaves * i) * G::kLatRow);
+    if (WITH_PARTNER) {
+      const char* partner = latent - kScoreWaves * a.latent.row_stride;
+#pragma unroll
+      for (int i = 0; i < kRowsPerWave; ++i) {
+        DirectLoad16(partner + i * pitch, il.partner_lat[i & 1], buf + (wave - kScoreWaves + kWaves * i) * G::kLatRow);
+      }
+    }
     if (rope_wave) DirectLoad16(rope, il.rope, buf + G::kLatRegion + rope_group * 8 * G::kRopeRow);
     return true;
   }
@@ -323,8 +335,9 @@ __device__ __forceinline__ bool IssueTileBf16(const AttnArgs& a, TileMap<ALIGNED
   // time, kept as a loop so that it costs little code.
   bool all_real = true;
 #pragma nounroll
-  for (int i = 0; i < kRowsPerWave; ++i) {
-    const int row = wave + kWaves * i;  // wave-uniform
+  for (int i = 0; i < (WITH_PARTNER ? 2 : 1) * kRowsPerWave; ++i) {
+    // wave-uniform; with a partner the wave walks rows (wave - 4) + 4 i, its partner's and its own in turn
+    const int row = WITH_PARTNER ? wave - kScoreWaves + kScoreWaves * i : wave + kWaves * i;
     int block, slot;
     const bool real = map.Row(tile, row, &block, &slot);
     all_real = all_real && real;
@@ -439,6 +452,10 @@ __device__ __forceinline__ bf16x8 CodesToBf16(unsigned lo, unsigned hi) {
 template <bool FP8, bool ALIGNED, bool MXQ, bool SPARSE>
 __global__ __launch_bounds__(kThreads) void MlaDecodeKernel(AttnArgs a) {
   static_assert(!(SPARSE && (ALIGNED || MXQ)), "selected-token attention uses the row-at-a-time path");
+  // bf16 tiles: the output waves, which have no query to wait for, issue the first tiles of the
+  // ring alone (their own rows and those of their partner score waves) as soon as they know the
+  // block-table entries; the score waves join from the first loop iteration on.
+  constexpr bool kSoloPrologue = !FP8 && !SPARSE;
   using G = Geom<FP8>;
   extern __shared__ __attribute__((aligned(16))) unsigned char lds[];
   const unsigned lds_base = static_cast<unsigned>(reinterpret_cast<size_t>((__attribute__((address_space(3))) unsigned char*)lds));
@@ -471,8 +488,8 @@ __global__ __launch_bounds__(kThreads) void MlaDecodeKernel(AttnArgs a) {
   // Q fragments (score waves): lane (head i16, k-group g) holds, for k-step ks, the eight query
   // elements that meet the lane's K fragment of that step: Q[head][32 ks + 8g .. +7] for bf16
   // tiles; for FP8 tiles one 16-byte K read feeds two k-steps, so the order inside each 64-wide
-  // window is Q[head][64 (ks/2) + 16g + 8 (ks&1) .. +7]. Issued first so that they travel while
-  // the lengths and the block table are fetched.
+  // window is Q[head][64 (ks/2) + 16g + 8 (ks&1) .. +7]. (Loaded further down, once the
+  // lengths and table entries have been asked for.)
   bf16x8 q[kKSteps];
   const auto load_q = [&]() __attribute__((always_inline)) {
     const char* q_latent = a.q_latent + seq * a.q_latent_seq_stride + head * a.q_latent_head_stride;
@@ -484,8 +501,6 @@ __global__ __launch_bounds__(kThreads) void MlaDecodeKernel(AttnArgs a) {
       q[ks] = __builtin_bit_cast(bf16x8, GlobalLoad16(p));
     }
   };
-  if (score_wave && active) load_q();
-  MLAKV_STAMP(32);
 
   // Stage this chunk's block-table entries in LDS. The range is bounded by the chunk and the
   // table row, not by the sequence length, so it does not wait for the length to arrive;
@@ -506,7 +521,9 @@ __global__ __launch_bounds__(kThreads) void MlaDecodeKernel(AttnArgs a) {
     int count = last_pos / a.block_size - map.first_block + 1;  // <= kTableEntries, ensured by the plan
     count = min(count, a.table_stride - map.first_block);
     const int32_t* table_row = a.block_table + static_cast<int64_t>(seq) * a.table_stride + map.first_block;
-    for (int i = tid; i < count; i += kThreads) {
+    // kSoloPrologue: every wave stages all entries itself (the same values to the same
+    // addresses), so that it can read them back without waiting for the other waves.
+    for (int i = kSoloPrologue ? lane : tid; i < count; i += kSoloPrologue ? 64 : kThreads) {
       const int entry = table_row[i];
       table_lds[i] = static_cast<unsigned>(entry) < static_cast<unsigned>(a.num_blocks) ? entry : -1;
     }
@@ -543,6 +560,11 @@ __global__ __launch_bounds__(kThreads) void MlaDecodeKernel(AttnArgs a) {
   }
   map.seq_len = seq_len;
   MLAKV_STAMP(33);
+  // Vector memory requests of a CU are served in order: the query (72 KB per workgroup) is asked
+  // for only now, behind the few bytes of lengths and table entries that the first tile
+  // addresses depend on.
+  if (score_wave && active) load_q();
+  MLAKV_STAMP(32);
   const int num_tiles = (seq_len + kTileTokens - 1) / kTileTokens;
   if (tile_begin >= num_tiles) {
     if (active && direct) {  // empty sequence: zeros, lse = -inf
@@ -579,7 +601,10 @@ __global__ __launch_bounds__(kThreads) void MlaDecodeKernel(AttnArgs a) {
     il8.rope = (lane >> 2) * static_cast<int>(a.rope.row_stride) + (((lane & 3) ^ SwizzleRope8(rope_row)) << 4);
   } else {
 #pragma unroll
-    for (int j = 0; j < 2; ++j) il.lat[j] = (lane ^ SwizzleLat(wave + kWaves * j)) << 4;
+    for (int j = 0; j < 2; ++j) {
+      il.lat[j] = (lane ^ SwizzleLat(wave + kWaves * j)) << 4;
+      il.partner_lat[j] = (lane ^ SwizzleLat((wave & (kScoreWaves - 1)) + kWaves * j)) << 4;
+    }
     il.rope_chunk = ((lane & 7) ^ SwizzleRope(8 * (wave - kScoreWaves) + (lane >> 3))) << 4;
     il.rope = (lane >> 3) * static_cast<int>(a.rope.row_stride) + il.rope_chunk;
   }
@@ -594,7 +619,7 @@ __global__ __launch_bounds__(kThreads) void MlaDecodeKernel(AttnArgs a) {
     }
   };
 
-  // The query must have arrived before the tile loads are issued: the compiler's own wait for
+  // The query must have arrived before this wave issues tile loads: the compiler's own wait for
   // it would otherwise also wait for every tile load issued in between.
   MLAKV_STAMP(35);
   if (score_wave && active) {
@@ -602,17 +627,34 @@ __global__ __launch_bounds__(kThreads) void MlaDecodeKernel(AttnArgs a) {
     for (int ks = 0; ks < kKSteps; ++ks) asm volatile("" ::"v"(q[ks]));
   }
   MLAKV_STAMP(1);
-  __syncthreads();  // table entries visible
+  if constexpr (!kSoloPrologue) __syncthreads();  // table entries visible
 
   // Prologue: tiles 0 .. kRing-2 on their way, tile 0 landed and published. A tile whose load
   // count is not known (rare path) makes every wait up to and including its own a full one.
   int last_unknown = -1;  // newest tile issued with an unknown number of loads
   int issued = 0;         // tiles issued so far
   for (; issued < G::kRing - 1 && issued < ntiles; ++issued) {
-    if (!issue(issued)) last_unknown = issued;
+    if constexpr (kSoloPrologue) {
+      if (score_wave) {
+        map.Begin(issued);  // keeps the cursor in step with the tiles this wave does not issue
+      } else if (!IssueTileBf16<ALIGNED, true>(a, map, il, tile_begin + issued, lds_base + ring(issued), lds + ring(issued), tid)) {
+        last_unknown = issued;
+      }
+    } else {
+      if (!issue(issued)) last_unknown = issued;
+    }
   }
+  // Loads this wave has in flight that are newer than those of tile t: the first `solo_tiles`
+  // tiles carry `solo_loads` each, the later ones `per_tile`.
+  const int solo_tiles = kSoloPrologue ? issued : 0;
+  const int solo_loads = score_wave ? 0 : per_tile + kRowsPerWave;
+  const auto newer_than = [&](int t) __attribute__((always_inline)) {
+    const int solo = max(0, min(issued, solo_tiles) - (t + 1));
+    const int shared = max(0, issued - max(t + 1, solo_tiles));
+    return solo * solo_loads + shared * per_tile;
+  };
   MLAKV_STAMP(2);
-  WaitLoads(last_unknown >= 0 ? 0 : (issued - 1) * per_tile);
+  WaitLoads(last_unknown >= 0 ? 0 : newer_than(0));
   __syncthreads();
   MLAKV_STAMP(3);
 
@@ -621,7 +663,7 @@ __global__ __launch_bounds__(kThreads) void MlaDecodeKernel(AttnArgs a) {
   // tile i-1, whose ring slot the next tile to be issued reuses.
   const auto publish = [&](int i) __attribute__((always_inline)) {
     MLAKV_STAMP((i) < 4 ? 4 + 6 * (i) : -1);
-    if (i + 1 < ntiles) WaitLoads(last_unknown >= i + 1 ? 0 : (issued - (i + 2)) * per_tile);
+    if (i + 1 < ntiles) WaitLoads(last_unknown >= i + 1 ? 0 : newer_than(i + 1));
     __syncthreads();
     MLAKV_STAMP((i) < 4 ? 5 + 6 * (i) : -1);
   };
