@@ -510,6 +510,84 @@ mlakvStatus mlakvAttnDecodeMxQuant(const mlakvAttnPlan* plan, const mlakvCacheVi
                         out_head_stride, quant, nullptr, 0, lse, workspace, workspace_bytes, stream);
 }
 
+uint64_t mlakvIndexerWorkspaceBytes(int32_t batch, int32_t max_seq_len) {
+  if (batch <= 0 || max_seq_len <= 0) return 0;
+  const uint64_t row = (static_cast<uint64_t>(max_seq_len) + 127) & ~127ull;  // 16-bit keys, rows 256-byte aligned
+  return static_cast<uint64_t>(batch) * row * 2;
+}
+
+mlakvStatus mlakvLightningIndexer(const mlakvIndexKeyView* keys, const void* query, int64_t query_seq_stride,
+                                  int64_t query_head_stride, const void* weights, int64_t weights_seq_stride,
+                                  const float* query_dequant_scale, int64_t query_scale_seq_stride, int32_t heads,
+                                  const int32_t* block_table, int32_t table_stride, const int32_t* seq_lens, int32_t batch,
+                                  int32_t max_seq_len, int32_t sparse_count, int32_t* sparse_indices,
+                                  int64_t sparse_indices_seq_stride, void* workspace, uint64_t workspace_bytes, void* stream) {
+  const char* who = "mlakvLightningIndexer";
+  if (keys == nullptr || keys->keys == nullptr || keys->scales == nullptr) return Fail(MLAKV_ERR_PARAM_NULLPTR, "%s: the index key pool is required", who);
+  if (batch < 0) return Fail(MLAKV_ERR_PARAM_INVALID, "%s: negative batch", who);
+  if (batch == 0) return MLAKV_SUCCESS;
+  if (query == nullptr || weights == nullptr || query_dequant_scale == nullptr || block_table == nullptr || seq_lens == nullptr ||
+      sparse_indices == nullptr) {
+    return Fail(MLAKV_ERR_PARAM_NULLPTR, "%s: query, weights, scales, block table, lengths and output are required", who);
+  }
+  if (keys->dim != 128) return Fail(MLAKV_ERR_PARAM_INVALID, "%s: index keys have 128 elements, not %d", who, keys->dim);
+  if (heads <= 0 || heads % 16 != 0 || heads > 64) {
+    return Fail(MLAKV_ERR_PARAM_INVALID, "%s: heads %d must be 16, 32, 48 or 64", who, heads);
+  }
+  if (sparse_count <= 0 || sparse_count > 2048) return Fail(MLAKV_ERR_PARAM_INVALID, "%s: sparse_count %d outside [1, 2048]", who, sparse_count);
+  if (keys->num_blocks <= 0 || keys->block_size <= 0 || max_seq_len <= 0 || batch > 65535) {
+    return Fail(MLAKV_ERR_PARAM_INVALID, "%s: sizes must be positive (batch at most 65535)", who);
+  }
+  if (static_cast<int64_t>(table_stride) * keys->block_size < max_seq_len) {
+    return Fail(MLAKV_ERR_PARAM_INVALID, "%s: a table row of %d blocks cannot address %d tokens", who, table_stride, max_seq_len);
+  }
+  if (!Aligned16(keys->keys) || keys->row_stride % 16 != 0 || keys->block_stride % 16 != 0 || keys->row_stride < 128 ||
+      reinterpret_cast<uintptr_t>(keys->scales) % 4 != 0) {
+    return Fail(MLAKV_ERR_PARAM_INVALID, "%s: key rows must be 16-byte aligned and hold 128 bytes", who);
+  }
+  if (!Aligned16(query) || query_seq_stride % 16 != 0 || query_head_stride % 16 != 0 || query_head_stride < 128 ||
+      reinterpret_cast<uintptr_t>(weights) % 2 != 0 || weights_seq_stride % 2 != 0) {
+    return Fail(MLAKV_ERR_PARAM_INVALID, "%s: query rows must be 16-byte aligned and hold 128 bytes; weights are bf16", who);
+  }
+  if (sparse_indices_seq_stride < sparse_count) return Fail(MLAKV_ERR_PARAM_INVALID, "%s: an output row holds %d entries", who, sparse_count);
+  const uint64_t needed = max_seq_len > sparse_count ? mlakvIndexerWorkspaceBytes(batch, max_seq_len) : 0;
+  if (needed > 0) {
+    if (workspace == nullptr) return Fail(MLAKV_ERR_PARAM_NULLPTR, "%s: %llu workspace bytes are needed", who, static_cast<unsigned long long>(needed));
+    if (workspace_bytes < needed || !Aligned16(workspace)) {
+      return Fail(MLAKV_ERR_PARAM_INVALID, "%s: workspace of %llu bytes (16-byte aligned) needed, %llu given", who,
+                  static_cast<unsigned long long>(needed), static_cast<unsigned long long>(workspace_bytes));
+    }
+  }
+  mlakv::IndexerArgs args{};
+  args.query = static_cast<const char*>(query);
+  args.query_seq_stride = query_seq_stride;
+  args.query_head_stride = query_head_stride;
+  args.weights = static_cast<const char*>(weights);
+  args.weights_seq_stride = weights_seq_stride;
+  args.query_scale = query_dequant_scale;
+  args.query_scale_seq_stride = query_scale_seq_stride;
+  args.key_base = static_cast<const char*>(keys->keys);
+  args.key_block_stride = keys->block_stride;
+  args.key_row_stride = keys->row_stride;
+  args.key_scale_base = keys->scales;
+  args.key_scale_block_stride = keys->scale_block_stride;
+  args.block_table = block_table;
+  args.table_stride = table_stride;
+  args.seq_lens = seq_lens;
+  args.keys = static_cast<unsigned short*>(workspace);
+  args.keys_stride = static_cast<int64_t>((static_cast<uint64_t>(max_seq_len) + 127) & ~127ull);
+  args.indices_out = sparse_indices;
+  args.indices_seq_stride = sparse_indices_seq_stride;
+  args.batch = batch;
+  args.heads = heads;
+  args.num_blocks = keys->num_blocks;
+  args.block_size = keys->block_size;
+  args.max_seq_len = max_seq_len;
+  args.sparse_count = sparse_count;
+  const hipError_t status = mlakv::LaunchIndexer(args, static_cast<hipStream_t>(stream));
+  return status == hipSuccess ? MLAKV_SUCCESS : HipFail(status, who);
+}
+
 mlakvStatus mlakvDynamicMxQuant(const void* x, int64_t x_row_stride, int64_t rows, int32_t cols, void* codes,
                                 int64_t codes_row_stride, void* scales, int64_t scales_row_stride, void* stream) {
   const char* who = "mlakvDynamicMxQuant";

@@ -133,6 +133,27 @@ struct MxQuantArgs {
   int32_t cols;
 };
 
+struct IndexerArgs {
+  const char* query;        // E4M3 [batch][heads][128]
+  int64_t query_seq_stride, query_head_stride;  // bytes
+  const char* weights;      // bf16 [batch][heads]
+  int64_t weights_seq_stride;                   // bytes
+  const float* query_scale; // fp32 [batch][heads]
+  int64_t query_scale_seq_stride;               // elements
+  const char* key_base;     // E4M3 [block][slot][128]
+  int64_t key_block_stride, key_row_stride;     // bytes
+  const float* key_scale_base;                  // fp32 [block][slot]
+  int64_t key_scale_block_stride;               // elements
+  const int32_t* block_table;
+  int32_t table_stride;
+  const int32_t* seq_lens;
+  unsigned short* keys;     // workspace [batch][keys_stride]
+  int64_t keys_stride;
+  int32_t* indices_out;     // int32 [batch][sparse_count]
+  int64_t indices_seq_stride;                   // elements
+  int32_t batch, heads, num_blocks, block_size, max_seq_len, sparse_count;
+};
+
 // MLA geometry the kernels are specialised for (include/moe/core/config.hpp:78-109 defaults).
 constexpr int kLatentDim = 512;
 constexpr int kRopeDim = 64;
@@ -144,6 +165,7 @@ hipError_t LaunchGather(const GatherArgs& args, hipStream_t stream);
 hipError_t LaunchCopyBlocks(const CopyBlocksArgs& args, hipStream_t stream);
 hipError_t LaunchAttnDecode(const AttnArgs& args, hipStream_t stream);
 hipError_t LaunchMxQuant(const MxQuantArgs& args, hipStream_t stream);
+hipError_t LaunchIndexer(const IndexerArgs& args, hipStream_t stream);
 // One-time per-process kernel attribute setup (dynamic LDS above 64 KB).
 hipError_t PrepareAttnKernels();
 

@@ -963,7 +963,7 @@ __global__ __launch_bounds__(kThreads) void MlaDecodeKernel(AttnArgs a) {
 // was never written), so all loads of a group of eight chunks are issued at once, with no
 // dependence on the sequence length.
 constexpr int kCombineHeads = 4;
-__global__ __launch_bounds__(256) void MlaCombineKernel(AttnArgs a) {
+__global__ __launch_bounds__(kCombineHeads * 64) void MlaCombineKernel(AttnArgs a) {
   const int head = blockIdx.x * kCombineHeads + (threadIdx.x >> 6), seq = blockIdx.y;
   const int lane = threadIdx.x & 63;
   if (head >= a.heads) return;
@@ -1075,7 +1075,7 @@ hipError_t LaunchAttnDecode(const AttnArgs& args_in, hipStream_t stream) {
   }
   if (e != hipSuccess) return e;
   if (args.max_chunks > 1) {
-    hipLaunchKernelGGL(MlaCombineKernel, dim3((args.heads + kCombineHeads - 1) / kCombineHeads, args.batch), dim3(256), 0,
+    hipLaunchKernelGGL(MlaCombineKernel, dim3((args.heads + kCombineHeads - 1) / kCombineHeads, args.batch), dim3(kCombineHeads * 64), 0,
                        stream, args);
     e = hipGetLastError();
   }

@@ -45,6 +45,12 @@ class MxQuantOut(C.Structure):
                 ("scales", C.c_void_p), ("scales_seq_stride", C.c_int64), ("scales_head_stride", C.c_int64)]
 
 
+class IndexKeyView(C.Structure):
+    _fields_ = [("keys", C.c_void_p), ("block_stride", C.c_int64), ("row_stride", C.c_int64), ("scales", C.c_void_p),
+                ("scale_block_stride", C.c_int64), ("num_blocks", C.c_int32), ("block_size", C.c_int32), ("dim", C.c_int32),
+                ("reserved", C.c_int32)]
+
+
 class AttnPlan(C.Structure):
     _fields_ = [
         ("batch", C.c_int32), ("heads", C.c_int32), ("max_seq_len", C.c_int32), ("block_size", C.c_int32),
@@ -89,6 +95,9 @@ PROTOTYPES = {
     "mlakvAttnSparsePlanInit": (_i32, [_i32, _i32, _i32, _i32, _i32, _P(AttnPlan)]),
     "mlakvAttnDecodeSparse": (_i32, [_P(AttnPlan), _P(CacheView), _i32, _vp, _i64, _i64, _vp, _i64, _i64, _vp, _i32, _vp, _vp, _i64,
                                      C.c_double, _vp, _i64, _i64, _vp, _vp, _u64, _vp]),
+    "mlakvIndexerWorkspaceBytes": (_u64, [_i32, _i32]),
+    "mlakvLightningIndexer": (_i32, [_P(IndexKeyView), _vp, _i64, _i64, _vp, _i64, _vp, _i64, _i32, _vp, _i32, _vp, _i32, _i32, _i32,
+                                     _vp, _i64, _vp, _u64, _vp]),
     "mlakvDynamicMxQuant": (_i32, [_vp, _i64, _i64, _i32, _vp, _i64, _vp, _i64, _vp]),
     "mlakvArenaCreate": (_i32, [_i32, _P(_vp)]),
     "mlakvArenaDestroy": (None, [_vp]),

@@ -287,6 +287,49 @@ def bench_attention(args, torch, np, ffi, fp8=False, batch=32, ctx=2048, heads=6
     return result
 
 
+def bench_indexer(args, torch, np, ffi, batch=32, ctx=8192, heads=64, k=512, bs=64, slices=4):
+    """Lightning Indexer at the shape the selected-token attention is timed on: FP8 index keys
+    (128 + 4 bytes per cached token) scored against one query token per sequence, top-k selected.
+    HIP-event time of the operator (score kernel + selection kernel) over rotating key pools."""
+    lib = ffi.load()
+    blocks = batch * (ctx // bs)
+    rng = np.random.default_rng(9)
+    keys = [torch.randint(0, 0x58, (blocks * bs, 128), dtype=torch.uint8, device="cuda") for _ in range(slices)]
+    scales = torch.rand(blocks * bs, device="cuda") * 0.04 + 0.01
+    table = torch.as_tensor(rng.permutation(blocks).astype(np.int32).reshape(batch, ctx // bs), device="cuda")
+    lens = torch.full((batch,), ctx, dtype=torch.int32, device="cuda")
+    query = torch.randint(0, 0x58, (batch, heads, 128), dtype=torch.uint8, device="cuda")
+    weights = torch.randn(batch, heads, device="cuda").to(torch.bfloat16)
+    q_scale = torch.rand(batch, heads, device="cuda") * 0.04 + 0.01
+    out = torch.empty(batch, k, dtype=torch.int32, device="cuda")
+    workspace = torch.empty(int(lib.mlakvIndexerWorkspaceBytes(batch, ctx)), dtype=torch.uint8, device="cuda")
+    views = [ffi.IndexKeyView(kp.data_ptr(), bs * 128, 128, scales.data_ptr(), bs, blocks, bs, 128, 0) for kp in keys]
+
+    def launch(i):
+        ffi.check(lib.mlakvLightningIndexer(C.byref(views[i % slices]), query.data_ptr(), heads * 128, 128, weights.data_ptr(),
+                                            heads * 2, q_scale.data_ptr(), heads, heads, table.data_ptr(), ctx // bs, lens.data_ptr(),
+                                            batch, ctx, k, out.data_ptr(), k, workspace.data_ptr(), workspace.numel(),
+                                            stream_ptr(torch)))
+    iters = 64
+    for i in range(8):
+        launch(i)
+    torch.cuda.synchronize()
+    start, stop = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+    start.record()
+    for i in range(iters):
+        launch(i)
+    stop.record()
+    torch.cuda.synchronize()
+    us = start.elapsed_time(stop) * 1e3 / iters
+    algorithmic = batch * ctx * (128 + 4) + batch * heads * (128 + 2 + 4) + 4 * batch * (ctx // bs) + 4 * batch * k
+    return {"us_per_step": us,
+            "workload": f"batch {batch}, ctx {ctx}, {heads} index heads x 128, top-{k}, block {bs}, e4m3 keys + fp32 row scale, "
+                        f"shuffled table, {slices} rotating key pools",
+            "roofline": {"bound": "hbm", "achieved": algorithmic / (us * 1e-6) / 1e9, "peak": HBM_PEAK_GBPS, "unit": "GB/s",
+                         "frac": algorithmic / (us * 1e-6) / 1e9 / HBM_PEAK_GBPS, "traffic": None},
+            "algorithmic_bytes": algorithmic, "launches_timed": iters}
+
+
 def bench_side_kernels(args, torch, np, ffi):
     """The other data-movement kernels of the path at configs[3]/[4]-like sizes (8 layers to bound
     memory): FP8 quantize-on-append, FP8 dequantising gather, bf16 compaction copy. HIP-event
@@ -488,7 +531,8 @@ def main():
                           "attention_long": bench_attention(args, torch, np, ffi, batch=128, ctx=8192, slices=2, iters=16,
                                                             label="configs[4]-scale decode shape (one workgroup per sequence)"),
                           "attention_sparse": bench_attention(args, torch, np, ffi, batch=32, ctx=8192, slices=4, sparse_k=512,
-                                                              label="selected-token decode (index_topk 512 of 8192)")}))
+                                                              label="selected-token decode (index_topk 512 of 8192)"),
+                          "indexer": bench_indexer(args, torch, np, ffi)}))
         return 0
     ag = bench_append_gather(args, torch, np, ffi)
     line = {
@@ -517,6 +561,7 @@ def main():
                                                  label="configs[4]-scale decode shape (one workgroup per sequence)")
         line["attention_sparse"] = bench_attention(args, torch, np, ffi, batch=32, ctx=8192, slices=4, sparse_k=512,
                                                    label="selected-token decode (index_topk 512 of 8192)")
+        line["indexer"] = bench_indexer(args, torch, np, ffi)
         line["side_kernels"] = bench_side_kernels(args, torch, np, ffi)
     if not args.no_cpu_baseline:
         line["cpu_baseline"] = cpu_baseline(np, ag)

@@ -220,6 +220,39 @@ mlakvStatus mlakvAttnDecodeSparse(const mlakvAttnPlan* plan, const mlakvCacheVie
                                   void* out, int64_t out_seq_stride, int64_t out_head_stride, float* lse, void* workspace,
                                   uint64_t workspace_bytes, void* stream);
 
+/* Lightning Indexer for decode (one query token per sequence): replaces the plan + launch of
+ * aclnnQuantLightningIndexer (contract include/moe/core/op_table.hpp:964-1006; kernel vendored
+ * under third_party/ops_transformer/attention/quant_lightning_indexer, formula in its README.md)
+ * with the engine's fixed attributes: E4M3 query and key, per-token-head quantization (mode 0),
+ * key layout PA_BSND with N2 = 1 and D = 128, causal sparse mode (for one query token: every
+ * cached token is eligible).
+ *   score[b][t] = key_scale[t] * sum_h (weights[b][h] * query_dequant_scale[b][h]) * ReLU(q[b][h] . k[t])
+ *   sparse_indices[b] = the sparse_count positions with the largest scores
+ * Scores are compared as bf16 (fp32 arithmetic in the vendored kernel's order, rounded with ties
+ * away from zero); equal scores go to the lower position. Output per sequence, as the vendored
+ * kernel writes it: a sequence no longer than sparse_count yields 0 .. len-1; otherwise the
+ * positions above the k-th score in increasing order, then those equal to it; the rest is -1.
+ * This is the list mlakvAttnDecodeSparse takes.
+ *   keys: the paged pool of index keys, E4M3 [block][slot][128] with one fp32 dequantization scale
+ *   per row, addressed through the same block table as the KV cache.
+ *   query E4M3 [batch][heads][128] (strides in bytes), weights bf16 [batch][heads] (byte stride),
+ *   query_dequant_scale fp32 [batch][heads] (element stride); heads in {16, 32, 48, 64}.
+ *   workspace: mlakvIndexerWorkspaceBytes(batch, max_seq_len) bytes (the 16-bit scores). */
+typedef struct mlakvIndexKeyView {
+  const void* keys;
+  int64_t block_stride, row_stride;  /* bytes */
+  const float* scales;
+  int64_t scale_block_stride;        /* elements */
+  int32_t num_blocks, block_size, dim, reserved;
+} mlakvIndexKeyView;
+uint64_t mlakvIndexerWorkspaceBytes(int32_t batch, int32_t max_seq_len);
+mlakvStatus mlakvLightningIndexer(const mlakvIndexKeyView* keys, const void* query, int64_t query_seq_stride,
+                                  int64_t query_head_stride, const void* weights, int64_t weights_seq_stride,
+                                  const float* query_dequant_scale, int64_t query_scale_seq_stride, int32_t heads,
+                                  const int32_t* block_table, int32_t table_stride, const int32_t* seq_lens, int32_t batch,
+                                  int32_t max_seq_len, int32_t sparse_count, int32_t* sparse_indices,
+                                  int64_t sparse_indices_seq_stride, void* workspace, uint64_t workspace_bytes, void* stream);
+
 /* ------------------------------------------------------------------------- */
 /* Static arena (host)                                                        */
 /* ------------------------------------------------------------------------- */

@@ -624,6 +624,73 @@ void kvo_mla_decode_sparse(const uint16_t* q_latent, int64_t q_latent_seq_stride
 }
 
 /* ------------------------------------------------------------------------- */
+/* Lightning Indexer: scores and top-k selection                               */
+/* ------------------------------------------------------------------------- */
+
+/* fp32 -> bf16 rounding to nearest with ties away from zero, then the order-preserving 16-bit key:
+ * a NaN gets the lowest key, a negative value has all bits inverted, any other value its sign bit
+ * set. */
+static uint16_t indexer_key(float score) {
+  uint32_t bits = f32_bits(score);
+  uint16_t b;
+  if ((bits & 0x7fffffffu) > 0x7f800000u) {
+    b = 0x7fc0u;
+  } else {
+    b = (uint16_t)((bits + 0x8000u) >> 16); /* magnitude + half, truncated: ties go away from zero */
+  }
+  if (b == 0x7fc0u) return 0x0000u;
+  return (b & 0x8000u) ? (uint16_t)~b : (uint16_t)(b | 0x8000u);
+}
+
+void kvo_indexer_scores(const uint8_t* query, const uint16_t* weights, const float* query_scale, int64_t heads,
+                        int64_t dim, const uint8_t* key_plane, int64_t key_block_stride, int64_t key_row_stride,
+                        const float* key_scale_plane, int64_t scale_block_stride, int64_t block_size,
+                        const int32_t* row_table, int64_t seq_len, uint16_t* keys_out) {
+  float* w = (float*)malloc((size_t)heads * sizeof(float));
+  for (int64_t h = 0; h < heads; ++h) w[h] = kvo_bf16_to_f32(weights[h]) * query_scale[h];
+  for (int64_t t = 0; t < seq_len; ++t) {
+    const int64_t slot = kvo_slot(row_table, t, block_size);
+    const int64_t block = slot / block_size, in_block = slot % block_size;
+    const uint8_t* k = key_plane + block * key_block_stride + in_block * key_row_stride;
+    float sum[2] = {0.0f, 0.0f}; /* even and odd heads, one fused multiply-add per head each */
+    for (int64_t h = 0; h < heads; ++h) {
+      /* every product of two E4M3 values is exact in double, and so is the sum of 128 of them */
+      double dot = 0.0;
+      for (int64_t d = 0; d < dim; ++d) dot += (double)kvo_e4m3_to_f32(query[h * dim + d]) * (double)kvo_e4m3_to_f32(k[d]);
+      float qk = (float)dot;
+      if (!(qk > 0.0f)) qk = 0.0f;
+      sum[h & 1] = fmaf(qk, w[h], sum[h & 1]);
+    }
+    const float score = (sum[0] + sum[1]) * key_scale_plane[block * scale_block_stride + in_block];
+    keys_out[t] = indexer_key(score);
+  }
+  free(w);
+}
+
+void kvo_indexer_topk(const uint16_t* keys, int64_t seq_len, int64_t sparse_count, int32_t* indices_out) {
+  int64_t written = 0;
+  if (seq_len <= sparse_count) {
+    for (int64_t t = 0; t < seq_len; ++t) indices_out[written++] = (int32_t)t;
+  } else {
+    /* the k-th largest key by counting, then everything above it in index order, then the lowest
+     * indices among the keys equal to it */
+    int64_t histogram[65536];
+    memset(histogram, 0, sizeof histogram);
+    for (int64_t t = 0; t < seq_len; ++t) ++histogram[keys[t]];
+    int64_t above = 0;
+    int32_t threshold = 65535;
+    while (above + histogram[threshold] < sparse_count) above += histogram[threshold--];
+    for (int64_t t = 0; t < seq_len; ++t) {
+      if (keys[t] > threshold) indices_out[written++] = (int32_t)t;
+    }
+    for (int64_t t = 0; t < seq_len && written < sparse_count; ++t) {
+      if (keys[t] == threshold) indices_out[written++] = (int32_t)t;
+    }
+  }
+  for (; written < sparse_count; ++written) indices_out[written] = -1;
+}
+
+/* ------------------------------------------------------------------------- */
 /* block pool                                                                 */
 /* ------------------------------------------------------------------------- */
 

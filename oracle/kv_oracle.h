@@ -237,6 +237,32 @@ void kvo_mla_decode_sparse(const uint16_t* q_latent, int64_t q_latent_seq_stride
                            const int32_t* seq_lens, const int32_t* sparse_indices, int64_t sparse_count,
                            int64_t sparse_stride, int64_t batch, int64_t heads, double scale, float* out, float* lse);
 
+/* Lightning Indexer (aclnnQuantLightningIndexer; contract include/moe/core/op_table.hpp:964-1006,
+ * kernel vendored under third_party/ops_transformer/attention/quant_lightning_indexer): for one
+ * query token of one sequence, the score of cached token t over the g = `heads` index heads
+ *   score[t] = key_scale[t] * sum_h (W[h] * query_scale[h]) * ReLU(q_h . k_t)
+ * (README.md "计算公式"), evaluated in the order of the vendored arch35 kernel
+ * (op_kernel/arch35/vf/quant_lightning_indexer_vector1.h:288-330): w[h] = W[h] * query_scale[h] in
+ * fp32; two fp32 accumulators, even and odd heads, one multiply-add per head; their sum times the
+ * key scale; rounded to bf16 with ties away from zero (CAST_ROUND) and mapped to an order-preserving
+ * 16-bit key (:66-96). q_h . k_t is the exact dot product of the E4M3 values rounded once to
+ * fp32 (the NPU's and the GPU's matrix units accumulate in fp32 in an order of their own, so a
+ * key may differ by one bf16 step from this restatement; parity with CANN unpinned).
+ * query: E4M3 [heads][dim]; weights bf16 [heads]; query_scale fp32 [heads]; key_plane E4M3
+ * [block][slot][dim] with key_scale_plane fp32 [block][slot] (layout PA_BSND, N2 = 1). */
+void kvo_indexer_scores(const uint8_t* query, const uint16_t* weights, const float* query_scale, int64_t heads,
+                        int64_t dim, const uint8_t* key_plane, int64_t key_block_stride, int64_t key_row_stride,
+                        const float* key_scale_plane, int64_t scale_block_stride, int64_t block_size,
+                        const int32_t* row_table, int64_t seq_len, uint16_t* keys_out);
+
+/* Top-k over the 16-bit keys as the vendored kernel selects (op_kernel/arch35/
+ * quant_lightning_indexer_service_vector.h:446-541, vf/vf_topk.h:634-670): a sequence no longer
+ * than sparse_count yields 0 .. seq_len-1; otherwise every token whose key is above the k-th
+ * largest key, in index order, followed by the lowest-indexed tokens whose key equals it; the rest
+ * of the sparse_count entries is -1. (The vendored kernel processes long sequences in trunks, which
+ * keeps the same set and may order it differently.) */
+void kvo_indexer_topk(const uint16_t* keys, int64_t seq_len, int64_t sparse_count, int32_t* indices_out);
+
 /* ---- block pool: free list, block tables, recycling, compaction ---------- */
 /* No reference counterpart (the reference is one sequence with identity paging and
  * never writes its block table, src/memory/static_arena_manager.cpp:298). Semantics:

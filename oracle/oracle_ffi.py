@@ -80,6 +80,8 @@ _PROTOTYPES = {
                               _vp, _vp, C.c_int]),
     "kvo_mla_decode_sparse": (None, [_vp, _i64, _i64, _vp, _i64, _i64, _P(CacheView), _vp, _i64, _vp, _vp, _i64, _i64, _i64, _i64,
                                      C.c_double, _vp, _vp]),
+    "kvo_indexer_scores": (None, [_vp, _vp, _vp, _i64, _i64, _vp, _i64, _i64, _vp, _i64, _i64, _vp, _i64, _vp]),
+    "kvo_indexer_topk": (None, [_vp, _i64, _i64, _vp]),
     "kvo_splitmix64": (_u64, [_P(_u64)]),
     "kvo_pool_new": (_vp, [_i64, _i64, _i64, _i64, _u64, C.c_int]),
     "kvo_pool_delete": (None, [_vp]),
@@ -260,6 +262,30 @@ def mx_quant_rows(x):
     scales = np.zeros((rows, -(-cols // 32)), dtype=np.uint8)
     load().kvo_mx_quant_rows(_ptr(x), cols, rows, cols, _ptr(codes), cols, _ptr(scales), scales.shape[1])
     return codes, scales
+
+
+def indexer_scores(query, weights, query_scale, key_plane, key_scale_plane, block_size, row_table, seq_len):
+    """One sequence: query uint8 [H, D] (E4M3 codes), weights uint16 [H] (bf16 bits), query_scale float32 [H],
+    key_plane uint8 [blocks*bs, D], key_scale_plane float32 [blocks*bs], row_table int32 [max_blocks].
+    Returns the 16-bit order-preserving score keys, uint16 [seq_len]."""
+    query = np.ascontiguousarray(query, dtype=np.uint8)
+    weights = np.ascontiguousarray(weights, dtype=np.uint16)
+    query_scale = np.ascontiguousarray(query_scale, dtype=np.float32)
+    key_plane = np.ascontiguousarray(key_plane, dtype=np.uint8)
+    key_scale_plane = np.ascontiguousarray(key_scale_plane, dtype=np.float32)
+    row_table = np.ascontiguousarray(row_table, dtype=np.int32)
+    heads, dim = query.shape
+    keys = np.zeros(max(seq_len, 1), dtype=np.uint16)
+    load().kvo_indexer_scores(_ptr(query), _ptr(weights), _ptr(query_scale), heads, dim, _ptr(key_plane), block_size * dim, dim,
+                              _ptr(key_scale_plane), block_size, block_size, _ptr(row_table), seq_len, _ptr(keys))
+    return keys[:seq_len]
+
+
+def indexer_topk(keys, sparse_count):
+    keys = np.ascontiguousarray(keys, dtype=np.uint16)
+    out = np.zeros(sparse_count, dtype=np.int32)
+    load().kvo_indexer_topk(_ptr(keys), len(keys), sparse_count, _ptr(out))
+    return out
 
 
 def gather_rows_fp8(latent_plane, rope_plane, scale_plane, block_size, table, seq_lens, latent_dim=512, rope_dim=64):

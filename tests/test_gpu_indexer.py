@@ -1,0 +1,178 @@
+"""GPU parity: Lightning Indexer (mlakvLightningIndexer) through the C ABI against the CPU oracle.
+The scores are compared as the values of the 16-bit keys the selection sorts by. The kernel sums
+the exact products in fp32 in the matrix unit's order and the head sum in a lane-tree order, the
+oracle rounds the exact dot product once and follows the vendored kernel's even/odd order, so a
+score may differ by fp32 rounding of a sum that can cancel (weights of either sign): the bound is
+one bf16 step of the score plus 1e-5 of the sum of the terms' magnitudes, and at most 0.5 % of the
+keys may differ at all. The selection itself is integer work and must be bit-exact on the keys the
+GPU produced, in the documented order."""
+import ctypes as C
+
+import numpy as np
+import pytest
+import torch
+
+import kv_testing as kt
+import mlakv_ffi as ffi
+import oracle_ffi as orc
+
+pytestmark = pytest.mark.gpu
+
+D = 128
+
+
+def _decode_table():
+    lib = orc.load()
+    return np.array([lib.kvo_e4m3_to_f32(c) for c in range(256)], dtype=np.float64)
+
+
+_E4M3 = _decode_table()
+
+
+def _key_value(keys):
+    keys = np.asarray(keys, dtype=np.uint16)
+    bits = np.where(keys & 0x8000, keys & 0x7FFF, ~keys & 0xFFFF).astype(np.uint32)
+    return (bits << 16).view(np.float32).astype(np.float64)
+
+
+def _codes(rng, shape, spread):
+    """Random E4M3 codes without NaN: magnitudes below `spread` exponent steps, either sign."""
+    magnitude = rng.integers(0, spread, shape).astype(np.uint8)
+    return (magnitude | (rng.integers(0, 2, shape).astype(np.uint8) << 7)).astype(np.uint8)
+
+
+def _run(seq_lens, bs, heads, k, seed, zero_query=False):
+    rng = np.random.default_rng(seed)
+    batch = len(seq_lens)
+    max_len = max(max(seq_lens), 1)
+    blocks = sum(-(-n // bs) for n in seq_lens) + 5
+    pool = kt.build_tables(seq_lens, bs, blocks, seed=seed, max_blocks=-(-max_len // bs))
+    table = pool.table()
+    key_plane = _codes(rng, (blocks * bs, D), 0x58)
+    key_scale = rng.uniform(0.01, 0.05, blocks * bs).astype(np.float32)
+    query = np.zeros((batch, heads, D), np.uint8) if zero_query else _codes(rng, (batch, heads, D), 0x58)
+    weights = kt.randn_bf16((batch, heads), seed=seed + 1)
+    q_scale = rng.uniform(0.01, 0.05, (batch, heads)).astype(np.float32)
+    lib = ffi.load()
+    keys_d = torch.as_tensor(key_plane, device="cuda")
+    scales_d = torch.as_tensor(key_scale, device="cuda")
+    view = ffi.IndexKeyView(keys_d.data_ptr(), bs * D, D, scales_d.data_ptr(), bs, blocks, bs, D, 0)
+    query_d, weights_d, q_scale_d = torch.as_tensor(query, device="cuda"), weights.cuda(), torch.as_tensor(q_scale, device="cuda")
+    table_d, lens_d = kt.dev_i32(table), kt.dev_i32(seq_lens)
+    out = torch.full((batch, k), -7, dtype=torch.int32, device="cuda")
+    ws_bytes = int(lib.mlakvIndexerWorkspaceBytes(batch, max_len))
+    workspace = torch.zeros(max(ws_bytes, 16), dtype=torch.uint8, device="cuda")
+    ffi.check(lib.mlakvLightningIndexer(C.byref(view), query_d.data_ptr(), heads * D, D, weights_d.data_ptr(), heads * 2,
+                                        q_scale_d.data_ptr(), heads, heads, table_d.data_ptr(), table.shape[1], lens_d.data_ptr(),
+                                        batch, max_len, k, out.data_ptr(), k, workspace.data_ptr(), workspace.numel(),
+                                        kt.stream_ptr()))
+    torch.cuda.synchronize()
+    got = out.cpu().numpy()
+    row = (max_len + 127) // 128 * 128
+    gpu_keys = workspace.view(torch.int16).cpu().numpy().view(np.uint16)[: batch * row].reshape(batch, row)
+    differing = total = 0
+    for b, n in enumerate(seq_lens):
+        if n <= k:
+            assert got[b].tolist() == list(range(n)) + [-1] * (k - n)
+            continue
+        want_keys = orc.indexer_scores(query[b], kt.bits16(weights[b]), q_scale[b], key_plane, key_scale, bs, table[b], n)
+        # fp32 rounding in a different order: one bf16 step of the score, plus the fp32 error of a
+        # 64-term sum that may cancel (weights of either sign), measured against the sum of magnitudes
+        slots = table[b][np.arange(n) // bs].astype(np.int64) * bs + np.arange(n) % bs
+        qk = np.maximum(_E4M3[query[b]] @ _E4M3[key_plane[slots]].T, 0.0)
+        w = (kt.bits16(weights[b]).astype(np.uint32) << 16).view(np.float32).astype(np.float64) * q_scale[b]
+        magnitude = (qk * np.abs(w)[:, None]).sum(axis=0) * key_scale[slots]
+        got_f, want_f = _key_value(gpu_keys[b, :n]), _key_value(want_keys)
+        tolerance = 2.0 ** -7 * np.abs(want_f) + 1e-5 * magnitude + 1e-30
+        assert (np.abs(got_f - want_f) <= tolerance).all(), (b, np.abs(got_f - want_f).max())
+        differing += int((gpu_keys[b, :n] != want_keys).sum())
+        total += n
+        # integer selection: bit-exact on the keys the GPU holds, in the documented order
+        assert got[b].tolist() == orc.indexer_topk(gpu_keys[b, :n], k).tolist()
+        # and against the oracle's own keys: the same set except where such a key difference
+        # moves a token across the threshold
+        want = orc.indexer_topk(want_keys, k)
+        odd = sorted(set(got[b].tolist()) ^ set(want.tolist()))
+        threshold = _key_value(np.sort(want_keys)[-k:])[0]
+        assert all(abs(want_f[t] - threshold) <= 2 * tolerance[t] for t in odd), (b, len(odd))
+        assert len(odd) <= max(2, k // 50)
+    assert total == 0 or differing <= 0.005 * total
+    return got
+
+
+@pytest.mark.parametrize("bs,heads,k", [(64, 64, 512), (16, 32, 100), (128, 16, 2048), (64, 48, 64)])
+def test_indexer_matches_oracle_ragged(bs, heads, k):
+    _run([3000, 513 if k == 512 else k + 1, 1, 0, 2600, k, 777], bs, heads, k, seed=101)
+
+
+def test_all_equal_scores_select_the_first_positions():
+    got = _run([1000, 300], 64, 64, 256, seed=102, zero_query=True)
+    assert got[0].tolist() == list(range(256)) and got[1].tolist() == list(range(256))
+
+
+def test_indices_feed_the_selected_token_attention():
+    """The two operators chained on one block table: the attention over the indexer's list equals
+    the oracle's attention over the same list."""
+    import math
+    bs, heads, k = 64, 64, 128
+    ctxs = [700, 90]
+    blocks = sum(-(-c // bs) for c in ctxs) + 2
+    pool = kt.build_tables(ctxs, bs, blocks, seed=103)
+    table = pool.table()
+    cache = kt.PagedCache(1, blocks, bs)
+    total = sum(ctxs)
+    kt.append(cache, kt.randn_bf16((1, total, kt.LATENT), seed=104).cuda(), kt.randn_bf16((1, total, kt.ROPE), seed=105).cuda(),
+              kt.dev_i32(kt.slots_for(table, ctxs, bs)))
+    rng = np.random.default_rng(106)
+    keys_d = torch.as_tensor(_codes(rng, (blocks * bs, D), 0x58), device="cuda")
+    scales_d = torch.as_tensor(rng.uniform(0.01, 0.05, blocks * bs).astype(np.float32), device="cuda")
+    view = ffi.IndexKeyView(keys_d.data_ptr(), bs * D, D, scales_d.data_ptr(), bs, blocks, bs, D, 0)
+    iq = torch.as_tensor(_codes(rng, (2, heads, D), 0x58), device="cuda")
+    iw = kt.randn_bf16((2, heads), seed=107).cuda()
+    iqs = torch.as_tensor(rng.uniform(0.01, 0.05, (2, heads)).astype(np.float32), device="cuda")
+    lib = ffi.load()
+    table_d, lens_d = kt.dev_i32(table), kt.dev_i32(ctxs)
+    selection = torch.zeros(2, k, dtype=torch.int32, device="cuda")
+    workspace = torch.zeros(int(lib.mlakvIndexerWorkspaceBytes(2, 700)), dtype=torch.uint8, device="cuda")
+    ffi.check(lib.mlakvLightningIndexer(C.byref(view), iq.data_ptr(), heads * D, D, iw.data_ptr(), heads * 2, iqs.data_ptr(), heads,
+                                        heads, table_d.data_ptr(), table.shape[1], lens_d.data_ptr(), 2, 700, k,
+                                        selection.data_ptr(), k, workspace.data_ptr(), workspace.numel(), kt.stream_ptr()))
+    q = kt.randn_bf16((2, heads, kt.LATENT + kt.ROPE), seed=108).cuda()
+    scale = 1.0 / math.sqrt(192.0)
+    out, lse, _ = kt.sparse_attention(cache, 0, q, table_d, lens_d, selection, scale)
+    chosen = selection.cpu().numpy()
+    assert (chosen[0] >= 0).all() and len(set(chosen[0].tolist())) == k
+    assert chosen[1].tolist() == list(range(90)) + [-1] * (k - 90)
+    expected, _ = kt.oracle_attention(cache, 0, q, table, ctxs, scale, sparse_indices=chosen)
+    peak = np.abs(expected).max()
+    assert np.abs(out.float().cpu().numpy() - expected).max() <= 2e-2 * peak
+
+
+def test_argument_checks():
+    lib = ffi.load()
+    keys = torch.zeros(4 * 64, D, dtype=torch.uint8, device="cuda")
+    scales = torch.ones(4 * 64, dtype=torch.float32, device="cuda")
+    query = torch.zeros(1, 64, D, dtype=torch.uint8, device="cuda")
+    weights = torch.ones(1, 64, dtype=torch.bfloat16, device="cuda")
+    q_scale = torch.ones(1, 64, dtype=torch.float32, device="cuda")
+    table, lens = kt.dev_i32(np.arange(4, dtype=np.int32).reshape(1, 4)), kt.dev_i32([200])
+    out = torch.zeros(1, 64, dtype=torch.int32, device="cuda")
+    workspace = torch.zeros(int(lib.mlakvIndexerWorkspaceBytes(1, 256)), dtype=torch.uint8, device="cuda")
+
+    def call(view=None, heads=64, k=64, max_len=256, ws=workspace.data_ptr(), ws_bytes=workspace.numel(), q=query.data_ptr(), stride=64):
+        view = view or ffi.IndexKeyView(keys.data_ptr(), 64 * D, D, scales.data_ptr(), 64, 4, 64, D, 0)
+        return lib.mlakvLightningIndexer(C.byref(view), q, 64 * D, D, weights.data_ptr(), 128, q_scale.data_ptr(), 64, heads,
+                                         table.data_ptr(), 4, lens.data_ptr(), 1, max_len, k, out.data_ptr(), stride, ws, ws_bytes,
+                                         kt.stream_ptr())
+
+    assert call() == 0
+    assert call(heads=24) == ffi.ERR_PARAM_INVALID
+    assert call(k=0) == ffi.ERR_PARAM_INVALID and call(k=4096) == ffi.ERR_PARAM_INVALID
+    assert call(max_len=257) == ffi.ERR_PARAM_INVALID          # the table row addresses 256 tokens
+    assert call(ws=None) == ffi.ERR_PARAM_NULLPTR
+    assert call(ws_bytes=16) == ffi.ERR_PARAM_INVALID
+    assert call(q=None) == ffi.ERR_PARAM_NULLPTR
+    assert call(stride=32) == ffi.ERR_PARAM_INVALID
+    assert call(view=ffi.IndexKeyView(keys.data_ptr(), 64 * D, D, scales.data_ptr(), 64, 4, 64, 64, 0)) == ffi.ERR_PARAM_INVALID
+    assert call(max_len=64, ws=None, ws_bytes=0) == 0          # nothing longer than k: no scores, no workspace
+    torch.cuda.synchronize()
