@@ -80,7 +80,7 @@ struct aclScalar { void* value = nullptr; aclDataType dtype = ACL_DT_UNDEFINED; 
 
 namespace {
 
-enum class OpKind { kScatter, kAttention, kGather };
+enum class OpKind { kScatter, kAttention, kGather, kMxQuant };
 enum class SlotKind { kNull, kTensor, kList, kIntArray };
 
 struct Slot {
@@ -654,6 +654,48 @@ aclnnStatus aclnnScatterPaKvCache(void* workspace, uint64_t workspace_size, aclO
   return status;
 }
 
+// ---- aclnnDynamicMxQuant ----------------------------------------------------------------------
+
+aclnnStatus aclnnDynamicMxQuantGetWorkspaceSize(const aclTensor* x, int64_t axis, char* round_mode_optional, int64_t dst_type,
+                                                int64_t blocksize, int64_t scale_alg, const aclTensor* y_out,
+                                                const aclTensor* mxscale_out, uint64_t* workspace_size, aclOpExecutor** executor) {
+  SHIM_REQUIRE(workspace_size && executor, ACLNN_ERR_PARAM_NULLPTR, "DynamicMxQuant: null workspace_size / executor output");
+  *executor = nullptr;
+  SHIM_REQUIRE(x && y_out && mxscale_out, ACLNN_ERR_PARAM_NULLPTR, "DynamicMxQuant: x, y and mxscale are required");
+  SHIM_REQUIRE(AsTensor(x) && AsTensor(y_out) && AsTensor(mxscale_out), ACLNN_ERR_PARAM_INVALID, "DynamicMxQuant: bad tensor handle");
+  const int64_t rank = static_cast<int64_t>(x->dims.size());
+  SHIM_REQUIRE(rank == 2, ACLNN_ERR_PARAM_INVALID, "DynamicMxQuant: x must be [rows, cols] (the engine quantizes flat activations)");
+  SHIM_REQUIRE(axis == -1 || axis == rank - 1, ACLNN_ERR_PARAM_INVALID, "DynamicMxQuant: only the last axis is served, got %lld",
+               static_cast<long long>(axis));
+  SHIM_REQUIRE(round_mode_optional == nullptr || std::strcmp(round_mode_optional, "rint") == 0, ACLNN_ERR_PARAM_INVALID,
+               "DynamicMxQuant: round mode '%s' is not served; the engine uses \"rint\"", round_mode_optional);
+  SHIM_REQUIRE(dst_type == ACL_FLOAT8_E4M3FN, ACLNN_ERR_PARAM_INVALID, "DynamicMxQuant: dst_type %lld is not served; the engine uses E4M3 (36)",
+               static_cast<long long>(dst_type));
+  SHIM_REQUIRE(blocksize == 32, ACLNN_ERR_PARAM_INVALID, "DynamicMxQuant: the microscale block is 32, got %lld", static_cast<long long>(blocksize));
+  SHIM_REQUIRE(scale_alg == 0, ACLNN_ERR_PARAM_INVALID, "DynamicMxQuant: only the OCP scale algorithm (0) is served");
+  SHIM_REQUIRE(x->dtype == ACL_BF16 && y_out->dtype == ACL_FLOAT8_E4M3FN && mxscale_out->dtype == ACL_FLOAT8_E8M0, ACLNN_ERR_PARAM_INVALID,
+               "DynamicMxQuant: BF16 input, E4M3 values and E8M0 scales expected");
+  const int64_t rows = x->dims[0], cols = x->dims[1];
+  SHIM_REQUIRE(rows > 0 && cols > 0 && cols % 32 == 0 && cols <= INT32_MAX, ACLNN_ERR_PARAM_INVALID,
+               "DynamicMxQuant: %lld columns are not a whole number of blocks of 32", static_cast<long long>(cols));
+  SHIM_REQUIRE(y_out->dims.size() == 2 && y_out->dims[0] == rows && y_out->dims[1] == cols, ACLNN_ERR_PARAM_INVALID,
+               "DynamicMxQuant: y must have the shape of x");
+  SHIM_REQUIRE(mxscale_out->dims.size() == 2 && mxscale_out->dims[0] == rows && mxscale_out->dims[1] == cols / 32, ACLNN_ERR_PARAM_INVALID,
+               "DynamicMxQuant: mxscale must be [rows, cols / 32]");
+  SHIM_REQUIRE(x->strides[1] == 1 && y_out->strides[1] == 1 && mxscale_out->strides[1] == 1, ACLNN_ERR_PARAM_INVALID,
+               "DynamicMxQuant: the last axis must be dense");
+  aclOpExecutor* e = NewExecutor(OpKind::kMxQuant, {TensorSlot(x), TensorSlot(y_out), TensorSlot(mxscale_out)});
+  e->tokens = static_cast<int32_t>(cols);  // columns
+  e->key_row_stride = x->strides[0] * 2;
+  e->value_row_stride = y_out->strides[0];
+  e->key_block_stride = mxscale_out->strides[0];
+  e->q_token_stride = rows;
+  e->workspace_bytes = 0;
+  *workspace_size = 0;
+  *executor = e;
+  return ACLNN_SUCCESS;
+}
+
 // ---- aclnnFusedInferAttentionScoreV5 ------------------------------------------------------------
 
 aclnnStatus aclnnFusedInferAttentionScoreV5GetWorkspaceSize(
@@ -776,6 +818,15 @@ aclnnStatus aclnnFusedInferAttentionScoreV5GetWorkspaceSize(
   *workspace_size = e->workspace_bytes;
   *executor = e;
   return ACLNN_SUCCESS;
+}
+
+aclnnStatus aclnnDynamicMxQuant(void* workspace, uint64_t workspace_size, aclOpExecutor* executor, aclrtStream stream) {
+  if (aclnnStatus s = BeginLaunch(executor, OpKind::kMxQuant, workspace, workspace_size, "aclnnDynamicMxQuant")) return s;
+  const mlakvStatus status = mlakvDynamicMxQuant(executor->slots[0].addresses[0], executor->key_row_stride, executor->q_token_stride,
+                                                 executor->tokens, executor->slots[1].addresses[0], executor->value_row_stride,
+                                                 executor->slots[2].addresses[0], executor->key_block_stride, stream);
+  if (status == MLAKV_SUCCESS) executor->launched = true;
+  return status;
 }
 
 aclnnStatus aclnnFusedInferAttentionScoreV5(void* workspace, uint64_t workspace_size, aclOpExecutor* executor, aclrtStream stream) {

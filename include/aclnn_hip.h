@@ -183,6 +183,16 @@ aclnnStatus aclnnFusedInferAttentionScoreV5GetWorkspaceSize(
 aclnnStatus aclnnFusedInferAttentionScoreV5(void* workspace, uint64_t workspace_size, aclOpExecutor* executor,
                                             aclrtStream stream);
 
+/* aclnnDynamicMxQuant, as the reference plans and launches it behind the attention (stage
+ * `attn_quant`, src/pipeline/pipeline.cpp:251-258; contract include/moe/core/op_table.hpp:205-233):
+ * x bf16 [rows, cols] (cols a multiple of 32, dense last axis) -> y E4M3 [rows, cols] and
+ * mxscale E8M0 [rows, cols / 32]; axis -1, round mode "rint" (or null), dst_type 36, blocksize
+ * 32, scale_alg 0 (OCP). IR indices: x 0, y 1, mxscale 2. No workspace. */
+aclnnStatus aclnnDynamicMxQuantGetWorkspaceSize(const aclTensor* x, int64_t axis, char* round_mode_optional, int64_t dst_type,
+                                                int64_t blocksize, int64_t scale_alg, const aclTensor* y_out,
+                                                const aclTensor* mxscale_out, uint64_t* workspace_size, aclOpExecutor** executor);
+aclnnStatus aclnnDynamicMxQuant(void* workspace, uint64_t workspace_size, aclOpExecutor* executor, aclrtStream stream);
+
 /* Block-table gather as a two-phase operator, for callers that want the paged read the
  * reference leaves inside its attention operator (addressing as in third_party/ops_transformer/
  * attention/quant_lightning_indexer/op_kernel/arch35/quant_lightning_indexer_service_cube.h:243-270).

@@ -52,7 +52,11 @@ using FusedInferAttentionScoreV5PlanFn = int (*)(
     const aclTensor*, const aclTensor*, const aclIntArray*, const aclIntArray*, int64_t, double, int64_t, int64_t, char*, int64_t,
     int64_t, int64_t, int64_t, int64_t, bool, int64_t, int64_t, int64_t, int64_t, const aclTensor*, const aclTensor*, uint64_t*,
     aclOpExecutor**);
+using DynamicMxQuantPlanFn = int (*)(const aclTensor*, int64_t, char*, int64_t, int64_t, int64_t, const aclTensor*, const aclTensor*,
+                                     uint64_t*, aclOpExecutor**);  // include/moe/core/op_table.hpp:230-233
 using AclnnLaunchFn = int (*)(void*, uint64_t, aclOpExecutor*, void*);
+static_assert(std::is_same_v<decltype(&aclnnDynamicMxQuantGetWorkspaceSize), DynamicMxQuantPlanFn>);
+static_assert(std::is_same_v<decltype(&aclnnDynamicMxQuant), AclnnLaunchFn>);
 static_assert(std::is_same_v<decltype(&aclnnScatterPaKvCacheGetWorkspaceSize), ScatterPaKvCachePlanFn>);
 static_assert(std::is_same_v<decltype(&aclnnFusedInferAttentionScoreV5GetWorkspaceSize), FusedInferAttentionScoreV5PlanFn>);
 static_assert(std::is_same_v<decltype(&aclnnScatterPaKvCache), AclnnLaunchFn>);
@@ -227,3 +231,34 @@ def test_no_device_fails_loudly_instead_of_falling_back():
     with pytest.raises(ffi.MlakvError) as info:
         ffi.Arena(ffi.BACKEND_HIP)
     assert "no HIP device" in str(info.value)
+
+
+def test_mx_quant_plan_contract():
+    """aclnnDynamicMxQuant plan phase with the attributes the reference passes (src/pipeline/pipeline.cpp:251-258:
+    axis -1, "rint", E4M3, block 32, OCP) and refusals for anything else; no device is touched."""
+    lib = acl.load()
+    keep = acl.Keep()
+    rows, cols = 3, 64 * 512
+    x = keep.tensor([rows, cols], acl.ACL_BF16, None)
+    y = keep.tensor([rows, cols], acl.ACL_FLOAT8_E4M3FN, None)
+    scales = keep.tensor([rows, cols // 32], 37, None)
+
+    def plan(x=x, axis=-1, mode=b"rint", dst=36, block=32, alg=0, y=y, scales=scales):
+        workspace, executor = C.c_uint64(99), C.c_void_p()
+        status = lib.aclnnDynamicMxQuantGetWorkspaceSize(x, axis, mode, dst, block, alg, y, scales, C.byref(workspace), C.byref(executor))
+        return status, workspace.value, executor.value
+
+    status, workspace, executor = plan()
+    assert status == 0 and workspace == 0 and executor
+    assert lib.aclDestroyAclOpExecutor(executor) == 0
+    assert plan(axis=1)[0] == 0 and plan(mode=None)[0] == 0
+    assert plan(axis=0)[0] == ffi.ERR_PARAM_INVALID
+    assert plan(mode=b"round")[0] == ffi.ERR_PARAM_INVALID
+    assert plan(dst=35)[0] == ffi.ERR_PARAM_INVALID
+    assert plan(block=16)[0] == ffi.ERR_PARAM_INVALID
+    assert plan(alg=1)[0] == ffi.ERR_PARAM_INVALID
+    assert plan(x=None)[0] == ffi.ERR_PARAM_NULLPTR
+    assert plan(y=keep.tensor([rows, cols], acl.ACL_BF16, None))[0] == ffi.ERR_PARAM_INVALID
+    assert plan(scales=keep.tensor([rows, cols // 16], 37, None))[0] == ffi.ERR_PARAM_INVALID
+    assert plan(x=keep.tensor([rows, 40], acl.ACL_BF16, None), y=keep.tensor([rows, 40], acl.ACL_FLOAT8_E4M3FN, None))[0] == ffi.ERR_PARAM_INVALID
+    assert "DynamicMxQuant" in acl.last_error()

@@ -140,3 +140,34 @@ def test_fused_entry_argument_checks():
     assert call(C.byref(ffi.MxQuantOut(codes.data_ptr(), heads * LATENT, 256, scales.data_ptr(), heads * 16, 16))) == ffi.ERR_PARAM_INVALID
     assert call(C.byref(ffi.MxQuantOut(codes.data_ptr(), heads * LATENT, LATENT, scales.data_ptr(), heads * 16, 8))) == ffi.ERR_PARAM_INVALID
     torch.cuda.synchronize()
+
+
+def test_two_phase_operator_matches_oracle_and_supports_address_swaps():
+    """aclnnDynamicMxQuant through the plan / launch boundary, as the reference drives stage
+    `attn_quant`: planned once on descriptors, made repeatable, launched with the tensors' addresses
+    and again after aclSetTensorAddr moved the input."""
+    import acl_ffi as acl
+    lib = acl.load()
+    keep = acl.Keep()
+    rows, cols = 5, 64 * 512
+    x = kt.randn_bf16((rows, cols), seed=77, outlier_fraction=0.01).cuda()
+    x2 = kt.randn_bf16((rows, cols), seed=78).cuda()
+    y = torch.zeros(rows, cols, dtype=torch.uint8, device="cuda")
+    scales = torch.zeros(rows, cols // 32, dtype=torch.uint8, device="cuda")
+    tx = keep.tensor([rows, cols], acl.ACL_BF16, x.data_ptr())
+    ty = keep.tensor([rows, cols], acl.ACL_FLOAT8_E4M3FN, y.data_ptr())
+    ts = keep.tensor([rows, cols // 32], 37, scales.data_ptr())
+    workspace, executor = C.c_uint64(1), C.c_void_p()
+    assert lib.aclnnDynamicMxQuantGetWorkspaceSize(tx, -1, b"rint", 36, 32, 0, ty, ts, C.byref(workspace), C.byref(executor)) == 0
+    assert workspace.value == 0
+    assert lib.aclSetAclOpExecutorRepeatable(executor) == 0
+    assert lib.aclnnDynamicMxQuant(None, 0, executor, kt.stream_ptr()) == 0
+    torch.cuda.synchronize()
+    want_codes, want_scales = orc.mx_quant_rows(kt.bits16(x))
+    assert np.array_equal(y.cpu().numpy(), want_codes) and np.array_equal(scales.cpu().numpy(), want_scales)
+    assert lib.aclSetTensorAddr(executor, 0, tx, x2.data_ptr()) == 0
+    assert lib.aclnnDynamicMxQuant(None, 0, executor, kt.stream_ptr()) == 0
+    torch.cuda.synchronize()
+    want_codes, want_scales = orc.mx_quant_rows(kt.bits16(x2))
+    assert np.array_equal(y.cpu().numpy(), want_codes) and np.array_equal(scales.cpu().numpy(), want_scales)
+    assert lib.aclDestroyAclOpExecutor(executor) == 0
