@@ -393,6 +393,25 @@ mlakvStatus AttnDecodeImpl(const char* who, const mlakvAttnPlan* plan, const mla
                 plan->dtype, plan->block_size, cache->dtype, cache->block_size);
   }
   if (!(scale > 0.0) || !std::isfinite(scale)) return Fail(MLAKV_ERR_PARAM_INVALID, "%s: a positive softmax scale is required", who);
+  // The kernels size their LDS staging and their grid from the plan: a plan that was not made by
+  // the init functions (or was altered since) is refused here instead of faulting there.
+  {
+    const int64_t max_tiles = (static_cast<int64_t>(plan->max_seq_len) + mlakv::kTileTokens - 1) / mlakv::kTileTokens;
+    const bool sane = plan->batch > 0 && plan->batch <= 65535 && plan->heads > 0 && plan->heads % 16 == 0 && plan->heads <= 128 &&
+                      plan->max_seq_len > 0 && plan->chunk_tiles >= 1 && plan->chunk_tiles <= max_tiles &&
+                      plan->max_chunks == (max_tiles + plan->chunk_tiles - 1) / plan->chunk_tiles &&
+                      (plan->reserved == 0 || plan->reserved == 1) &&
+                      (plan->reserved == 1
+                           ? plan->chunk_tiles * mlakv::kTileTokens <= 1024 && plan->max_seq_len <= 2048
+                           : (static_cast<int64_t>(plan->chunk_tiles) * mlakv::kTileTokens + plan->block_size - 1) / plan->block_size + 1 <= 1024 ||
+                                 plan->chunk_tiles == 1);
+    const uint64_t rows = static_cast<uint64_t>(plan->batch > 0 ? plan->batch : 0) * (plan->max_chunks > 0 ? plan->max_chunks : 0) *
+                          (plan->heads > 0 ? plan->heads : 0);
+    const uint64_t expected = plan->max_chunks > 1 ? rows * mlakv::kLatentDim * 2 + ((rows * sizeof(float) + 255) & ~255ull) : 0;
+    if (!sane || plan->workspace_bytes != expected) {
+      return Fail(MLAKV_ERR_PARAM_INVALID, "%s: the plan is not one made by mlakvAttnPlanInit / mlakvAttnSparsePlanInit", who);
+    }
+  }
   const bool sparse = sparse_indices != nullptr;
   if (sparse != (plan->reserved == 1)) {
     return Fail(MLAKV_ERR_PARAM_INVALID, "%s: the plan was made by %s", who,

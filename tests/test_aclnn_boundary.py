@@ -224,6 +224,25 @@ def test_thin_abi_argument_validation_without_a_device():
     fp8 = ffi.CacheView.from_buffer_copy(view)
     fp8.dtype = ffi.DTYPE_FP8_E4M3
     assert lib.mlakvCopyBlocks(C.byref(fp8), 0, 1, FAKE, 1, None) == ffi.ERR_PARAM_NULLPTR  # FP8 without a scale plane
+    # a plan altered after its init call is refused at launch (the kernels size LDS staging from it)
+    assert lib.mlakvAttnPlanInit(32, 64, 2048, 64, ffi.DTYPE_BF16, C.byref(plan)) == 0
+    row = 1152
+
+    def decode(p):
+        return lib.mlakvAttnDecode(C.byref(p), C.byref(view), 0, FAKE, 64 * row, row, FAKE + 1024, 64 * row, row, FAKE, 32, FAKE,
+                                   0.07, FAKE, 64 * 1024, 1024, None, None, 0, None)
+
+    assert decode(plan) == ffi.ERR_PARAM_NULLPTR          # everything fine up to the missing workspace
+    for field, value in (("chunk_tiles", 4096), ("chunk_tiles", 0), ("max_chunks", 9), ("heads", 60), ("workspace_bytes", 16),
+                         ("reserved", 2), ("batch", 0)):
+        altered = ffi.AttnPlan.from_buffer_copy(plan)
+        setattr(altered, field, value)
+        assert decode(altered) == ffi.ERR_PARAM_INVALID, field
+        assert "not one made by" in ffi.last_error()
+    sparse = ffi.AttnPlan()
+    assert lib.mlakvAttnSparsePlanInit(32, 64, 512, 64, ffi.DTYPE_BF16, C.byref(sparse)) == 0
+    assert sparse.reserved == 1 and sparse.max_seq_len == 512 and sparse.chunk_tiles * 32 <= 1024
+    assert decode(sparse) == ffi.ERR_PARAM_INVALID        # a selection plan handed to the whole-context entry
 
 
 @pytest.mark.skipif(ffi.load().mlakvDeviceCount() > 0, reason="checks the no-device behaviour")
