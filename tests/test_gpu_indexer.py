@@ -176,3 +176,57 @@ def test_argument_checks():
     assert call(view=ffi.IndexKeyView(keys.data_ptr(), 64 * D, D, scales.data_ptr(), 64, 4, 64, 64, 0)) == ffi.ERR_PARAM_INVALID
     assert call(max_len=64, ws=None, ws_bytes=0) == 0          # nothing longer than k: no scores, no workspace
     torch.cuda.synchronize()
+
+
+def test_full_size_indexer_and_selected_attention_on_sampled_sequences():
+    """The shape the bench times (batch 32, context 8192, 64 index heads, top-512, block 64): the
+    indexer's keys and selection for three sampled sequences against the oracle, every sequence's
+    list checked for being 512 distinct in-range positions, then the selected-token attention over
+    those lists against the oracle for the same three sequences."""
+    import math
+    bs, heads, k, batch, ctx = 64, 64, 512, 32, 8192
+    blocks = batch * (ctx // bs) + 7
+    rng = np.random.default_rng(120)
+    pool = kt.build_tables([ctx] * batch, bs, blocks, seed=121)
+    table = pool.table()
+    key_plane = _codes(rng, (blocks * bs, D), 0x58)
+    key_scale = rng.uniform(0.01, 0.05, blocks * bs).astype(np.float32)
+    query = _codes(rng, (batch, heads, D), 0x58)
+    weights = kt.randn_bf16((batch, heads), seed=122)
+    q_scale = rng.uniform(0.01, 0.05, (batch, heads)).astype(np.float32)
+    lib = ffi.load()
+    keys_d, scales_d = torch.as_tensor(key_plane, device="cuda"), torch.as_tensor(key_scale, device="cuda")
+    view = ffi.IndexKeyView(keys_d.data_ptr(), bs * D, D, scales_d.data_ptr(), bs, blocks, bs, D, 0)
+    query_d, weights_d, q_scale_d = torch.as_tensor(query, device="cuda"), weights.cuda(), torch.as_tensor(q_scale, device="cuda")
+    table_d, lens_d = kt.dev_i32(table), kt.dev_i32([ctx] * batch)
+    selection = torch.full((batch, k), -7, dtype=torch.int32, device="cuda")
+    workspace = torch.zeros(int(lib.mlakvIndexerWorkspaceBytes(batch, ctx)), dtype=torch.uint8, device="cuda")
+    ffi.check(lib.mlakvLightningIndexer(C.byref(view), query_d.data_ptr(), heads * D, D, weights_d.data_ptr(), heads * 2,
+                                        q_scale_d.data_ptr(), heads, heads, table_d.data_ptr(), table.shape[1], lens_d.data_ptr(),
+                                        batch, ctx, k, selection.data_ptr(), k, workspace.data_ptr(), workspace.numel(),
+                                        kt.stream_ptr()))
+    torch.cuda.synchronize()
+    chosen = selection.cpu().numpy()
+    assert ((chosen >= 0) & (chosen < ctx)).all()
+    assert all(len(set(row.tolist())) == k for row in chosen)
+    gpu_keys = workspace.view(torch.int16).cpu().numpy().view(np.uint16).reshape(batch, ctx)
+    sample = (0, 13, 31)
+    for b in sample:
+        want_keys = orc.indexer_scores(query[b], kt.bits16(weights[b]), q_scale[b], key_plane, key_scale, bs, table[b], ctx)
+        assert (gpu_keys[b] != want_keys).mean() <= 0.005
+        assert chosen[b].tolist() == orc.indexer_topk(gpu_keys[b], k).tolist()
+    # the MLA cache behind the same table, filled on the device; attention over the selected lists
+    cache = kt.PagedCache(1, blocks, bs)
+    cache.latent.copy_(torch.randn(cache.latent.shape, device="cuda", generator=torch.Generator(device="cuda").manual_seed(123)).to(torch.bfloat16))
+    cache.rope.copy_(torch.randn(cache.rope.shape, device="cuda", generator=torch.Generator(device="cuda").manual_seed(124)).to(torch.bfloat16))
+    q = kt.randn_bf16((batch, 64, kt.LATENT + kt.ROPE), seed=125).cuda()
+    scale = 1.0 / math.sqrt(192.0)
+    out, lse, plan = kt.sparse_attention(cache, 0, q, table_d, lens_d, selection, scale)
+    assert plan.max_chunks * batch >= 128
+    got = out.float().cpu().numpy()
+    assert np.isfinite(got).all()
+    for b in sample:
+        expected, expected_lse = kt.oracle_attention(cache, 0, q[b:b + 1], table[b:b + 1], [ctx], scale, sparse_indices=chosen[b:b + 1])
+        peak = np.abs(expected).max()
+        assert np.abs(got[b] - expected[0]).max() <= 2e-2 * peak
+        assert np.abs(lse[b].cpu().numpy() - expected_lse[0]).max() <= 2e-2
