@@ -166,7 +166,8 @@ def bench_attention(args, torch, np, ffi, fp8=False, batch=32, ctx=2048, heads=6
     pool_blocks = batch * blocks_per_seq + 8
     arena = ffi.Arena(ffi.BACKEND_HIP)
     cache = ffi.KvCache(arena, num_layers=slices, block_size=bs, max_context_len=ctx, max_batch=batch,
-                        pool_blocks=pool_blocks, seed=7, shuffle=1, dtype=ffi.DTYPE_FP8_E4M3 if fp8 else ffi.DTYPE_BF16)
+                        pool_blocks=pool_blocks, seed=7, shuffle=int(os.environ.get("MLAKV_BENCH_SHUFFLE", "1")),
+                        dtype=ffi.DTYPE_FP8_E4M3 if fp8 else ffi.DTYPE_BF16)
     plan = ffi.AttnPlan()
     if sparse_k:
         ffi.check(lib.mlakvAttnSparsePlanInit(batch, heads, sparse_k, bs, cache.config.dtype, C.byref(plan)))
