@@ -97,28 +97,53 @@ __device__ __forceinline__ u32x4 Dequant8(u32x2 codes, float scale) {
 
 // ---- append -----------------------------------------------------------------
 
-// One wavefront per (token, layer). bf16: 64 lanes move the latent row, 8 lanes the rope row.
+// One wavefront per (four consecutive tokens, layer). bf16: 64 lanes move a latent row, 8 lanes a
+// rope row. The source rows do not depend on the slots, so all of a wavefront's loads (slots and
+// rows) are issued together: with one row per wavefront and the row fetched only after its slot
+// had arrived, a prefill-sized append was bound by two memory latencies per 1152 bytes.
+constexpr int kAppendRows = 4;
+
 __global__ __launch_bounds__(kThreads) void AppendBf16Kernel(AppendArgs a) {
   const int lane = threadIdx.x & (kWave - 1);
-  const int token = blockIdx.x * kWavesPerGroup + (threadIdx.x >> 6);
+  const int token0 = Uniform((blockIdx.x * kWavesPerGroup + (threadIdx.x >> 6)) * kAppendRows);
   const int layer = blockIdx.y;
-  if (token >= a.num_tokens) return;
-  const int slot = Uniform(a.slots[token]);
-  if (slot < 0) return;
-  const int block = slot / a.block_size;
-  const int in_block = slot - block * a.block_size;
-  if (block >= a.num_blocks) return;
-  const char* latent_src = a.latent_src.base + layer * a.latent_src.layer_stride + token * a.latent_src.row_stride;
-  const char* rope_src = a.rope_src.base + layer * a.rope_src.layer_stride + token * a.rope_src.row_stride;
-  char* latent_dst = a.latent.base + layer * a.latent.layer_stride + block * a.latent.block_stride +
-                     in_block * a.latent.row_stride;
-  char* rope_dst = a.rope.base + layer * a.rope.layer_stride + block * a.rope.block_stride + in_block * a.rope.row_stride;
+  if (token0 >= a.num_tokens) return;
+  int my_slot = -1;
+  if (lane < kAppendRows && token0 + lane < a.num_tokens) my_slot = a.slots[token0 + lane];
   static_assert(kLatentDim * 2 / 16 == kWave, "one latent row is one wave access");
-  const u32x4 v = Load16(latent_src + lane * 16);
-  u32x4 r;
-  if (lane < kRopeDim * 2 / 16) r = Load16(rope_src + lane * 16);
-  Store16(latent_dst + lane * 16, v);
-  if (lane < kRopeDim * 2 / 16) Store16(rope_dst + lane * 16, r);
+  const bool rope_lane = lane < kRopeDim * 2 / 16;
+  const char* latent_src = a.latent_src.base + layer * a.latent_src.layer_stride;
+  const char* rope_src = a.rope_src.base + layer * a.rope_src.layer_stride;
+  u32x4 v[kAppendRows], r[kAppendRows];
+  // a row past the end repeats the last one: loaded, never stored (its slot lane holds -1)
+#pragma unroll
+  for (int i = 0; i < kAppendRows; ++i) v[i] = Load16(latent_src + min(token0 + i, a.num_tokens - 1) * a.latent_src.row_stride + lane * 16);
+  if (rope_lane) {  // one branch around all rope loads: a branch per row made the compiler wait between the rows
+#pragma unroll
+    for (int i = 0; i < kAppendRows; ++i) r[i] = Load16(rope_src + min(token0 + i, a.num_tokens - 1) * a.rope_src.row_stride + lane * 16);
+  }
+  char* latent_dst[kAppendRows];
+  char* rope_dst[kAppendRows];
+  bool live[kAppendRows];
+#pragma unroll
+  for (int i = 0; i < kAppendRows; ++i) {
+    const int slot = __builtin_amdgcn_readlane(my_slot, i);
+    const int block = slot < 0 ? 0 : slot / a.block_size;
+    const int in_block = slot < 0 ? 0 : slot - block * a.block_size;
+    live[i] = slot >= 0 && block < a.num_blocks;
+    latent_dst[i] = a.latent.base + layer * a.latent.layer_stride + block * a.latent.block_stride + in_block * a.latent.row_stride;
+    rope_dst[i] = a.rope.base + layer * a.rope.layer_stride + block * a.rope.block_stride + in_block * a.rope.row_stride;
+  }
+#pragma unroll
+  for (int i = 0; i < kAppendRows; ++i) {
+    if (live[i]) Store16(latent_dst[i] + lane * 16, v[i]);
+  }
+  if (rope_lane) {
+#pragma unroll
+    for (int i = 0; i < kAppendRows; ++i) {
+      if (live[i]) Store16(rope_dst[i] + lane * 16, r[i]);
+    }
+  }
 }
 
 // Two quotients -> two E4M3 codes in the low half of a dword. v_cvt_pk_fp8_f32 rounds to nearest
@@ -142,10 +167,36 @@ __device__ __forceinline__ void QuantizeRowAndStore(const AppendArgs& a, int lay
 #pragma unroll
   for (int offset = 32; offset >= 1; offset >>= 1) absmax = fmaxf(absmax, __shfl_xor(absmax, offset));
   const float scale = absmax == 0.0f ? 1.0f : absmax / 448.0f;
+  // code = e4m3(x / scale) with the correctly rounded fp32 quotient. Nine divisions per lane made
+  // this kernel compute-bound, so the quotient is first taken as x * (1 / scale), which is within
+  // 2^-22 relative of the rounded quotient; the encoding is monotone, so if the two ends of that
+  // interval (widened to 2^-21) encode alike, so does the exact quotient. Only a lane that holds
+  // a value this close to a rounding boundary of the E4M3 grid (about one in 10^5 values) divides.
+  const float inverse = 1.0f / scale;
+  float q[9];
+#pragma unroll
+  for (int i = 0; i < 8; ++i) q[i] = fminf(fmaxf(x[i] * inverse, -448.0f), 448.0f);
+  q[8] = fminf(fmaxf(y * inverse, -448.0f), 448.0f);
+  constexpr float kWiden = 4.76837158203125e-07f;  // 2^-21
+  unsigned below[5], above[5];
+#pragma unroll
+  for (int i = 0; i < 5; ++i) {
+    const float a = q[2 * i], b = i < 4 ? q[2 * i + 1] : 0.0f;
+    below[i] = static_cast<unsigned>(__builtin_amdgcn_cvt_pk_fp8_f32(__builtin_fmaf(a, -kWiden, a), __builtin_fmaf(b, -kWiden, b), 0, false)) & 0xffffu;
+    above[i] = static_cast<unsigned>(__builtin_amdgcn_cvt_pk_fp8_f32(__builtin_fmaf(a, kWiden, a), __builtin_fmaf(b, kWiden, b), 0, false)) & 0xffffu;
+  }
+  const bool settled = below[0] == above[0] && below[1] == above[1] && below[2] == above[2] && below[3] == above[3] && below[4] == above[4];
   u32x2 lq;
-  lq.x = E4m3EncodePair(x[0] / scale, x[1] / scale) | (E4m3EncodePair(x[2] / scale, x[3] / scale) << 16);
-  lq.y = E4m3EncodePair(x[4] / scale, x[5] / scale) | (E4m3EncodePair(x[6] / scale, x[7] / scale) << 16);
-  const unsigned int rq = E4m3EncodePair(y / scale, 0.0f) & 0xffu;
+  unsigned int rq;
+  if (settled) {
+    lq.x = below[0] | (below[1] << 16);
+    lq.y = below[2] | (below[3] << 16);
+    rq = below[4] & 0xffu;
+  } else {
+    lq.x = E4m3EncodePair(x[0] / scale, x[1] / scale) | (E4m3EncodePair(x[2] / scale, x[3] / scale) << 16);
+    lq.y = E4m3EncodePair(x[4] / scale, x[5] / scale) | (E4m3EncodePair(x[6] / scale, x[7] / scale) << 16);
+    rq = E4m3EncodePair(y / scale, 0.0f) & 0xffu;
+  }
   char* latent_dst = a.latent.base + layer * a.latent.layer_stride + block * a.latent.block_stride +
                      in_block * a.latent.row_stride;
   char* rope_dst = a.rope.base + layer * a.rope.layer_stride + block * a.rope.block_stride + in_block * a.rope.row_stride;
@@ -163,25 +214,34 @@ __device__ __forceinline__ void QuantizeRowAndStore(const AppendArgs& a, int lay
 __global__ __launch_bounds__(kThreads) void AppendFp8Kernel(AppendArgs a) {
   static_assert(kRopeDim == kWave, "one rope element per lane");
   const int lane = threadIdx.x & (kWave - 1);
-  const int token = blockIdx.x * kWavesPerGroup + (threadIdx.x >> 6);
+  const int token0 = Uniform((blockIdx.x * kWavesPerGroup + (threadIdx.x >> 6)) * kAppendRows);
   const int layer = blockIdx.y;
-  if (token >= a.num_tokens) return;
-  const int slot = Uniform(a.slots[token]);
-  if (slot < 0) return;
-  const int block = slot / a.block_size;
-  const int in_block = slot - block * a.block_size;
-  if (block >= a.num_blocks) return;
-  const char* latent_src = a.latent_src.base + layer * a.latent_src.layer_stride + token * a.latent_src.row_stride;
-  const char* rope_src = a.rope_src.base + layer * a.rope_src.layer_stride + token * a.rope_src.row_stride;
-  const u32x4 lv = Load16(latent_src + lane * 16);
-  const float y = Bf16ToF32(*reinterpret_cast<const unsigned short*>(rope_src + lane * 2));
-  float x[8];
+  if (token0 >= a.num_tokens) return;
+  int my_slot = -1;
+  if (lane < kAppendRows && token0 + lane < a.num_tokens) my_slot = a.slots[token0 + lane];
+  u32x4 lv[kAppendRows];
+  unsigned short rv[kAppendRows];
 #pragma unroll
-  for (int i = 0; i < 4; ++i) {
-    x[2 * i] = Bf16ToF32(lv[i] & 0xffffu);
-    x[2 * i + 1] = Bf16ToF32(lv[i] >> 16);
+  for (int i = 0; i < kAppendRows; ++i) {
+    const int token = min(token0 + i, a.num_tokens - 1);  // a repeated row is loaded and never stored
+    lv[i] = Load16(a.latent_src.base + layer * a.latent_src.layer_stride + token * a.latent_src.row_stride + lane * 16);
+    rv[i] = *reinterpret_cast<const unsigned short*>(a.rope_src.base + layer * a.rope_src.layer_stride + token * a.rope_src.row_stride + lane * 2);
   }
-  QuantizeRowAndStore(a, layer, block, in_block, lane, x, y);
+#pragma unroll
+  for (int i = 0; i < kAppendRows; ++i) {
+    const int slot = __builtin_amdgcn_readlane(my_slot, i);
+    if (slot < 0) continue;
+    const int block = slot / a.block_size;
+    const int in_block = slot - block * a.block_size;
+    if (block >= a.num_blocks) continue;
+    float x[8];
+#pragma unroll
+    for (int j = 0; j < 4; ++j) {
+      x[2 * j] = Bf16ToF32(lv[i][j] & 0xffffu);
+      x[2 * j + 1] = Bf16ToF32(lv[i][j] >> 16);
+    }
+    QuantizeRowAndStore(a, layer, block, in_block, lane, x, Bf16ToF32(rv[i]));
+  }
 }
 
 // ---- latent RMSNorm + key RoPE + append ---------------------------------------------------
@@ -470,7 +530,7 @@ int DivUp(int a, int b) { return (a + b - 1) / b; }
 
 hipError_t LaunchAppend(const AppendArgs& args, hipStream_t stream) {
   if (args.num_tokens <= 0 || args.num_layers <= 0) return hipSuccess;
-  const dim3 grid(DivUp(args.num_tokens, kWavesPerGroup), args.num_layers);
+  const dim3 grid(DivUp(args.num_tokens, kWavesPerGroup * kAppendRows), args.num_layers);
   if (args.fp8) {
     hipLaunchKernelGGL(AppendFp8Kernel, grid, dim3(kThreads), 0, stream, args);
   } else {
