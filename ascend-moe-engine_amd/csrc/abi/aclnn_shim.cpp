@@ -80,7 +80,7 @@ struct aclScalar { void* value = nullptr; aclDataType dtype = ACL_DT_UNDEFINED; 
 
 namespace {
 
-enum class OpKind { kScatter, kAttention, kGather, kMxQuant };
+enum class OpKind { kScatter, kAttention, kGather, kMxQuant, kIndexer };
 enum class SlotKind { kNull, kTensor, kList, kIntArray };
 
 struct Slot {
@@ -134,6 +134,8 @@ struct aclOpExecutor {
   double scale = 0.0;
   bool want_lse = false;
   mlakvAttnPlan plan{};
+  int64_t aux_stride[4] = {0, 0, 0, 0};  // indexer: weights / query scale / key scale block / output strides
+  int32_t sparse_count = 0;
   uint64_t workspace_bytes = 0;
   uint64_t lens_offset = 0;  // attention: where the int32 lengths live inside the workspace
   const aclIntArray* host_lens = nullptr;
@@ -696,6 +698,91 @@ aclnnStatus aclnnDynamicMxQuantGetWorkspaceSize(const aclTensor* x, int64_t axis
   return ACLNN_SUCCESS;
 }
 
+// ---- aclnnQuantLightningIndexer ---------------------------------------------------------------
+
+aclnnStatus aclnnQuantLightningIndexerGetWorkspaceSize(const aclTensor* query, const aclTensor* key, const aclTensor* weights,
+                                                       const aclTensor* query_dequant_scale, const aclTensor* key_dequant_scale,
+                                                       const aclTensor* actual_seq_lengths_query_optional,
+                                                       const aclTensor* actual_seq_lengths_key_optional,
+                                                       const aclTensor* block_table_optional, int64_t query_quant_mode,
+                                                       int64_t key_quant_mode, char* layout_query_optional,
+                                                       char* layout_key_optional, int64_t sparse_count, int64_t sparse_mode,
+                                                       int64_t pre_tokens, int64_t next_tokens, const aclTensor* out,
+                                                       uint64_t* workspace_size, aclOpExecutor** executor) {
+  const char* who = "QuantLightningIndexer";
+  SHIM_REQUIRE(workspace_size && executor, ACLNN_ERR_PARAM_NULLPTR, "%s: null workspace_size / executor output", who);
+  *executor = nullptr;
+  SHIM_REQUIRE(query && key && weights && query_dequant_scale && key_dequant_scale && out, ACLNN_ERR_PARAM_NULLPTR,
+               "%s: query, key, weights, both dequant scales and out are required", who);
+  SHIM_REQUIRE(actual_seq_lengths_key_optional && block_table_optional, ACLNN_ERR_PARAM_NULLPTR,
+               "%s: the paged key layout needs actual_seq_lengths_key and block_table", who);
+  SHIM_REQUIRE(AsTensor(query) && AsTensor(key) && AsTensor(weights) && AsTensor(query_dequant_scale) && AsTensor(key_dequant_scale) &&
+                   AsTensor(actual_seq_lengths_key_optional) && AsTensor(block_table_optional) && AsTensor(out) &&
+                   (actual_seq_lengths_query_optional == nullptr || AsTensor(actual_seq_lengths_query_optional)),
+               ACLNN_ERR_PARAM_INVALID, "%s: bad tensor handle", who);
+  SHIM_REQUIRE(query_quant_mode == 0 && key_quant_mode == 0, ACLNN_ERR_PARAM_INVALID, "%s: only per-token-head quantization (mode 0) is served", who);
+  SHIM_REQUIRE(layout_query_optional == nullptr || std::strcmp(layout_query_optional, "BSND") == 0, ACLNN_ERR_PARAM_INVALID,
+               "%s: query layout '%s' is not served; decode uses \"BSND\"", who, layout_query_optional);
+  SHIM_REQUIRE(layout_key_optional != nullptr && std::strcmp(layout_key_optional, "PA_BSND") == 0, ACLNN_ERR_PARAM_INVALID,
+               "%s: only the paged key layout \"PA_BSND\" is served", who);
+  SHIM_REQUIRE(sparse_count >= 1 && sparse_count <= 2048, ACLNN_ERR_PARAM_INVALID, "%s: sparse_count %lld outside [1, 2048]", who,
+               static_cast<long long>(sparse_count));
+  SHIM_REQUIRE(sparse_mode == 0 || sparse_mode == 3, ACLNN_ERR_PARAM_INVALID, "%s: sparse_mode %lld is not one of 0, 3", who,
+               static_cast<long long>(sparse_mode));
+  SHIM_REQUIRE(pre_tokens == INT64_MAX && next_tokens == INT64_MAX, ACLNN_ERR_PARAM_INVALID, "%s: only the unrestricted window is served", who);
+  SHIM_REQUIRE(query->dtype == ACL_FLOAT8_E4M3FN && key->dtype == ACL_FLOAT8_E4M3FN, ACLNN_ERR_PARAM_INVALID, "%s: E4M3 query and key expected", who);
+  SHIM_REQUIRE(weights->dtype == ACL_BF16 && query_dequant_scale->dtype == ACL_FLOAT32 && key_dequant_scale->dtype == ACL_FLOAT32,
+               ACLNN_ERR_PARAM_INVALID, "%s: BF16 weights and FP32 dequant scales expected", who);
+  SHIM_REQUIRE(block_table_optional->dtype == ACL_INT32 && actual_seq_lengths_key_optional->dtype == ACL_INT32 && out->dtype == ACL_INT32,
+               ACLNN_ERR_PARAM_INVALID, "%s: block table, key lengths and out must be INT32", who);
+  // query [B, 1, N1, 128]: one decode token per sequence
+  SHIM_REQUIRE(query->dims.size() == 4 && query->dims[1] == 1 && query->dims[3] == 128 && query->strides[3] == 1, ACLNN_ERR_PARAM_INVALID,
+               "%s: query must be [B, 1, N1, 128] (one decode token per sequence)", who);
+  const int64_t batch = query->dims[0], heads = query->dims[2];
+  SHIM_REQUIRE(batch > 0 && batch <= 65535 && (heads == 16 || heads == 32 || heads == 48 || heads == 64), ACLNN_ERR_PARAM_INVALID,
+               "%s: N1 = %lld is not one of 16, 32, 48, 64", who, static_cast<long long>(heads));
+  int64_t blocks = 0, bs = 0, kb = 0, ks = 0;
+  SHIM_REQUIRE(PagedCacheShape(key, 128, &blocks, &bs, &kb, &ks), ACLNN_ERR_PARAM_INVALID, "%s: key must be paged [blocks, block, 1, 128]", who);
+  SHIM_REQUIRE(weights->dims.size() == 3 && weights->dims[0] == batch && weights->dims[1] == 1 && weights->dims[2] == heads && weights->strides[2] == 1 &&
+                   query_dequant_scale->dims.size() == 3 && query_dequant_scale->dims[0] == batch && query_dequant_scale->dims[2] == heads &&
+                   query_dequant_scale->strides[2] == 1,
+               ACLNN_ERR_PARAM_INVALID, "%s: weights and query_dequant_scale must be [B, 1, N1]", who);
+  SHIM_REQUIRE(key_dequant_scale->dims.size() == 3 && key_dequant_scale->dims[0] == blocks && key_dequant_scale->dims[1] == bs &&
+                   key_dequant_scale->dims[2] == 1 && key_dequant_scale->strides[1] == 1,
+               ACLNN_ERR_PARAM_INVALID, "%s: key_dequant_scale must be [blocks, block, 1] with dense slots", who);
+  SHIM_REQUIRE(block_table_optional->dims.size() == 2 && block_table_optional->dims[0] == batch && block_table_optional->contiguous() &&
+                   actual_seq_lengths_key_optional->numel() == batch && actual_seq_lengths_key_optional->contiguous(),
+               ACLNN_ERR_PARAM_INVALID, "%s: block table [B, W] and key lengths [B] must be dense", who);
+  SHIM_REQUIRE(out->dims.size() == 4 && out->dims[0] == batch && out->dims[1] == 1 && out->dims[2] == 1 && out->dims[3] == sparse_count &&
+                   out->strides[3] == 1,
+               ACLNN_ERR_PARAM_INVALID, "%s: out must be [B, 1, 1, sparse_count]", who);
+  const int64_t width = block_table_optional->dims[1];
+  SHIM_REQUIRE(width * bs <= INT32_MAX && blocks <= INT32_MAX, ACLNN_ERR_PARAM_INVALID, "%s: sizes overflow INT32", who);
+  aclOpExecutor* e = NewExecutor(OpKind::kIndexer, {TensorSlot(query), TensorSlot(key), TensorSlot(weights), TensorSlot(query_dequant_scale),
+                                                    TensorSlot(key_dequant_scale), TensorSlot(actual_seq_lengths_query_optional),
+                                                    TensorSlot(actual_seq_lengths_key_optional), TensorSlot(block_table_optional),
+                                                    TensorSlot(out)});
+  e->batch = static_cast<int32_t>(batch);
+  e->heads = static_cast<int32_t>(heads);
+  e->num_blocks = static_cast<int32_t>(blocks);
+  e->block_size = static_cast<int32_t>(bs);
+  e->table_width = static_cast<int32_t>(width);
+  e->max_seq_len = static_cast<int32_t>(width * bs);  // every length the table can address
+  e->sparse_count = static_cast<int32_t>(sparse_count);
+  e->key_block_stride = kb;
+  e->key_slot_stride = ks;
+  e->q_token_stride = query->strides[0];
+  e->q_head_stride = query->strides[2];
+  e->aux_stride[0] = weights->strides[0] * 2;
+  e->aux_stride[1] = query_dequant_scale->strides[0];
+  e->aux_stride[2] = key_dequant_scale->strides[0];
+  e->aux_stride[3] = out->strides[0];
+  e->workspace_bytes = mlakvIndexerWorkspaceBytes(e->batch, e->max_seq_len);
+  *workspace_size = e->workspace_bytes;
+  *executor = e;
+  return ACLNN_SUCCESS;
+}
+
 // ---- aclnnFusedInferAttentionScoreV5 ------------------------------------------------------------
 
 aclnnStatus aclnnFusedInferAttentionScoreV5GetWorkspaceSize(
@@ -818,6 +905,27 @@ aclnnStatus aclnnFusedInferAttentionScoreV5GetWorkspaceSize(
   *workspace_size = e->workspace_bytes;
   *executor = e;
   return ACLNN_SUCCESS;
+}
+
+aclnnStatus aclnnQuantLightningIndexer(void* workspace, uint64_t workspace_size, aclOpExecutor* executor, aclrtStream stream) {
+  if (aclnnStatus s = BeginLaunch(executor, OpKind::kIndexer, workspace, workspace_size, "aclnnQuantLightningIndexer")) return s;
+  aclOpExecutor* e = executor;
+  mlakvIndexKeyView keys{};
+  keys.keys = e->slots[1].addresses[0];
+  keys.block_stride = e->key_block_stride;
+  keys.row_stride = e->key_slot_stride;
+  keys.scales = static_cast<const float*>(e->slots[4].addresses[0]);
+  keys.scale_block_stride = e->aux_stride[2];
+  keys.num_blocks = e->num_blocks;
+  keys.block_size = e->block_size;
+  keys.dim = 128;
+  const mlakvStatus status = mlakvLightningIndexer(
+      &keys, e->slots[0].addresses[0], e->q_token_stride, e->q_head_stride, e->slots[2].addresses[0], e->aux_stride[0],
+      static_cast<const float*>(e->slots[3].addresses[0]), e->aux_stride[1], e->heads, static_cast<const int32_t*>(e->slots[7].addresses[0]),
+      e->table_width, static_cast<const int32_t*>(e->slots[6].addresses[0]), e->batch, e->max_seq_len, e->sparse_count,
+      static_cast<int32_t*>(e->slots[8].addresses[0]), e->aux_stride[3], workspace, workspace_size, stream);
+  if (status == MLAKV_SUCCESS) e->launched = true;
+  return status;
 }
 
 aclnnStatus aclnnDynamicMxQuant(void* workspace, uint64_t workspace_size, aclOpExecutor* executor, aclrtStream stream) {

@@ -193,6 +193,27 @@ aclnnStatus aclnnDynamicMxQuantGetWorkspaceSize(const aclTensor* x, int64_t axis
                                                 const aclTensor* mxscale_out, uint64_t* workspace_size, aclOpExecutor** executor);
 aclnnStatus aclnnDynamicMxQuant(void* workspace, uint64_t workspace_size, aclOpExecutor* executor, aclrtStream stream);
 
+/* aclnnQuantLightningIndexer for decode (contract include/moe/core/op_table.hpp:964-1006; the
+ * reference's op table requires the symbol, src/core/op_table.cpp:87-88): query E4M3
+ * [B, 1, N1, 128] with N1 in {16, 32, 48, 64}; key E4M3 paged [blocks, block, 1, 128] (layout
+ * "PA_BSND"); weights BF16 [B, 1, N1]; query_dequant_scale FP32 [B, 1, N1]; key_dequant_scale FP32
+ * [blocks, block, 1]; actual_seq_lengths_key INT32 [B] and block_table INT32 [B, W] (device
+ * tensors, both required); quant modes 0; layout_query "BSND" or null; sparse_count in [1, 2048];
+ * sparse_mode 0 or 3 (the same thing for one query token); pre/next tokens INT64_MAX; out INT32
+ * [B, 1, 1, sparse_count]. IR indices: query 0, key 1, weights 2, query_dequant_scale 3,
+ * key_dequant_scale 4, actual_seq_lengths_query 5, actual_seq_lengths_key 6, block_table 7,
+ * out 8. The workspace holds the 16-bit scores of W * block tokens per sequence. */
+aclnnStatus aclnnQuantLightningIndexerGetWorkspaceSize(const aclTensor* query, const aclTensor* key, const aclTensor* weights,
+                                                       const aclTensor* query_dequant_scale, const aclTensor* key_dequant_scale,
+                                                       const aclTensor* actual_seq_lengths_query_optional,
+                                                       const aclTensor* actual_seq_lengths_key_optional,
+                                                       const aclTensor* block_table_optional, int64_t query_quant_mode,
+                                                       int64_t key_quant_mode, char* layout_query_optional,
+                                                       char* layout_key_optional, int64_t sparse_count, int64_t sparse_mode,
+                                                       int64_t pre_tokens, int64_t next_tokens, const aclTensor* out,
+                                                       uint64_t* workspace_size, aclOpExecutor** executor);
+aclnnStatus aclnnQuantLightningIndexer(void* workspace, uint64_t workspace_size, aclOpExecutor* executor, aclrtStream stream);
+
 /* Block-table gather as a two-phase operator, for callers that want the paged read the
  * reference leaves inside its attention operator (addressing as in third_party/ops_transformer/
  * attention/quant_lightning_indexer/op_kernel/arch35/quant_lightning_indexer_service_cube.h:243-270).

@@ -46,6 +46,9 @@ PROTOTYPES = {
     "aclnnMlaKvBindSeqLens": (_i32, [_vp, _vp]),
     "aclnnDynamicMxQuantGetWorkspaceSize": (_i32, [_vp, _i64, C.c_char_p, _i64, _i64, _i64, _vp, _vp, _P(_u64), _P(_vp)]),
     "aclnnDynamicMxQuant": (_i32, [_vp, _u64, _vp, _vp]),
+    "aclnnQuantLightningIndexerGetWorkspaceSize": (_i32, [_vp] * 8 + [_i64, _i64, C.c_char_p, C.c_char_p, _i64, _i64, _i64, _i64, _vp,
+                                                          _P(_u64), _P(_vp)]),
+    "aclnnQuantLightningIndexer": (_i32, [_vp, _u64, _vp, _vp]),
 }
 
 _lib = None

@@ -54,7 +54,13 @@ using FusedInferAttentionScoreV5PlanFn = int (*)(
     aclOpExecutor**);
 using DynamicMxQuantPlanFn = int (*)(const aclTensor*, int64_t, char*, int64_t, int64_t, int64_t, const aclTensor*, const aclTensor*,
                                      uint64_t*, aclOpExecutor**);  // include/moe/core/op_table.hpp:230-233
+using QuantLightningIndexerPlanFn = int (*)(const aclTensor*, const aclTensor*, const aclTensor*, const aclTensor*, const aclTensor*,
+                                            const aclTensor*, const aclTensor*, const aclTensor*, int64_t, int64_t, char*, char*,
+                                            int64_t, int64_t, int64_t, int64_t, const aclTensor*, uint64_t*,
+                                            aclOpExecutor**);  // include/moe/core/op_table.hpp:998-1006
 using AclnnLaunchFn = int (*)(void*, uint64_t, aclOpExecutor*, void*);
+static_assert(std::is_same_v<decltype(&aclnnQuantLightningIndexerGetWorkspaceSize), QuantLightningIndexerPlanFn>);
+static_assert(std::is_same_v<decltype(&aclnnQuantLightningIndexer), AclnnLaunchFn>);
 static_assert(std::is_same_v<decltype(&aclnnDynamicMxQuantGetWorkspaceSize), DynamicMxQuantPlanFn>);
 static_assert(std::is_same_v<decltype(&aclnnDynamicMxQuant), AclnnLaunchFn>);
 static_assert(std::is_same_v<decltype(&aclnnScatterPaKvCacheGetWorkspaceSize), ScatterPaKvCachePlanFn>);
@@ -281,3 +287,44 @@ def test_mx_quant_plan_contract():
     assert plan(scales=keep.tensor([rows, cols // 16], 37, None))[0] == ffi.ERR_PARAM_INVALID
     assert plan(x=keep.tensor([rows, 40], acl.ACL_BF16, None), y=keep.tensor([rows, 40], acl.ACL_FLOAT8_E4M3FN, None))[0] == ffi.ERR_PARAM_INVALID
     assert "DynamicMxQuant" in acl.last_error()
+
+
+def test_indexer_plan_contract():
+    """aclnnQuantLightningIndexer plan phase for the decode shape (one query token per sequence, paged E4M3 keys) and
+    its refusals; no device is touched."""
+    lib = acl.load()
+    keep = acl.Keep()
+    batch, heads, blocks, bs, width, k = 4, 64, 40, 64, 8, 512
+    E8 = acl.ACL_FLOAT8_E4M3FN
+    t = dict(query=keep.tensor([batch, 1, heads, 128], E8, None), key=keep.tensor([blocks, bs, 1, 128], E8, None),
+             weights=keep.tensor([batch, 1, heads], acl.ACL_BF16, None), q_scale=keep.tensor([batch, 1, heads], acl.ACL_FLOAT32, None),
+             k_scale=keep.tensor([blocks, bs, 1], acl.ACL_FLOAT32, None), lens=keep.tensor([batch], acl.ACL_INT32, None),
+             table=keep.tensor([batch, width], acl.ACL_INT32, None), out=keep.tensor([batch, 1, 1, k], acl.ACL_INT32, None))
+    big = 2 ** 63 - 1
+
+    def plan(qmode=0, kmode=0, lq=b"BSND", lk=b"PA_BSND", count=k, mode=3, pre=big, nxt=big, **over):
+        a = dict(t)
+        a.update(over)
+        workspace, executor = C.c_uint64(7), C.c_void_p()
+        status = lib.aclnnQuantLightningIndexerGetWorkspaceSize(a["query"], a["key"], a["weights"], a["q_scale"], a["k_scale"], None, a["lens"],
+                                                                a["table"], qmode, kmode, lq, lk, count, mode, pre, nxt, a["out"],
+                                                                C.byref(workspace), C.byref(executor))
+        return status, workspace.value, executor.value
+
+    status, workspace, executor = plan()
+    assert status == 0 and executor and workspace == batch * width * bs * 2      # 16-bit scores of every addressable token
+    assert lib.aclDestroyAclOpExecutor(executor) == 0
+    assert plan(mode=0)[0] == 0 and plan(lq=None)[0] == 0
+    assert plan(qmode=1)[0] == ffi.ERR_PARAM_INVALID
+    assert plan(lk=b"BSND")[0] == ffi.ERR_PARAM_INVALID and plan(lk=None)[0] == ffi.ERR_PARAM_INVALID
+    assert plan(count=4096)[0] == ffi.ERR_PARAM_INVALID
+    assert plan(mode=1)[0] == ffi.ERR_PARAM_INVALID
+    assert plan(pre=128)[0] == ffi.ERR_PARAM_INVALID
+    assert plan(table=None)[0] == ffi.ERR_PARAM_NULLPTR and plan(lens=None)[0] == ffi.ERR_PARAM_NULLPTR
+    assert plan(query=keep.tensor([batch, 2, heads, 128], E8, None))[0] == ffi.ERR_PARAM_INVALID   # more than one query token
+    assert plan(query=keep.tensor([batch, 1, 24, 128], E8, None), weights=keep.tensor([batch, 1, 24], acl.ACL_BF16, None),
+                q_scale=keep.tensor([batch, 1, 24], acl.ACL_FLOAT32, None))[0] == ffi.ERR_PARAM_INVALID
+    assert plan(key=keep.tensor([blocks, bs, 1, 64], E8, None))[0] == ffi.ERR_PARAM_INVALID
+    assert plan(out=keep.tensor([batch, 1, 1, k + 1], acl.ACL_INT32, None))[0] == ffi.ERR_PARAM_INVALID
+    assert plan(weights=keep.tensor([batch, 1, heads], acl.ACL_FLOAT32, None))[0] == ffi.ERR_PARAM_INVALID
+    assert "QuantLightningIndexer" in acl.last_error()

@@ -230,3 +230,52 @@ def test_full_size_indexer_and_selected_attention_on_sampled_sequences():
         peak = np.abs(expected).max()
         assert np.abs(got[b] - expected[0]).max() <= 2e-2 * peak
         assert np.abs(lse[b].cpu().numpy() - expected_lse[0]).max() <= 2e-2
+
+
+def test_two_phase_operator_equals_the_direct_entry():
+    """aclnnQuantLightningIndexer through plan / launch on descriptors shaped as the operator's
+    contract names them, against mlakvLightningIndexer on the same buffers."""
+    import acl_ffi as acl
+    lib, alib = ffi.load(), acl.load()
+    keep = acl.Keep()
+    rng = np.random.default_rng(130)
+    batch, heads, bs, k = 3, 64, 64, 128
+    seq_lens = [900, 64, 333]
+    width = -(-max(seq_lens) // bs)
+    blocks = sum(-(-n // bs) for n in seq_lens) + 2
+    pool = kt.build_tables(seq_lens, bs, blocks, seed=131, max_blocks=width)
+    table = pool.table()
+    keys_d = torch.as_tensor(_codes(rng, (blocks, bs, 1, D), 0x58), device="cuda")
+    scales_d = torch.as_tensor(rng.uniform(0.01, 0.05, (blocks, bs, 1)).astype(np.float32), device="cuda")
+    query_d = torch.as_tensor(_codes(rng, (batch, 1, heads, D), 0x58), device="cuda")
+    weights_d = kt.randn_bf16((batch, 1, heads), seed=132).cuda()
+    q_scale_d = torch.as_tensor(rng.uniform(0.01, 0.05, (batch, 1, heads)).astype(np.float32), device="cuda")
+    table_d, lens_d = kt.dev_i32(table), kt.dev_i32(seq_lens)
+    out_shim = torch.full((batch, 1, 1, k), -7, dtype=torch.int32, device="cuda")
+    E8 = acl.ACL_FLOAT8_E4M3FN
+    handles = [keep.tensor([batch, 1, heads, D], E8, query_d.data_ptr()), keep.tensor([blocks, bs, 1, D], E8, keys_d.data_ptr()),
+               keep.tensor([batch, 1, heads], acl.ACL_BF16, weights_d.data_ptr()),
+               keep.tensor([batch, 1, heads], acl.ACL_FLOAT32, q_scale_d.data_ptr()),
+               keep.tensor([blocks, bs, 1], acl.ACL_FLOAT32, scales_d.data_ptr())]
+    t_lens = keep.tensor([batch], acl.ACL_INT32, lens_d.data_ptr())
+    t_table = keep.tensor([batch, width], acl.ACL_INT32, table_d.data_ptr())
+    t_out = keep.tensor([batch, 1, 1, k], acl.ACL_INT32, out_shim.data_ptr())
+    big = 2 ** 63 - 1
+    workspace_bytes, executor = C.c_uint64(0), C.c_void_p()
+    assert alib.aclnnQuantLightningIndexerGetWorkspaceSize(*handles, None, t_lens, t_table, 0, 0, b"BSND", b"PA_BSND", k, 3, big, big, t_out,
+                                                           C.byref(workspace_bytes), C.byref(executor)) == 0, acl.last_error()
+    workspace = torch.zeros(max(workspace_bytes.value, 16), dtype=torch.uint8, device="cuda")
+    assert alib.aclnnQuantLightningIndexer(workspace.data_ptr(), workspace.numel(), executor, kt.stream_ptr()) == 0, acl.last_error()
+    torch.cuda.synchronize()
+    assert alib.aclDestroyAclOpExecutor(executor) == 0
+    out_direct = torch.full((batch, k), -7, dtype=torch.int32, device="cuda")
+    view = ffi.IndexKeyView(keys_d.data_ptr(), bs * D, D, scales_d.data_ptr(), bs, blocks, bs, D, 0)
+    ws2 = torch.zeros(int(lib.mlakvIndexerWorkspaceBytes(batch, width * bs)), dtype=torch.uint8, device="cuda")
+    ffi.check(lib.mlakvLightningIndexer(C.byref(view), query_d.data_ptr(), heads * D, D, weights_d.data_ptr(), heads * 2, q_scale_d.data_ptr(),
+                                        heads, heads, table_d.data_ptr(), width, lens_d.data_ptr(), batch, width * bs, k,
+                                        out_direct.data_ptr(), k, ws2.data_ptr(), ws2.numel(), kt.stream_ptr()))
+    torch.cuda.synchronize()
+    assert torch.equal(out_shim.reshape(batch, k), out_direct)
+    got = out_direct.cpu().numpy()
+    assert got[1].tolist() == list(range(64)) + [-1] * (k - 64)
+    assert (got[0] >= 0).all() and (got[0] < 900).all() and len(set(got[0].tolist())) == k
