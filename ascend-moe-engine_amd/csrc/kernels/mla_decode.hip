@@ -82,6 +82,7 @@ typedef __attribute__((ext_vector_type(2))) __bf16 bf16x2;
 typedef __attribute__((ext_vector_type(4))) float f32x4;
 typedef __attribute__((ext_vector_type(2))) float f32x2;
 typedef __attribute__((ext_vector_type(4))) unsigned int u32x4;
+typedef __attribute__((ext_vector_type(4))) int i32x4;
 typedef __attribute__((ext_vector_type(2))) unsigned int u32x2;
 typedef __attribute__((ext_vector_type(4))) short s16x4;
 typedef __attribute__((ext_vector_type(8))) short s16x8;
@@ -121,7 +122,7 @@ constexpr int kRowsPerWave = kTileTokens / kWaves;           // bf16: latent row
 constexpr float kRescaleThreshold = 8.0f;                    // log2 domain
 constexpr int kKAhead = 8;                                   // bf16 K fragments in flight ahead of their MFMA
 constexpr int kKAhead8 = 4;                                  // FP8 K reads (two fragments each) in flight
-constexpr int kVAhead = 4;                                   // V fragments in flight
+constexpr int kVAhead = 3;                                   // V fragments in flight (of the eight an output wave fetches per tile)
 
 __device__ __forceinline__ int Uniform(int v) { return __builtin_amdgcn_readfirstlane(v); }
 
@@ -855,101 +856,158 @@ __global__ __launch_bounds__(kThreads) void MlaDecodeKernel(AttnArgs a) {
       }
     };
 
-    f32x4 o[kDvTiles];
+    // Output wave w owns the 128 output columns [128 w, 128 w + 128) of all 64 heads of the group:
+    // every V^T fragment is then fetched (and, for FP8, converted) by one wave only, and meets the
+    // P fragments of the four score waves. (With one head block per output wave, each of the four
+    // read and converted all of V.) Head blocks past the group's heads are computed on whatever
+    // their LDS slots hold and never written.
+    constexpr int kDvPerWave = kDvTiles / (kWaves - kScoreWaves);
+    const int hba = min(kScoreWaves, (a.heads - static_cast<int>(blockIdx.z) * 64 + 15) >> 4);  // head blocks in use
+    const unsigned char* p_all = lds + G::kPOff + lane * 16;                                   // + (parity * 4 + hb) * 64 * 16
+    const float* alpha_all = reinterpret_cast<const float*>(lds + G::kAlphaOff) + lane;      // + (parity * 4 + hb) * 64
+    const float* inv_all = reinterpret_cast<const float*>(lds + G::kInvOff) + lane;          // + hb * 64
+    const int* flag_all = reinterpret_cast<const int*>(lds + G::kFlagOff);                   // [parity * 4 + hb]
+    f32x4 o[kScoreWaves][kDvPerWave];
 #pragma unroll
-    for (int n = 0; n < kDvTiles; ++n) o[n] = f32x4{0.f, 0.f, 0.f, 0.f};
+    for (int hb = 0; hb < kScoreWaves; ++hb) {
+#pragma unroll
+      for (int n = 0; n < kDvPerWave; ++n) o[hb][n] = f32x4{0.f, 0.f, 0.f, 0.f};
+    }
 
     for (int i = 0; i < ntiles; ++i) {
       publish(i);
       issue_next(i);
-      if (active) {
+      {
         const unsigned char* buf = lds + ring(i);
         const int parity = i & 1;
+        // the four rescale flags of the tile in one read; a moved reference maximum is the exception
+        const i32x4 flags = *reinterpret_cast<const i32x4*>(flag_all + parity * kScoreWaves);
+        if (Uniform(flags.x | flags.y | flags.z | flags.w) != 0) {
+          const int moved[kScoreWaves] = {flags.x, flags.y, flags.z, flags.w};
+#pragma unroll
+          for (int hb = 0; hb < kScoreWaves; ++hb) {
+            if (Uniform(moved[hb]) != 0) {  // that block's reference maximum moved: rescale its O first
+              const float alpha = alpha_all[(parity * kScoreWaves + hb) * 64];
+#pragma unroll
+              for (int n = 0; n < kDvPerWave; ++n) o[hb][n] *= alpha;
+            }
+          }
+        }
         u32x4 vf[kVAhead];
 #pragma unroll
-        for (int d = 0; d < kVAhead; ++d) vf[d] = v_fetch(buf, d);
-        const bf16x8 p = *reinterpret_cast<const bf16x8*>(p_lds + parity * kScoreWaves * 64 * 16);
-        if (Uniform(flag_lds[parity * kScoreWaves]) != 0) {  // the reference maximum moved: rescale O first
-          const float alpha = alpha_lds[parity * kScoreWaves * 64];
+        for (int d = 0; d < kVAhead; ++d) vf[d] = v_fetch(buf, kDvPerWave * hw + d);
+        bf16x8 p[kScoreWaves];
 #pragma unroll
-          for (int n = 0; n < kDvTiles; ++n) o[n] *= alpha;
-        }
+        for (int hb = 0; hb < kScoreWaves; ++hb) p[hb] = *reinterpret_cast<const bf16x8*>(p_all + (parity * kScoreWaves + hb) * 64 * 16);
         __builtin_amdgcn_sched_barrier(0);
-        StaticFor<kDvTiles>([&](auto n_c) __attribute__((always_inline)) {
-          constexpr int n = decltype(n_c)::value;
-          o[n] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(v_operand(vf[n % kVAhead]), p, o[n], 0, 0, 0);
-          if constexpr (n + kVAhead < kDvTiles) vf[n % kVAhead] = v_fetch(buf, n + kVAhead);
-          __builtin_amdgcn_sched_barrier(0);
-        });
+        if constexpr (FP8) {
+          // the next fragment is converted while this one's four MFMAs run
+          bf16x8 v = v_operand(vf[0]);
+          if constexpr (kVAhead < kDvPerWave) vf[0] = v_fetch(buf, kDvPerWave * hw + kVAhead);
+          StaticFor<kDvPerWave>([&](auto n_c) __attribute__((always_inline)) {
+            constexpr int n = decltype(n_c)::value;
+            bf16x8 v_next = v;
+            if constexpr (n + 1 < kDvPerWave) v_next = v_operand(vf[(n + 1) % kVAhead]);
+#pragma unroll
+            for (int hb = 0; hb < kScoreWaves; ++hb) o[hb][n] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(v, p[hb], o[hb][n], 0, 0, 0);
+            if constexpr (n + 1 + kVAhead < kDvPerWave) vf[(n + 1) % kVAhead] = v_fetch(buf, kDvPerWave * hw + n + 1 + kVAhead);
+            v = v_next;
+            __builtin_amdgcn_sched_barrier(0);
+          });
+        } else {
+          StaticFor<kDvPerWave>([&](auto n_c) __attribute__((always_inline)) {
+            constexpr int n = decltype(n_c)::value;
+            const bf16x8 v = v_operand(vf[n % kVAhead]);
+#pragma unroll
+            for (int hb = 0; hb < kScoreWaves; ++hb) o[hb][n] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(v, p[hb], o[hb][n], 0, 0, 0);
+            if constexpr (n + kVAhead < kDvPerWave) vf[n % kVAhead] = v_fetch(buf, kDvPerWave * hw + n + kVAhead);
+            __builtin_amdgcn_sched_barrier(0);
+          });
+        }
         MLAKV_STAMP((i) < 4 ? 7 + 6 * (i) : -1);
       }
     }
     MLAKV_STAMP(29);
     __syncthreads();  // 1/denominator from the score waves
     MLAKV_STAMP(30);
-    if (active) {
-      const float inv = *inv_lds;
-      char* out_row;
-      if (direct) {
-        out_row = MXQ && a.out == nullptr ? nullptr : a.out + seq * a.out_seq_stride + head * a.out_head_stride;
-      } else {
-        const int64_t row = (static_cast<int64_t>(seq) * a.max_chunks + chunk_index) * a.heads + head;
-        out_row = a.partial_out + row * (kLatentDim * 2);
-      }
-      if (MXQ && direct) {
-        // Quantising epilogue of the single-chunk case: a block of 32 columns is the tile pair
-        // (2k, 2k+1) over the four lanes that share this head.
-        char* codes_row = a.out_codes + seq * a.out_codes_seq_stride + head * a.out_codes_head_stride;
-        unsigned scale_codes[4] = {0u, 0u, 0u, 0u};
+    const int group_head0 = static_cast<int>(blockIdx.z) * 64;
+    // Row (bf16 [512]) of head `h` of this group in the launch's output: the final output when
+    // there is one chunk, this chunk's partial otherwise.
+    const auto row_of = [&](int h) __attribute__((always_inline)) -> char* {
+      if (direct) return a.out + seq * a.out_seq_stride + (group_head0 + h) * a.out_head_stride;
+      const int64_t row = (static_cast<int64_t>(seq) * a.max_chunks + chunk_index) * a.heads + group_head0 + h;
+      return a.partial_out + row * (kLatentDim * 2);
+    };
+    if (MXQ && direct) {
+      // Quantising epilogue of the single-chunk case: a block of 32 columns is a pair of this
+      // wave's column tiles over the four lanes that share a head; the wave covers blocks
+      // 4 w .. 4 w + 3 of every head.
 #pragma unroll
-        for (int k = 0; k < kDvTiles / 2; ++k) {
+      for (int hb = 0; hb < kScoreWaves; ++hb) {
+        if (hb >= hba) continue;
+        const int h = 16 * hb + i16;
+        const float inv = inv_all[hb * 64];
+        char* codes_row = a.out_codes + seq * a.out_codes_seq_stride + (group_head0 + h) * a.out_codes_head_stride;
+        char* out_row = a.out == nullptr ? nullptr : row_of(h);
+        unsigned scale_codes = 0u;
+#pragma unroll
+        for (int k = 0; k < kDvPerWave / 2; ++k) {
           u32x2 packed[2];
           unsigned magnitude = 0u;
 #pragma unroll
-          for (int h = 0; h < 2; ++h) {
-            const int n = 2 * k + h;
-            packed[h].x = PackBf16(o[n][0] * inv, o[n][1] * inv);
-            packed[h].y = PackBf16(o[n][2] * inv, o[n][3] * inv);
-            magnitude = MxMagnitudeMax(packed[h].y, MxMagnitudeMax(packed[h].x, magnitude));
-            if (out_row != nullptr) __builtin_nontemporal_store(packed[h], reinterpret_cast<u32x2*>(out_row + (16 * n + 4 * g) * 2));
+          for (int half = 0; half < 2; ++half) {
+            const int n = 2 * k + half;
+            packed[half].x = PackBf16(o[hb][n][0] * inv, o[hb][n][1] * inv);
+            packed[half].y = PackBf16(o[hb][n][2] * inv, o[hb][n][3] * inv);
+            magnitude = MxMagnitudeMax(packed[half].y, MxMagnitudeMax(packed[half].x, magnitude));
+            if (out_row != nullptr) {
+              __builtin_nontemporal_store(packed[half], reinterpret_cast<u32x2*>(out_row + (16 * (kDvPerWave * hw + n) + 4 * g) * 2));
+            }
           }
           magnitude = UMaxAcrossHeadLanes(magnitude);
           const MxScale s = MxScaleFromMaxBits(magnitude);
 #pragma unroll
-          for (int h = 0; h < 2; ++h) {
-            const unsigned four = MxEncodeWord(packed[h].x, s) | (MxEncodeWord(packed[h].y, s) << 16);
-            __builtin_nontemporal_store(four, reinterpret_cast<unsigned*>(codes_row + 16 * (2 * k + h) + 4 * g));
+          for (int half = 0; half < 2; ++half) {
+            const unsigned four = MxEncodeWord(packed[half].x, s) | (MxEncodeWord(packed[half].y, s) << 16);
+            __builtin_nontemporal_store(four, reinterpret_cast<unsigned*>(codes_row + 16 * (kDvPerWave * hw + 2 * k + half) + 4 * g));
           }
-          scale_codes[k >> 2] |= s.code << (8 * (k & 3));
+          scale_codes |= s.code << (8 * k);
         }
         if (g == 0) {
-          *reinterpret_cast<u32x4*>(a.out_scales + seq * a.out_scales_seq_stride + head * a.out_scales_head_stride) =
-              u32x4{scale_codes[0], scale_codes[1], scale_codes[2], scale_codes[3]};
+          *reinterpret_cast<unsigned*>(a.out_scales + seq * a.out_scales_seq_stride + (group_head0 + h) * a.out_scales_head_stride +
+                                       (kDvPerWave / 2) * hw) = scale_codes;
         }
-      } else {
-        // The accumulators hold O^T (lane = head i16, four columns per 16-column tile), which
-        // stored as it is would write 32-byte pieces of sixteen different rows per instruction.
-        // The tile ring is dead after the last barrier: each output wave transposes its sixteen
-        // rows through its own part of it and writes whole 1-KB rows, 16 bytes per lane. A row
-        // stride of 1040 bytes (= 4 banks mod 64) spreads the 8-byte writes of a half-wave over
-        // all banks.
-        constexpr int kStageRow = kLatentDim * 2 + 16;
-        static_assert((kWaves - kScoreWaves) * 16 * kStageRow <= G::kRing * G::kTileBytes, "the staging rows fit in the ring");
-        unsigned char* stage = lds + G::Slot(0) + hw * (16 * kStageRow);
+      }
+    } else {
+      // The accumulators hold O^T (lane = head i16 of a block, four columns per 16-column tile),
+      // which stored as it is would write 8-byte pieces of sixteen different rows per
+      // instruction. The tile ring is dead after the last barrier: each output wave transposes
+      // its 256-byte slices of the 64 rows through its own part of it and writes them 16 bytes per
+      // lane, four whole slices per instruction. A row stride of 272 bytes (= 4 banks mod 64)
+      // spreads the 8-byte writes of a half-wave over all banks.
+      constexpr int kSliceBytes = kDvPerWave * 16 * 2;  // 256
+      constexpr int kStageRow = kSliceBytes + 16;
+      static_assert((kWaves - kScoreWaves) * 64 * kStageRow <= G::kRing * G::kTileBytes, "the staging rows fit in the ring");
+      unsigned char* stage = lds + G::Slot(0) + hw * (64 * kStageRow);
 #pragma unroll
-        for (int n = 0; n < kDvTiles; ++n) {
+      for (int hb = 0; hb < kScoreWaves; ++hb) {
+        const float inv = inv_all[hb * 64];
+#pragma unroll
+        for (int n = 0; n < kDvPerWave; ++n) {
           u32x2 packed;
-          packed.x = PackBf16(o[n][0] * inv, o[n][1] * inv);
-          packed.y = PackBf16(o[n][2] * inv, o[n][3] * inv);
-          *reinterpret_cast<u32x2*>(stage + i16 * kStageRow + (16 * n + 4 * g) * 2) = packed;
+          packed.x = PackBf16(o[hb][n][0] * inv, o[hb][n][1] * inv);
+          packed.y = PackBf16(o[hb][n][2] * inv, o[hb][n][3] * inv);
+          *reinterpret_cast<u32x2*>(stage + (16 * hb + i16) * kStageRow + (16 * n + 4 * g) * 2) = packed;
         }
-        // Same wave wrote and reads: the LDS queue is in order, no barrier needed.
-        const int64_t row_stride = direct ? a.out_head_stride : kLatentDim * 2;
-        char* first_row = out_row - i16 * row_stride;  // row of this wave's head 0
+      }
+      // Same wave wrote and reads: the LDS queue is in order, no barrier needed.
+      const int piece = lane & 15, sub = lane >> 4;
 #pragma unroll
-        for (int r = 0; r < 16; ++r) {
-          const u32x4 v = *reinterpret_cast<const u32x4*>(stage + r * kStageRow + lane * 16);
-          __builtin_nontemporal_store(v, reinterpret_cast<u32x4*>(first_row + r * row_stride + lane * 16));
+      for (int it = 0; it < 16; ++it) {
+        const int h = 4 * it + sub;
+        if (h < 16 * hba) {
+          const u32x4 v = *reinterpret_cast<const u32x4*>(stage + h * kStageRow + piece * 16);
+          __builtin_nontemporal_store(v, reinterpret_cast<u32x4*>(row_of(h) + kSliceBytes * hw + piece * 16));
         }
       }
     }
