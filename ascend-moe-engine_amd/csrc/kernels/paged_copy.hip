@@ -97,36 +97,38 @@ __device__ __forceinline__ u32x4 Dequant8(u32x2 codes, float scale) {
 
 // ---- append -----------------------------------------------------------------
 
-// One wavefront per (four consecutive tokens, layer). bf16: 64 lanes move a latent row, 8 lanes a
-// rope row. The source rows do not depend on the slots, so all of a wavefront's loads (slots and
-// rows) are issued together: with one row per wavefront and the row fetched only after its slot
-// had arrived, a prefill-sized append was bound by two memory latencies per 1152 bytes.
-constexpr int kAppendRows = 4;
+// One wavefront per (run of consecutive tokens, layer). bf16: 64 lanes move a latent row, 8 lanes
+// a rope row. The source rows do not depend on the slots, so all of a wavefront's loads (slots
+// and rows) are issued together: with the row fetched only after its slot had arrived, a
+// prefill-sized append was bound by two memory latencies per row. The quantising kernel, which has
+// a shuffle reduction and a division per row to hide, takes four rows per wavefront.
+constexpr int kAppendRows = 4;      // FP8: rows per wavefront
+constexpr int kAppendRowsBf16 = 1;  // bf16: a pure copy ran fastest with one row per wavefront (8 layers x 311k rows: 984 us, 1081 with two, 1106 with four)
 
 __global__ __launch_bounds__(kThreads) void AppendBf16Kernel(AppendArgs a) {
   const int lane = threadIdx.x & (kWave - 1);
-  const int token0 = Uniform((blockIdx.x * kWavesPerGroup + (threadIdx.x >> 6)) * kAppendRows);
+  const int token0 = Uniform((blockIdx.x * kWavesPerGroup + (threadIdx.x >> 6)) * kAppendRowsBf16);
   const int layer = blockIdx.y;
   if (token0 >= a.num_tokens) return;
   int my_slot = -1;
-  if (lane < kAppendRows && token0 + lane < a.num_tokens) my_slot = a.slots[token0 + lane];
+  if (lane < kAppendRowsBf16 && token0 + lane < a.num_tokens) my_slot = a.slots[token0 + lane];
   static_assert(kLatentDim * 2 / 16 == kWave, "one latent row is one wave access");
   const bool rope_lane = lane < kRopeDim * 2 / 16;
   const char* latent_src = a.latent_src.base + layer * a.latent_src.layer_stride;
   const char* rope_src = a.rope_src.base + layer * a.rope_src.layer_stride;
-  u32x4 v[kAppendRows], r[kAppendRows];
+  u32x4 v[kAppendRowsBf16], r[kAppendRowsBf16];
   // a row past the end repeats the last one: loaded, never stored (its slot lane holds -1)
 #pragma unroll
-  for (int i = 0; i < kAppendRows; ++i) v[i] = Load16(latent_src + min(token0 + i, a.num_tokens - 1) * a.latent_src.row_stride + lane * 16);
+  for (int i = 0; i < kAppendRowsBf16; ++i) v[i] = Load16(latent_src + min(token0 + i, a.num_tokens - 1) * a.latent_src.row_stride + lane * 16);
   if (rope_lane) {  // one branch around all rope loads: a branch per row made the compiler wait between the rows
 #pragma unroll
-    for (int i = 0; i < kAppendRows; ++i) r[i] = Load16(rope_src + min(token0 + i, a.num_tokens - 1) * a.rope_src.row_stride + lane * 16);
+    for (int i = 0; i < kAppendRowsBf16; ++i) r[i] = Load16(rope_src + min(token0 + i, a.num_tokens - 1) * a.rope_src.row_stride + lane * 16);
   }
-  char* latent_dst[kAppendRows];
-  char* rope_dst[kAppendRows];
-  bool live[kAppendRows];
+  char* latent_dst[kAppendRowsBf16];
+  char* rope_dst[kAppendRowsBf16];
+  bool live[kAppendRowsBf16];
 #pragma unroll
-  for (int i = 0; i < kAppendRows; ++i) {
+  for (int i = 0; i < kAppendRowsBf16; ++i) {
     const int slot = __builtin_amdgcn_readlane(my_slot, i);
     const int block = slot < 0 ? 0 : slot / a.block_size;
     const int in_block = slot < 0 ? 0 : slot - block * a.block_size;
@@ -135,12 +137,12 @@ __global__ __launch_bounds__(kThreads) void AppendBf16Kernel(AppendArgs a) {
     rope_dst[i] = a.rope.base + layer * a.rope.layer_stride + block * a.rope.block_stride + in_block * a.rope.row_stride;
   }
 #pragma unroll
-  for (int i = 0; i < kAppendRows; ++i) {
+  for (int i = 0; i < kAppendRowsBf16; ++i) {
     if (live[i]) Store16(latent_dst[i] + lane * 16, v[i]);
   }
   if (rope_lane) {
 #pragma unroll
-    for (int i = 0; i < kAppendRows; ++i) {
+    for (int i = 0; i < kAppendRowsBf16; ++i) {
       if (live[i]) Store16(rope_dst[i] + lane * 16, r[i]);
     }
   }
@@ -530,10 +532,11 @@ int DivUp(int a, int b) { return (a + b - 1) / b; }
 
 hipError_t LaunchAppend(const AppendArgs& args, hipStream_t stream) {
   if (args.num_tokens <= 0 || args.num_layers <= 0) return hipSuccess;
-  const dim3 grid(DivUp(args.num_tokens, kWavesPerGroup * kAppendRows), args.num_layers);
   if (args.fp8) {
+    const dim3 grid(DivUp(args.num_tokens, kWavesPerGroup * kAppendRows), args.num_layers);
     hipLaunchKernelGGL(AppendFp8Kernel, grid, dim3(kThreads), 0, stream, args);
   } else {
+    const dim3 grid(DivUp(args.num_tokens, kWavesPerGroup * kAppendRowsBf16), args.num_layers);
     hipLaunchKernelGGL(AppendBf16Kernel, grid, dim3(kThreads), 0, stream, args);
   }
   return hipGetLastError();
