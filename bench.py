@@ -37,6 +37,24 @@ LATENT, ROPE, ROW = 512, 64, 576
 ROW_BYTES = ROW * 2
 
 
+def sustained_us(torch, fn, min_iters, warm_ms=250.0, timed_ms=100.0):
+    """Average microseconds per fn(i) launch with the shader clock settled: the clock climbs for
+    some 100 ms under load (the long attention shape measured 284 us per launch over 2 launches,
+    254 over 32, 227 over 512), so the launches run back to back for `warm_ms` before the timed
+    ones, which then cover at least `timed_ms`."""
+    def run(n):
+        start, stop = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+        start.record()
+        for i in range(n):
+            fn(i)
+        stop.record()
+        torch.cuda.synchronize()
+        return start.elapsed_time(stop) * 1e3 / n
+    rough = run(16)
+    run(max(16, int(warm_ms * 1e3 / rough)))
+    return run(max(min_iters, int(timed_ms * 1e3 / rough)))
+
+
 def parse_args():
     p = argparse.ArgumentParser()
     p.add_argument("--gpus", type=int, default=1)
@@ -240,16 +258,7 @@ def bench_attention(args, torch, np, ffi, fp8=False, batch=32, ctx=2048, heads=6
     iters = iters or max(args.steps * 8, 64)
 
     def timed_us(fn):
-        for i in range(16):
-            fn(i)
-        torch.cuda.synchronize()
-        start, stop = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
-        start.record()
-        for i in range(iters):
-            fn(i)
-        stop.record()
-        torch.cuda.synchronize()
-        return start.elapsed_time(stop) * 1e3 / iters
+        return sustained_us(torch, fn, iters)
 
     us = timed_us(launch)
     mx = None
@@ -293,7 +302,7 @@ def bench_attention(args, torch, np, ffi, fp8=False, batch=32, ctx=2048, heads=6
         "mfma_tflops": flops / (us * 1e-6) / 1e12,
         "mfma_frac_of_bf16_peak": flops / (us * 1e-6) / 1e12 / MFMA_BF16_PEAK_TFLOPS,
         "chunk_tiles": int(plan.chunk_tiles), "max_chunks": int(plan.max_chunks),
-        "workspace_bytes": int(plan.workspace_bytes), "launches_timed": iters,
+        "workspace_bytes": int(plan.workspace_bytes), "timing": "250 ms of back-to-back launches untimed, then at least 100 ms of them timed",
     }
     if mx is not None:
         result["mx_quant_output"] = mx
@@ -325,24 +334,14 @@ def bench_indexer(args, torch, np, ffi, batch=32, ctx=8192, heads=64, k=512, bs=
                                             heads * 2, q_scale.data_ptr(), heads, heads, table.data_ptr(), ctx // bs, lens.data_ptr(),
                                             batch, ctx, k, out.data_ptr(), k, workspace.data_ptr(), workspace.numel(),
                                             stream_ptr(torch)))
-    iters = 64
-    for i in range(8):
-        launch(i)
-    torch.cuda.synchronize()
-    start, stop = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
-    start.record()
-    for i in range(iters):
-        launch(i)
-    stop.record()
-    torch.cuda.synchronize()
-    us = start.elapsed_time(stop) * 1e3 / iters
+    us = sustained_us(torch, launch, 64)
     algorithmic = batch * ctx * (128 + 4) + batch * heads * (128 + 2 + 4) + 4 * batch * (ctx // bs) + 4 * batch * k
     return {"us_per_step": us,
             "workload": f"batch {batch}, ctx {ctx}, {heads} index heads x 128, top-{k}, block {bs}, e4m3 keys + fp32 row scale, "
                         f"shuffled table, {slices} rotating key pools",
             "roofline": {"bound": "hbm", "achieved": algorithmic / (us * 1e-6) / 1e9, "peak": HBM_PEAK_GBPS, "unit": "GB/s",
                          "frac": algorithmic / (us * 1e-6) / 1e9 / HBM_PEAK_GBPS, "traffic": None},
-            "algorithmic_bytes": algorithmic, "launches_timed": iters}
+            "algorithmic_bytes": algorithmic, "timing": "250 ms of back-to-back launches untimed, then at least 100 ms of them timed"}
 
 
 def bench_side_kernels(args, torch, np, ffi):
@@ -358,15 +357,7 @@ def bench_side_kernels(args, torch, np, ffi):
     out = {}
 
     def timed(fn, reps=5):
-        fn()
-        torch.cuda.synchronize()
-        start, stop = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
-        start.record()
-        for _ in range(reps):
-            fn()
-        stop.record()
-        torch.cuda.synchronize()
-        return start.elapsed_time(stop) / reps
+        return sustained_us(torch, lambda i: fn(), reps, warm_ms=100.0, timed_ms=50.0) * 1e-3
 
     gen = torch.Generator(device="cuda").manual_seed(5)
     lat = torch.randn(layers, total, LATENT, generator=gen, device="cuda").to(torch.bfloat16)
