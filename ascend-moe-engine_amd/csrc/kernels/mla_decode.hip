@@ -75,6 +75,7 @@ namespace mlakv {
 namespace {
 
 constexpr int kXcds = 8;
+constexpr bool kLateIssue = true;
 
 typedef __attribute__((ext_vector_type(8))) __bf16 bf16x8;
 typedef __attribute__((ext_vector_type(4))) __bf16 bf16x4;
@@ -623,10 +624,12 @@ __global__ __launch_bounds__(kThreads) void MlaDecodeKernel(AttnArgs a) {
   // The query must have arrived before this wave issues tile loads: the compiler's own wait for
   // it would otherwise also wait for every tile load issued in between.
   MLAKV_STAMP(35);
-  if (score_wave && active) {
+  // Every wave passes through it, whether it asked for the query or not: were it skipped on
+  // some path, the compiler would have to assume the query still in flight wherever the paths
+  // meet again, and would wait for it -- with counts that know nothing of the tile loads, so in
+  // effect for every tile in flight -- inside the score loop, at every use.
 #pragma unroll
-    for (int ks = 0; ks < kKSteps; ++ks) asm volatile("" ::"v"(q[ks]));
-  }
+  for (int ks = 0; ks < kKSteps; ++ks) asm volatile("" ::"v"(q[ks]));
   MLAKV_STAMP(1);
   if constexpr (!kSoloPrologue) __syncthreads();  // table entries visible
 
@@ -720,7 +723,7 @@ __global__ __launch_bounds__(kThreads) void MlaDecodeKernel(AttnArgs a) {
 
     // S^T of tile `tile_rel`, its softmax against the running reference, P and the rescale
     // request into the LDS slots of the tile's parity.
-    const auto score_tile = [&](int tile_rel) __attribute__((always_inline)) {
+    const auto score_tile = [&](int tile_rel, int issue_iteration) __attribute__((always_inline)) {
       const unsigned char* buf = lds + ring(tile_rel);
       f32x4 acc[4];
 #pragma unroll
@@ -757,6 +760,7 @@ __global__ __launch_bounds__(kThreads) void MlaDecodeKernel(AttnArgs a) {
         });
       }
       MLAKV_STAMP(tile_rel >= 1 && tile_rel <= 4 ? 7 + 6 * (tile_rel - 1) : -1);
+      if (kLateIssue && issue_iteration >= 0) issue_next(issue_iteration);
       // lane holds tokens 4g+j (x[0..3]) and 16+4g+j (x[4..7]) of head i16
       float x[8];
 #pragma unroll
@@ -801,11 +805,12 @@ __global__ __launch_bounds__(kThreads) void MlaDecodeKernel(AttnArgs a) {
       MLAKV_STAMP(tile_rel >= 1 && tile_rel <= 4 ? 8 + 6 * (tile_rel - 1) : -1);
     };
 
-    if (active) score_tile(0);
+    if (active) score_tile(0, -1);
     for (int i = 0; i < ntiles; ++i) {
       publish(i);
-      issue_next(i);
-      if (active && i + 1 < ntiles) score_tile(i + 1);
+      const bool scores = active && i + 1 < ntiles;
+      if (!kLateIssue || !scores) issue_next(i);
+      if (scores) score_tile(i + 1, i);
     }
     if (active) {
       const float l_total = SumAcrossHeadLanes(l_run);
@@ -1022,7 +1027,16 @@ __global__ __launch_bounds__(kThreads) void MlaDecodeKernel(AttnArgs a) {
 // dependence on the sequence length.
 constexpr int kCombineHeads = 4;
 __global__ __launch_bounds__(kCombineHeads * 64) void MlaCombineKernel(AttnArgs a) {
-  const int head = blockIdx.x * kCombineHeads + (threadIdx.x >> 6), seq = blockIdx.y;
+  // Workgroups go to the XCDs round-robin by linear id; the main kernel put all chunks of a
+  // sequence on XCD seq / (batch / 8), and the partials are most likely still in that L2.
+  int group = blockIdx.x, seq = blockIdx.y;
+  if ((gridDim.y & (kXcds - 1)) == 0) {
+    const int linear = blockIdx.y * gridDim.x + blockIdx.x;
+    const int within = linear / kXcds;
+    seq = (linear & (kXcds - 1)) * (gridDim.y / kXcds) + within / static_cast<int>(gridDim.x);
+    group = within % static_cast<int>(gridDim.x);
+  }
+  const int head = group * kCombineHeads + (threadIdx.x >> 6);
   const int lane = threadIdx.x & 63;
   if (head >= a.heads) return;
   const int chunks = a.max_chunks;

@@ -58,8 +58,8 @@ def sustained_us(torch, fn, min_iters, warm_ms=250.0, timed_ms=100.0):
 def parse_args():
     p = argparse.ArgumentParser()
     p.add_argument("--gpus", type=int, default=1)
-    p.add_argument("--steps", type=int, default=20)
-    p.add_argument("--warmup", type=int, default=5)
+    p.add_argument("--steps", type=int, default=60)
+    p.add_argument("--warmup", type=int, default=60)
     p.add_argument("--no-cpu-baseline", action="store_true")
     p.add_argument("--no-attention", action="store_true")
     p.add_argument("--side-only", action="store_true", help="development aid: time only the FP8 append/gather and compaction kernels")
@@ -74,10 +74,11 @@ def stream_ptr(torch):
 
 def bench_append_gather(args, torch, np, ffi):
     lib = ffi.load()
-    layers, batch, bs, max_ctx = 43, 32, 64, 2048 + 128
+    layers, batch, bs = 43, 32, 64
     rng = np.random.default_rng(20251125)
     ctxs = [int(v) for v in rng.integers(128, 2049, size=batch)]
     total_steps = args.warmup + args.steps
+    max_ctx = 2048 + max(128, -(-total_steps // bs) * bs)  # every sequence grows by one token per step
     pool_blocks = sum(-(-(c + total_steps) // bs) for c in ctxs) + 32
     arena = ffi.Arena(ffi.BACKEND_HIP)
     cache = ffi.KvCache(arena, num_layers=layers, block_size=bs, max_context_len=max_ctx, max_batch=batch,
