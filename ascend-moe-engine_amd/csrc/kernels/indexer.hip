@@ -23,10 +23,11 @@ typedef __attribute__((ext_vector_type(4))) float f32x4;
 typedef __attribute__((ext_vector_type(8))) __bf16 bf16x8;
 typedef __attribute__((ext_vector_type(2))) __bf16 bf16x2;
 typedef __attribute__((ext_vector_type(4))) unsigned int u32x4;
+typedef __attribute__((ext_vector_type(2))) unsigned int u32x2;
 
 constexpr int kIndexDim = 128;
 static_assert(kIndexDim == 4 * 32, "four lane groups of 32 elements cover an index key");
-constexpr int kScoreThreads = 256;
+constexpr int kScoreThreads = 512;
 constexpr int kTokensPerWave = 64;
 constexpr int kTokensPerGroup = (kScoreThreads / 64) * kTokensPerWave;
 
@@ -50,84 +51,199 @@ __device__ __forceinline__ unsigned ScoreKey(float score) {
   return (b & 0x8000u) ? (~b & 0xffffu) : (b | 0x8000u);
 }
 
-// Address pieces of cached token `token` of sequence `seq` (clamped into the sequence).
-__device__ __forceinline__ void LocateToken(const IndexerArgs& a, const int32_t* table_row, int token, int seq_len, int* block,
+// Address pieces of cached token `token` of a sequence, clamped to the last position `limit - 1`
+// that the table row can address. The limit does not depend on the sequence length, so the
+// lookup need not wait for it; a token past the end of its sequence resolves to some readable
+// row whose score is never written.
+__device__ __forceinline__ void LocateToken(const IndexerArgs& a, const int32_t* table_row, int token, int limit, int* block,
                                             int* slot) {
-  const int clamped = token < seq_len ? token : seq_len - 1;
+  const int clamped = token < limit ? token : limit - 1;
   const int logical = clamped / a.block_size;
   const int entry = table_row[logical];
   *block = static_cast<unsigned>(entry) < static_cast<unsigned>(a.num_blocks) ? entry : 0;
   *slot = clamped - logical * a.block_size;
 }
 
-// One wavefront scores 64 consecutive tokens in four groups of 16: A = keys (16 tokens x 32
-// elements per MFMA, converted to bf16), B = query (32 elements x 16 heads), four k-steps and HB head blocks. Lane
-// (r = lane % 16, g = lane / 16) holds elements [32g, 32g + 32) of token r (A) and of head r (B); a
-// k-step takes eight of them from both, so the element order inside the dot product is the same
-// on both sides.
+// Sum over the four lanes {r, r + 16, r + 32, r + 48}, left in all of them.
+__device__ __forceinline__ float SumAcrossGroups(float x) {
+  unsigned bits = __builtin_bit_cast(unsigned, x);
+  u32x2 swapped = __builtin_amdgcn_permlane16_swap(bits, bits, false, false);
+  const float s = __builtin_bit_cast(float, static_cast<unsigned>(swapped.x)) + __builtin_bit_cast(float, static_cast<unsigned>(swapped.y));
+  bits = __builtin_bit_cast(unsigned, s);
+  swapped = __builtin_amdgcn_permlane32_swap(bits, bits, false, false);
+  return __builtin_bit_cast(float, static_cast<unsigned>(swapped.x)) + __builtin_bit_cast(float, static_cast<unsigned>(swapped.y));
+}
+
+// Direct global->LDS load: lane L's 16 bytes land at lds_wave_base + 16 * L (the LDS base travels
+// in M0 and is wave-uniform). Issued from inline assembly, so the kernel waits for it itself.
+__device__ __forceinline__ void DirectLoad16PerLane(const char* lane_pointer, unsigned lds_wave_base) {
+  asm volatile("s_mov_b32 m0, %1\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %0, off"
+               :
+               : "v"(lane_pointer), "s"(__builtin_amdgcn_readfirstlane(lds_wave_base))
+               : "memory", "m0");
+}
+
+// Rows of 128 bytes (an index key, or the 128 query codes of a head) sit in LDS as eight 16-byte
+// pieces, piece c of row t at position c ^ Swizzle(t): the sixteen rows that the lanes of an MFMA
+// operand read together then fall into sixteen different bank groups.
+__device__ __forceinline__ int Swizzle(int row) { return (row >> 1) & 7; }
+
+// One wavefront scores 64 consecutive tokens in four groups of 16: A = query (16 heads x 32
+// elements per MFMA), B = keys (32 elements x 16 tokens), both converted to bf16 exactly; four
+// k-steps and HB head blocks. Lane (r = lane % 16, g = lane / 16) holds elements [32g, 32g + 32)
+// of head r (A) and of token r (B); a k-step takes eight of them from both, so the element order
+// inside the dot product is the same on both sides. The product leaves heads 4g .. 4g + 3 of
+// token r in lane (r, g): the weighted sum over the heads is a few additions inside the lane and
+// two lane exchanges, and lane (r, g) ends up writing the key of token 16g + r: one 128-byte
+// store per wavefront.
+// A lane that fetched its operand rows itself would touch sixteen different 128-byte lines per
+// quarter-wave (measured: 4.9 M cache accesses for 35 MB, the L1's lookup rate was the bound),
+// so keys and query come in through LDS instead: every load instruction moves eight whole rows
+// (1 KB, consecutive lanes fetch consecutive pieces), and the operand reads are LDS reads. A
+// wavefront reads only the keys it fetched itself; the query is shared by the workgroup.
 template <int HB>
 __global__ __launch_bounds__(kScoreThreads) void IndexerScoreKernel(IndexerArgs a) {
+  extern __shared__ __attribute__((aligned(16))) unsigned char lds[];
+  const unsigned lds_base = static_cast<unsigned>(reinterpret_cast<size_t>((__attribute__((address_space(3))) unsigned char*)lds));
+  constexpr int kQueryBytes = HB * 16 * kIndexDim;
   const int seq = blockIdx.y;
-  const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+  const int lane = threadIdx.x & 63, wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
   const int r = lane & 15, g = lane >> 4;
-  const int seq_len = min(a.seq_lens[seq], a.max_seq_len);
-  const int token0 = blockIdx.x * kTokensPerGroup + wave * kTokensPerWave;
-  if (seq_len <= a.sparse_count || token0 >= seq_len) return;  // short sequences select everything without scores
+  const int group0 = blockIdx.x * kTokensPerGroup;
+  const int token0 = group0 + wave * kTokensPerWave;
+  if (group0 >= a.max_seq_len) return;
   const int32_t* table_row = a.block_table + static_cast<int64_t>(seq) * a.table_stride;
+  // Rounds of loads, each behind the one it depends on and nothing else: the sequence length, the
+  // table entries, the query and the weights together; then the keys; the scores leave last.
+  const int raw_len = a.seq_lens[seq];
+  const int limit = a.max_seq_len;  // the caller's table rows address at least this many positions (checked on the host)
 
+  // Query codes: HB * 16 rows, eight per load instruction, the instructions dealt to the waves.
+  for (int j = wave; j < 2 * HB; j += kScoreThreads / 64) {
+    const int head = 8 * j + (lane >> 3);
+    const char* src = a.query + seq * a.query_seq_stride + head * a.query_head_stride + (((lane & 7) ^ Swizzle(head)) << 4);
+    DirectLoad16PerLane(src, lds_base + j * 1024);
+  }
+  // wave-uniform: whether the weight and scale rows of every sequence start on 8 and 16 bytes
+  const bool rows_aligned = ((reinterpret_cast<uintptr_t>(a.weights) | static_cast<uintptr_t>(a.weights_seq_stride)) & 7) == 0 &&
+                            ((reinterpret_cast<uintptr_t>(a.query_scale) | static_cast<uintptr_t>(a.query_scale_seq_stride) * 4) & 15) == 0;
+  float w[HB][4];  // heads 16 hb + 4 g + j: the rows this lane holds of every product
+#pragma unroll
+  for (int hb = 0; hb < HB; ++hb) {
+    // four consecutive heads: 8 bytes of weights, 16 bytes of scales
+    const char* weights = a.weights + seq * a.weights_seq_stride + (16 * hb + 4 * g) * 2;
+    const float* scales = a.query_scale + seq * a.query_scale_seq_stride + 16 * hb + 4 * g;
+    if (rows_aligned) {
+      const u32x2 pair = *reinterpret_cast<const u32x2*>(weights);
+      const f32x4 four = *reinterpret_cast<const f32x4*>(scales);
+      w[hb][0] = Bf16BitsToF32(pair.x & 0xffffu) * four[0];
+      w[hb][1] = Bf16BitsToF32(pair.x >> 16) * four[1];
+      w[hb][2] = Bf16BitsToF32(pair.y & 0xffffu) * four[2];
+      w[hb][3] = Bf16BitsToF32(pair.y >> 16) * four[3];
+    } else {
+#pragma unroll
+      for (int j = 0; j < 4; ++j) w[hb][j] = Bf16BitsToF32(reinterpret_cast<const unsigned short*>(weights)[j]) * scales[j];
+    }
+  }
+
+  // Where this wave's tokens live: lane L needs token L / 8 + 8 i for load i and token L for its
+  // scale. With blocks of at least 64 tokens the 64 tokens span at most two table entries.
+  const bool wave_in_range = token0 < limit;
+  const bool two_entries = a.block_size >= kTokensPerWave && token0 + kTokensPerWave <= limit;
+  int logical0 = 0, slot0 = 0, entry0 = 0, entry1 = 0;
+  if (two_entries) {
+    logical0 = token0 / a.block_size;
+    slot0 = token0 - logical0 * a.block_size;
+    entry0 = table_row[logical0];
+    entry1 = table_row[min(logical0 + 1, a.table_stride - 1)];
+    entry0 = static_cast<unsigned>(entry0) < static_cast<unsigned>(a.num_blocks) ? entry0 : 0;
+    entry1 = static_cast<unsigned>(entry1) < static_cast<unsigned>(a.num_blocks) ? entry1 : 0;
+  }
+  const auto locate = [&](int offset, int* block, int* slot) __attribute__((always_inline)) {
+    if (two_entries) {
+      const int at = slot0 + offset;
+      const bool next = at >= a.block_size;
+      *block = next ? entry1 : entry0;
+      *slot = next ? at - a.block_size : at;
+    } else {
+      LocateToken(a, table_row, token0 + offset, limit, block, slot);
+    }
+  };
+
+  const int seq_len = min(raw_len, a.max_seq_len);
+  if (seq_len <= a.sparse_count || group0 >= seq_len) {  // the whole workgroup; short sequences select everything without scores
+    asm volatile("s_waitcnt vmcnt(0)" ::: "memory");  // no load may land in LDS that is no longer this workgroup's
+    return;
+  }
+
+  const unsigned key_lds = lds_base + kQueryBytes + wave * (kTokensPerWave * kIndexDim);
+  float my_scale = 0.0f;  // of token token0 + lane
+  if (wave_in_range && token0 < seq_len) {
+    if (two_entries && slot0 + kTokensPerWave <= a.block_size) {
+      // the usual case, all 64 tokens in one block: one address, a constant step between the loads
+      const char* src = a.key_base + entry0 * a.key_block_stride + (slot0 + (lane >> 3)) * a.key_row_stride;
+      const int64_t step = 8 * a.key_row_stride;
+#pragma unroll
+      for (int i = 0; i < 8; ++i) {
+        DirectLoad16PerLane(src + i * step + (((lane & 7) ^ Swizzle(8 * i + (lane >> 3))) << 4), key_lds + i * 1024);
+      }
+    } else {
+#pragma unroll
+      for (int i = 0; i < 8; ++i) {
+        const int t = 8 * i + (lane >> 3);
+        int block, slot;
+        locate(t, &block, &slot);
+        const char* src = a.key_base + block * a.key_block_stride + slot * a.key_row_stride + (((lane & 7) ^ Swizzle(t)) << 4);
+        DirectLoad16PerLane(src, key_lds + i * 1024);
+      }
+    }
+    int block, slot;
+    locate(lane, &block, &slot);
+    my_scale = a.key_scale_base[block * a.key_scale_block_stride + slot];
+  }
+  // Loads return in issue order: query, keys (two loads per group of 16 tokens), the scale. A
+  // group is scored while the later ones are still on their way.
+  asm volatile("s_waitcnt vmcnt(7)" ::: "memory");
+  __syncthreads();  // the query rows the other waves fetched
+  if (token0 >= seq_len) return;
+
+  const unsigned char* q_lds = lds;
+  const unsigned char* k_lds = lds + kQueryBytes + wave * (kTokensPerWave * kIndexDim);
   bf16x8 q[HB][4];
-  float w[HB];
 #pragma unroll
   for (int hb = 0; hb < HB; ++hb) {
     const int head = 16 * hb + r;
-    const char* src = a.query + seq * a.query_seq_stride + head * a.query_head_stride + 32 * g;
-    const u32x4 lo = *reinterpret_cast<const u32x4*>(src), hi = *reinterpret_cast<const u32x4*>(src + 16);
+    const u32x4 lo = *reinterpret_cast<const u32x4*>(q_lds + head * kIndexDim + (((2 * g) ^ Swizzle(head)) << 4));
+    const u32x4 hi = *reinterpret_cast<const u32x4*>(q_lds + head * kIndexDim + (((2 * g + 1) ^ Swizzle(head)) << 4));
     q[hb][0] = CodesToBf16(lo.x, lo.y);
     q[hb][1] = CodesToBf16(lo.z, lo.w);
     q[hb][2] = CodesToBf16(hi.x, hi.y);
     q[hb][3] = CodesToBf16(hi.z, hi.w);
-    const unsigned short weight = *reinterpret_cast<const unsigned short*>(a.weights + seq * a.weights_seq_stride + head * 2);
-    w[hb] = Bf16BitsToF32(weight) * a.query_scale[seq * a.query_scale_seq_stride + head];
   }
-
-  u32x4 k_lo[4], k_hi[4];
-  float k_scale[4];  // of token 16 rg + r, fetched with its key so that no load depends on the MFMA results
+  float mine = 0.0f;  // score of token 16 g + r before its key scale
 #pragma unroll
   for (int rg = 0; rg < 4; ++rg) {
-    int block, slot;
-    LocateToken(a, table_row, token0 + 16 * rg + r, seq_len, &block, &slot);
-    const char* src = a.key_base + block * a.key_block_stride + slot * a.key_row_stride + 32 * g;
-    k_lo[rg] = __builtin_nontemporal_load(reinterpret_cast<const u32x4*>(src));
-    k_hi[rg] = __builtin_nontemporal_load(reinterpret_cast<const u32x4*>(src + 16));
-    k_scale[rg] = a.key_scale_base[block * a.key_scale_block_stride + slot];
-  }
-#pragma unroll
-  for (int rg = 0; rg < 4; ++rg) {
-    const bf16x8 k[4] = {CodesToBf16(k_lo[rg].x, k_lo[rg].y), CodesToBf16(k_lo[rg].z, k_lo[rg].w),
-                         CodesToBf16(k_hi[rg].x, k_hi[rg].y), CodesToBf16(k_hi[rg].z, k_hi[rg].w)};
-    // lane (r, g) ends up with sum over its head column of w * relu(q . k) for tokens 4g + j
-    float sum[4] = {0.0f, 0.0f, 0.0f, 0.0f};
+    if (rg == 1) asm volatile("s_waitcnt vmcnt(5)" ::: "memory");
+    if (rg == 2) asm volatile("s_waitcnt vmcnt(3)" ::: "memory");
+    if (rg == 3) asm volatile("s_waitcnt vmcnt(1)" ::: "memory");
+    const int t = 16 * rg + r;
+    const u32x4 lo = *reinterpret_cast<const u32x4*>(k_lds + t * kIndexDim + (((2 * g) ^ Swizzle(t)) << 4));
+    const u32x4 hi = *reinterpret_cast<const u32x4*>(k_lds + t * kIndexDim + (((2 * g + 1) ^ Swizzle(t)) << 4));
+    const bf16x8 k[4] = {CodesToBf16(lo.x, lo.y), CodesToBf16(lo.z, lo.w), CodesToBf16(hi.x, hi.y), CodesToBf16(hi.z, hi.w)};
+    float sum[2] = {0.0f, 0.0f};  // heads 4g + {0, 2} and 4g + {1, 3} of every block, token 16 rg + r
 #pragma unroll
     for (int hb = 0; hb < HB; ++hb) {
       f32x4 acc = {0.0f, 0.0f, 0.0f, 0.0f};
 #pragma unroll
-      for (int s = 0; s < 4; ++s) acc = __builtin_amdgcn_mfma_f32_16x16x32_bf16(k[s], q[hb][s], acc, 0, 0, 0);
+      for (int s = 0; s < 4; ++s) acc = __builtin_amdgcn_mfma_f32_16x16x32_bf16(q[hb][s], k[s], acc, 0, 0, 0);
 #pragma unroll
-      for (int j = 0; j < 4; ++j) sum[j] = __builtin_fmaf(fmaxf(acc[j], 0.0f), w[hb], sum[j]);
+      for (int j = 0; j < 4; ++j) sum[j & 1] = __builtin_fmaf(fmaxf(acc[j], 0.0f), w[hb][j], sum[j & 1]);
     }
-#pragma unroll
-    for (int j = 0; j < 4; ++j) {
-#pragma unroll
-      for (int offset = 1; offset < 16; offset <<= 1) sum[j] += __shfl_xor(sum[j], offset);
-    }
-    // lanes r < 4 of each group finish token 4g + r, whose scale lane 4g + r holds
-    const int token = token0 + 16 * rg + 4 * g + r;
-    const float scale = __shfl(k_scale[rg], (4 * g + r) & 15);
-    if (r < 4 && token < seq_len) {
-      const float mine = r == 0 ? sum[0] : r == 1 ? sum[1] : r == 2 ? sum[2] : sum[3];
-      a.keys[seq * a.keys_stride + token] = static_cast<unsigned short>(ScoreKey(mine * scale));
-    }
+    const float total = SumAcrossGroups(sum[0] + sum[1]);  // every lane (r, *) has token 16 rg + r
+    if (rg == g) mine = total;
   }
+  const int token = token0 + lane;  // = token0 + 16 g + r
+  if (token < seq_len) a.keys[seq * a.keys_stride + token] = static_cast<unsigned short>(ScoreKey(mine * my_scale));
 }
 
 constexpr int kSelectThreads = 1024;
@@ -287,6 +403,17 @@ __global__ __launch_bounds__(kSelectThreads) void IndexerSelectKernel(IndexerArg
   }
 }
 
+template <int HB>
+hipError_t LaunchScore(const IndexerArgs& args, const dim3& grid, hipStream_t stream) {
+  constexpr int kLdsBytes = HB * 16 * kIndexDim + kTokensPerGroup * kIndexDim;  // query codes + the keys of eight waves
+  // Dynamic LDS above 64 KB needs the attribute once per kernel and process.
+  static const hipError_t prepared = hipFuncSetAttribute(reinterpret_cast<const void*>(&IndexerScoreKernel<HB>),
+                                                         hipFuncAttributeMaxDynamicSharedMemorySize, kLdsBytes);
+  if (prepared != hipSuccess) return prepared;
+  hipLaunchKernelGGL(IndexerScoreKernel<HB>, grid, dim3(kScoreThreads), kLdsBytes, stream, args);
+  return hipGetLastError();
+}
+
 }  // namespace
 
 hipError_t LaunchIndexer(const IndexerArgs& args, hipStream_t stream) {
@@ -294,14 +421,14 @@ hipError_t LaunchIndexer(const IndexerArgs& args, hipStream_t stream) {
   const int groups = (args.max_seq_len + kTokensPerGroup - 1) / kTokensPerGroup;
   if (args.max_seq_len > args.sparse_count) {
     const dim3 grid(groups, args.batch);
+    hipError_t e;
     switch (args.heads / 16) {
-      case 1: hipLaunchKernelGGL(IndexerScoreKernel<1>, grid, dim3(kScoreThreads), 0, stream, args); break;
-      case 2: hipLaunchKernelGGL(IndexerScoreKernel<2>, grid, dim3(kScoreThreads), 0, stream, args); break;
-      case 3: hipLaunchKernelGGL(IndexerScoreKernel<3>, grid, dim3(kScoreThreads), 0, stream, args); break;
-      case 4: hipLaunchKernelGGL(IndexerScoreKernel<4>, grid, dim3(kScoreThreads), 0, stream, args); break;
+      case 1: e = LaunchScore<1>(args, grid, stream); break;
+      case 2: e = LaunchScore<2>(args, grid, stream); break;
+      case 3: e = LaunchScore<3>(args, grid, stream); break;
+      case 4: e = LaunchScore<4>(args, grid, stream); break;
       default: return hipErrorInvalidValue;
     }
-    const hipError_t e = hipGetLastError();
     if (e != hipSuccess) return e;
   }
   hipLaunchKernelGGL(IndexerSelectKernel, dim3(args.batch), dim3(kSelectThreads), 0, stream, args);
