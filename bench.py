@@ -38,10 +38,10 @@ ROW_BYTES = ROW * 2
 
 
 def sustained_us(torch, fn, min_iters, warm_ms=250.0, timed_ms=100.0):
-    """Average microseconds per fn(i) launch with the shader clock settled: the clock climbs for
-    some 100 ms under load (the long attention shape measured 284 us per launch over 2 launches,
-    254 over 32, 227 over 512), so the launches run back to back for `warm_ms` before the timed
-    ones, which then cover at least `timed_ms`."""
+    """Average microseconds per fn(i) launch once the device has settled: launches get faster for
+    some 100 ms of sustained load (the long attention shape measured 284 us per launch over 2
+    launches, 254 over 32, 227 over 512; most likely clock and power management), so the launches
+    run back to back for `warm_ms` before the timed ones, which then cover at least `timed_ms`."""
     def run(n):
         start, stop = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
         start.record()
