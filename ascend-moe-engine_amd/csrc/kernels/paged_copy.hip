@@ -283,64 +283,86 @@ __device__ __forceinline__ void RotateQueryHeads(const NormRopeAppendArgs& n, in
   Store16(q, out);
 }
 
-template <bool FP8>
+// R rows per wavefront when no query heads ride along: a row's table loads wait for its position,
+// so a wavefront spends two memory latencies on a row, and two rows share them.
+template <bool FP8, int R>
 __global__ __launch_bounds__(kThreads) void NormRopeAppendKernel(NormRopeAppendArgs n) {
   static_assert(kRopeDim == kWave && kLatentDim == 8 * kWave, "lane = 8 latent + 1 rope element");
   const AppendArgs& a = n.append;
   const int lane = threadIdx.x & (kWave - 1);
   const int wave_item = blockIdx.x * kWavesPerGroup + (threadIdx.x >> 6);
-  const int token = wave_item / n.items_per_token;
-  const int sub_item = wave_item - token * n.items_per_token;
-  if (token >= a.num_tokens) return;
+  const int item_token = wave_item / n.items_per_token;  // items_per_token == 1 whenever R > 1
+  const int sub_item = wave_item - item_token * n.items_per_token;
+  const int token0 = Uniform(item_token * R);
+  if (token0 >= a.num_tokens) return;
   if (sub_item > 0) {
-    RotateQueryHeads(n, token, (sub_item - 1) * kQueryHeadsPerItem, lane);
+    RotateQueryHeads(n, token0, (sub_item - 1) * kQueryHeadsPerItem, lane);
     return;
   }
-  const char* row = n.kv_a + token * n.kv_a_row_stride;
-  const u32x4 lv = Load16(row + lane * 16);
   const u32x4 gv = *reinterpret_cast<const u32x4*>(n.gamma + lane * 16);
-  const float r = Bf16ToF32(*reinterpret_cast<const unsigned short*>(row + kLatentDim * 2 + lane * 2));
-  const int position = Uniform(n.positions[token]);
-  const float c = Bf16ToF32(*reinterpret_cast<const unsigned short*>(n.rope_cos + position * n.rope_table_row_stride + lane * 2));
-  const float s = Bf16ToF32(*reinterpret_cast<const unsigned short*>(n.rope_sin + position * n.rope_table_row_stride + lane * 2));
-  float x[8], g[8];
+  u32x4 lv[R];
+  unsigned short rv[R], cv[R], sv[R];
+  int slot[R];
+  bool live[R];
+#pragma unroll
+  for (int k = 0; k < R; ++k) {
+    live[k] = token0 + k < a.num_tokens;  // wave-uniform
+    const int token = live[k] ? token0 + k : token0;
+    const char* row = n.kv_a + token * n.kv_a_row_stride;
+    lv[k] = Load16(row + lane * 16);
+    rv[k] = *reinterpret_cast<const unsigned short*>(row + kLatentDim * 2 + lane * 2);
+    const int position = Uniform(n.positions[token]);
+    cv[k] = *reinterpret_cast<const unsigned short*>(n.rope_cos + position * n.rope_table_row_stride + lane * 2);
+    sv[k] = *reinterpret_cast<const unsigned short*>(n.rope_sin + position * n.rope_table_row_stride + lane * 2);
+    slot[k] = Uniform(a.slots[token]);
+  }
+  float g[8];
 #pragma unroll
   for (int i = 0; i < 4; ++i) {
-    x[2 * i] = Bf16ToF32(lv[i] & 0xffffu);
-    x[2 * i + 1] = Bf16ToF32(lv[i] >> 16);
     g[2 * i] = Bf16ToF32(gv[i] & 0xffffu);
     g[2 * i + 1] = Bf16ToF32(gv[i] >> 16);
   }
-  float sum_squares = 0.0f;
 #pragma unroll
-  for (int i = 0; i < 8; ++i) sum_squares += x[i] * x[i];
+  for (int k = 0; k < R; ++k) {
+    if (!live[k]) continue;
+    const int token = token0 + k;
+    const float r = Bf16ToF32(rv[k]), c = Bf16ToF32(cv[k]), s = Bf16ToF32(sv[k]);
+    float x[8];
 #pragma unroll
-  for (int offset = 32; offset >= 1; offset >>= 1) sum_squares += __shfl_xor(sum_squares, offset);
-  const float rstd = 1.0f / __builtin_sqrtf(sum_squares * (1.0f / kLatentDim) + n.epsilon);
-  u32x4 yv;
+    for (int i = 0; i < 4; ++i) {
+      x[2 * i] = Bf16ToF32(lv[k][i] & 0xffffu);
+      x[2 * i + 1] = Bf16ToF32(lv[k][i] >> 16);
+    }
+    float sum_squares = 0.0f;
 #pragma unroll
-  for (int i = 0; i < 4; ++i) {
-    const unsigned lo = F32ToBf16(x[2 * i] * rstd * g[2 * i]), hi = F32ToBf16(x[2 * i + 1] * rstd * g[2 * i + 1]);
-    yv[i] = lo | (hi << 16);
-    x[2 * i] = Bf16ToF32(lo);
-    x[2 * i + 1] = Bf16ToF32(hi);
-  }
-  const float partner = __shfl_xor(r, 32);
-  const unsigned rotated = F32ToBf16(lane < 32 ? r * c - partner * s : r * c + partner * s);
-  if (n.latent_out != nullptr) Store16(n.latent_out + token * n.latent_out_row_stride + lane * 16, yv);
-  if (n.rope_out != nullptr) *reinterpret_cast<unsigned short*>(n.rope_out + token * n.rope_out_row_stride + lane * 2) = static_cast<unsigned short>(rotated);
-  const int slot = Uniform(a.slots[token]);
-  if (slot < 0) return;
-  const int block = slot / a.block_size;
-  const int in_block = slot - block * a.block_size;
-  if (block >= a.num_blocks) return;
-  if (FP8) {
-    QuantizeRowAndStore(a, 0, block, in_block, lane, x, Bf16ToF32(rotated));
-  } else {
-    char* latent_dst = a.latent.base + block * a.latent.block_stride + in_block * a.latent.row_stride;
-    char* rope_dst = a.rope.base + block * a.rope.block_stride + in_block * a.rope.row_stride;
-    Store16(latent_dst + lane * 16, yv);
-    *reinterpret_cast<unsigned short*>(rope_dst + lane * 2) = static_cast<unsigned short>(rotated);
+    for (int i = 0; i < 8; ++i) sum_squares += x[i] * x[i];
+#pragma unroll
+    for (int offset = 32; offset >= 1; offset >>= 1) sum_squares += __shfl_xor(sum_squares, offset);
+    const float rstd = 1.0f / __builtin_sqrtf(sum_squares * (1.0f / kLatentDim) + n.epsilon);
+    u32x4 yv;
+#pragma unroll
+    for (int i = 0; i < 4; ++i) {
+      const unsigned lo = F32ToBf16(x[2 * i] * rstd * g[2 * i]), hi = F32ToBf16(x[2 * i + 1] * rstd * g[2 * i + 1]);
+      yv[i] = lo | (hi << 16);
+      x[2 * i] = Bf16ToF32(lo);
+      x[2 * i + 1] = Bf16ToF32(hi);
+    }
+    const float partner = __shfl_xor(r, 32);
+    const unsigned rotated = F32ToBf16(lane < 32 ? r * c - partner * s : r * c + partner * s);
+    if (n.latent_out != nullptr) Store16(n.latent_out + token * n.latent_out_row_stride + lane * 16, yv);
+    if (n.rope_out != nullptr) *reinterpret_cast<unsigned short*>(n.rope_out + token * n.rope_out_row_stride + lane * 2) = static_cast<unsigned short>(rotated);
+    if (slot[k] < 0) continue;
+    const int block = slot[k] / a.block_size;
+    const int in_block = slot[k] - block * a.block_size;
+    if (block >= a.num_blocks) continue;
+    if (FP8) {
+      QuantizeRowAndStore(a, 0, block, in_block, lane, x, Bf16ToF32(rotated));
+    } else {
+      char* latent_dst = a.latent.base + block * a.latent.block_stride + in_block * a.latent.row_stride;
+      char* rope_dst = a.rope.base + block * a.rope.block_stride + in_block * a.rope.row_stride;
+      Store16(latent_dst + lane * 16, yv);
+      *reinterpret_cast<unsigned short*>(rope_dst + lane * 2) = static_cast<unsigned short>(rotated);
+    }
   }
 }
 
@@ -546,13 +568,17 @@ hipError_t LaunchNormRopeAppend(const NormRopeAppendArgs& args, hipStream_t stre
   if (args.append.num_tokens <= 0) return hipSuccess;
   NormRopeAppendArgs launch = args;
   launch.items_per_token = 1 + (args.q_rope != nullptr ? DivUp(args.num_heads, kQueryHeadsPerItem) : 0);
-  const int64_t items = static_cast<int64_t>(args.append.num_tokens) * launch.items_per_token;
+  constexpr int kRowsAlone = 2;  // rows per wavefront when there are no query heads
+  const int rows = launch.items_per_token == 1 ? kRowsAlone : 1;
+  const int64_t items = static_cast<int64_t>(DivUp(args.append.num_tokens, rows)) * launch.items_per_token;
   if (items > 0x7fffffff - kWavesPerGroup) return hipErrorInvalidValue;  // the kernel indexes work items in 32 bits
   const dim3 grid(DivUp(static_cast<int>(items), kWavesPerGroup));
   if (args.append.fp8) {
-    hipLaunchKernelGGL(NormRopeAppendKernel<true>, grid, dim3(kThreads), 0, stream, launch);
+    if (rows == 1) hipLaunchKernelGGL((NormRopeAppendKernel<true, 1>), grid, dim3(kThreads), 0, stream, launch);
+    else hipLaunchKernelGGL((NormRopeAppendKernel<true, kRowsAlone>), grid, dim3(kThreads), 0, stream, launch);
   } else {
-    hipLaunchKernelGGL(NormRopeAppendKernel<false>, grid, dim3(kThreads), 0, stream, launch);
+    if (rows == 1) hipLaunchKernelGGL((NormRopeAppendKernel<false, 1>), grid, dim3(kThreads), 0, stream, launch);
+    else hipLaunchKernelGGL((NormRopeAppendKernel<false, kRowsAlone>), grid, dim3(kThreads), 0, stream, launch);
   }
   return hipGetLastError();
 }
