@@ -41,7 +41,7 @@ def _codes(rng, shape, spread):
     return (magnitude | (rng.integers(0, 2, shape).astype(np.uint8) << 7)).astype(np.uint8)
 
 
-def _run(seq_lens, bs, heads, k, seed, zero_query=False):
+def _run(seq_lens, bs, heads, k, seed, zero_query=False, row_padding=0):
     rng = np.random.default_rng(seed)
     batch = len(seq_lens)
     max_len = max(max(seq_lens), 1)
@@ -57,13 +57,19 @@ def _run(seq_lens, bs, heads, k, seed, zero_query=False):
     keys_d = torch.as_tensor(key_plane, device="cuda")
     scales_d = torch.as_tensor(key_scale, device="cuda")
     view = ffi.IndexKeyView(keys_d.data_ptr(), bs * D, D, scales_d.data_ptr(), bs, blocks, bs, D, 0)
-    query_d, weights_d, q_scale_d = torch.as_tensor(query, device="cuda"), weights.cuda(), torch.as_tensor(q_scale, device="cuda")
+    query_d = torch.as_tensor(query, device="cuda")
+    # `row_padding` extra elements behind every sequence's weights and scales: rows that do not
+    # start on 8 / 16 bytes take the kernel's element-wise loads
+    weights_d = torch.zeros(batch, heads + row_padding, dtype=torch.bfloat16, device="cuda")
+    weights_d[:, :heads] = weights.cuda()
+    q_scale_d = torch.zeros(batch, heads + row_padding, dtype=torch.float32, device="cuda")
+    q_scale_d[:, :heads] = torch.as_tensor(q_scale, device="cuda")
     table_d, lens_d = kt.dev_i32(table), kt.dev_i32(seq_lens)
     out = torch.full((batch, k), -7, dtype=torch.int32, device="cuda")
     ws_bytes = int(lib.mlakvIndexerWorkspaceBytes(batch, max_len))
     workspace = torch.zeros(max(ws_bytes, 16), dtype=torch.uint8, device="cuda")
-    ffi.check(lib.mlakvLightningIndexer(C.byref(view), query_d.data_ptr(), heads * D, D, weights_d.data_ptr(), heads * 2,
-                                        q_scale_d.data_ptr(), heads, heads, table_d.data_ptr(), table.shape[1], lens_d.data_ptr(),
+    ffi.check(lib.mlakvLightningIndexer(C.byref(view), query_d.data_ptr(), heads * D, D, weights_d.data_ptr(), (heads + row_padding) * 2,
+                                        q_scale_d.data_ptr(), heads + row_padding, heads, table_d.data_ptr(), table.shape[1], lens_d.data_ptr(),
                                         batch, max_len, k, out.data_ptr(), k, workspace.data_ptr(), workspace.numel(),
                                         kt.stream_ptr()))
     torch.cuda.synchronize()
@@ -103,6 +109,10 @@ def _run(seq_lens, bs, heads, k, seed, zero_query=False):
 @pytest.mark.parametrize("bs,heads,k", [(64, 64, 512), (16, 32, 100), (128, 16, 2048), (64, 48, 64)])
 def test_indexer_matches_oracle_ragged(bs, heads, k):
     _run([3000, 513 if k == 512 else k + 1, 1, 0, 2600, k, 777], bs, heads, k, seed=101)
+
+
+def test_weight_and_scale_rows_need_no_alignment():
+    _run([900, 300, 1200], 64, 32, 128, seed=105, row_padding=1)
 
 
 def test_all_equal_scores_select_the_first_positions():
