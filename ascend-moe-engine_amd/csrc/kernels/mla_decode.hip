@@ -55,14 +55,14 @@
 
 #pragma clang diagnostic ignored "-Winline-asm"
 
-// Development timeline (built only with -DMLAKV_ATTN_TRACE): lane 0 of waves 0 and 4 of every
+// Development timeline (built only with -DMLAKV_ATTN_TRACE): lane 0 of every wave of every
 // workgroup stamps the 100 MHz wall clock into a caller-provided buffer.
 #ifdef MLAKV_ATTN_TRACE
 #include <cstdlib>
 #define MLAKV_STAMP(slot)                                                                              \
   do {                                                                                                 \
-    if (a.trace != nullptr && lane == 0 && (wave == 0 || wave == 4) && (slot) >= 0 && (slot) < 40) {                     \
-      a.trace[((blockIdx.y * gridDim.x + blockIdx.x) * 2 + (wave >> 2)) * 40 + (slot)] = __builtin_amdgcn_s_memrealtime(); \
+    if (a.trace != nullptr && lane == 0 && (slot) >= 0 && (slot) < 40) {                                                 \
+      a.trace[((blockIdx.y * gridDim.x + blockIdx.x) * 8 + wave) * 40 + (slot)] = __builtin_amdgcn_s_memrealtime();       \
     }                                                                                                  \
   } while (0)
 #else
