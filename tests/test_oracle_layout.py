@@ -41,7 +41,7 @@ def test_ledger_goldens_sizes_and_blocks(oracle, goldens):
         assert oracle.kvo_backbone_device_bytes(512, 64, bs, ctx) == entry["backbone_device_bytes"]
         assert ffi.load().mlakvBackboneDeviceBytes(512, 64, bs, ctx) == entry["backbone_device_bytes"]
         assert entry["total_blocks_allocated"] == entry["num_blocks"] * 43
-    # the values the survey of the reference recorded from its own dry runs
+    # values the reference records from its own dry runs (docs/examples/inference_diagnostics_dry_run.json and the arena ledger)
     by_key = {(e["block_size"], e["max_context"]): e for e in goldens["ledger"]}
     assert by_key[(64, 8192)]["kv"]["kv.latent_cache"]["bytes"] == 360710144
     assert by_key[(64, 8192)]["kv"]["kv.rope_cache"]["bytes"] == 45088768
