@@ -323,21 +323,32 @@ void KvCacheManager::UploadStep(void* stream) {
   MOE_HIP_REQUIRE(bound_, "UploadStep before Bind");
   RefreshSeqLens();
   IDeviceBackend& backend = arena_.backend();
-  const int k = staging_next_;
-  staging_next_ ^= 1;
-  if (staging_busy_[k]) backend.SynchronizeEvent(staging_event_[k]);  // copy from two steps ago
-  uint8_t* staging = static_cast<uint8_t*>(staging_[k]);
   const size_t table_bytes = host_table_.size() * sizeof(int32_t);
   const size_t small_bytes = host_small_.size() * sizeof(int32_t);
-  if (table_dirty_) {
-    std::memcpy(staging, host_table_.data(), table_bytes);
-    backend.MemcpyAsync(d_table_, arena_.Bytes(h_table_), staging, table_bytes, CopyKind::kHostToDevice, stream);
-    table_dirty_ = false;
+  // The usual step changes only the small arrays (slot mapping, lengths, their prefix sums). On
+  // a device that runs kernels they ride in the argument block of a one-workgroup kernel: no
+  // pinned staging, no copy engine and no event per step, which together cost more stream time
+  // than the append itself.
+  const bool by_kernel = backend.runs_kernels() && !table_dirty_ && host_small_.size() <= static_cast<size_t>(mlakv::kMaxStoreWords);
+  if (by_kernel) {
+    const hipError_t e = mlakv::LaunchStoreWords(host_small_.data(), static_cast<int>(host_small_.size()),
+                                                 static_cast<int32_t*>(d_small_), static_cast<hipStream_t>(stream));
+    MOE_HIP_REQUIRE(e == hipSuccess, "UploadStep: metadata kernel launch failed");
+  } else {
+    const int k = staging_next_;
+    staging_next_ ^= 1;
+    if (staging_busy_[k]) backend.SynchronizeEvent(staging_event_[k]);  // copy from two steps ago
+    uint8_t* staging = static_cast<uint8_t*>(staging_[k]);
+    if (table_dirty_) {
+      std::memcpy(staging, host_table_.data(), table_bytes);
+      backend.MemcpyAsync(d_table_, arena_.Bytes(h_table_), staging, table_bytes, CopyKind::kHostToDevice, stream);
+      table_dirty_ = false;
+    }
+    std::memcpy(staging + table_bytes, host_small_.data(), small_bytes);
+    backend.MemcpyAsync(d_small_, small_bytes, staging + table_bytes, small_bytes, CopyKind::kHostToDevice, stream);
+    backend.RecordEvent(staging_event_[k], stream);
+    staging_busy_[k] = true;
   }
-  std::memcpy(staging + table_bytes, host_small_.data(), small_bytes);
-  backend.MemcpyAsync(d_small_, small_bytes, staging + table_bytes, small_bytes, CopyKind::kHostToDevice, stream);
-  backend.RecordEvent(staging_event_[k], stream);
-  staging_busy_[k] = true;
   for (int64_t s = 0; s < config_.max_batch; ++s) host_small_[static_cast<size_t>(s)] = -1;
 }
 

@@ -163,6 +163,11 @@ hipError_t LaunchAppend(const AppendArgs& args, hipStream_t stream);
 hipError_t LaunchNormRopeAppend(const NormRopeAppendArgs& args, hipStream_t stream);
 hipError_t LaunchGather(const GatherArgs& args, hipStream_t stream);
 hipError_t LaunchCopyBlocks(const CopyBlocksArgs& args, hipStream_t stream);
+// Writes `count` (<= kMaxStoreWords) 32-bit words to device memory at `dst`. The words travel in
+// the kernel's argument block, which the runtime copies when the launch is queued: the caller's
+// buffer is free again on return, with no staging buffer, copy engine or event involved.
+constexpr int kMaxStoreWords = 960;
+hipError_t LaunchStoreWords(const int32_t* host_words, int count, int32_t* dst, hipStream_t stream);
 hipError_t LaunchAttnDecode(const AttnArgs& args, hipStream_t stream);
 hipError_t LaunchMxQuant(const MxQuantArgs& args, hipStream_t stream);
 hipError_t LaunchIndexer(const IndexerArgs& args, hipStream_t stream);

@@ -550,6 +550,16 @@ int RowsPerItem(int block_size, int want) {
 
 int DivUp(int a, int b) { return (a + b - 1) / b; }
 
+// ---- per-step metadata ---------------------------------------------------------
+
+struct StoreWordsArgs {
+  int32_t words[kMaxStoreWords];
+};
+
+__global__ __launch_bounds__(kThreads) void StoreWordsKernel(StoreWordsArgs args, int count, int32_t* dst) {
+  for (int i = threadIdx.x; i < count; i += kThreads) dst[i] = args.words[i];
+}
+
 }  // namespace
 
 hipError_t LaunchAppend(const AppendArgs& args, hipStream_t stream) {
@@ -602,6 +612,15 @@ hipError_t LaunchGather(const GatherArgs& args, hipStream_t stream) {
   } else {
     hipLaunchKernelGGL(GatherBf16Kernel, grid, dim3(kThreads), 0, stream, args, rows_per_item);
   }
+  return hipGetLastError();
+}
+
+hipError_t LaunchStoreWords(const int32_t* host_words, int count, int32_t* dst, hipStream_t stream) {
+  if (count <= 0) return hipSuccess;
+  if (count > kMaxStoreWords || host_words == nullptr || dst == nullptr) return hipErrorInvalidValue;
+  StoreWordsArgs args;
+  for (int i = 0; i < count; ++i) args.words[i] = host_words[i];
+  hipLaunchKernelGGL(StoreWordsKernel, dim3(1), dim3(kThreads), 0, stream, args, count, dst);
   return hipGetLastError();
 }
 
