@@ -607,6 +607,38 @@ mlakvStatus mlakvLightningIndexer(const mlakvIndexKeyView* keys, const void* que
   return status == hipSuccess ? MLAKV_SUCCESS : HipFail(status, who);
 }
 
+mlakvStatus mlakvIndexKeyAppend(const mlakvIndexKeyView* keys, const void* k, int64_t k_row_stride,
+                                const int32_t* slot_mapping, int32_t num_tokens, void* stream) {
+  const char* who = "mlakvIndexKeyAppend";
+  if (keys == nullptr || keys->keys == nullptr || keys->scales == nullptr) return Fail(MLAKV_ERR_PARAM_NULLPTR, "%s: the index key pool is required", who);
+  if (num_tokens < 0) return Fail(MLAKV_ERR_PARAM_INVALID, "%s: negative num_tokens", who);
+  if (num_tokens == 0) return MLAKV_SUCCESS;
+  if (k == nullptr || slot_mapping == nullptr) return Fail(MLAKV_ERR_PARAM_NULLPTR, "%s: rows and slot mapping are required", who);
+  if (keys->dim != 128) return Fail(MLAKV_ERR_PARAM_INVALID, "%s: index keys have 128 elements, not %d", who, keys->dim);
+  if (keys->num_blocks <= 0 || keys->block_size <= 0) return Fail(MLAKV_ERR_PARAM_INVALID, "%s: the pool needs blocks of a positive size", who);
+  if (!Aligned16(keys->keys) || keys->row_stride % 16 != 0 || keys->block_stride % 16 != 0 || keys->row_stride < 128 ||
+      reinterpret_cast<uintptr_t>(keys->scales) % 4 != 0) {
+    return Fail(MLAKV_ERR_PARAM_INVALID, "%s: key rows must be 16-byte aligned and hold 128 bytes", who);
+  }
+  if (!Aligned16(k) || k_row_stride % 16 != 0 || k_row_stride < 256) {
+    return Fail(MLAKV_ERR_PARAM_INVALID, "%s: source rows must be 16-byte aligned and hold 128 bf16 values", who);
+  }
+  mlakv::IndexKeyAppendArgs args{};
+  args.key_base = static_cast<char*>(const_cast<void*>(keys->keys));
+  args.key_block_stride = keys->block_stride;
+  args.key_row_stride = keys->row_stride;
+  args.key_scale_base = const_cast<float*>(keys->scales);
+  args.key_scale_block_stride = keys->scale_block_stride;
+  args.num_blocks = keys->num_blocks;
+  args.block_size = keys->block_size;
+  args.src = static_cast<const char*>(k);
+  args.src_row_stride = k_row_stride;
+  args.slots = slot_mapping;
+  args.num_tokens = num_tokens;
+  const hipError_t status = mlakv::LaunchIndexKeyAppend(args, static_cast<hipStream_t>(stream));
+  return status == hipSuccess ? MLAKV_SUCCESS : HipFail(status, who);
+}
+
 mlakvStatus mlakvDynamicMxQuant(const void* x, int64_t x_row_stride, int64_t rows, int32_t cols, void* codes,
                                 int64_t codes_row_stride, void* scales, int64_t scales_row_stride, void* stream) {
   const char* who = "mlakvDynamicMxQuant";

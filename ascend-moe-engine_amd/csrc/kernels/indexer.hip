@@ -403,6 +403,47 @@ __global__ __launch_bounds__(kSelectThreads) void IndexerSelectKernel(IndexerArg
   }
 }
 
+// Index-key append: sixteen lanes per token (eight bf16 values each), four tokens per wavefront.
+// The row's absmax by four lane exchanges, scale = absmax / 448, codes from the correctly rounded
+// quotient (the E4M3 conversion saturates behind a clamp to +-448).
+__global__ __launch_bounds__(256) void IndexKeyAppendKernel(IndexKeyAppendArgs a) {
+  const int lane = threadIdx.x & 63;
+  const int token = (blockIdx.x * 4 + (threadIdx.x >> 6)) * 4 + (lane >> 4);
+  const int piece = lane & 15;
+  const bool real = token < a.num_tokens;
+  const int row = real ? token : a.num_tokens - 1;  // a repeated row is loaded and never stored
+  const u32x4 words = *reinterpret_cast<const u32x4*>(a.src + row * a.src_row_stride + piece * 16);
+  const int slot = a.slots[row];
+  float x[8];
+#pragma unroll
+  for (int i = 0; i < 4; ++i) {
+    x[2 * i] = Bf16BitsToF32(words[i] & 0xffffu);
+    x[2 * i + 1] = Bf16BitsToF32(words[i] >> 16);
+  }
+  float absmax = 0.0f;
+#pragma unroll
+  for (int i = 0; i < 8; ++i) absmax = fmaxf(absmax, fabsf(x[i]));
+#pragma unroll
+  for (int offset = 1; offset < 16; offset <<= 1) absmax = fmaxf(absmax, __shfl_xor(absmax, offset));
+  const float scale = absmax == 0.0f ? 1.0f : absmax / 448.0f;
+  u32x2 codes;
+#pragma unroll
+  for (int half = 0; half < 2; ++half) {
+    float q[4];
+#pragma unroll
+    for (int i = 0; i < 4; ++i) q[i] = fminf(fmaxf(x[4 * half + i] / scale, -448.0f), 448.0f);
+    int word = __builtin_amdgcn_cvt_pk_fp8_f32(q[0], q[1], 0, false);
+    word = __builtin_amdgcn_cvt_pk_fp8_f32(q[2], q[3], word, true);
+    codes[half] = static_cast<unsigned>(word);
+  }
+  if (!real || slot < 0) return;
+  const int block = slot / a.block_size;
+  if (block >= a.num_blocks) return;
+  const int in_block = slot - block * a.block_size;
+  *reinterpret_cast<u32x2*>(a.key_base + block * a.key_block_stride + in_block * a.key_row_stride + piece * 8) = codes;
+  if (piece == 0) a.key_scale_base[block * a.key_scale_block_stride + in_block] = scale;
+}
+
 template <int HB>
 hipError_t LaunchScore(const IndexerArgs& args, const dim3& grid, hipStream_t stream) {
   constexpr int kLdsBytes = HB * 16 * kIndexDim + kTokensPerGroup * kIndexDim;  // query codes + the keys of eight waves
@@ -415,6 +456,12 @@ hipError_t LaunchScore(const IndexerArgs& args, const dim3& grid, hipStream_t st
 }
 
 }  // namespace
+
+hipError_t LaunchIndexKeyAppend(const IndexKeyAppendArgs& args, hipStream_t stream) {
+  if (args.num_tokens <= 0) return hipSuccess;
+  hipLaunchKernelGGL(IndexKeyAppendKernel, dim3((args.num_tokens + 15) / 16), dim3(256), 0, stream, args);
+  return hipGetLastError();
+}
 
 hipError_t LaunchIndexer(const IndexerArgs& args, hipStream_t stream) {
   if (args.batch <= 0) return hipSuccess;

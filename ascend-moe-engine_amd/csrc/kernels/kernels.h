@@ -171,6 +171,19 @@ hipError_t LaunchStoreWords(const int32_t* host_words, int count, int32_t* dst, 
 hipError_t LaunchAttnDecode(const AttnArgs& args, hipStream_t stream);
 hipError_t LaunchMxQuant(const MxQuantArgs& args, hipStream_t stream);
 hipError_t LaunchIndexer(const IndexerArgs& args, hipStream_t stream);
+
+struct IndexKeyAppendArgs {
+  char* key_base;
+  int64_t key_block_stride, key_row_stride;  // bytes
+  float* key_scale_base;
+  int64_t key_scale_block_stride;            // elements
+  int32_t num_blocks, block_size;
+  const char* src;                           // bf16 [num_tokens][128]
+  int64_t src_row_stride;                    // bytes
+  const int32_t* slots;
+  int32_t num_tokens;
+};
+hipError_t LaunchIndexKeyAppend(const IndexKeyAppendArgs& args, hipStream_t stream);
 // One-time per-process kernel attribute setup (dynamic LDS above 64 KB).
 hipError_t PrepareAttnKernels();
 

@@ -96,6 +96,7 @@ PROTOTYPES = {
     "mlakvAttnDecodeSparse": (_i32, [_P(AttnPlan), _P(CacheView), _i32, _vp, _i64, _i64, _vp, _i64, _i64, _vp, _i32, _vp, _vp, _i64,
                                      C.c_double, _vp, _i64, _i64, _vp, _vp, _u64, _vp]),
     "mlakvIndexerWorkspaceBytes": (_u64, [_i32, _i32]),
+    "mlakvIndexKeyAppend": (_i32, [_P(IndexKeyView), _vp, _i64, _vp, _i32, _vp]),
     "mlakvLightningIndexer": (_i32, [_P(IndexKeyView), _vp, _i64, _i64, _vp, _i64, _vp, _i64, _i32, _vp, _i32, _vp, _i32, _i32, _i32,
                                      _vp, _i64, _vp, _u64, _vp]),
     "mlakvDynamicMxQuant": (_i32, [_vp, _i64, _i64, _i32, _vp, _i64, _vp, _i64, _vp]),

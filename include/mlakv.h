@@ -246,6 +246,16 @@ typedef struct mlakvIndexKeyView {
   int32_t num_blocks, block_size, dim, reserved;
 } mlakvIndexKeyView;
 uint64_t mlakvIndexerWorkspaceBytes(int32_t batch, int32_t max_seq_len);
+/* Writes index keys into that pool: row t of `k` (bf16 [num_tokens][128], stride in bytes) is
+ * quantised like a row of the FP8 KV cache (scale = absmax / 448 in fp32, 1.0 for a zero row;
+ * code = E4M3 of the correctly rounded x / scale, saturating) and lands at slot_mapping[t] =
+ * block * block_size + slot of the pool (`keys->keys` and `keys->scales` are written through); a
+ * negative slot or a block outside the pool skips the row, as in mlakvAppend. The reference has no
+ * such stage (it reserves no index-key pool, src/pipeline/pipeline.cpp:576-578): the write side of
+ * the vendored operator's key input (third_party/ops_transformer/attention/quant_lightning_indexer,
+ * key + key_dequant_scale, "PA_BSND"), for callers that keep the keys paged beside the KV cache. */
+mlakvStatus mlakvIndexKeyAppend(const mlakvIndexKeyView* keys, const void* k, int64_t k_row_stride,
+                                const int32_t* slot_mapping, int32_t num_tokens, void* stream);
 mlakvStatus mlakvLightningIndexer(const mlakvIndexKeyView* keys, const void* query, int64_t query_seq_stride,
                                   int64_t query_head_stride, const void* weights, int64_t weights_seq_stride,
                                   const float* query_dequant_scale, int64_t query_scale_seq_stride, int32_t heads,

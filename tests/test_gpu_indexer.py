@@ -115,6 +115,39 @@ def test_weight_and_scale_rows_need_no_alignment():
     _run([900, 300, 1200], 64, 32, 128, seed=105, row_padding=1)
 
 
+@pytest.mark.parametrize("bs", [16, 64])
+def test_index_key_append_matches_the_oracle_quantiser(bs):
+    """The write side of the key pool: bit-exact with the oracle's E4M3 row quantiser (the one the
+    FP8 KV cache is pinned with) at 128 elements per row; untouched slots stay as they were."""
+    rng = np.random.default_rng(131)
+    tokens, blocks = 203, 9 if bs == 64 else 30
+    rows = kt.randn_bf16((tokens, D), seed=132, outlier_fraction=0.02)
+    rows[7] = 0                                  # a zero row: scale 1, zero codes
+    rows[11, 5] = 1e30                           # one huge value: the rest of the row rounds to zero codes
+    slots = rng.permutation(blocks * bs)[:tokens].astype(np.int32)
+    slots[3] = -1                                # skipped
+    slots[4] = blocks * bs + 5                   # a block outside the pool: skipped
+    lib = ffi.load()
+    keys_d = torch.full((blocks * bs, D), 0x11, dtype=torch.uint8, device="cuda")
+    scales_d = torch.full((blocks * bs,), 7.0, dtype=torch.float32, device="cuda")
+    view = ffi.IndexKeyView(keys_d.data_ptr(), bs * D, D, scales_d.data_ptr(), bs, blocks, bs, D, 0)
+    rows_d, slots_d = rows.cuda(), kt.dev_i32(slots)
+    ffi.check(lib.mlakvIndexKeyAppend(C.byref(view), rows_d.data_ptr(), D * 2, slots_d.data_ptr(), tokens, kt.stream_ptr()))
+    torch.cuda.synchronize()
+    want_keys = np.full(blocks * bs * D, 0x11, dtype=np.uint8)
+    want_scales = np.full(blocks * bs, 7.0, dtype=np.float32)
+    live = (slots >= 0) & (slots < blocks * bs)
+    unused = np.zeros((tokens, 1), dtype=np.uint16)
+    finite = kt.bits16(rows).copy()
+    orc.append_rows_fp8(want_keys, np.zeros(1, np.uint8), want_scales, bs, finite[live], unused[live], slots[live],
+                        latent_dim=D, rope_dim=0)
+    assert np.array_equal(keys_d.cpu().numpy().reshape(-1), want_keys)
+    assert np.array_equal(scales_d.cpu().numpy(), want_scales)
+    assert lib.mlakvIndexKeyAppend(C.byref(view), None, D * 2, slots_d.data_ptr(), tokens, kt.stream_ptr()) == ffi.ERR_PARAM_NULLPTR
+    assert lib.mlakvIndexKeyAppend(C.byref(view), rows_d.data_ptr(), D, slots_d.data_ptr(), tokens, kt.stream_ptr()) == ffi.ERR_PARAM_INVALID
+    assert lib.mlakvIndexKeyAppend(C.byref(view), rows_d.data_ptr(), D * 2, slots_d.data_ptr(), 0, kt.stream_ptr()) == 0
+
+
 def test_all_equal_scores_select_the_first_positions():
     got = _run([1000, 300], 64, 64, 256, seed=102, zero_query=True)
     assert got[0].tolist() == list(range(256)) and got[1].tolist() == list(range(256))
