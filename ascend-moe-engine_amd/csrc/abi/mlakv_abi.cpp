@@ -18,6 +18,8 @@
 #include "moe_hip/kv_cache_manager.hpp"
 #include "moe_hip/static_arena.hpp"
 
+static_assert(MLAKV_NOALLOC_SCRATCH_BYTES == mlakv::kAttnStaticScratchBytes, "header and kernel file agree on the scratch size");
+
 namespace mlakv_abi {
 
 static thread_local std::string g_last_error;
@@ -499,6 +501,29 @@ mlakvStatus mlakvAttnDecode(const mlakvAttnPlan* plan, const mlakvCacheView* cac
   return AttnDecodeImpl("mlakvAttnDecode", plan, cache, layer, q_latent, q_latent_seq_stride, q_latent_head_stride, q_rope,
                         q_rope_seq_stride, q_rope_head_stride, block_table, table_stride, seq_lens, scale, out, out_seq_stride,
                         out_head_stride, nullptr, nullptr, 0, lse, workspace, workspace_bytes, stream);
+}
+
+mlakvStatus mlakvAttnDecodeNoAlloc(const mlakvAttnPlan* plan, const mlakvCacheView* cache, int32_t layer, const void* q_latent,
+                                   int64_t q_latent_seq_stride, int64_t q_latent_head_stride, const void* q_rope,
+                                   int64_t q_rope_seq_stride, int64_t q_rope_head_stride, const int32_t* block_table,
+                                   int32_t table_stride, const int32_t* seq_lens, double scale, void* out, int64_t out_seq_stride,
+                                   int64_t out_head_stride, float* lse, void* stream) {
+  const char* who = "mlakvAttnDecodeNoAlloc";
+  if (plan == nullptr) return Fail(MLAKV_ERR_PARAM_NULLPTR, "%s: plan is null", who);
+  if (out == nullptr) return Fail(MLAKV_ERR_PARAM_NULLPTR, "%s: the output is required", who);
+  if (plan->workspace_bytes > MLAKV_NOALLOC_SCRATCH_BYTES) {
+    return Fail(MLAKV_ERR_PARAM_INVALID,
+                "%s: the plan needs %llu bytes of split-KV partials, the library's static scratch holds %llu; use "
+                "mlakvAttnDecode with a workspace of the caller's",
+                who, static_cast<unsigned long long>(plan->workspace_bytes),
+                static_cast<unsigned long long>(MLAKV_NOALLOC_SCRATCH_BYTES));
+  }
+  char* scratch = nullptr;
+  const hipError_t resolved = mlakv::AttnStaticScratch(&scratch);
+  if (resolved != hipSuccess) return HipFail(resolved, who);
+  return AttnDecodeImpl(who, plan, cache, layer, q_latent, q_latent_seq_stride, q_latent_head_stride, q_rope, q_rope_seq_stride,
+                        q_rope_head_stride, block_table, table_stride, seq_lens, scale, out, out_seq_stride, out_head_stride,
+                        nullptr, nullptr, 0, lse, scratch, mlakv::kAttnStaticScratchBytes, stream);
 }
 
 mlakvStatus mlakvAttnDecodeSparse(const mlakvAttnPlan* plan, const mlakvCacheView* cache, int32_t layer, const void* q_latent,

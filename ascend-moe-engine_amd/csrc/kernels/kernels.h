@@ -186,5 +186,10 @@ struct IndexKeyAppendArgs {
 hipError_t LaunchIndexKeyAppend(const IndexKeyAppendArgs& args, hipStream_t stream);
 // One-time per-process kernel attribute setup (dynamic LDS above 64 KB).
 hipError_t PrepareAttnKernels();
+// Device memory owned by the library for the split-KV partials of attention launches whose
+// caller brings no workspace: kAttnStaticScratchBytes per GPU, resolved on first use on the
+// current device. Launches that use it on one GPU share it.
+constexpr uint64_t kAttnStaticScratchBytes = uint64_t{24} << 20;
+hipError_t AttnStaticScratch(char** address);
 
 }  // namespace mlakv

@@ -48,6 +48,7 @@
 //
 // Chunks of one sequence are merged by a second small kernel from partials (normalised O in
 // bf16, log2-domain LSE in fp32) held in the caller's workspace.
+#include <mutex>
 #include <utility>
 
 #include "kernels.h"
@@ -1130,6 +1131,30 @@ hipError_t LaunchByCache(const AttnArgs& args, const dim3& grid, hipStream_t str
 }  // namespace
 
 hipError_t PrepareAttnKernels() { return hipSuccess; }
+
+// Split-KV partials for callers that cannot allocate: one array per GPU, held from module load to
+// process exit. In host code the array's name only stands for the symbol; its address on the
+// current device comes from hipGetSymbolAddress, once per device, and everything (kernel
+// arguments included) uses that address.
+static __device__ __align__(256) unsigned char scratch[kAttnStaticScratchBytes];
+
+hipError_t AttnStaticScratch(char** address) {
+  constexpr int kMaxDevices = 64;
+  static std::mutex guard;
+  static char* per_device[kMaxDevices] = {};
+  int device = 0;
+  if (hipError_t e = hipGetDevice(&device); e != hipSuccess) return e;
+  if (device < 0 || device >= kMaxDevices) return hipErrorInvalidDevice;
+  std::lock_guard<std::mutex> lock(guard);
+  if (per_device[device] == nullptr) {
+    void* resolved = nullptr;
+    if (hipError_t e = hipGetSymbolAddress(&resolved, HIP_SYMBOL(scratch)); e != hipSuccess) return e;
+    if (resolved == nullptr) return hipErrorInvalidSymbol;
+    per_device[device] = static_cast<char*>(resolved);
+  }
+  *address = per_device[device];
+  return hipSuccess;
+}
 
 hipError_t LaunchAttnDecode(const AttnArgs& args_in, hipStream_t stream) {
   AttnArgs args = args_in;

@@ -160,6 +160,24 @@ mlakvStatus mlakvAttnDecode(const mlakvAttnPlan* plan, const mlakvCacheView* cac
                             void* out, int64_t out_seq_stride, int64_t out_head_stride, float* lse, void* workspace,
                             uint64_t workspace_bytes, void* stream);
 
+/* mlakvAttnDecode for callers that cannot allocate device memory and have no workspace to pass
+ * (code under HIP graph capture, tight serving loops, harnesses that forbid hipMalloc). It has no
+ * counterpart in the reference, whose operators always receive the arena's shared workspace
+ * (src/memory/static_arena.cpp:270-295). The split-KV partials go to a static device array of
+ * MLAKV_NOALLOC_SCRATCH_BYTES that the library holds on every GPU it runs on until the process
+ * ends; the call allocates nothing (no hipMalloc / hipFree, no allocating library routine) and
+ * otherwise behaves like mlakvAttnDecode: same arguments without the workspace pair, same
+ * results bit for bit. A plan whose workspace_bytes exceeds MLAKV_NOALLOC_SCRATCH_BYTES is
+ * refused with MLAKV_ERR_PARAM_INVALID. The first call on a device resolves the array's address
+ * (make it outside any stream capture). All calls on one GPU share the array: launches that may
+ * overlap there (different streams without an ordering between them) race on the partials. */
+#define MLAKV_NOALLOC_SCRATCH_BYTES (24ull << 20)
+mlakvStatus mlakvAttnDecodeNoAlloc(const mlakvAttnPlan* plan, const mlakvCacheView* cache, int32_t layer,
+                                   const void* q_latent, int64_t q_latent_seq_stride, int64_t q_latent_head_stride,
+                                   const void* q_rope, int64_t q_rope_seq_stride, int64_t q_rope_head_stride,
+                                   const int32_t* block_table, int32_t table_stride, const int32_t* seq_lens, double scale,
+                                   void* out, int64_t out_seq_stride, int64_t out_head_stride, float* lse, void* stream);
+
 /* Block-32 MX quantization of bf16 rows along the last axis: replaces the plan + launch of
  * aclnnDynamicMxQuant (contract include/moe/core/op_table.hpp:205-233; the reference's stages
  * `attn_quant` src/pipeline/pipeline.cpp:251-258 and `shared_act_quant`), with the reference's
