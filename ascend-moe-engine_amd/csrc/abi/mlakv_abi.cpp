@@ -297,8 +297,45 @@ mlakvStatus mlakvCopyBlocks(const mlakvCacheView* cache, int32_t layer_begin, in
 }  // extern "C"
 
 namespace {
+
+constexpr int32_t kDefaultMergeSpinUs = 50;
+
+// The largest unit (in tiles) whose block-table entries fit the kernel's LDS staging whatever
+// the unit's offset inside a block; a selection stages one entry per selected token.
+int64_t CapUnitTiles(int32_t block_size, bool sparse) {
+  if (sparse) return mlakv::kAttnTableEntries / mlakv::kTileTokens;
+  const int64_t cap = ((static_cast<int64_t>(mlakv::kAttnTableEntries) - 2) * block_size + 2) / mlakv::kTileTokens;
+  return cap < 1 ? 1 : cap;
+}
+
+struct PlanShape {
+  int64_t max_tiles, head_groups, cap, units;
+  uint64_t workspace;
+};
+
+// What follows from a plan's own fields; the launch recomputes it to refuse a plan that was not
+// made by the init functions.
+PlanShape ShapeOf(int32_t batch, int32_t heads, int32_t max_seq_len, int32_t block_size, bool sparse, int32_t chunk_tiles,
+                  int32_t work_groups) {
+  PlanShape shape;
+  shape.max_tiles = (static_cast<int64_t>(max_seq_len) + mlakv::kTileTokens - 1) / mlakv::kTileTokens;
+  shape.head_groups = (heads + 63) / 64;
+  shape.cap = CapUnitTiles(block_size, sparse);
+  const int64_t total = static_cast<int64_t>(batch) * shape.max_tiles;
+  if (chunk_tiles > 0) {
+    shape.units = (total + chunk_tiles - 1) / chunk_tiles;
+  } else {
+    const int64_t capped = (total + shape.cap - 1) / shape.cap;
+    shape.units = capped > work_groups ? capped : work_groups;
+  }
+  const uint64_t rows = static_cast<uint64_t>(shape.head_groups) * static_cast<uint64_t>(shape.units + batch) * 64;
+  // bf16 partial outputs, then fp32 partial log-sum-exps
+  shape.workspace = rows * mlakv::kLatentDim * 2 + ((rows * sizeof(float) + 255) & ~255ull);
+  return shape;
+}
+
 mlakvStatus AttnPlanImpl(const char* who, int32_t batch, int32_t heads, int32_t max_seq_len, int32_t block_size,
-                         int32_t dtype, bool sparse, mlakvAttnPlan* plan) {
+                         int32_t dtype, bool sparse, const mlakvAttnPlanOptions* options, mlakvAttnPlan* plan) {
   if (plan == nullptr) return Fail(MLAKV_ERR_PARAM_NULLPTR, "%s: plan is null", who);
   if (batch <= 0 || batch > 65535) return Fail(MLAKV_ERR_PARAM_INVALID, "%s: batch %d outside [1, 65535]", who, batch);
   if (heads <= 0 || heads % 16 != 0 || heads > 128) {
@@ -308,40 +345,44 @@ mlakvStatus AttnPlanImpl(const char* who, int32_t batch, int32_t heads, int32_t 
   if (dtype != MLAKV_DTYPE_BF16 && dtype != MLAKV_DTYPE_FP8_E4M3) {
     return Fail(MLAKV_ERR_PARAM_INVALID, "%s: unknown cache dtype %d", who, dtype);
   }
-  const int max_tiles = (max_seq_len + mlakv::kTileTokens - 1) / mlakv::kTileTokens;
-  const int head_groups = (heads + 63) / 64;
-  // One workgroup occupies a whole CU (a ring of four 36 KB tile buffers), so aim for one chunk per CU.
-  int chunks_wanted = ComputeUnits() / (batch * head_groups);
-  if (chunks_wanted < 1) chunks_wanted = 1;
-  int chunk_tiles = (max_tiles + chunks_wanted - 1) / chunks_wanted;
-  // Amortise the query load over at least 128 tokens; a selection is short and latency-bound, where
-  // 64-token chunks measured faster (18.8 against 20.8 us for 512 of 8192 tokens, batch 32).
-  const int min_tiles = sparse ? 2 : 4;
-  if (chunk_tiles < min_tiles) chunk_tiles = max_tiles < min_tiles ? max_tiles : min_tiles;
-  if (const char* forced = std::getenv("MLAKV_ATTN_CHUNK_TILES")) {
-    const int value = std::atoi(forced);
-    if (value > 0) chunk_tiles = value;
+  mlakvAttnPlanOptions chosen{};
+  if (options != nullptr) chosen = *options;
+  if (chosen.chunk_tiles < 0 || chosen.work_groups < 0 || chosen.work_groups > 65535 || chosen.merge_mode < 0 ||
+      chosen.merge_mode > MLAKV_ATTN_MERGE_SECOND_LAUNCH || chosen.merge_spin_us > 1000000) {
+    return Fail(MLAKV_ERR_PARAM_INVALID, "%s: options outside their ranges", who);
   }
-  if (chunk_tiles > max_tiles) chunk_tiles = max_tiles;
-  // A chunk's block-table entries are staged in LDS (1024 entries); a selection stages one entry
-  // per selected token.
-  while (chunk_tiles > 1 && (chunk_tiles * mlakv::kTileTokens + block_size - 1) / block_size + 1 > 1024) --chunk_tiles;
-  if (sparse && chunk_tiles > 1024 / mlakv::kTileTokens) chunk_tiles = 1024 / mlakv::kTileTokens;
+  const int64_t head_groups = (heads + 63) / 64;
+  const int64_t cap = CapUnitTiles(block_size, sparse);
+  int32_t work_groups = chosen.work_groups;
+  if (work_groups == 0) {
+    // One workgroup occupies a whole CU (a ring of four 36 KB tile buffers).
+    work_groups = static_cast<int32_t>(ComputeUnits() / head_groups);
+    if (work_groups < 1) work_groups = 1;
+  }
+  int32_t chunk_tiles = chosen.chunk_tiles;
+  if (chunk_tiles > cap) chunk_tiles = static_cast<int32_t>(cap);
+  const PlanShape shape = ShapeOf(batch, heads, max_seq_len, block_size, sparse, chunk_tiles, work_groups);
+  if (shape.units > (int64_t{1} << 30)) return Fail(MLAKV_ERR_PARAM_INVALID, "%s: too many work units (%lld)", who, static_cast<long long>(shape.units));
   plan->batch = batch;
   plan->heads = heads;
   plan->max_seq_len = max_seq_len;
   plan->block_size = block_size;
   plan->dtype = dtype;
   plan->chunk_tiles = chunk_tiles;
-  plan->max_chunks = (max_tiles + chunk_tiles - 1) / chunk_tiles;
+  plan->work_groups = work_groups;
+  plan->max_units = static_cast<int32_t>(shape.units);
+  // The in-launch merge meets on counters the library holds for kAttnSyncSequences (head group,
+  // sequence) pairs; beyond that the merge is a launch of its own.
+  // (and a sequence's partials are counted in 16 bits)
+  const bool fits = static_cast<int64_t>(batch) * head_groups <= mlakv::kAttnSyncSequences && shape.units < 65535;
+  // Measured on MI355X: announcing and polling at agent scope costs about as much as the second
+  // launch it replaces (a counter round trip is ~2 us, as is the partial read), so the second
+  // launch, which needs no counters, is the default.
+  plan->merge_mode = chosen.merge_mode == MLAKV_ATTN_MERGE_IN_LAUNCH && fits ? MLAKV_ATTN_MERGE_IN_LAUNCH : MLAKV_ATTN_MERGE_SECOND_LAUNCH;
+  plan->merge_spin_us = chosen.merge_spin_us == 0 ? kDefaultMergeSpinUs : (chosen.merge_spin_us < 0 ? -1 : chosen.merge_spin_us);
   plan->reserved = sparse ? 1 : 0;
-  if (plan->max_chunks > 1) {
-    const uint64_t rows = static_cast<uint64_t>(batch) * plan->max_chunks * heads;
-    // bf16 partial outputs, then fp32 partial log-sum-exps
-    plan->workspace_bytes = rows * mlakv::kLatentDim * 2 + ((rows * sizeof(float) + 255) & ~255ull);
-  } else {
-    plan->workspace_bytes = 0;
-  }
+  plan->reserved2 = 0;
+  plan->workspace_bytes = shape.workspace;
   return MLAKV_SUCCESS;
 }
 
@@ -351,7 +392,20 @@ extern "C" {
 
 mlakvStatus mlakvAttnPlanInit(int32_t batch, int32_t heads, int32_t max_seq_len, int32_t block_size, int32_t dtype,
                               mlakvAttnPlan* plan) {
-  return AttnPlanImpl("mlakvAttnPlanInit", batch, heads, max_seq_len, block_size, dtype, false, plan);
+  return AttnPlanImpl("mlakvAttnPlanInit", batch, heads, max_seq_len, block_size, dtype, false, nullptr, plan);
+}
+
+mlakvStatus mlakvAttnPlanInitEx(int32_t batch, int32_t heads, int32_t max_seq_len, int32_t block_size, int32_t dtype,
+                                const mlakvAttnPlanOptions* options, mlakvAttnPlan* plan) {
+  const bool selection = options != nullptr && options->selection != 0;
+  if (options != nullptr && (options->selection < 0 || options->selection > 1 || options->reserved[0] != 0 ||
+                             options->reserved[1] != 0 || options->reserved[2] != 0)) {
+    return Fail(MLAKV_ERR_PARAM_INVALID, "mlakvAttnPlanInitEx: options outside their ranges");
+  }
+  if (selection && (max_seq_len <= 0 || max_seq_len > 2048)) {
+    return Fail(MLAKV_ERR_PARAM_INVALID, "mlakvAttnPlanInitEx: sparse_count %d outside [1, 2048]", max_seq_len);
+  }
+  return AttnPlanImpl("mlakvAttnPlanInitEx", batch, heads, max_seq_len, block_size, dtype, selection, options, plan);
 }
 
 mlakvStatus mlakvAttnSparsePlanInit(int32_t batch, int32_t heads, int32_t sparse_count, int32_t block_size, int32_t dtype,
@@ -359,7 +413,7 @@ mlakvStatus mlakvAttnSparsePlanInit(int32_t batch, int32_t heads, int32_t sparse
   if (sparse_count <= 0 || sparse_count > 2048) {
     return Fail(MLAKV_ERR_PARAM_INVALID, "mlakvAttnSparsePlanInit: sparse_count %d outside [1, 2048]", sparse_count);
   }
-  return AttnPlanImpl("mlakvAttnSparsePlanInit", batch, heads, sparse_count, block_size, dtype, true, plan);
+  return AttnPlanImpl("mlakvAttnSparsePlanInit", batch, heads, sparse_count, block_size, dtype, true, nullptr, plan);
 }
 
 }  // extern "C"
@@ -395,22 +449,25 @@ mlakvStatus AttnDecodeImpl(const char* who, const mlakvAttnPlan* plan, const mla
                 plan->dtype, plan->block_size, cache->dtype, cache->block_size);
   }
   if (!(scale > 0.0) || !std::isfinite(scale)) return Fail(MLAKV_ERR_PARAM_INVALID, "%s: a positive softmax scale is required", who);
-  // The kernels size their LDS staging and their grid from the plan: a plan that was not made by
-  // the init functions (or was altered since) is refused here instead of faulting there.
+  // The kernels size their LDS staging, their grid and their partial slots from the plan: a plan
+  // that was not made by the init functions (or was altered since) is refused here instead of
+  // faulting there.
   {
-    const int64_t max_tiles = (static_cast<int64_t>(plan->max_seq_len) + mlakv::kTileTokens - 1) / mlakv::kTileTokens;
-    const bool sane = plan->batch > 0 && plan->batch <= 65535 && plan->heads > 0 && plan->heads % 16 == 0 && plan->heads <= 128 &&
-                      plan->max_seq_len > 0 && plan->chunk_tiles >= 1 && plan->chunk_tiles <= max_tiles &&
-                      plan->max_chunks == (max_tiles + plan->chunk_tiles - 1) / plan->chunk_tiles &&
-                      (plan->reserved == 0 || plan->reserved == 1) &&
-                      (plan->reserved == 1
-                           ? plan->chunk_tiles * mlakv::kTileTokens <= 1024 && plan->max_seq_len <= 2048
-                           : (static_cast<int64_t>(plan->chunk_tiles) * mlakv::kTileTokens + plan->block_size - 1) / plan->block_size + 1 <= 1024 ||
-                                 plan->chunk_tiles == 1);
-    const uint64_t rows = static_cast<uint64_t>(plan->batch > 0 ? plan->batch : 0) * (plan->max_chunks > 0 ? plan->max_chunks : 0) *
-                          (plan->heads > 0 ? plan->heads : 0);
-    const uint64_t expected = plan->max_chunks > 1 ? rows * mlakv::kLatentDim * 2 + ((rows * sizeof(float) + 255) & ~255ull) : 0;
-    if (!sane || plan->workspace_bytes != expected) {
+    const bool fields = plan->batch > 0 && plan->batch <= 65535 && plan->heads > 0 && plan->heads % 16 == 0 && plan->heads <= 128 &&
+                        plan->max_seq_len > 0 && plan->block_size > 0 && plan->chunk_tiles >= 0 && plan->work_groups >= 1 &&
+                        plan->work_groups <= 65535 && (plan->reserved == 0 || plan->reserved == 1) && plan->reserved2 == 0 &&
+                        (plan->reserved == 0 || plan->max_seq_len <= 2048) &&
+                        (plan->merge_mode == MLAKV_ATTN_MERGE_IN_LAUNCH || plan->merge_mode == MLAKV_ATTN_MERGE_SECOND_LAUNCH) &&
+                        (plan->merge_spin_us == -1 || (plan->merge_spin_us > 0 && plan->merge_spin_us <= 1000000));
+    bool sane = fields;
+    if (fields) {
+      const PlanShape shape = ShapeOf(plan->batch, plan->heads, plan->max_seq_len, plan->block_size, plan->reserved == 1,
+                                      plan->chunk_tiles, plan->work_groups);
+      sane = plan->chunk_tiles <= shape.cap && plan->max_units == shape.units && plan->workspace_bytes == shape.workspace &&
+             (plan->merge_mode != MLAKV_ATTN_MERGE_IN_LAUNCH ||
+              (static_cast<int64_t>(plan->batch) * shape.head_groups <= mlakv::kAttnSyncSequences && shape.units < 65535));
+    }
+    if (!sane) {
       return Fail(MLAKV_ERR_PARAM_INVALID, "%s: the plan is not one made by mlakvAttnPlanInit / mlakvAttnSparsePlanInit", who);
     }
   }
@@ -434,13 +491,11 @@ mlakvStatus AttnDecodeImpl(const char* who, const mlakvAttnPlan* plan, const mla
   if (out != nullptr && (!Aligned16(out) || out_seq_stride % 16 != 0 || out_head_stride % 16 != 0)) {
     return Fail(MLAKV_ERR_PARAM_INVALID, "%s: output rows must be 16-byte aligned with 16-byte-multiple strides", who);
   }
-  if (plan->workspace_bytes > 0) {
-    if (workspace == nullptr) return Fail(MLAKV_ERR_PARAM_NULLPTR, "%s: the plan needs %llu workspace bytes", who,
-                                          static_cast<unsigned long long>(plan->workspace_bytes));
-    if (workspace_bytes < plan->workspace_bytes || !Aligned16(workspace)) {
-      return Fail(MLAKV_ERR_PARAM_INVALID, "%s: workspace of %llu bytes (16-byte aligned) needed, %llu given", who,
-                  static_cast<unsigned long long>(plan->workspace_bytes), static_cast<unsigned long long>(workspace_bytes));
-    }
+  if (workspace == nullptr) return Fail(MLAKV_ERR_PARAM_NULLPTR, "%s: the plan needs %llu workspace bytes", who,
+                                        static_cast<unsigned long long>(plan->workspace_bytes));
+  if (workspace_bytes < plan->workspace_bytes || !Aligned16(workspace)) {
+    return Fail(MLAKV_ERR_PARAM_INVALID, "%s: workspace of %llu bytes (16-byte aligned) needed, %llu given", who,
+                static_cast<unsigned long long>(plan->workspace_bytes), static_cast<unsigned long long>(workspace_bytes));
   }
   static std::once_flag prepared;
   static hipError_t prepare_status = hipSuccess;
@@ -473,16 +528,27 @@ mlakvStatus AttnDecodeImpl(const char* who, const mlakvAttnPlan* plan, const mla
     args.out_scales_seq_stride = quant->scales_seq_stride;
     args.out_scales_head_stride = quant->scales_head_stride;
   }
-  const uint64_t rows = static_cast<uint64_t>(plan->batch) * plan->max_chunks * plan->heads;
+  const uint64_t rows = static_cast<uint64_t>((plan->heads + 63) / 64) * (static_cast<uint64_t>(plan->max_units) + plan->batch) * 64;
   args.partial_out = static_cast<char*>(workspace);
-  args.partial_lse = workspace == nullptr ? nullptr : reinterpret_cast<float*>(static_cast<char*>(workspace) + rows * mlakv::kLatentDim * 2);
+  args.partial_lse = reinterpret_cast<float*>(static_cast<char*>(workspace) + rows * mlakv::kLatentDim * 2);
   args.scale_log2 = static_cast<float>(scale * 1.4426950408889634);
   args.batch = plan->batch;
   args.heads = plan->heads;
   args.num_blocks = cache->num_blocks;
   args.block_size = cache->block_size;
-  args.chunk_tiles = plan->chunk_tiles;
-  args.max_chunks = plan->max_chunks;
+  {
+    const int64_t addressable = static_cast<int64_t>(table_stride) * cache->block_size;
+    args.max_tokens = sparse ? plan->max_seq_len : static_cast<int32_t>(addressable < plan->max_seq_len ? addressable : plan->max_seq_len);
+  }
+  args.work_groups = plan->work_groups;
+  args.max_units = plan->max_units;
+  args.forced_unit_tiles = plan->chunk_tiles;
+  // Amortise the query load over at least 128 tokens; a selection is short and latency-bound, where
+  // 64-token units measured faster.
+  args.min_unit_tiles = sparse ? 2 : 4;
+  args.cap_unit_tiles = static_cast<int32_t>(CapUnitTiles(plan->block_size, sparse));
+  args.spin_ticks = plan->merge_spin_us < 0 ? 0 : plan->merge_spin_us * 100;
+  args.merge_in_launch = plan->merge_mode == MLAKV_ATTN_MERGE_IN_LAUNCH;
   args.fp8 = cache->dtype == MLAKV_DTYPE_FP8_E4M3;
   const hipError_t status = mlakv::LaunchAttnDecode(args, static_cast<hipStream_t>(stream));
   return status == hipSuccess ? MLAKV_SUCCESS : HipFail(status, who);

@@ -107,19 +107,25 @@ struct AttnArgs {
   const int32_t* sparse_indices;
   int64_t sparse_seq_stride;  // elements
   int32_t sparse_count;
-  char* partial_out;     // workspace: [batch][max_chunks][heads][512] bf16
-  float* partial_lse;    // workspace: [batch][max_chunks][heads] fp32, log2 domain
+  // Workspace: partials of the segments that do not hold a whole sequence, per group of 64 heads
+  // [max_units + batch][64][512] bf16 and the same rows of fp32 log2-domain LSE.
+  char* partial_out;
+  float* partial_lse;
   float scale_log2;      // softmax scale * log2(e)
   int32_t batch;
   int32_t heads;
   int32_t num_blocks;
   int32_t block_size;
-  int32_t chunk_tiles;
-  int32_t max_chunks;
+  int32_t max_tokens;         // lengths are clamped to min(plan's max_seq_len, table_stride * block_size)
+  int32_t work_groups;        // workgroups per group of 64 heads
+  int32_t max_units;          // bound on the work units of a launch (per head group)
+  int32_t forced_unit_tiles;  // tiles per work unit; 0: from the live lengths
+  int32_t min_unit_tiles;     // the smallest unit worth a query load
+  int32_t cap_unit_tiles;     // what a segment's staged block-table entries can address
+  int32_t spin_ticks;         // bound of the in-launch merge's wait, in 10 ns ticks
+  bool merge_in_launch;       // false: the merge is a second launch
   bool fp8;
-#ifdef MLAKV_ATTN_TRACE
-  unsigned long long* trace;  // development timeline, see mla_decode.hip
-#endif
+  unsigned* sync;             // set by the launcher: this launch's counters, null for a second-launch merge
 };
 
 struct MxQuantArgs {
@@ -158,6 +164,8 @@ struct IndexerArgs {
 constexpr int kLatentDim = 512;
 constexpr int kRopeDim = 64;
 constexpr int kTileTokens = 32;
+constexpr int kAttnTableEntries = 512;     // block-table entries (or selected tokens) of one segment staged in LDS
+constexpr int kAttnSyncSequences = 4096;   // (head group, sequence) pairs a launch can merge in place
 
 hipError_t LaunchAppend(const AppendArgs& args, hipStream_t stream);
 hipError_t LaunchNormRopeAppend(const NormRopeAppendArgs& args, hipStream_t stream);

@@ -7,8 +7,10 @@
 // as both K (with the 64 rope columns appended) and V.
 //
 // Work decomposition
-//   workgroup = (kv chunk, sequence, group of 64 heads), one workgroup per CU, 8 wavefronts in
-//   two roles, one of each role per SIMD:
+//   The contexts of the batch, in 32-token tiles, laid end to end, are cut into as many equal
+//   work units as there are CUs; a workgroup (one per CU, all 64 heads of a group) walks the
+//   segments of its unit, each a tile range of one sequence (see "work decomposition" below).
+//   8 wavefronts in two roles, one of each role per SIMD:
 //     score waves 0..3 (16 heads each) hold the query in registers, compute S^T = K Q^T for a
 //       tile, run the online softmax and publish P (bf16, already in MFMA operand layout)
 //       through LDS, one tile ahead of
@@ -17,11 +19,11 @@
 //   every stall exposed); with the two roles the softmax VALU work, the LDS traffic and the
 //   MFMAs of neighbouring tiles overlap in hardware, and neither role has to hold both the
 //   query (72 registers) and O (128 registers).
-//   A chunk is `chunk_tiles` tiles of 32 tokens. LDS holds a ring of four tile buffers: while
+//   LDS holds a ring of four tile buffers: while
 //   tile i feeds the second product and tile i+1 the first, tiles i+2 and i+3 are in flight
 //   from HBM. bf16 tiles are filled by direct global->LDS loads (global_load_lds_dwordx4: no
-//   staging registers, no ds_write) issued by all eight waves; FP8 tiles are dequantised to
-//   bf16 through registers on their way into LDS. One workgroup barrier per tile publishes
+//   staging registers, no ds_write) issued by all eight waves; FP8 tiles arrive the same way as
+//   codes and are converted at the MFMA operand. One workgroup barrier per tile publishes
 //   tile i+1 and P(i) and retires tile i-1.
 //
 // MFMA formulation (v_mfma_f32_16x16x32_bf16; A: lane holds row l%16, k = 8*(l/16)..+7;
@@ -46,8 +48,10 @@
 // exceeds it by more than 2^8, so exponentials stay below 256; when it moves, the score wave
 // hands the factor to its output wave, which rescales O before adding the tile.
 //
-// Chunks of one sequence are merged by a second small kernel from partials (normalised O in
-// bf16, log2-domain LSE in fp32) held in the caller's workspace.
+// Segments that do not hold a whole sequence leave partials (normalised O in bf16, log2-domain
+// LSE in fp32) in the caller's workspace; they are merged inside the same launch, or by a second
+// small kernel when the launch has no counters to meet on.
+#include <algorithm>
 #include <mutex>
 #include <utility>
 
@@ -55,22 +59,6 @@
 #include "mx_quant_device.h"
 
 #pragma clang diagnostic ignored "-Winline-asm"
-
-// Development timeline (built only with -DMLAKV_ATTN_TRACE): lane 0 of every wave of every
-// workgroup stamps the 100 MHz wall clock into a caller-provided buffer.
-#ifdef MLAKV_ATTN_TRACE
-#include <cstdlib>
-#define MLAKV_STAMP(slot)                                                                              \
-  do {                                                                                                 \
-    if (a.trace != nullptr && lane == 0 && (slot) >= 0 && (slot) < 40) {                                                 \
-      a.trace[((blockIdx.y * gridDim.x + blockIdx.x) * 8 + wave) * 40 + (slot)] = __builtin_amdgcn_s_memrealtime();       \
-    }                                                                                                  \
-  } while (0)
-#else
-#define MLAKV_STAMP(slot) \
-  do {                    \
-  } while (0)
-#endif
 
 namespace mlakv {
 namespace {
@@ -96,7 +84,8 @@ constexpr int kScoreWaves = 4;
 constexpr int kKSteps = (kLatentDim + kRopeDim) / 32;        // 18
 constexpr int kQkSteps = 2 * kKSteps;                        // 36 MFMAs: 18 k-steps x 2 token subtiles
 constexpr int kDvTiles = kLatentDim / 16;                    // 32
-constexpr int kTableEntries = 1024;                          // block-table entries of one chunk staged in LDS
+constexpr int kTableEntries = kAttnTableEntries;             // block-table entries of one segment staged in LDS
+constexpr int kMaxDuties = 64;                               // merges a workgroup has promised and not yet carried out
 static_assert(kTileTokens == 32, "the fragment maps below are written for 32-token tiles");
 
 // LDS geometry. A bf16 tile is 32 latent rows of 1024 B followed by 32 rope rows of 128 B. An
@@ -117,7 +106,9 @@ struct Geom {
   static constexpr int kAlphaOff = kPOff + 2 * kScoreWaves * 64 * 16;  // alpha[2][4][64] fp32
   static constexpr int kInvOff = kAlphaOff + 2 * kScoreWaves * 64 * 4; // 1/denominator[4][64] fp32
   static constexpr int kFlagOff = kInvOff + kScoreWaves * 64 * 4;      // rescale flag[2][4] int
-  static constexpr int kLdsBytes = kFlagOff + 64;
+  static constexpr int kDutyOff = kFlagOff + 64;                       // i32x4[kMaxDuties]
+  static constexpr int kFoundOff = kDutyOff + kMaxDuties * 16;         // unsigned[kMaxDuties]
+  static constexpr int kLdsBytes = kFoundOff + kMaxDuties * 4;
   static_assert(kLdsBytes <= 160 * 1024, "one workgroup owns the LDS of a CU");
   __device__ static __forceinline__ int Slot(int i) { return (kRing == 4 ? (i & 3) : (i % kRing)) * kTileBytes; }
 };
@@ -447,620 +438,150 @@ __device__ __forceinline__ bf16x8 CodesToBf16(unsigned lo, unsigned hi) {
   return bf16x8{a.x, a.y, b.x, b.y, c.x, c.y, d.x, d.y};
 }
 
-// ---- main kernel -------------------------------------------------------------------
+// ---- work decomposition --------------------------------------------------------------------
+//
+// The sequences' contexts, counted in 32-token tiles, are laid end to end on one flat tile axis,
+// and that axis is cut into work units of `tiles_per_unit` tiles: as many units as the launch
+// has workgroups (per group of 64 heads) when the batch is large enough, so that every CU streams
+// the same number of tiles whatever the individual lengths are. Every workgroup derives the cut
+// from the live lengths itself (one prefix sum over the batch); nothing depends on the host
+// knowing them. A unit is a run of segments, each a tile range of one sequence:
+//   * a segment that holds a whole sequence writes the final output;
+//   * any other segment writes a partial (normalised O in bf16, log2-domain LSE in fp32) to the
+//     caller's workspace: slot `max_units + seq` for the segment with the sequence's first tile,
+//     slot `unit` for a later one (a unit starts inside at most one sequence).
+// The partials of a sequence are merged inside the same launch: every contributor announces its
+// partial on a per-sequence counter and then merges its share of the heads once the counter is
+// full. Waiting is bounded, and a share whose owner gave up (or has not claimed it by then) is
+// taken by the contributor that arrived last, so the launch finishes whatever the order in which
+// workgroups get to run.
 
-// MXQ: the single-chunk launch also quantises its output (and its bf16 output is optional). Kept
-// out of the common instantiation, whose register allocation has no room to spare.
-// SPARSE: the sequence attends to the tokens listed in a.sparse_indices instead of to its whole
-// context (never ALIGNED: every row is located on its own).
-template <bool FP8, bool ALIGNED, bool MXQ, bool SPARSE>
-__global__ __launch_bounds__(kThreads) void MlaDecodeKernel(AttnArgs a) {
-  static_assert(!(SPARSE && (ALIGNED || MXQ)), "selected-token attention uses the row-at-a-time path");
-  // bf16 tiles: the output waves, which have no query to wait for, issue the first tiles of the
-  // ring alone (their own rows and those of their partner score waves) as soon as they know the
-  // block-table entries; the score waves join from the first loop iteration on.
-  constexpr bool kSoloPrologue = !FP8 && !SPARSE;
-  using G = Geom<FP8>;
-  extern __shared__ __attribute__((aligned(16))) unsigned char lds[];
-  const unsigned lds_base = static_cast<unsigned>(reinterpret_cast<size_t>((__attribute__((address_space(3))) unsigned char*)lds));
-  const int tid = threadIdx.x;
-  const int lane = tid & 63, wave = Uniform(tid >> 6);
-  const bool score_wave = wave < kScoreWaves;   // wave-uniform role
-  const int hw = wave & (kScoreWaves - 1);      // which 16 heads of the 64
-  const int g = lane >> 4, i16 = lane & 15;
-  // Workgroups are handed to the eight XCDs round-robin by linear id, and each XCD has its own
-  // L2. The chunks of one sequence all read the same 72 KB of Q, so they are placed on one XCD:
-  // XCD x takes the contiguous range of (sequence, chunk) pairs [x, x+1) * pairs / 8.
-  int chunk_index = blockIdx.x;
-  int seq = blockIdx.y;
-  {
-    const int pairs = gridDim.x * gridDim.y;
-    if ((pairs & (kXcds - 1)) == 0) {
-      const int linear = blockIdx.y * gridDim.x + blockIdx.x;
-      const int pair = (linear & (kXcds - 1)) * (pairs / kXcds) + linear / kXcds;
-      seq = pair / static_cast<int>(gridDim.x);
-      chunk_index = pair - seq * static_cast<int>(gridDim.x);
-    }
-  }
-  const int head_base = blockIdx.z * 64 + hw * 16;
-  const bool active = head_base < a.heads;  // wave-uniform
-  const int head = head_base + i16;
-  const bool direct = a.max_chunks == 1;  // single chunk: write the final output here
-  const int per_tile = FP8 ? LoadsPerTile8(wave) : LoadsPerTile(wave);
-  MLAKV_STAMP(0);
+typedef unsigned long long u64;
 
-  // Q fragments (score waves): lane (head i16, k-group g) holds, for k-step ks, the eight query
-  // elements that meet the lane's K fragment of that step: Q[head][32 ks + 8g .. +7] for bf16
-  // tiles; for FP8 tiles one 16-byte K read feeds two k-steps, so the order inside each 64-wide
-  // window is Q[head][64 (ks/2) + 16g + 8 (ks&1) .. +7]. (Loaded further down, once the
-  // lengths and table entries have been asked for.)
-  bf16x8 q[kKSteps];
-  const auto load_q = [&]() __attribute__((always_inline)) {
-    const char* q_latent = a.q_latent + seq * a.q_latent_seq_stride + head * a.q_latent_head_stride;
-    const char* q_rope = a.q_rope + seq * a.q_rope_seq_stride + head * a.q_rope_head_stride;
-#pragma unroll
-    for (int ks = 0; ks < kKSteps; ++ks) {
-      const int d0 = FP8 ? 64 * (ks >> 1) + 16 * g + 8 * (ks & 1) : 32 * ks + 8 * g;
-      const char* p = d0 < kLatentDim ? q_latent + d0 * 2 : q_rope + (d0 - kLatentDim) * 2;
-      q[ks] = __builtin_bit_cast(bf16x8, GlobalLoad16(p));
-    }
-  };
+constexpr int kMergeHeads = 8;   // heads of one merge step: one per wave
 
-  // Stage this chunk's block-table entries in LDS. The range is bounded by the chunk and the
-  // table row, not by the sequence length, so it does not wait for the length to arrive;
-  // entries past the sequence are never used.
-  const int tile_begin = chunk_index * a.chunk_tiles;
-  int* table_lds = reinterpret_cast<int*>(lds + G::kTableOff);
-  TileMap<ALIGNED> map;
-  map.entries = table_lds;
-  map.block_size = a.block_size;
-  map.sparse = SPARSE;
-  map.first_pos = tile_begin * kTileTokens;
-  if constexpr (!SPARSE) {
-    const int first_pos = tile_begin * kTileTokens;
-    const int last_pos = first_pos + a.chunk_tiles * kTileTokens - 1;
-    map.first_block = first_pos / a.block_size;
-    map.next_entry = 0;
-    map.next_slot0 = first_pos - map.first_block * a.block_size;
-    int count = last_pos / a.block_size - map.first_block + 1;  // <= kTableEntries, ensured by the plan
-    count = min(count, a.table_stride - map.first_block);
-    const int32_t* table_row = a.block_table + static_cast<int64_t>(seq) * a.table_stride + map.first_block;
-    // kSoloPrologue: every wave stages all entries itself (the same values to the same
-    // addresses), so that it can read them back without waiting for the other waves.
-    for (int i = kSoloPrologue ? lane : tid; i < count; i += kSoloPrologue ? 64 : kThreads) {
-      const int entry = table_row[i];
-      table_lds[i] = static_cast<unsigned>(entry) < static_cast<unsigned>(a.num_blocks) ? entry : -1;
-    }
-  }
-  MLAKV_STAMP(34);
-  // A length beyond what the table row can address is clamped: every position below it has a
-  // staged entry.
-  int seq_len = static_cast<int>(
-      min(static_cast<int64_t>(Uniform(a.seq_lens[seq])), static_cast<int64_t>(a.table_stride) * a.block_size));
-  if constexpr (SPARSE) {
-    // The selection ends at its first entry that is negative or not inside the context. Then
-    // this chunk's part of it is resolved to pool slots through the block table.
-    const int context = seq_len;
-    const int32_t* selection = a.sparse_indices + static_cast<int64_t>(seq) * a.sparse_seq_stride;
-    int* count_lds = reinterpret_cast<int*>(lds + G::kFlagOff) + 2 * kScoreWaves;
-    if (tid == 0) *count_lds = a.sparse_count;
-    __syncthreads();
-    for (int i = tid; i < a.sparse_count; i += kThreads) {
-      const int index = selection[i];
-      if (index < 0 || index >= context) atomicMin(count_lds, i);
-    }
-    __syncthreads();
-    seq_len = Uniform(*count_lds);
-    const int32_t* table_row = a.block_table + static_cast<int64_t>(seq) * a.table_stride;
-    const int chunk_tokens = min(a.chunk_tiles * kTileTokens, seq_len - map.first_pos);  // <= kTableEntries, ensured by the plan
-    for (int i = tid; i < chunk_tokens; i += kThreads) {
-      const int index = selection[map.first_pos + i];  // inside [0, context): before the end of the selection
-      const int logical = index / a.block_size;
-      const int entry = table_row[logical];
-      table_lds[i] = static_cast<unsigned>(entry) < static_cast<unsigned>(a.num_blocks)
-                         ? entry * a.block_size + (index - logical * a.block_size)
-                         : -1;
-    }
-  }
-  map.seq_len = seq_len;
-  MLAKV_STAMP(33);
-  // Vector memory requests of a CU are served in order: the query (72 KB per workgroup) is asked
-  // for only now, behind the few bytes of lengths and table entries that the first tile
-  // addresses depend on.
-  if (score_wave && active) load_q();
-  MLAKV_STAMP(32);
-  const int num_tiles = (seq_len + kTileTokens - 1) / kTileTokens;
-  if (tile_begin >= num_tiles) {
-    if (active && direct) {  // empty sequence: zeros, lse = -inf
-      if (score_wave) {
-        if (a.lse != nullptr && g == 0) a.lse[seq * a.heads + head] = -__builtin_inff();
+// Inclusive prefix sum over the 64 lanes with data-parallel-primitive moves: four shifted adds
+// inside each row of 16 lanes, then lane 15 of rows 0 and 2 onto rows 1 and 3, then lane 31 onto
+// the upper half. Lanes a move does not reach add zero.
+__device__ __forceinline__ int WaveInclusiveScan(int v) {
+  v += __builtin_amdgcn_update_dpp(0, v, 0x111, 0xf, 0xf, false);  // row_shr:1
+  v += __builtin_amdgcn_update_dpp(0, v, 0x112, 0xf, 0xf, false);  // row_shr:2
+  v += __builtin_amdgcn_update_dpp(0, v, 0x114, 0xf, 0xf, false);  // row_shr:4
+  v += __builtin_amdgcn_update_dpp(0, v, 0x118, 0xf, 0xf, false);  // row_shr:8
+  v += __builtin_amdgcn_update_dpp(0, v, 0x142, 0xa, 0xf, false);  // row_bcast:15 into rows 1 and 3
+  v += __builtin_amdgcn_update_dpp(0, v, 0x143, 0xc, 0xf, false);  // row_bcast:31 into rows 2 and 3
+  return v;
+}
+
+// 64 consecutive sequences, one per lane: tokens that count, tiles, and the running tile total
+// up to and including the lane's sequence. Windows are visited in increasing order.
+template <bool SPARSE>
+struct SeqWindow {
+  int base;   // first sequence of the window; uniform
+  int tok, tiles, incl;
+
+  __device__ __forceinline__ void Load(const AttnArgs& a, int lane, int new_base, int carry) {
+    base = new_base;
+    const int seq = base + lane;
+    int n = 0;
+    if (seq < a.batch) {
+      if (SPARSE) {
+        n = a.sparse_count;
       } else {
-        if (!MXQ || a.out != nullptr) {
-          char* out = a.out + seq * a.out_seq_stride + head * a.out_head_stride;
-          for (int n = g; n < kLatentDim / 8; n += 4) *reinterpret_cast<u32x4*>(out + n * 16) = u32x4{0u, 0u, 0u, 0u};
-        }
-        if constexpr (MXQ) {  // zeros quantise to zero codes under the smallest scale
-          char* codes = a.out_codes + seq * a.out_codes_seq_stride + head * a.out_codes_head_stride;
-          for (int n = g; n < kLatentDim / 16; n += 4) *reinterpret_cast<u32x4*>(codes + n * 16) = u32x4{0u, 0u, 0u, 0u};
-          if (g == 0) *reinterpret_cast<u32x4*>(a.out_scales + seq * a.out_scales_seq_stride + head * a.out_scales_head_stride) = u32x4{0u, 0u, 0u, 0u};
-        }
+        n = min(max(a.seq_lens[seq], 0), a.max_tokens);
       }
-    } else if (active && score_wave && g == 0) {  // empty chunk: the merge reads every chunk's LSE
-      a.partial_lse[(static_cast<int64_t>(seq) * a.max_chunks + chunk_index) * a.heads + head] = -__builtin_inff();
     }
-    return;
+    tok = n;
+    tiles = (n + kTileTokens - 1) / kTileTokens;
+    incl = carry + WaveInclusiveScan(tiles);
   }
-  const int ntiles = min(a.chunk_tiles, num_tiles - tile_begin);  // tiles of this chunk, >= 1
+  __device__ __forceinline__ int End() const { return __builtin_amdgcn_readlane(incl, 63); }
+  __device__ __forceinline__ int Tok(int seq) const { return __builtin_amdgcn_readlane(tok, seq - base); }
+  __device__ __forceinline__ int Tiles(int seq) const { return __builtin_amdgcn_readlane(tiles, seq - base); }
+  __device__ __forceinline__ int Incl(int seq) const { return __builtin_amdgcn_readlane(incl, seq - base); }
+};
 
-  // Direct loads: lane L of a latent row fetches chunk L ^ swizzle(row); rows of this wave.
-  IssueLane il;
-  IssueLane8 il8;
-  if (FP8) {
-#pragma unroll
-    for (int j = 0; j < 2; ++j) {
-      const int row = 2 * wave + 16 * j + (lane >> 5);
-      il8.lat[j] = (lane >> 5) * static_cast<int>(a.latent.row_stride) + (((lane & 31) ^ SwizzleLat8(row)) << 4);
+// Stores and loads that other CUs' accesses of the same kind see without a cache write-back or
+// invalidate in between (agent scope: the sc1 bit): the partials and the counters travel through
+// these. The 16-byte forms have no builtin; a load's result is ready after WaitAgentLoads on it.
+__device__ __forceinline__ void StoreAgent16(char* p, const u32x4& v) {
+  asm volatile("global_store_dwordx4 %0, %1, off sc1" : : "v"(p), "v"(v) : "memory");
+}
+__device__ __forceinline__ u32x4 LoadAgent16(const char* p) {
+  u32x4 v;
+  asm volatile("global_load_dwordx4 %0, %1, off sc1" : "=v"(v) : "v"(p) : "memory");
+  return v;
+}
+// Waits for every outstanding vector-memory operation of the wave; the loaded registers pass
+// through the statement so that no use of them can be scheduled ahead of it.
+__device__ __forceinline__ void WaitAgentLoads(u32x4 (&v)[8]) {
+  asm volatile("s_waitcnt vmcnt(0)"
+               : "+v"(v[0]), "+v"(v[1]), "+v"(v[2]), "+v"(v[3]), "+v"(v[4]), "+v"(v[5]), "+v"(v[6]), "+v"(v[7])
+               :
+               : "memory");
+}
+__device__ __forceinline__ void StoreAgentF32(float* p, float v) {
+  __hip_atomic_store(reinterpret_cast<unsigned*>(p), __builtin_bit_cast(unsigned, v), __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+}
+__device__ __forceinline__ float LoadAgentF32(const float* p) {
+  return __builtin_bit_cast(float, __hip_atomic_load(reinterpret_cast<unsigned*>(const_cast<float*>(p)), __ATOMIC_RELAXED,
+                                                     __HIP_MEMORY_SCOPE_AGENT));
+}
+
+// Row index of (head group z, partial slot, head of the group) in the partial arrays.
+__device__ __forceinline__ int64_t PartialRow(const AttnArgs& a, int z, int slot, int head_in_group) {
+  return (static_cast<int64_t>(z) * (a.max_units + a.batch) + slot) * 64 + head_in_group;
+}
+
+// Final output rows of an empty sequence (zeros, lse = -inf): wave w takes heads w, w + 8, ... of the group.
+template <bool MXQ>
+__device__ __forceinline__ void ZeroFill(const AttnArgs& a, int z, int seq, int wave, int lane) {
+  const int heads_here = min(64, a.heads - 64 * z);
+  for (int h = wave; h < heads_here; h += kWaves) {
+    const int head = 64 * z + h;
+    if (a.out != nullptr) *reinterpret_cast<u32x4*>(a.out + seq * a.out_seq_stride + head * a.out_head_stride + lane * 16) = u32x4{0u, 0u, 0u, 0u};
+    if (a.lse != nullptr && lane == 0) a.lse[seq * a.heads + head] = -__builtin_inff();
+    if constexpr (MXQ) {  // zeros quantise to zero codes under the smallest scale
+      if (lane < kLatentDim / 16) *reinterpret_cast<u32x4*>(a.out_codes + seq * a.out_codes_seq_stride + head * a.out_codes_head_stride + lane * 16) = u32x4{0u, 0u, 0u, 0u};
+      if (lane == 0) *reinterpret_cast<u32x4*>(a.out_scales + seq * a.out_scales_seq_stride + head * a.out_scales_head_stride) = u32x4{0u, 0u, 0u, 0u};
     }
-    const int rope_row = 16 * (wave & 1) + (lane >> 2);
-    il8.rope = (lane >> 2) * static_cast<int>(a.rope.row_stride) + (((lane & 3) ^ SwizzleRope8(rope_row)) << 4);
-  } else {
-#pragma unroll
-    for (int j = 0; j < 2; ++j) {
-      il.lat[j] = (lane ^ SwizzleLat(wave + kWaves * j)) << 4;
-      il.partner_lat[j] = (lane ^ SwizzleLat((wave & (kScoreWaves - 1)) + kWaves * j)) << 4;
-    }
-    il.rope_chunk = ((lane & 7) ^ SwizzleRope(8 * (wave - kScoreWaves) + (lane >> 3))) << 4;
-    il.rope = (lane >> 3) * static_cast<int>(a.rope.row_stride) + il.rope_chunk;
-  }
-
-  const auto ring = [&](int i) __attribute__((always_inline)) { return G::Slot(i); };
-  // Issues this wave's loads of chunk-relative tile t; returns whether their number is known.
-  const auto issue = [&](int t) __attribute__((always_inline)) {
-    if constexpr (FP8) {
-      return IssueTileFp8(a, map, il8, tile_begin + t, lds_base + ring(t), lds + ring(t), tid);
-    } else {
-      return IssueTileBf16(a, map, il, tile_begin + t, lds_base + ring(t), lds + ring(t), tid);
-    }
-  };
-
-  // The query must have arrived before this wave issues tile loads: the compiler's own wait for
-  // it would otherwise also wait for every tile load issued in between.
-  MLAKV_STAMP(35);
-  // Every wave passes through it, whether it asked for the query or not: were it skipped on
-  // some path, the compiler would have to assume the query still in flight wherever the paths
-  // meet again, and would wait for it -- with counts that know nothing of the tile loads, so in
-  // effect for every tile in flight -- inside the score loop, at every use.
-#pragma unroll
-  for (int ks = 0; ks < kKSteps; ++ks) asm volatile("" ::"v"(q[ks]));
-  MLAKV_STAMP(1);
-  if constexpr (!kSoloPrologue) __syncthreads();  // table entries visible
-
-  // Prologue: tiles 0 .. kRing-2 on their way, tile 0 landed and published. A tile whose load
-  // count is not known (rare path) makes every wait up to and including its own a full one.
-  int last_unknown = -1;  // newest tile issued with an unknown number of loads
-  int issued = 0;         // tiles issued so far
-  for (; issued < G::kRing - 1 && issued < ntiles; ++issued) {
-    if constexpr (kSoloPrologue) {
-      if (score_wave) {
-        map.Begin(issued);  // keeps the cursor in step with the tiles this wave does not issue
-      } else if (!IssueTileBf16<ALIGNED, true>(a, map, il, tile_begin + issued, lds_base + ring(issued), lds + ring(issued), tid)) {
-        last_unknown = issued;
-      }
-    } else {
-      if (!issue(issued)) last_unknown = issued;
-    }
-  }
-  // Loads this wave has in flight that are newer than those of tile t: the first `solo_tiles`
-  // tiles carry `solo_loads` each, the later ones `per_tile`.
-  const int solo_tiles = kSoloPrologue ? issued : 0;
-  const int solo_loads = score_wave ? 0 : per_tile + kRowsPerWave;
-  const auto newer_than = [&](int t) __attribute__((always_inline)) {
-    const int solo = max(0, min(issued, solo_tiles) - (t + 1));
-    const int shared = max(0, issued - max(t + 1, solo_tiles));
-    return solo * solo_loads + shared * per_tile;
-  };
-  MLAKV_STAMP(2);
-  WaitLoads(last_unknown >= 0 ? 0 : newer_than(0));
-  __syncthreads();
-  MLAKV_STAMP(3);
-
-  // Top of iteration i, both roles: tile i+1 must have landed (later tiles may still be in
-  // flight); the barrier publishes it together with P(i) and retires every wave's reads of
-  // tile i-1, whose ring slot the next tile to be issued reuses.
-  const auto publish = [&](int i) __attribute__((always_inline)) {
-    MLAKV_STAMP((i) < 4 ? 4 + 6 * (i) : -1);
-    if (i + 1 < ntiles) WaitLoads(last_unknown >= i + 1 ? 0 : newer_than(i + 1));
-    __syncthreads();
-    MLAKV_STAMP((i) < 4 ? 5 + 6 * (i) : -1);
-  };
-  // Issues the next tile of the ring (tile i + kRing - 1 during iteration i), right after
-  // publish(i): the memory-bound shapes want every load in flight as early as possible (issuing
-  // after the score waves' MFMA phase, to skew the two MFMA phases of a SIMD, gained 6 % where
-  // the kernel is compute-bound and lost 4 % where it is not).
-  const auto issue_next = [&](int i) __attribute__((always_inline)) {
-    if (issued < ntiles) {
-      if (!issue(issued)) last_unknown = issued;
-      ++issued;
-    }
-    MLAKV_STAMP((i) < 4 ? 6 + 6 * (i) : -1);
-  };
-
-  unsigned char* p_lds = lds + G::kPOff + (hw * 64 + lane) * 16;           // + parity * kScoreWaves * 64 * 16
-  float* alpha_lds = reinterpret_cast<float*>(lds + G::kAlphaOff) + hw * 64 + lane;  // + parity * kScoreWaves * 64
-  float* inv_lds = reinterpret_cast<float*>(lds + G::kInvOff) + hw * 64 + lane;
-  int* flag_lds = reinterpret_cast<int*>(lds + G::kFlagOff) + hw;          // + parity * kScoreWaves
-
-  if (score_wave) {
-    // ---------------------------------------------------------------- score waves
-    // bf16 K reads: token = 16t + i16, chunk = 4 ks + g (latent, ks < 16) or 4 (ks - 16) + g (rope).
-    const int k_lat = i16 * Geom<false>::kLatRow, k_rope = Geom<false>::kLatRegion + i16 * Geom<false>::kRopeRow;
-    int k_e[4], kr_e[2];
-#pragma unroll
-    for (int j = 0; j < 4; ++j) k_e[j] = ((4 * j + g) ^ SwizzleLat(i16)) << 4;
-#pragma unroll
-    for (int j = 0; j < 2; ++j) kr_e[j] = ((4 * j + g) ^ SwizzleRope(i16)) << 4;
-    // K fragment of pipeline step `step` (k-step step/2, token subtile step&1) of the tile at `buf`.
-    const auto k_frag = [&](const unsigned char* buf, int step) __attribute__((always_inline)) {
-      const int ks = step >> 1, t = step & 1;
-      const int offset = ks < 16 ? k_lat + (ks >> 2) * 256 + k_e[ks & 3] + t * 16 * Geom<false>::kLatRow
-                                 : k_rope + kr_e[ks & 1] + t * 16 * Geom<false>::kRopeRow;
-      return *reinterpret_cast<const bf16x8*>(buf + offset);
-    };
-    // FP8 K reads: read u = 2 kp + t fetches the 16 codes k = 64 kp + 16 g .. +15 of token 16t + i16
-    // (k-steps 2kp and 2kp+1): chunk (4 kp + g) ^ swizzle(token) of the 512-byte row; kp = 8 is the
-    // rope row (chunk g ^ swizzle). The tile base is a multiple of 512, so the XOR with kp << 6 is
-    // applied to the lane-constant part.
-    int k8_lat[2];
-#pragma unroll
-    for (int t = 0; t < 2; ++t) k8_lat[t] = (16 * t + i16) * Geom<true>::kLatRow + ((g ^ SwizzleLat8(16 * t + i16)) << 4);
-    const int k8_rope = Geom<true>::kLatRegion + i16 * Geom<true>::kRopeRow + ((g ^ SwizzleRope8(i16)) << 4);
-    const auto k8_read = [&](const unsigned char* buf, int u) __attribute__((always_inline)) {
-      const int kp = u >> 1, t = u & 1;
-      const int offset = kp < 8 ? (k8_lat[t] ^ (kp << 6)) : k8_rope + t * 16 * Geom<true>::kRopeRow;
-      return *reinterpret_cast<const u32x4*>(buf + offset);
-    };
-
-    float m_ref = -__builtin_inff();  // reference maximum of the exponentials, log2 domain
-    float l_run = 0.0f;               // this lane's share of the running denominator
-
-    // S^T of tile `tile_rel`, its softmax against the running reference, P and the rescale
-    // request into the LDS slots of the tile's parity.
-    const auto score_tile = [&](int tile_rel, int issue_iteration) __attribute__((always_inline)) {
-      const unsigned char* buf = lds + ring(tile_rel);
-      f32x4 acc[4];
-#pragma unroll
-      for (int j = 0; j < 4; ++j) acc[j] = f32x4{0.f, 0.f, 0.f, 0.f};
-      f32x4 row_scale[2];  // FP8: scales of tokens 4g+j and 16+4g+j
-      if constexpr (FP8) {
-        const float* scales = reinterpret_cast<const float*>(buf + G::kScaleOff);
-        row_scale[0] = *reinterpret_cast<const f32x4*>(scales + 4 * g);
-        row_scale[1] = *reinterpret_cast<const f32x4*>(scales + 16 + 4 * g);
-        u32x4 kr[kKAhead8];
-#pragma unroll
-        for (int d = 0; d < kKAhead8; ++d) kr[d] = k8_read(buf, d);
-        __builtin_amdgcn_sched_barrier(0);
-        StaticFor<kKSteps>([&](auto u_c) __attribute__((always_inline)) {
-          constexpr int u = decltype(u_c)::value;  // kp = u / 2, token subtile t = u & 1
-          const u32x4 codes = kr[u % kKAhead8];
-          if constexpr (u + kKAhead8 < kKSteps) kr[u % kKAhead8] = k8_read(buf, u + kKAhead8);
-          constexpr int t = u & 1, kp = u >> 1;
-          acc[2 * t] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(CodesToBf16(codes.x, codes.y), q[2 * kp], acc[2 * t], 0, 0, 0);
-          acc[2 * t + 1] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(CodesToBf16(codes.z, codes.w), q[2 * kp + 1], acc[2 * t + 1], 0, 0, 0);
-          __builtin_amdgcn_sched_barrier(0);
-        });
-      } else {
-        bf16x8 kf[kKAhead];
-#pragma unroll
-        for (int d = 0; d < kKAhead; ++d) kf[d] = k_frag(buf, d);
-        __builtin_amdgcn_sched_barrier(0);
-        StaticFor<kQkSteps>([&](auto step_c) __attribute__((always_inline)) {
-          constexpr int step = decltype(step_c)::value;
-          constexpr int slot = (step & 1) * 2 + ((step >> 1) & 1);  // two accumulators per token subtile
-          acc[slot] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(kf[step % kKAhead], q[step >> 1], acc[slot], 0, 0, 0);
-          if constexpr (step + kKAhead < kQkSteps) kf[step % kKAhead] = k_frag(buf, step + kKAhead);
-          __builtin_amdgcn_sched_barrier(0);
-        });
-      }
-      MLAKV_STAMP(tile_rel >= 1 && tile_rel <= 4 ? 7 + 6 * (tile_rel - 1) : -1);
-      if (kLateIssue && issue_iteration >= 0) issue_next(issue_iteration);
-      // lane holds tokens 4g+j (x[0..3]) and 16+4g+j (x[4..7]) of head i16
-      float x[8];
-#pragma unroll
-      for (int j = 0; j < 4; ++j) {
-        x[j] = (acc[0][j] + acc[1][j]) * a.scale_log2;
-        x[4 + j] = (acc[2][j] + acc[3][j]) * a.scale_log2;
-        if constexpr (FP8) {  // the codes were multiplied unscaled
-          x[j] *= row_scale[0][j];
-          x[4 + j] *= row_scale[1][j];
-        }
-      }
-      const int valid = seq_len - (tile_begin + tile_rel) * kTileTokens;  // >= 1
-      if (valid < kTileTokens) {  // wave-uniform: only the last tile of a sequence
-#pragma unroll
-        for (int j = 0; j < 8; ++j) {
-          if (16 * (j >> 2) + 4 * g + (j & 3) >= valid) x[j] = -__builtin_inff();
-        }
-      }
-      float tile_max = fmaxf(fmaxf(fmaxf(x[0], x[1]), fmaxf(x[2], x[3])), fmaxf(fmaxf(x[4], x[5]), fmaxf(x[6], x[7])));
-      tile_max = MaxAcrossHalves(MaxAcrossRows16(tile_max));
-      const int parity = tile_rel & 1;
-      // Move the reference only when some head's maximum outgrew it by more than the threshold.
-      const bool moved = __builtin_amdgcn_ballot_w64(tile_max > m_ref + kRescaleThreshold) != 0;
-      if (moved) {
-        const float m_new = fmaxf(m_ref, tile_max);  // finite: token 0 of the tile is valid
-        const float alpha = __builtin_amdgcn_exp2f(m_ref - m_new);
-        l_run *= alpha;
-        m_ref = m_new;
-        alpha_lds[parity * kScoreWaves * 64] = alpha;
-      }
-      if (lane == 0) flag_lds[parity * kScoreWaves] = moved && tile_rel != 0 ? 1 : 0;  // O is still zero on the first tile
-      bf16x8 p;
-      float sum = 0.0f;
-#pragma unroll
-      for (int j = 0; j < 8; ++j) {
-        const float e = __builtin_amdgcn_exp2f(x[j] - m_ref);
-        sum += e;
-        p[j] = static_cast<__bf16>(FP8 ? e * row_scale[j >> 2][j & 3] : e);  // FP8: V is multiplied unscaled as well
-      }
-      l_run += sum;
-      *reinterpret_cast<bf16x8*>(p_lds + parity * kScoreWaves * 64 * 16) = p;
-      MLAKV_STAMP(tile_rel >= 1 && tile_rel <= 4 ? 8 + 6 * (tile_rel - 1) : -1);
-    };
-
-    if (active) score_tile(0, -1);
-    for (int i = 0; i < ntiles; ++i) {
-      publish(i);
-      const bool scores = active && i + 1 < ntiles;
-      if (!kLateIssue || !scores) issue_next(i);
-      if (scores) score_tile(i + 1, i);
-    }
-    if (active) {
-      const float l_total = SumAcrossHeadLanes(l_run);
-      *inv_lds = 1.0f / l_total;
-      const float lse2 = m_ref + __builtin_amdgcn_logf(l_total);  // v_log_f32 is log2
-      if (g == 0) {
-        if (direct) {
-          if (a.lse != nullptr) a.lse[seq * a.heads + head] = lse2 * 0.6931471805599453f;
-        } else {
-          a.partial_lse[(static_cast<int64_t>(seq) * a.max_chunks + chunk_index) * a.heads + head] = lse2;
-        }
-      }
-    }
-    MLAKV_STAMP(29);
-    __syncthreads();  // 1/denominator visible to the output waves
-    MLAKV_STAMP(30);
-  } else {
-    // ---------------------------------------------------------------- output waves
-    // bf16 V reads: token = (16 +) 4g + i16/4, chunk = 2n + (i16 & 3) / 2, 8-byte half i16 & 1.
-    const int v_row = 4 * g + (i16 >> 2);
-    const int v_lane = v_row * Geom<false>::kLatRow + (i16 & 1) * 8;
-    int v_e[8];
-#pragma unroll
-    for (int j = 0; j < 8; ++j) v_e[j] = ((2 * j + ((i16 & 3) >> 1)) ^ SwizzleLat(v_row)) << 4;
-    // FP8 V reads (ds_read_b64_tr_b8: output lane i of a 16-lane group, element e <- byte i & 7 of
-    // the 8 bytes addressed by lane 2e + (i >> 3)): as a source, lane j addresses bytes
-    // 16n + 8 (j & 1) .. +7 of the row of token kappa = j >> 1 (tokens 4g + kappa, 16 + 4g + kappa - 4).
-    const int v8_token = 4 * g + ((i16 >> 1) & 3) + 16 * (i16 >> 3);
-    const int v8_base = v8_token * Geom<true>::kLatRow + (SwizzleLat8(v8_token) << 4) + 8 * (i16 & 1);
-    // Raw V^T fragment of output tile n (dv 16n..16n+15) over the 32 tokens of the tile at `buf`:
-    // eight bf16 for bf16 tiles, eight codes in the low two dwords for FP8 tiles.
-    const auto v_fetch = [&](const unsigned char* buf, int n) __attribute__((always_inline)) {
-      if constexpr (FP8) {
-        const i32x2 codes = __builtin_amdgcn_ds_read_tr8_b64_v2i32((__attribute__((address_space(3))) i32x2*)(buf + (v8_base ^ (n << 4))));
-        return u32x4{static_cast<unsigned>(codes.x), static_cast<unsigned>(codes.y), 0u, 0u};
-      } else {
-        const unsigned char* addr = buf + v_lane + (n >> 3) * 256 + v_e[n & 7];
-        const s16x4 lo = __builtin_amdgcn_ds_read_tr16_b64_v4i16((__attribute__((address_space(3))) s16x4*)(addr));
-        const s16x4 hi = __builtin_amdgcn_ds_read_tr16_b64_v4i16((__attribute__((address_space(3))) s16x4*)(addr + 16 * Geom<false>::kLatRow));
-        return __builtin_bit_cast(u32x4, __builtin_shufflevector(lo, hi, 0, 1, 2, 3, 4, 5, 6, 7));
-      }
-    };
-    const auto v_operand = [&](const u32x4& raw) __attribute__((always_inline)) {
-      if constexpr (FP8) {
-        return CodesToBf16(raw.x, raw.y);
-      } else {
-        return __builtin_bit_cast(bf16x8, raw);
-      }
-    };
-
-    // Output wave w owns the 128 output columns [128 w, 128 w + 128) of all 64 heads of the group:
-    // every V^T fragment is then fetched (and, for FP8, converted) by one wave only, and meets the
-    // P fragments of the four score waves. (With one head block per output wave, each of the four
-    // read and converted all of V.) Head blocks past the group's heads are computed on whatever
-    // their LDS slots hold and never written.
-    constexpr int kDvPerWave = kDvTiles / (kWaves - kScoreWaves);
-    const int hba = min(kScoreWaves, (a.heads - static_cast<int>(blockIdx.z) * 64 + 15) >> 4);  // head blocks in use
-    const unsigned char* p_all = lds + G::kPOff + lane * 16;                                   // + (parity * 4 + hb) * 64 * 16
-    const float* alpha_all = reinterpret_cast<const float*>(lds + G::kAlphaOff) + lane;      // + (parity * 4 + hb) * 64
-    const float* inv_all = reinterpret_cast<const float*>(lds + G::kInvOff) + lane;          // + hb * 64
-    const int* flag_all = reinterpret_cast<const int*>(lds + G::kFlagOff);                   // [parity * 4 + hb]
-    f32x4 o[kScoreWaves][kDvPerWave];
-#pragma unroll
-    for (int hb = 0; hb < kScoreWaves; ++hb) {
-#pragma unroll
-      for (int n = 0; n < kDvPerWave; ++n) o[hb][n] = f32x4{0.f, 0.f, 0.f, 0.f};
-    }
-
-    for (int i = 0; i < ntiles; ++i) {
-      publish(i);
-      issue_next(i);
-      {
-        const unsigned char* buf = lds + ring(i);
-        const int parity = i & 1;
-        // the four rescale flags of the tile in one read; a moved reference maximum is the exception
-        const i32x4 flags = *reinterpret_cast<const i32x4*>(flag_all + parity * kScoreWaves);
-        if (Uniform(flags.x | flags.y | flags.z | flags.w) != 0) {
-          const int moved[kScoreWaves] = {flags.x, flags.y, flags.z, flags.w};
-#pragma unroll
-          for (int hb = 0; hb < kScoreWaves; ++hb) {
-            if (Uniform(moved[hb]) != 0) {  // that block's reference maximum moved: rescale its O first
-              const float alpha = alpha_all[(parity * kScoreWaves + hb) * 64];
-#pragma unroll
-              for (int n = 0; n < kDvPerWave; ++n) o[hb][n] *= alpha;
-            }
-          }
-        }
-        u32x4 vf[kVAhead];
-#pragma unroll
-        for (int d = 0; d < kVAhead; ++d) vf[d] = v_fetch(buf, kDvPerWave * hw + d);
-        bf16x8 p[kScoreWaves];
-#pragma unroll
-        for (int hb = 0; hb < kScoreWaves; ++hb) p[hb] = *reinterpret_cast<const bf16x8*>(p_all + (parity * kScoreWaves + hb) * 64 * 16);
-        __builtin_amdgcn_sched_barrier(0);
-        if constexpr (FP8) {
-          // the next fragment is converted while this one's four MFMAs run
-          bf16x8 v = v_operand(vf[0]);
-          if constexpr (kVAhead < kDvPerWave) vf[0] = v_fetch(buf, kDvPerWave * hw + kVAhead);
-          StaticFor<kDvPerWave>([&](auto n_c) __attribute__((always_inline)) {
-            constexpr int n = decltype(n_c)::value;
-            bf16x8 v_next = v;
-            if constexpr (n + 1 < kDvPerWave) v_next = v_operand(vf[(n + 1) % kVAhead]);
-#pragma unroll
-            for (int hb = 0; hb < kScoreWaves; ++hb) o[hb][n] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(v, p[hb], o[hb][n], 0, 0, 0);
-            if constexpr (n + 1 + kVAhead < kDvPerWave) vf[(n + 1) % kVAhead] = v_fetch(buf, kDvPerWave * hw + n + 1 + kVAhead);
-            v = v_next;
-            __builtin_amdgcn_sched_barrier(0);
-          });
-        } else {
-          StaticFor<kDvPerWave>([&](auto n_c) __attribute__((always_inline)) {
-            constexpr int n = decltype(n_c)::value;
-            const bf16x8 v = v_operand(vf[n % kVAhead]);
-#pragma unroll
-            for (int hb = 0; hb < kScoreWaves; ++hb) o[hb][n] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(v, p[hb], o[hb][n], 0, 0, 0);
-            if constexpr (n + kVAhead < kDvPerWave) vf[n % kVAhead] = v_fetch(buf, kDvPerWave * hw + n + kVAhead);
-            __builtin_amdgcn_sched_barrier(0);
-          });
-        }
-        MLAKV_STAMP((i) < 4 ? 7 + 6 * (i) : -1);
-      }
-    }
-    MLAKV_STAMP(29);
-    __syncthreads();  // 1/denominator from the score waves
-    MLAKV_STAMP(30);
-    const int group_head0 = static_cast<int>(blockIdx.z) * 64;
-    // Row (bf16 [512]) of head `h` of this group in the launch's output: the final output when
-    // there is one chunk, this chunk's partial otherwise.
-    const auto row_of = [&](int h) __attribute__((always_inline)) -> char* {
-      if (direct) return a.out + seq * a.out_seq_stride + (group_head0 + h) * a.out_head_stride;
-      const int64_t row = (static_cast<int64_t>(seq) * a.max_chunks + chunk_index) * a.heads + group_head0 + h;
-      return a.partial_out + row * (kLatentDim * 2);
-    };
-    if (MXQ && direct) {
-      // Quantising epilogue of the single-chunk case: a block of 32 columns is a pair of this
-      // wave's column tiles over the four lanes that share a head; the wave covers blocks
-      // 4 w .. 4 w + 3 of every head.
-#pragma unroll
-      for (int hb = 0; hb < kScoreWaves; ++hb) {
-        if (hb >= hba) continue;
-        const int h = 16 * hb + i16;
-        const float inv = inv_all[hb * 64];
-        char* codes_row = a.out_codes + seq * a.out_codes_seq_stride + (group_head0 + h) * a.out_codes_head_stride;
-        char* out_row = a.out == nullptr ? nullptr : row_of(h);
-        unsigned scale_codes = 0u;
-#pragma unroll
-        for (int k = 0; k < kDvPerWave / 2; ++k) {
-          u32x2 packed[2];
-          unsigned magnitude = 0u;
-#pragma unroll
-          for (int half = 0; half < 2; ++half) {
-            const int n = 2 * k + half;
-            packed[half].x = PackBf16(o[hb][n][0] * inv, o[hb][n][1] * inv);
-            packed[half].y = PackBf16(o[hb][n][2] * inv, o[hb][n][3] * inv);
-            magnitude = MxMagnitudeMax(packed[half].y, MxMagnitudeMax(packed[half].x, magnitude));
-            if (out_row != nullptr) {
-              __builtin_nontemporal_store(packed[half], reinterpret_cast<u32x2*>(out_row + (16 * (kDvPerWave * hw + n) + 4 * g) * 2));
-            }
-          }
-          magnitude = UMaxAcrossHeadLanes(magnitude);
-          const MxScale s = MxScaleFromMaxBits(magnitude);
-#pragma unroll
-          for (int half = 0; half < 2; ++half) {
-            const unsigned four = MxEncodeWord(packed[half].x, s) | (MxEncodeWord(packed[half].y, s) << 16);
-            __builtin_nontemporal_store(four, reinterpret_cast<unsigned*>(codes_row + 16 * (kDvPerWave * hw + 2 * k + half) + 4 * g));
-          }
-          scale_codes |= s.code << (8 * k);
-        }
-        if (g == 0) {
-          *reinterpret_cast<unsigned*>(a.out_scales + seq * a.out_scales_seq_stride + (group_head0 + h) * a.out_scales_head_stride +
-                                       (kDvPerWave / 2) * hw) = scale_codes;
-        }
-      }
-    } else {
-      // The accumulators hold O^T (lane = head i16 of a block, four columns per 16-column tile),
-      // which stored as it is would write 8-byte pieces of sixteen different rows per
-      // instruction. The tile ring is dead after the last barrier: each output wave transposes
-      // its 256-byte slices of the 64 rows through its own part of it and writes them 16 bytes per
-      // lane, four whole slices per instruction. A row stride of 272 bytes (= 4 banks mod 64)
-      // spreads the 8-byte writes of a half-wave over all banks.
-      constexpr int kSliceBytes = kDvPerWave * 16 * 2;  // 256
-      constexpr int kStageRow = kSliceBytes + 16;
-      static_assert((kWaves - kScoreWaves) * 64 * kStageRow <= G::kRing * G::kTileBytes, "the staging rows fit in the ring");
-      unsigned char* stage = lds + G::Slot(0) + hw * (64 * kStageRow);
-#pragma unroll
-      for (int hb = 0; hb < kScoreWaves; ++hb) {
-        const float inv = inv_all[hb * 64];
-#pragma unroll
-        for (int n = 0; n < kDvPerWave; ++n) {
-          u32x2 packed;
-          packed.x = PackBf16(o[hb][n][0] * inv, o[hb][n][1] * inv);
-          packed.y = PackBf16(o[hb][n][2] * inv, o[hb][n][3] * inv);
-          *reinterpret_cast<u32x2*>(stage + (16 * hb + i16) * kStageRow + (16 * n + 4 * g) * 2) = packed;
-        }
-      }
-      // Same wave wrote and reads: the LDS queue is in order, no barrier needed.
-      const int piece = lane & 15, sub = lane >> 4;
-#pragma unroll
-      for (int it = 0; it < 16; ++it) {
-        const int h = 4 * it + sub;
-        if (h < 16 * hba) {
-          const u32x4 v = *reinterpret_cast<const u32x4*>(stage + h * kStageRow + piece * 16);
-          __builtin_nontemporal_store(v, reinterpret_cast<u32x4*>(row_of(h) + kSliceBytes * hw + piece * 16));
-        }
-      }
-    }
-    MLAKV_STAMP(31);
   }
 }
 
-// Merges the chunks of one (sequence, head): out = sum_c w_c O_c / sum_c w_c with
-// w_c = 2^(lse2_c - max lse2). 256 threads = 4 heads x 64 lanes, 8 output columns per lane.
-// Every chunk slot carries an LSE (-inf for a chunk past the end of its sequence, whose O slot
-// was never written), so all loads of a group of eight chunks are issued at once, with no
-// dependence on the sequence length.
-constexpr int kCombineHeads = 4;
-__global__ __launch_bounds__(kCombineHeads * 64) void MlaCombineKernel(AttnArgs a) {
-  // Workgroups go to the XCDs round-robin by linear id; the main kernel put all chunks of a
-  // sequence on XCD seq / (batch / 8), and the partials are most likely still in that L2.
-  int group = blockIdx.x, seq = blockIdx.y;
-  if ((gridDim.y & (kXcds - 1)) == 0) {
-    const int linear = blockIdx.y * gridDim.x + blockIdx.x;
-    const int within = linear / kXcds;
-    seq = (linear & (kXcds - 1)) * (gridDim.y / kXcds) + within / static_cast<int>(gridDim.x);
-    group = within % static_cast<int>(gridDim.x);
-  }
-  const int head = group * kCombineHeads + (threadIdx.x >> 6);
-  const int lane = threadIdx.x & 63;
-  if (head >= a.heads) return;
-  const int chunks = a.max_chunks;
-  const int64_t row0 = static_cast<int64_t>(seq) * chunks * a.heads + head;
+// Merges the `n` partials of (sequence, head): out = sum_c w_c O_c / sum_c w_c with
+// w_c = 2^(lse2_c - max lse2), in the order of the sequence's tiles. One wave, 8 output columns
+// per lane. Partial 0 sits in slot `first_slot`, partial i > 0 in slot `u0 + i`. Every partial
+// carries an LSE (-inf for an empty one, whose O row is not data), so the loads of a group of
+// eight partials are issued together.
+// AGENT: the partials were written by other CUs of this launch (agent-scope loads); otherwise by
+// an earlier launch (plain streaming loads).
+template <bool MXQ, bool AGENT>
+__device__ __forceinline__ void MergeHead(const AttnArgs& a, int z, int seq, int head_in_group, int first_slot, int u0, int n, int lane) {
+  const int head = 64 * z + head_in_group;
   float acc[8];
 #pragma unroll
   for (int j = 0; j < 8; ++j) acc[j] = 0.0f;
   float m = -__builtin_inff(), denom = 0.0f;
-  for (int c0 = 0; c0 < chunks; c0 += 8) {
+  for (int c0 = 0; c0 < n; c0 += 8) {
     u32x4 v[8];
     float l[8];
 #pragma unroll
     for (int u = 0; u < 8; ++u) {
-      const int c = min(c0 + u, chunks - 1);
-      const int64_t row = row0 + static_cast<int64_t>(c) * a.heads;
-      l[u] = c0 + u < chunks ? a.partial_lse[row] : -__builtin_inff();
-      v[u] = __builtin_nontemporal_load(reinterpret_cast<const u32x4*>(a.partial_out + row * (kLatentDim * 2) + lane * 16));
+      const int c = min(c0 + u, n - 1);
+      const int64_t row = PartialRow(a, z, c == 0 ? first_slot : u0 + c, head_in_group);
+      if constexpr (AGENT) {
+        l[u] = c0 + u < n ? LoadAgentF32(a.partial_lse + row) : -__builtin_inff();
+        v[u] = LoadAgent16(a.partial_out + row * (kLatentDim * 2) + lane * 16);
+      } else {
+        l[u] = c0 + u < n ? a.partial_lse[row] : -__builtin_inff();
+        v[u] = __builtin_nontemporal_load(reinterpret_cast<const u32x4*>(a.partial_out + row * (kLatentDim * 2) + lane * 16));
+      }
     }
+    if constexpr (AGENT) WaitAgentLoads(v);
     float group_max = m;
 #pragma unroll
     for (int u = 0; u < 8; ++u) group_max = fmaxf(group_max, l[u]);
-    if (group_max == -__builtin_inff()) continue;  // nothing but empty chunks so far
+    if (group_max == -__builtin_inff()) continue;  // nothing but empty partials so far
     const float rescale = __builtin_amdgcn_exp2f(m - group_max);  // 0 on the first group
     m = group_max;
     denom *= rescale;
@@ -1068,7 +589,7 @@ __global__ __launch_bounds__(kCombineHeads * 64) void MlaCombineKernel(AttnArgs 
     for (int j = 0; j < 8; ++j) acc[j] *= rescale;
 #pragma unroll
     for (int u = 0; u < 8; ++u) {
-      if (l[u] == -__builtin_inff()) continue;  // empty or padding slot: its O bytes are not data
+      if (l[u] == -__builtin_inff()) continue;  // empty or padding slot
       const float w = __builtin_amdgcn_exp2f(l[u] - m);
       denom += w;
       const unsigned words[4] = {v[u].x, v[u].y, v[u].z, v[u].w};
@@ -1079,7 +600,7 @@ __global__ __launch_bounds__(kCombineHeads * 64) void MlaCombineKernel(AttnArgs 
       }
     }
   }
-  // An empty sequence (no live chunk) yields zeros and lse = -inf.
+  // Nothing but empty partials yields zeros and lse = -inf.
   const float inv = denom == 0.0f ? 0.0f : 1.0f / denom;
   u32x4 packed;
   packed.x = PackBf16(acc[0] * inv, acc[1] * inv);
@@ -1087,7 +608,7 @@ __global__ __launch_bounds__(kCombineHeads * 64) void MlaCombineKernel(AttnArgs 
   packed.z = PackBf16(acc[4] * inv, acc[5] * inv);
   packed.w = PackBf16(acc[6] * inv, acc[7] * inv);
   if (a.out != nullptr) *reinterpret_cast<u32x4*>(a.out + seq * a.out_seq_stride + head * a.out_head_stride + lane * 16) = packed;
-  if (a.out_codes != nullptr) {
+  if constexpr (MXQ) {
     // Quantising epilogue (the reference's stage behind the attention): the four lanes of a
     // block of 32 columns are neighbours; the codes come from the bf16-rounded values, as they
     // would from the bf16 tensor.
@@ -1111,6 +632,751 @@ __global__ __launch_bounds__(kCombineHeads * 64) void MlaCombineKernel(AttnArgs 
   }
 }
 
+// ---- main kernel -------------------------------------------------------------------
+
+// MXQ: the launch also quantises its output (and its bf16 output is optional). Kept out of the
+// common instantiation, whose register allocation has no room to spare.
+// SPARSE: every sequence attends to the tokens listed in a.sparse_indices instead of to its whole
+// context (never ALIGNED: every row is located on its own); on the flat tile axis every sequence
+// counts with the full length of the list.
+template <bool FP8, bool ALIGNED, bool MXQ, bool SPARSE>
+__global__ __launch_bounds__(kThreads) void MlaDecodeKernel(AttnArgs a) {
+  static_assert(!(SPARSE && ALIGNED), "selected-token attention uses the row-at-a-time path");
+  // bf16 tiles: the output waves, which have no query to wait for, issue the first tiles of the
+  // ring alone (their own rows and those of their partner score waves) as soon as they know the
+  // block-table entries; the score waves join from the first loop iteration on.
+  constexpr bool kSoloPrologue = !FP8 && !SPARSE;
+  using G = Geom<FP8>;
+  extern __shared__ __attribute__((aligned(16))) unsigned char lds[];
+  const unsigned lds_base = static_cast<unsigned>(reinterpret_cast<size_t>((__attribute__((address_space(3))) unsigned char*)lds));
+  const int tid0 = threadIdx.x;
+  const int lane0 = tid0 & 63, wave0 = Uniform(tid0 >> 6);
+  // Workgroups are handed to the eight XCDs round-robin by linear id, and each XCD has its own
+  // L2. Neighbouring units mostly belong to one sequence and read the same 72 KB of Q, so XCD x
+  // takes the contiguous range of units [x, x+1) * W / 8.
+  const int work_groups = gridDim.x;
+  int wg = blockIdx.x;
+  if ((work_groups & (kXcds - 1)) == 0) wg = (wg & (kXcds - 1)) * (work_groups / kXcds) + wg / kXcds;
+  const int z = blockIdx.y;  // group of 64 heads
+
+  // Every wave walks the batch itself: the total number of tiles fixes the cut of the flat axis.
+  // On the way the empty sequences (no tile, so no unit) get their zeros, spread over the workgroups.
+  SeqWindow<SPARSE> win;
+  win.Load(a, lane0, 0, 0);
+  for (;;) {
+    if constexpr (!SPARSE) {
+      u64 empties = __builtin_amdgcn_ballot_w64(win.base + lane0 < a.batch && win.tiles == 0);
+      while (empties != 0) {
+        const int s = win.base + __builtin_ctzll(empties);
+        if (s % work_groups == wg) ZeroFill<MXQ>(a, z, s, wave0, lane0);
+        empties &= empties - 1;
+      }
+    }
+    if (win.base + 64 >= a.batch) break;
+    win.Load(a, lane0, win.base + 64, win.End());
+  }
+  const int total_tiles = win.End();
+  int tiles_per_unit = a.forced_unit_tiles > 0 ? a.forced_unit_tiles : max(a.min_unit_tiles, (total_tiles + work_groups - 1) / work_groups);
+  tiles_per_unit = min(tiles_per_unit, a.cap_unit_tiles);
+  const int units = (total_tiles + tiles_per_unit - 1) / tiles_per_unit;  // <= a.max_units, ensured by the plan
+  if (wg >= units) return;
+  if (win.base != 0) win.Load(a, lane0, 0, 0);
+
+  // Q fragments (score waves): lane (head i16, k-group g) holds, for k-step ks, the eight query
+  // elements that meet the lane's K fragment of that step: Q[head][32 ks + 8g .. +7] for bf16
+  // tiles; for FP8 tiles one 16-byte K read feeds two k-steps, so the order inside each 64-wide
+  // window is Q[head][64 (ks/2) + 16g + 8 (ks&1) .. +7]. (Loaded per segment, once the table
+  // entries have been asked for.)
+
+  const auto ring = [&](int i) __attribute__((always_inline)) { return G::Slot(i); };
+  int* table_lds = reinterpret_cast<int*>(lds + G::kTableOff);
+  int* scalar_lds = reinterpret_cast<int*>(lds + G::kFlagOff) + 2 * kScoreWaves;  // a few words for workgroup-wide values
+  i32x4* duty_lds = reinterpret_cast<i32x4*>(lds + G::kDutyOff);
+  int duties = 0;  // uniform over the workgroup
+  const int group_head0 = z * 64;
+  const int heads_here = min(64, a.heads - group_head0);
+  const int hba = (heads_here + 15) >> 4;  // head blocks in use
+  unsigned* const sync_group = a.sync == nullptr ? nullptr : a.sync + static_cast<int64_t>(z) * a.batch * 2;
+
+  // Carries out the merges promised so far; entry: (sequence, first unit, partials, rank). Two
+  // words per (head group, sequence), zero between launches:
+  //   word 0: partials announced (low 16 bits) | contributors that gave up waiting (high 16 bits)
+  //   word 1: contributors that are through with word 0; the last of them clears both.
+  // A contributor announces its partial, waits (bounded) until all are announced and merges its
+  // share of the heads, rank, rank + n, ... in steps of eight heads. One that gives up before the
+  // count is full says so in the same word and leaves; the contributor whose announcement fills
+  // the count sees that somebody gave up (not who) and merges every share. A share may then be
+  // merged twice, by its owner as well: both write the same bytes.
+  const auto flush_duties = [&]() __attribute__((always_inline)) {
+    const int merge_units = (heads_here + kMergeHeads - 1) / kMergeHeads;
+    asm volatile("s_waitcnt vmcnt(0)" ::: "memory");  // this wave's partial stores are complete
+    __syncthreads();                                  // every wave's are, and the entries are visible
+    // All announcements first (a workgroup with several units may hold several partials of one
+    // sequence); thread 0 keeps what each found.
+    unsigned* found_lds = reinterpret_cast<unsigned*>(lds + G::kFoundOff);
+    if (tid0 == 0) {
+      for (int d = 0; d < duties; ++d) {
+        found_lds[d] = __hip_atomic_fetch_add(sync_group + duty_lds[d].x * 2, 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+      }
+    }
+    for (int d = 0; d < duties; ++d) {
+      const i32x4 duty = duty_lds[d];
+      const int seq = Uniform(duty.x), u0 = Uniform(duty.y), n = Uniform(duty.z), rank = Uniform(duty.w);
+      unsigned* words = sync_group + seq * 2;
+      unsigned through = 0u;
+      if (tid0 == 0) {
+        const unsigned before = found_lds[d];
+        int share = 1;  // 0: leave it to the last contributor, 1: own share, 2: every share
+        if ((before & 0xffffu) == static_cast<unsigned>(n - 1)) {
+          share = (before >> 16) != 0u ? 2 : 1;
+        } else {
+          const u64 t0 = __builtin_amdgcn_s_memrealtime();
+          for (;;) {
+            if ((__hip_atomic_load(words, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT) & 0xffffu) == static_cast<unsigned>(n)) break;
+            if (__builtin_amdgcn_s_memrealtime() - t0 >= static_cast<u64>(a.spin_ticks)) {
+              // giving up: unless the count filled in the meantime, the last contributor will know
+              const unsigned found = __hip_atomic_fetch_add(words, 0x10000u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+              if ((found & 0xffffu) != static_cast<unsigned>(n)) share = 0;
+              break;
+            }
+            __builtin_amdgcn_s_sleep(2);
+          }
+        }
+        // through with word 0; the answer is looked at after the merge
+        through = __hip_atomic_fetch_add(words + 1, 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+        scalar_lds[1] = share;
+      }
+      __syncthreads();
+      const int share = Uniform(scalar_lds[1]);
+      if (share != 0) {
+        for (int u = share == 2 ? 0 : rank; u < merge_units; u += share == 2 ? 1 : n) {
+          const int h = u * kMergeHeads + wave0;
+          if (h < heads_here) MergeHead<MXQ, true>(a, z, seq, h, a.max_units + seq, u0, n, lane0);
+        }
+      }
+      __syncthreads();  // scalar_lds[1] is free again
+      if (tid0 == 0 && through == static_cast<unsigned>(n - 1)) {
+        __hip_atomic_store(words, 0u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+        __hip_atomic_store(words + 1, 0u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+      }
+    }
+    duties = 0;
+  };
+
+  for (int unit = wg; unit < units; unit += work_groups) {
+    const int flat_end = min(total_tiles, (unit + 1) * tiles_per_unit);
+    int flat = unit * tiles_per_unit;
+    while (win.End() <= flat) win.Load(a, lane0, win.base + 64, win.End());
+    int seq = win.base + __builtin_ctzll(__builtin_amdgcn_ballot_w64(win.incl > flat));
+    while (flat < flat_end) {
+      // Segment: tiles [flat, segment_end) of the flat axis, inside sequence `seq`.
+      const int seq_end = win.Incl(seq), seq_begin = seq_end - win.Tiles(seq);
+      const int segment_end = min(flat_end, seq_end);
+      const int tile_begin = flat - seq_begin;          // first tile of the segment inside its sequence
+      const int segment_tiles = segment_end - flat;     // >= 1
+      const bool holds_first = flat == seq_begin, holds_last = segment_end == seq_end;
+      const bool direct = holds_first && holds_last;    // the whole sequence: write the final output here
+      const int slot = holds_first ? a.max_units + seq : unit;
+      int seq_len = win.Tok(seq);
+
+      __syncthreads();  // the previous segment's staging rows, table entries and P slots are free
+
+      // Everything that depends on the thread id alone is formed here, per segment, from a copy
+      // of the id that the compiler cannot see through: hoisted out of the segment loop, these
+      // values would stay live through both roles' tile loops, where no register is to spare.
+      int tid = tid0;
+      asm volatile("" : "+v"(tid));
+      const int lane = tid & 63, wave = Uniform(tid >> 6);
+      const bool score_wave = wave < kScoreWaves;   // wave-uniform role
+      const int hw = wave & (kScoreWaves - 1);      // which 16 heads of the 64
+      const int g = lane >> 4, i16 = lane & 15;
+      const int head_base = z * 64 + hw * 16;
+      const bool active = head_base < a.heads;  // wave-uniform
+      const int head = head_base + i16;
+      const int per_tile = FP8 ? LoadsPerTile8(wave) : LoadsPerTile(wave);
+      // Direct loads: lane L of a latent row fetches chunk L ^ swizzle(row); rows of this wave.
+      IssueLane il;
+      IssueLane8 il8;
+      if (FP8) {
+    #pragma unroll
+        for (int j = 0; j < 2; ++j) {
+          const int row = 2 * wave + 16 * j + (lane >> 5);
+          il8.lat[j] = (lane >> 5) * static_cast<int>(a.latent.row_stride) + (((lane & 31) ^ SwizzleLat8(row)) << 4);
+        }
+        const int rope_row = 16 * (wave & 1) + (lane >> 2);
+        il8.rope = (lane >> 2) * static_cast<int>(a.rope.row_stride) + (((lane & 3) ^ SwizzleRope8(rope_row)) << 4);
+      } else {
+    #pragma unroll
+        for (int j = 0; j < 2; ++j) {
+          il.lat[j] = (lane ^ SwizzleLat(wave + kWaves * j)) << 4;
+          il.partner_lat[j] = (lane ^ SwizzleLat((wave & (kScoreWaves - 1)) + kWaves * j)) << 4;
+        }
+        il.rope_chunk = ((lane & 7) ^ SwizzleRope(8 * (wave - kScoreWaves) + (lane >> 3))) << 4;
+        il.rope = (lane >> 3) * static_cast<int>(a.rope.row_stride) + il.rope_chunk;
+      }
+
+      unsigned char* p_lds = lds + G::kPOff + (hw * 64 + lane) * 16;           // + parity * kScoreWaves * 64 * 16
+      float* alpha_lds = reinterpret_cast<float*>(lds + G::kAlphaOff) + hw * 64 + lane;  // + parity * kScoreWaves * 64
+      float* inv_lds = reinterpret_cast<float*>(lds + G::kInvOff) + hw * 64 + lane;
+      int* flag_lds = reinterpret_cast<int*>(lds + G::kFlagOff) + hw;          // + parity * kScoreWaves
+
+      // Stage this segment's block-table entries in LDS.
+      TileMap<ALIGNED> map;
+      map.entries = table_lds;
+      map.block_size = a.block_size;
+      map.sparse = SPARSE;
+      map.first_pos = tile_begin * kTileTokens;
+      map.first_block = 0;
+      map.next_entry = 0;
+      map.next_slot0 = 0;
+      map.tile_block = 0;
+      map.tile_slot0 = 0;
+      int staged[kTableEntries / 64];  // kSoloPrologue: this lane's table entries on their way to LDS
+      int staged_count = 0;
+      const auto write_table = [&]() __attribute__((always_inline)) {
+        if constexpr (kSoloPrologue) {
+#pragma unroll
+          for (int j = 0; j < kTableEntries / 64; ++j) {
+            const int i = lane + 64 * j;
+            if (i < staged_count) table_lds[i] = static_cast<unsigned>(staged[j]) < static_cast<unsigned>(a.num_blocks) ? staged[j] : -1;
+          }
+        }
+      };
+      if constexpr (!SPARSE) {
+        const int first_pos = tile_begin * kTileTokens;
+        const int last_pos = first_pos + segment_tiles * kTileTokens - 1;
+        map.first_block = first_pos / a.block_size;
+        map.next_slot0 = first_pos - map.first_block * a.block_size;
+        int count = last_pos / a.block_size - map.first_block + 1;  // <= kTableEntries, ensured by the plan's cap
+        count = min(count, a.table_stride - map.first_block);
+        const int32_t* table_row = a.block_table + static_cast<int64_t>(seq) * a.table_stride + map.first_block;
+        if constexpr (kSoloPrologue) {
+          // Every wave stages all entries itself (the same values to the same addresses), so that it
+          // can read them back without waiting for the other waves. Here they are only asked for;
+          // each role writes them to LDS where it first needs them (write_table below).
+          staged_count = count;
+#pragma unroll
+          for (int j = 0; j < kTableEntries / 64; ++j) {
+            const int i = lane + 64 * j;
+            staged[j] = i < count ? table_row[i] : -1;
+          }
+        } else {
+          for (int i = tid; i < count; i += kThreads) {
+            const int entry = table_row[i];
+            table_lds[i] = static_cast<unsigned>(entry) < static_cast<unsigned>(a.num_blocks) ? entry : -1;
+          }
+        }
+      } else {
+        // The selection ends at its first entry that is negative or not inside the context. Then
+        // this segment's part of it is resolved to pool slots through the block table.
+        const int context = static_cast<int>(
+            min(static_cast<int64_t>(max(Uniform(a.seq_lens[seq]), 0)), static_cast<int64_t>(a.table_stride) * a.block_size));
+        const int32_t* selection = a.sparse_indices + static_cast<int64_t>(seq) * a.sparse_seq_stride;
+        if (tid == 0) scalar_lds[0] = a.sparse_count;
+        __syncthreads();
+        for (int i = tid; i < a.sparse_count; i += kThreads) {
+          const int index = selection[i];
+          if (index < 0 || index >= context) atomicMin(scalar_lds, i);
+        }
+        __syncthreads();
+        seq_len = Uniform(scalar_lds[0]);
+        const int32_t* table_row = a.block_table + static_cast<int64_t>(seq) * a.table_stride;
+        const int segment_tokens = min(segment_tiles * kTileTokens, seq_len - map.first_pos);  // <= kTableEntries, ensured by the plan's cap
+        for (int i = tid; i < segment_tokens; i += kThreads) {
+          const int index = selection[map.first_pos + i];  // inside [0, context): before the end of the selection
+          const int logical = index / a.block_size;
+          const int entry = table_row[logical];
+          table_lds[i] = static_cast<unsigned>(entry) < static_cast<unsigned>(a.num_blocks)
+                             ? entry * a.block_size + (index - logical * a.block_size)
+                             : -1;
+        }
+      }
+      map.seq_len = seq_len;
+      const int num_tiles = (seq_len + kTileTokens - 1) / kTileTokens;
+      // tiles of this segment that exist (a selection may end before the list does)
+      const int ntiles = min(segment_tiles, num_tiles - tile_begin);
+      if (SPARSE && ntiles <= 0) {
+        if (direct) {
+          ZeroFill<MXQ>(a, z, seq, wave, lane);
+        } else if (active && score_wave && g == 0) {  // empty partial: the merge reads every partial's LSE
+          StoreAgentF32(a.partial_lse + PartialRow(a, z, slot, hw * 16 + i16), -__builtin_inff());
+        }
+      } else {
+        const auto issue = [&](int t) __attribute__((always_inline)) {
+          if constexpr (FP8) {
+            return IssueTileFp8(a, map, il8, tile_begin + t, lds_base + ring(t), lds + ring(t), tid);
+          } else {
+            return IssueTileBf16(a, map, il, tile_begin + t, lds_base + ring(t), lds + ring(t), tid);
+          }
+        };
+        // Prologue (each role runs its own copy, below): tiles 0 .. kRing-2 on their way, tile 0
+        // landed and published. A tile whose load count is not known (rare path) makes every wait
+        // up to and including its own a full one.
+        int last_unknown = -1;  // newest tile issued with an unknown number of loads
+        int issued = 0;         // tiles issued so far
+        // Loads this wave has in flight that are newer than those of tile t: the first `solo_tiles`
+        // tiles carry `solo_loads` each, the later ones `per_tile`.
+        const int solo_tiles = kSoloPrologue ? min(G::kRing - 1, ntiles) : 0;
+        const int solo_loads = score_wave ? 0 : per_tile + kRowsPerWave;
+        const auto newer_than = [&](int t) __attribute__((always_inline)) {
+          const int solo = max(0, min(issued, solo_tiles) - (t + 1));
+          const int shared = max(0, issued - max(t + 1, solo_tiles));
+          return solo * solo_loads + shared * per_tile;
+        };
+        // Top of iteration i, both roles: tile i+1 must have landed (later tiles may still be in
+        // flight); the barrier publishes it together with P(i) and retires every wave's reads of
+        // tile i-1, whose ring slot the next tile to be issued reuses.
+        const auto publish = [&](int i) __attribute__((always_inline)) {
+          if (i + 1 < ntiles) WaitLoads(last_unknown >= i + 1 ? 0 : newer_than(i + 1));
+          __syncthreads();
+        };
+        // Issues the next tile of the ring (tile i + kRing - 1 during iteration i).
+        const auto issue_next = [&](int i) __attribute__((always_inline)) {
+          if (issued < ntiles) {
+            if (!issue(issued)) last_unknown = issued;
+            ++issued;
+          }
+        };
+
+        if (score_wave) {
+          // ---------------------------------------------------------------- score waves
+          // Vector memory requests of a CU are served in order: the query (72 KB per workgroup) is
+          // asked for behind the few bytes of table entries that the first tile addresses depend on.
+          // It lives in this role's branch only; the output waves' prologue has no room for it.
+          bf16x8 q[kKSteps];
+          if (active) {
+            const char* q_latent = a.q_latent + seq * a.q_latent_seq_stride + head * a.q_latent_head_stride;
+            const char* q_rope = a.q_rope + seq * a.q_rope_seq_stride + head * a.q_rope_head_stride;
+#pragma unroll
+            for (int ks = 0; ks < kKSteps; ++ks) {
+              const int d0 = FP8 ? 64 * (ks >> 1) + 16 * g + 8 * (ks & 1) : 32 * ks + 8 * g;
+              const char* p = d0 < kLatentDim ? q_latent + d0 * 2 : q_rope + (d0 - kLatentDim) * 2;
+              q[ks] = __builtin_bit_cast(bf16x8, GlobalLoad16(p));
+            }
+          } else {
+#pragma unroll
+            for (int ks = 0; ks < kKSteps; ++ks) q[ks] = __builtin_bit_cast(bf16x8, u32x4{0u, 0u, 0u, 0u});
+          }
+          write_table();  // asked for before the query, so it is here first
+          // The query must have arrived before this wave issues tile loads: the compiler's own wait
+          // for it would otherwise also wait for every tile load issued in between. Both paths above
+          // pass through the statement: were it skipped on one, the compiler would have to assume the
+          // query still in flight where they meet again, and would wait for it -- with counts that
+          // know nothing of the tile loads, so in effect for every tile in flight -- inside the
+          // score loop, at every use.
+#pragma unroll
+          for (int ks = 0; ks < kKSteps; ++ks) asm volatile("" ::"v"(q[ks]));
+          if constexpr (!kSoloPrologue) __syncthreads();  // table entries visible
+          for (; issued < G::kRing - 1 && issued < ntiles; ++issued) {
+            if constexpr (kSoloPrologue) {
+              map.Begin(issued);  // keeps the cursor in step with the tiles this wave does not issue
+            } else {
+              if (!issue(issued)) last_unknown = issued;
+            }
+          }
+          WaitLoads(last_unknown >= 0 ? 0 : newer_than(0));
+          __syncthreads();
+
+          // bf16 K reads: token = 16t + i16, chunk = 4 ks + g (latent, ks < 16) or 4 (ks - 16) + g (rope).
+          const int k_lat = i16 * Geom<false>::kLatRow, k_rope = Geom<false>::kLatRegion + i16 * Geom<false>::kRopeRow;
+          int k_e[4], kr_e[2];
+#pragma unroll
+          for (int j = 0; j < 4; ++j) k_e[j] = ((4 * j + g) ^ SwizzleLat(i16)) << 4;
+#pragma unroll
+          for (int j = 0; j < 2; ++j) kr_e[j] = ((4 * j + g) ^ SwizzleRope(i16)) << 4;
+          // K fragment of pipeline step `step` (k-step step/2, token subtile step&1) of the tile at `buf`.
+          const auto k_frag = [&](const unsigned char* buf, int step) __attribute__((always_inline)) {
+            const int ks = step >> 1, t = step & 1;
+            const int offset = ks < 16 ? k_lat + (ks >> 2) * 256 + k_e[ks & 3] + t * 16 * Geom<false>::kLatRow
+                                       : k_rope + kr_e[ks & 1] + t * 16 * Geom<false>::kRopeRow;
+            return *reinterpret_cast<const bf16x8*>(buf + offset);
+          };
+          // FP8 K reads: read u = 2 kp + t fetches the 16 codes k = 64 kp + 16 g .. +15 of token 16t + i16
+          // (k-steps 2kp and 2kp+1): chunk (4 kp + g) ^ swizzle(token) of the 512-byte row; kp = 8 is the
+          // rope row (chunk g ^ swizzle). The tile base is a multiple of 512, so the XOR with kp << 6 is
+          // applied to the lane-constant part.
+          int k8_lat[2];
+#pragma unroll
+          for (int t = 0; t < 2; ++t) k8_lat[t] = (16 * t + i16) * Geom<true>::kLatRow + ((g ^ SwizzleLat8(16 * t + i16)) << 4);
+          const int k8_rope = Geom<true>::kLatRegion + i16 * Geom<true>::kRopeRow + ((g ^ SwizzleRope8(i16)) << 4);
+          const auto k8_read = [&](const unsigned char* buf, int u) __attribute__((always_inline)) {
+            const int kp = u >> 1, t = u & 1;
+            const int offset = kp < 8 ? (k8_lat[t] ^ (kp << 6)) : k8_rope + t * 16 * Geom<true>::kRopeRow;
+            return *reinterpret_cast<const u32x4*>(buf + offset);
+          };
+
+          float m_ref = -__builtin_inff();  // reference maximum of the exponentials, log2 domain
+          float l_run = 0.0f;               // this lane's share of the running denominator
+
+          // S^T of tile `tile_rel`, its softmax against the running reference, P and the rescale
+          // request into the LDS slots of the tile's parity.
+          const auto score_tile = [&](int tile_rel, int issue_iteration) __attribute__((always_inline)) {
+            const unsigned char* buf = lds + ring(tile_rel);
+            f32x4 acc[4];
+#pragma unroll
+            for (int j = 0; j < 4; ++j) acc[j] = f32x4{0.f, 0.f, 0.f, 0.f};
+            f32x4 row_scale[2];  // FP8: scales of tokens 4g+j and 16+4g+j
+            if constexpr (FP8) {
+              const float* scales = reinterpret_cast<const float*>(buf + G::kScaleOff);
+              row_scale[0] = *reinterpret_cast<const f32x4*>(scales + 4 * g);
+              row_scale[1] = *reinterpret_cast<const f32x4*>(scales + 16 + 4 * g);
+              u32x4 kr[kKAhead8];
+#pragma unroll
+              for (int d = 0; d < kKAhead8; ++d) kr[d] = k8_read(buf, d);
+              __builtin_amdgcn_sched_barrier(0);
+              StaticFor<kKSteps>([&](auto u_c) __attribute__((always_inline)) {
+                constexpr int u = decltype(u_c)::value;  // kp = u / 2, token subtile t = u & 1
+                const u32x4 codes = kr[u % kKAhead8];
+                if constexpr (u + kKAhead8 < kKSteps) kr[u % kKAhead8] = k8_read(buf, u + kKAhead8);
+                constexpr int t = u & 1, kp = u >> 1;
+                acc[2 * t] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(CodesToBf16(codes.x, codes.y), q[2 * kp], acc[2 * t], 0, 0, 0);
+                acc[2 * t + 1] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(CodesToBf16(codes.z, codes.w), q[2 * kp + 1], acc[2 * t + 1], 0, 0, 0);
+                __builtin_amdgcn_sched_barrier(0);
+              });
+            } else {
+              bf16x8 kf[kKAhead];
+#pragma unroll
+              for (int d = 0; d < kKAhead; ++d) kf[d] = k_frag(buf, d);
+              __builtin_amdgcn_sched_barrier(0);
+              StaticFor<kQkSteps>([&](auto step_c) __attribute__((always_inline)) {
+                constexpr int step = decltype(step_c)::value;
+                constexpr int slot_acc = (step & 1) * 2 + ((step >> 1) & 1);  // two accumulators per token subtile
+                acc[slot_acc] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(kf[step % kKAhead], q[step >> 1], acc[slot_acc], 0, 0, 0);
+                if constexpr (step + kKAhead < kQkSteps) kf[step % kKAhead] = k_frag(buf, step + kKAhead);
+                __builtin_amdgcn_sched_barrier(0);
+              });
+            }
+            // the score waves ask for their rows of the next ring tile behind the QK phase
+            if (kLateIssue && issue_iteration >= 0) issue_next(issue_iteration);
+            // lane holds tokens 4g+j (x[0..3]) and 16+4g+j (x[4..7]) of head i16
+            float x[8];
+#pragma unroll
+            for (int j = 0; j < 4; ++j) {
+              x[j] = (acc[0][j] + acc[1][j]) * a.scale_log2;
+              x[4 + j] = (acc[2][j] + acc[3][j]) * a.scale_log2;
+              if constexpr (FP8) {  // the codes were multiplied unscaled
+                x[j] *= row_scale[0][j];
+                x[4 + j] *= row_scale[1][j];
+              }
+            }
+            const int valid = seq_len - (tile_begin + tile_rel) * kTileTokens;  // >= 1
+            if (valid < kTileTokens) {  // wave-uniform: only the last tile of a sequence
+#pragma unroll
+              for (int j = 0; j < 8; ++j) {
+                if (16 * (j >> 2) + 4 * g + (j & 3) >= valid) x[j] = -__builtin_inff();
+              }
+            }
+            float tile_max = fmaxf(fmaxf(fmaxf(x[0], x[1]), fmaxf(x[2], x[3])), fmaxf(fmaxf(x[4], x[5]), fmaxf(x[6], x[7])));
+            tile_max = MaxAcrossHalves(MaxAcrossRows16(tile_max));
+            const int parity = tile_rel & 1;
+            // Move the reference only when some head's maximum outgrew it by more than the threshold.
+            const bool moved = __builtin_amdgcn_ballot_w64(tile_max > m_ref + kRescaleThreshold) != 0;
+            if (moved) {
+              const float m_new = fmaxf(m_ref, tile_max);  // finite: token 0 of the tile is valid
+              const float alpha = __builtin_amdgcn_exp2f(m_ref - m_new);
+              l_run *= alpha;
+              m_ref = m_new;
+              alpha_lds[parity * kScoreWaves * 64] = alpha;
+            }
+            if (lane == 0) flag_lds[parity * kScoreWaves] = moved && tile_rel != 0 ? 1 : 0;  // O is still zero on the first tile
+            bf16x8 p;
+            float sum = 0.0f;
+#pragma unroll
+            for (int j = 0; j < 8; ++j) {
+              const float e = __builtin_amdgcn_exp2f(x[j] - m_ref);
+              sum += e;
+              p[j] = static_cast<__bf16>(FP8 ? e * row_scale[j >> 2][j & 3] : e);  // FP8: V is multiplied unscaled as well
+            }
+            l_run += sum;
+            *reinterpret_cast<bf16x8*>(p_lds + parity * kScoreWaves * 64 * 16) = p;
+          };
+
+          if (active) score_tile(0, -1);
+          for (int i = 0; i < ntiles; ++i) {
+            publish(i);
+            const bool scores = active && i + 1 < ntiles;
+            if (!kLateIssue || !scores) issue_next(i);
+            if (scores) score_tile(i + 1, i);
+          }
+          if (active) {
+            const float l_total = SumAcrossHeadLanes(l_run);
+            *inv_lds = 1.0f / l_total;
+            const float lse2 = m_ref + __builtin_amdgcn_logf(l_total);  // v_log_f32 is log2
+            if (g == 0) {
+              if (direct) {
+                if (a.lse != nullptr) a.lse[seq * a.heads + head] = lse2 * 0.6931471805599453f;
+              } else {
+                StoreAgentF32(a.partial_lse + PartialRow(a, z, slot, hw * 16 + i16), lse2);
+              }
+            }
+          }
+          __syncthreads();  // 1/denominator visible to the output waves
+        } else {
+          // ---------------------------------------------------------------- output waves
+          write_table();
+          if constexpr (!kSoloPrologue) __syncthreads();  // table entries visible
+          for (; issued < G::kRing - 1 && issued < ntiles; ++issued) {
+            if constexpr (kSoloPrologue) {
+              // bf16 tiles: these waves have no query to wait for and issue the first tiles of the ring
+              // alone, their own rows and those of their partner score waves
+              if (!IssueTileBf16<ALIGNED, true>(a, map, il, tile_begin + issued, lds_base + ring(issued), lds + ring(issued), tid)) {
+                last_unknown = issued;
+              }
+            } else {
+              if (!issue(issued)) last_unknown = issued;
+            }
+          }
+          WaitLoads(last_unknown >= 0 ? 0 : newer_than(0));
+          __syncthreads();
+
+          // bf16 V reads: token = (16 +) 4g + i16/4, chunk = 2n + (i16 & 3) / 2, 8-byte half i16 & 1.
+          const int v_row = 4 * g + (i16 >> 2);
+          const int v_lane = v_row * Geom<false>::kLatRow + (i16 & 1) * 8;
+          int v_e[8];
+#pragma unroll
+          for (int j = 0; j < 8; ++j) v_e[j] = ((2 * j + ((i16 & 3) >> 1)) ^ SwizzleLat(v_row)) << 4;
+          // FP8 V reads (ds_read_b64_tr_b8: output lane i of a 16-lane group, element e <- byte i & 7 of
+          // the 8 bytes addressed by lane 2e + (i >> 3)): as a source, lane j addresses bytes
+          // 16n + 8 (j & 1) .. +7 of the row of token kappa = j >> 1 (tokens 4g + kappa, 16 + 4g + kappa - 4).
+          const int v8_token = 4 * g + ((i16 >> 1) & 3) + 16 * (i16 >> 3);
+          const int v8_base = v8_token * Geom<true>::kLatRow + (SwizzleLat8(v8_token) << 4) + 8 * (i16 & 1);
+          // Raw V^T fragment of output tile n (dv 16n..16n+15) over the 32 tokens of the tile at `buf`:
+          // eight bf16 for bf16 tiles, eight codes in the low two dwords for FP8 tiles.
+          const auto v_fetch = [&](const unsigned char* buf, int n) __attribute__((always_inline)) {
+            if constexpr (FP8) {
+              const i32x2 codes = __builtin_amdgcn_ds_read_tr8_b64_v2i32((__attribute__((address_space(3))) i32x2*)(buf + (v8_base ^ (n << 4))));
+              return u32x4{static_cast<unsigned>(codes.x), static_cast<unsigned>(codes.y), 0u, 0u};
+            } else {
+              const unsigned char* addr = buf + v_lane + (n >> 3) * 256 + v_e[n & 7];
+              const s16x4 lo = __builtin_amdgcn_ds_read_tr16_b64_v4i16((__attribute__((address_space(3))) s16x4*)(addr));
+              const s16x4 hi = __builtin_amdgcn_ds_read_tr16_b64_v4i16((__attribute__((address_space(3))) s16x4*)(addr + 16 * Geom<false>::kLatRow));
+              return __builtin_bit_cast(u32x4, __builtin_shufflevector(lo, hi, 0, 1, 2, 3, 4, 5, 6, 7));
+            }
+          };
+          const auto v_operand = [&](const u32x4& raw) __attribute__((always_inline)) {
+            if constexpr (FP8) {
+              return CodesToBf16(raw.x, raw.y);
+            } else {
+              return __builtin_bit_cast(bf16x8, raw);
+            }
+          };
+
+          // Output wave w owns the 128 output columns [128 w, 128 w + 128) of all 64 heads of the group:
+          // every V^T fragment is then fetched (and, for FP8, converted) by one wave only, and meets the
+          // P fragments of the four score waves. Head blocks past the group's heads are computed on
+          // whatever their LDS slots hold and never written.
+          constexpr int kDvPerWave = kDvTiles / (kWaves - kScoreWaves);
+          const unsigned char* p_all = lds + G::kPOff + lane * 16;                                   // + (parity * 4 + hb) * 64 * 16
+          const float* alpha_all = reinterpret_cast<const float*>(lds + G::kAlphaOff) + lane;      // + (parity * 4 + hb) * 64
+          const float* inv_all = reinterpret_cast<const float*>(lds + G::kInvOff) + lane;          // + hb * 64
+          const int* flag_all = reinterpret_cast<const int*>(lds + G::kFlagOff);                   // [parity * 4 + hb]
+          f32x4 o[kScoreWaves][kDvPerWave];
+#pragma unroll
+          for (int hb = 0; hb < kScoreWaves; ++hb) {
+#pragma unroll
+            for (int n = 0; n < kDvPerWave; ++n) o[hb][n] = f32x4{0.f, 0.f, 0.f, 0.f};
+          }
+
+          for (int i = 0; i < ntiles; ++i) {
+            publish(i);
+            issue_next(i);
+            {
+              const unsigned char* buf = lds + ring(i);
+              const int parity = i & 1;
+              // the four rescale flags of the tile in one read; a moved reference maximum is the exception
+              const i32x4 flags = *reinterpret_cast<const i32x4*>(flag_all + parity * kScoreWaves);
+              if (Uniform(flags.x | flags.y | flags.z | flags.w) != 0) {
+                const int moved[kScoreWaves] = {flags.x, flags.y, flags.z, flags.w};
+#pragma unroll
+                for (int hb = 0; hb < kScoreWaves; ++hb) {
+                  if (Uniform(moved[hb]) != 0) {  // that block's reference maximum moved: rescale its O first
+                    const float alpha = alpha_all[(parity * kScoreWaves + hb) * 64];
+#pragma unroll
+                    for (int n = 0; n < kDvPerWave; ++n) o[hb][n] *= alpha;
+                  }
+                }
+              }
+              u32x4 vf[kVAhead];
+#pragma unroll
+              for (int d = 0; d < kVAhead; ++d) vf[d] = v_fetch(buf, kDvPerWave * hw + d);
+              bf16x8 p[kScoreWaves];
+#pragma unroll
+              for (int hb = 0; hb < kScoreWaves; ++hb) p[hb] = *reinterpret_cast<const bf16x8*>(p_all + (parity * kScoreWaves + hb) * 64 * 16);
+              __builtin_amdgcn_sched_barrier(0);
+              if constexpr (FP8) {
+                // the next fragment is converted while this one's four MFMAs run
+                bf16x8 v = v_operand(vf[0]);
+                if constexpr (kVAhead < kDvPerWave) vf[0] = v_fetch(buf, kDvPerWave * hw + kVAhead);
+                StaticFor<kDvPerWave>([&](auto n_c) __attribute__((always_inline)) {
+                  constexpr int n = decltype(n_c)::value;
+                  bf16x8 v_next = v;
+                  if constexpr (n + 1 < kDvPerWave) v_next = v_operand(vf[(n + 1) % kVAhead]);
+#pragma unroll
+                  for (int hb = 0; hb < kScoreWaves; ++hb) o[hb][n] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(v, p[hb], o[hb][n], 0, 0, 0);
+                  if constexpr (n + 1 + kVAhead < kDvPerWave) vf[(n + 1) % kVAhead] = v_fetch(buf, kDvPerWave * hw + n + 1 + kVAhead);
+                  v = v_next;
+                  __builtin_amdgcn_sched_barrier(0);
+                });
+              } else {
+                StaticFor<kDvPerWave>([&](auto n_c) __attribute__((always_inline)) {
+                  constexpr int n = decltype(n_c)::value;
+                  const bf16x8 v = v_operand(vf[n % kVAhead]);
+#pragma unroll
+                  for (int hb = 0; hb < kScoreWaves; ++hb) o[hb][n] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(v, p[hb], o[hb][n], 0, 0, 0);
+                  if constexpr (n + kVAhead < kDvPerWave) vf[n % kVAhead] = v_fetch(buf, kDvPerWave * hw + n + kVAhead);
+                  __builtin_amdgcn_sched_barrier(0);
+                });
+              }
+            }
+          }
+          __syncthreads();  // 1/denominator from the score waves
+          if (MXQ && direct) {
+            // Quantising epilogue of a whole sequence: a block of 32 columns is a pair of this
+            // wave's column tiles over the four lanes that share a head; the wave covers blocks
+            // 4 w .. 4 w + 3 of every head.
+#pragma unroll
+            for (int hb = 0; hb < kScoreWaves; ++hb) {
+              if (hb >= hba) continue;
+              const int h = 16 * hb + i16;
+              const float inv = inv_all[hb * 64];
+              char* codes_row = a.out_codes + seq * a.out_codes_seq_stride + (group_head0 + h) * a.out_codes_head_stride;
+              char* out_row = a.out == nullptr ? nullptr : a.out + seq * a.out_seq_stride + (group_head0 + h) * a.out_head_stride;
+              unsigned scale_codes = 0u;
+#pragma unroll
+              for (int k = 0; k < kDvPerWave / 2; ++k) {
+                u32x2 packed[2];
+                unsigned magnitude = 0u;
+#pragma unroll
+                for (int half = 0; half < 2; ++half) {
+                  const int n = 2 * k + half;
+                  packed[half].x = PackBf16(o[hb][n][0] * inv, o[hb][n][1] * inv);
+                  packed[half].y = PackBf16(o[hb][n][2] * inv, o[hb][n][3] * inv);
+                  magnitude = MxMagnitudeMax(packed[half].y, MxMagnitudeMax(packed[half].x, magnitude));
+                  if (out_row != nullptr) {
+                    __builtin_nontemporal_store(packed[half], reinterpret_cast<u32x2*>(out_row + (16 * (kDvPerWave * hw + n) + 4 * g) * 2));
+                  }
+                }
+                magnitude = UMaxAcrossHeadLanes(magnitude);
+                const MxScale s = MxScaleFromMaxBits(magnitude);
+#pragma unroll
+                for (int half = 0; half < 2; ++half) {
+                  const unsigned four = MxEncodeWord(packed[half].x, s) | (MxEncodeWord(packed[half].y, s) << 16);
+                  __builtin_nontemporal_store(four, reinterpret_cast<unsigned*>(codes_row + 16 * (kDvPerWave * hw + 2 * k + half) + 4 * g));
+                }
+                scale_codes |= s.code << (8 * k);
+              }
+              if (g == 0) {
+                *reinterpret_cast<unsigned*>(a.out_scales + seq * a.out_scales_seq_stride + (group_head0 + h) * a.out_scales_head_stride +
+                                             (kDvPerWave / 2) * hw) = scale_codes;
+              }
+            }
+          } else {
+            // The accumulators hold O^T (lane = head i16 of a block, four columns per 16-column tile),
+            // which stored as it is would write 8-byte pieces of sixteen different rows per
+            // instruction. The tile ring is dead after the last barrier: each output wave transposes
+            // its 256-byte slices of the 64 rows through its own part of it and writes them 16 bytes per
+            // lane, four whole slices per instruction. A row stride of 272 bytes (= 4 banks mod 64)
+            // spreads the 8-byte writes of a half-wave over all banks.
+            constexpr int kSliceBytes = kDvPerWave * 16 * 2;  // 256
+            constexpr int kStageRow = kSliceBytes + 16;
+            static_assert((kWaves - kScoreWaves) * 64 * kStageRow <= G::kRing * G::kTileBytes, "the staging rows fit in the ring");
+            unsigned char* stage = lds + G::Slot(0) + hw * (64 * kStageRow);
+#pragma unroll
+            for (int hb = 0; hb < kScoreWaves; ++hb) {
+              const float inv = inv_all[hb * 64];
+#pragma unroll
+              for (int n = 0; n < kDvPerWave; ++n) {
+                u32x2 packed;
+                packed.x = PackBf16(o[hb][n][0] * inv, o[hb][n][1] * inv);
+                packed.y = PackBf16(o[hb][n][2] * inv, o[hb][n][3] * inv);
+                *reinterpret_cast<u32x2*>(stage + (16 * hb + i16) * kStageRow + (16 * n + 4 * g) * 2) = packed;
+              }
+            }
+            // Same wave wrote and reads: the LDS queue is in order, no barrier needed.
+            const int piece = lane & 15, sub = lane >> 4;
+            if (direct) {
+              char* out0 = a.out + seq * a.out_seq_stride + group_head0 * a.out_head_stride + kSliceBytes * hw + piece * 16;
+#pragma unroll
+              for (int it = 0; it < 16; ++it) {
+                const int h = 4 * it + sub;
+                if (h < 16 * hba) {
+                  const u32x4 v = *reinterpret_cast<const u32x4*>(stage + h * kStageRow + piece * 16);
+                  __builtin_nontemporal_store(v, reinterpret_cast<u32x4*>(out0 + h * a.out_head_stride));
+                }
+              }
+            } else {
+              char* out0 = a.partial_out + PartialRow(a, z, slot, 0) * (kLatentDim * 2) + kSliceBytes * hw + piece * 16;
+#pragma unroll
+              for (int it = 0; it < 16; ++it) {
+                const int h = 4 * it + sub;
+                if (h < 16 * hba) {
+                  const u32x4 v = *reinterpret_cast<const u32x4*>(stage + h * kStageRow + piece * 16);
+                  if (sync_group != nullptr) {
+                    StoreAgent16(out0 + h * (kLatentDim * 2), v);
+                  } else {
+                    __builtin_nontemporal_store(v, reinterpret_cast<u32x4*>(out0 + h * (kLatentDim * 2)));
+                  }
+                }
+              }
+            }
+          }
+        }
+      }
+
+      if (!direct && sync_group != nullptr) {
+        // A merge to take part in once this workgroup's units are done (all its partials are
+        // announced together then: nothing waits in between).
+        if (tid == 0) {
+          const int first_unit = seq_begin / tiles_per_unit;
+          const int partials = (seq_end - 1) / tiles_per_unit - first_unit + 1;
+          duty_lds[duties] = i32x4{seq, first_unit, partials, unit - first_unit};
+        }
+        ++duties;
+        if (duties == kMaxDuties) flush_duties();
+      }
+
+      flat = segment_end;
+      if (flat < flat_end) {  // the next sequence that has tiles
+        do {
+          ++seq;
+          if (seq >= win.base + 64) win.Load(a, lane0, win.base + 64, win.End());
+        } while (win.Tiles(seq) == 0);
+      }
+    }
+  }
+  if (duties != 0) flush_duties();
+}
+
+// The merge as a launch of its own, for launches that have no counters to meet on: block =
+// (eight heads, sequence, head group); every wave repeats the cut of the flat tile axis and merges
+// one head.
+template <bool MXQ, bool SPARSE>
+__global__ __launch_bounds__(kMergeHeads * 64) void MlaMergeKernel(AttnArgs a) {
+  const int lane = threadIdx.x & 63, wave = Uniform(threadIdx.x >> 6);
+  const int seq = blockIdx.y, z = blockIdx.z;
+  const int h = blockIdx.x * kMergeHeads + wave;
+  if (h >= min(64, a.heads - 64 * z)) return;
+  SeqWindow<SPARSE> win;
+  win.Load(a, lane, 0, 0);
+  int seq_end = 0, seq_tiles = 0;
+  for (;;) {
+    if (seq >= win.base && seq < win.base + 64) {
+      seq_end = win.Incl(seq);
+      seq_tiles = win.Tiles(seq);
+    }
+    if (win.base + 64 >= a.batch) break;
+    win.Load(a, lane, win.base + 64, win.End());
+  }
+  const int total_tiles = win.End();
+  if (seq_tiles == 0) return;
+  int tiles_per_unit = a.forced_unit_tiles > 0 ? a.forced_unit_tiles : max(a.min_unit_tiles, (total_tiles + a.work_groups - 1) / a.work_groups);
+  tiles_per_unit = min(tiles_per_unit, a.cap_unit_tiles);
+  const int first_unit = (seq_end - seq_tiles) / tiles_per_unit;
+  const int partials = (seq_end - 1) / tiles_per_unit - first_unit + 1;
+  if (partials == 1) return;  // written by the workgroup that held the whole sequence
+  MergeHead<MXQ, false>(a, z, seq, h, a.max_units + seq, first_unit, partials, lane);
+}
+
 template <bool FP8, bool ALIGNED, bool MXQ, bool SPARSE>
 hipError_t Launch(const AttnArgs& args, const dim3& grid, hipStream_t stream) {
   // Dynamic LDS above 64 KB needs the attribute once per kernel and process.
@@ -1128,9 +1394,65 @@ hipError_t LaunchByCache(const AttnArgs& args, const dim3& grid, hipStream_t str
   return aligned ? Launch<false, true, MXQ, false>(args, grid, stream) : Launch<false, false, MXQ, false>(args, grid, stream);
 }
 
+// Meeting points of the in-launch merge: two words per (head group, sequence), all zero between
+// launches (the last contributor to leave a sequence clears its words). A launch takes the next of kSyncRegions
+// regions, so that launches running side by side on different streams do not share counters.
+constexpr int kSyncRegions = 16;
+static __device__ __align__(256) unsigned int sync_words[kSyncRegions][kAttnSyncSequences * 2];
+
+hipError_t SyncRegion(unsigned** region) {
+  constexpr int kMaxDevices = 64;
+  static std::mutex guard;
+  static unsigned* per_device[kMaxDevices] = {};
+  static unsigned next[kMaxDevices] = {};
+  int device = 0;
+  if (hipError_t e = hipGetDevice(&device); e != hipSuccess) return e;
+  if (device < 0 || device >= kMaxDevices) return hipErrorInvalidDevice;
+  std::lock_guard<std::mutex> lock(guard);
+  if (per_device[device] == nullptr) {
+    void* resolved = nullptr;
+    if (hipError_t e = hipGetSymbolAddress(&resolved, HIP_SYMBOL(sync_words)); e != hipSuccess) return e;
+    if (resolved == nullptr) return hipErrorInvalidSymbol;
+    per_device[device] = static_cast<unsigned*>(resolved);
+  }
+  *region = per_device[device] + static_cast<size_t>(next[device]++ % kSyncRegions) * (kAttnSyncSequences * 2);
+  return hipSuccess;
+}
+
 }  // namespace
 
 hipError_t PrepareAttnKernels() { return hipSuccess; }
+
+hipError_t LaunchAttnDecode(const AttnArgs& args_in, hipStream_t stream) {
+  AttnArgs args = args_in;
+  if (args.batch <= 0) return hipSuccess;
+  const int head_groups = (args.heads + 63) / 64;
+  const bool merge_in_launch = args.merge_in_launch && static_cast<int64_t>(args.batch) * head_groups <= kAttnSyncSequences;
+  args.sync = nullptr;
+  if (merge_in_launch) {
+    if (hipError_t e = SyncRegion(&args.sync); e != hipSuccess) return e;
+  }
+  const dim3 grid(args.work_groups, head_groups);
+  const bool quantise = args.out_codes != nullptr;
+  const bool sparse = args.sparse_indices != nullptr;
+  hipError_t e;
+  if (sparse) {
+    if (quantise) return hipErrorInvalidValue;
+    e = args.fp8 ? Launch<true, false, false, true>(args, grid, stream) : Launch<false, false, false, true>(args, grid, stream);
+  } else {
+    e = quantise ? LaunchByCache<true>(args, grid, stream) : LaunchByCache<false>(args, grid, stream);
+  }
+  if (e != hipSuccess || merge_in_launch) return e;
+  const dim3 merge_grid((std::min(64, args.heads) + kMergeHeads - 1) / kMergeHeads, args.batch, head_groups);
+  if (sparse) {
+    hipLaunchKernelGGL((MlaMergeKernel<false, true>), merge_grid, dim3(kMergeHeads * 64), 0, stream, args);
+  } else if (quantise) {
+    hipLaunchKernelGGL((MlaMergeKernel<true, false>), merge_grid, dim3(kMergeHeads * 64), 0, stream, args);
+  } else {
+    hipLaunchKernelGGL((MlaMergeKernel<false, false>), merge_grid, dim3(kMergeHeads * 64), 0, stream, args);
+  }
+  return hipGetLastError();
+}
 
 // Split-KV partials for callers that cannot allocate: one array per GPU, held from module load to
 // process exit. In host code the array's name only stands for the symbol; its address on the
@@ -1154,30 +1476,6 @@ hipError_t AttnStaticScratch(char** address) {
   }
   *address = per_device[device];
   return hipSuccess;
-}
-
-hipError_t LaunchAttnDecode(const AttnArgs& args_in, hipStream_t stream) {
-  AttnArgs args = args_in;
-#ifdef MLAKV_ATTN_TRACE
-  args.trace = std::getenv("MLAKV_ATTN_TRACE_PTR") ? reinterpret_cast<unsigned long long*>(std::strtoull(std::getenv("MLAKV_ATTN_TRACE_PTR"), nullptr, 0)) : nullptr;
-#endif
-  if (args.batch <= 0) return hipSuccess;
-  const dim3 grid(args.max_chunks, args.batch, (args.heads + 63) / 64);
-  // With several chunks the merge kernel owns the final output and the optional quantisation.
-  const bool quantise_here = args.max_chunks == 1 && args.out_codes != nullptr;
-  hipError_t e;
-  if (args.sparse_indices != nullptr) {
-    e = args.fp8 ? Launch<true, false, false, true>(args, grid, stream) : Launch<false, false, false, true>(args, grid, stream);
-  } else {
-    e = quantise_here ? LaunchByCache<true>(args, grid, stream) : LaunchByCache<false>(args, grid, stream);
-  }
-  if (e != hipSuccess) return e;
-  if (args.max_chunks > 1) {
-    hipLaunchKernelGGL(MlaCombineKernel, dim3((args.heads + kCombineHeads - 1) / kCombineHeads, args.batch), dim3(kCombineHeads * 64), 0,
-                       stream, args);
-    e = hipGetLastError();
-  }
-  return e;
 }
 
 }  // namespace mlakv

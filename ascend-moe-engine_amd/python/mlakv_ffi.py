@@ -54,9 +54,18 @@ class IndexKeyView(C.Structure):
 class AttnPlan(C.Structure):
     _fields_ = [
         ("batch", C.c_int32), ("heads", C.c_int32), ("max_seq_len", C.c_int32), ("block_size", C.c_int32),
-        ("dtype", C.c_int32), ("chunk_tiles", C.c_int32), ("max_chunks", C.c_int32), ("reserved", C.c_int32),
+        ("dtype", C.c_int32), ("chunk_tiles", C.c_int32), ("work_groups", C.c_int32), ("max_units", C.c_int32),
+        ("merge_mode", C.c_int32), ("merge_spin_us", C.c_int32), ("reserved", C.c_int32), ("reserved2", C.c_int32),
         ("workspace_bytes", C.c_uint64),
     ]
+
+
+class AttnPlanOptions(C.Structure):
+    _fields_ = [("chunk_tiles", C.c_int32), ("work_groups", C.c_int32), ("merge_mode", C.c_int32), ("merge_spin_us", C.c_int32),
+                ("selection", C.c_int32), ("reserved", C.c_int32 * 3)]
+
+
+ATTN_MERGE_AUTO, ATTN_MERGE_IN_LAUNCH, ATTN_MERGE_SECOND_LAUNCH = 0, 1, 2
 
 
 class KvConfig(C.Structure):
@@ -88,6 +97,7 @@ PROTOTYPES = {
     "mlakvGather": (_i32, [_P(CacheView), _i32, _i32, _vp, _i32, _vp, _vp, _i32, _i32, _vp, _i64, _i64, _vp, _i64, _i64, _vp]),
     "mlakvCopyBlocks": (_i32, [_P(CacheView), _i32, _i32, _vp, _i32, _vp]),
     "mlakvAttnPlanInit": (_i32, [_i32, _i32, _i32, _i32, _i32, _P(AttnPlan)]),
+    "mlakvAttnPlanInitEx": (_i32, [_i32, _i32, _i32, _i32, _i32, _P(AttnPlanOptions), _P(AttnPlan)]),
     "mlakvAttnDecode": (_i32, [_P(AttnPlan), _P(CacheView), _i32, _vp, _i64, _i64, _vp, _i64, _i64, _vp, _i32, _vp,
                                C.c_double, _vp, _i64, _i64, _vp, _vp, _u64, _vp]),
     "mlakvAttnDecodeNoAlloc": (_i32, [_P(AttnPlan), _P(CacheView), _i32, _vp, _i64, _i64, _vp, _i64, _i64, _vp, _i32, _vp,

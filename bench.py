@@ -302,7 +302,8 @@ def bench_attention(args, torch, np, ffi, fp8=False, batch=32, ctx=2048, heads=6
         "algorithmic_bytes": algorithmic,
         "mfma_tflops": flops / (us * 1e-6) / 1e12,
         "mfma_frac_of_bf16_peak": flops / (us * 1e-6) / 1e12 / MFMA_BF16_PEAK_TFLOPS,
-        "chunk_tiles": int(plan.chunk_tiles), "max_chunks": int(plan.max_chunks),
+        "work_groups": int(plan.work_groups), "max_units": int(plan.max_units),
+        "merge": "in launch" if plan.merge_mode == ffi.ATTN_MERGE_IN_LAUNCH else "second launch",
         "workspace_bytes": int(plan.workspace_bytes), "timing": "250 ms of back-to-back launches untimed, then at least 100 ms of them timed",
     }
     if mx is not None:

@@ -134,21 +134,52 @@ mlakvStatus mlakvCopyBlocks(const mlakvCacheView* cache, int32_t layer_begin, in
  *   s_i = scale * (q_latent[b,h] . c_i + q_rope[b,h] . r_i), p = softmax_i(s),
  *   out[b,h] = sum_i p_i c_i     over the seq_lens[b] cached rows of sequence b,
  * one query token per sequence, `heads` query heads sharing one latent KV head.
- * The plan fixes shapes and the workspace; the launch only enqueues. */
+ * The plan fixes shapes and the workspace; the launch only enqueues.
+ *
+ * How the work is cut: the contexts of the batch, counted in 32-token tiles and laid end to end,
+ * are divided into equal work units, one per workgroup (one workgroup per CU and group of 64
+ * heads), at every launch from the live seq_lens on the device; a sequence shorter than
+ * its neighbours costs its own tiles and no more. A unit that holds a whole sequence writes that
+ * sequence's output; the others leave partial results in the workspace, which a second small
+ * launch merges (MLAKV_ATTN_MERGE_SECOND_LAUNCH, the default) or the same launch does
+ * (MLAKV_ATTN_MERGE_IN_LAUNCH: contributors meet on counters the library keeps in a static device
+ * array, with a bounded wait; measured no faster on MI355X, kept for callers that want one
+ * launch). seq_lens[b] is read as min(max(seq_lens[b], 0), max_seq_len). */
+#define MLAKV_ATTN_MERGE_AUTO 0
+#define MLAKV_ATTN_MERGE_IN_LAUNCH 1
+#define MLAKV_ATTN_MERGE_SECOND_LAUNCH 2
 typedef struct mlakvAttnPlan {
   int32_t batch;
   int32_t heads;           /* multiple of 16, at most 128 */
   int32_t max_seq_len;
   int32_t block_size;
   int32_t dtype;           /* cache dtype */
-  int32_t chunk_tiles;     /* 32-token tiles per workgroup; chosen by the plan */
-  int32_t max_chunks;      /* ceil(ceil(max_seq_len / 32) / chunk_tiles) */
+  int32_t chunk_tiles;     /* tiles per work unit when fixed by mlakvAttnPlanInitEx; 0: from the live lengths */
+  int32_t work_groups;     /* workgroups per group of 64 heads */
+  int32_t max_units;       /* bound on the work units of one launch (sizes the workspace) */
+  int32_t merge_mode;      /* MLAKV_ATTN_MERGE_IN_LAUNCH or _SECOND_LAUNCH */
+  int32_t merge_spin_us;   /* bound of the in-launch merge's wait for a sequence's other partials */
   int32_t reserved;        /* 1: made by mlakvAttnSparsePlanInit (max_seq_len holds sparse_count) */
+  int32_t reserved2;
   uint64_t workspace_bytes;
 } mlakvAttnPlan;
 
 mlakvStatus mlakvAttnPlanInit(int32_t batch, int32_t heads, int32_t max_seq_len, int32_t block_size, int32_t dtype,
                               mlakvAttnPlan* plan);
+
+/* The same with the planner's choices spelled out (tests and measurements use it to force many
+ * small units, a single unit per sequence, the second-launch merge or a wait that gives up at
+ * once); a zero field keeps the default. No reference counterpart. */
+typedef struct mlakvAttnPlanOptions {
+  int32_t chunk_tiles;    /* tiles per work unit, fixed instead of derived from the live lengths */
+  int32_t work_groups;    /* workgroups per group of 64 heads (default: CUs / head groups) */
+  int32_t merge_mode;     /* MLAKV_ATTN_MERGE_* */
+  int32_t merge_spin_us;  /* > 0: microseconds; < 0: do not wait at all (the last contributor merges) */
+  int32_t selection;      /* 1: a plan for mlakvAttnDecodeSparse; max_seq_len then holds sparse_count */
+  int32_t reserved[3];    /* zero */
+} mlakvAttnPlanOptions;
+mlakvStatus mlakvAttnPlanInitEx(int32_t batch, int32_t heads, int32_t max_seq_len, int32_t block_size, int32_t dtype,
+                                const mlakvAttnPlanOptions* options, mlakvAttnPlan* plan);
 
 /* q strides: bytes between sequences / between heads. out is bf16 [batch, heads, latent_dim]
  * with its own strides; lse (optional) is fp32 [batch, heads], natural log of the softmax

@@ -120,7 +120,24 @@ def gather(cache, table, seq_lens, fused_out=False, layer_begin=0, layer_count=N
     return latent_out[:, :total], rope_out[:, :total]
 
 
-def attention(cache, layer, q, table, seq_lens, scale, max_seq_len=None, want_lse=True, quant=False, want_out=True):
+def make_plan(batch, heads, max_seq_len, block_size, fp8, chunk_tiles=0, work_groups=0, merge_mode=0, merge_spin_us=0,
+              selection=False):
+    """The default plan, or one with the planner's choices forced (mlakvAttnPlanInitEx). With
+    selection=True, max_seq_len is the length of the selection (mlakvAttnSparsePlanInit)."""
+    lib = ffi.load()
+    plan = ffi.AttnPlan()
+    dtype = ffi.DTYPE_FP8_E4M3 if fp8 else ffi.DTYPE_BF16
+    if chunk_tiles or work_groups or merge_mode or merge_spin_us:
+        options = ffi.AttnPlanOptions(chunk_tiles, work_groups, merge_mode, merge_spin_us, 1 if selection else 0)
+        ffi.check(lib.mlakvAttnPlanInitEx(batch, heads, max_seq_len, block_size, dtype, C.byref(options), C.byref(plan)))
+    elif selection:
+        ffi.check(lib.mlakvAttnSparsePlanInit(batch, heads, max_seq_len, block_size, dtype, C.byref(plan)))
+    else:
+        ffi.check(lib.mlakvAttnPlanInit(batch, heads, max_seq_len, block_size, dtype, C.byref(plan)))
+    return plan
+
+
+def attention(cache, layer, q, table, seq_lens, scale, max_seq_len=None, want_lse=True, quant=False, want_out=True, **plan_options):
     """q [B, H, 576] bf16 cuda (latent | rope per head). Returns (out [B,H,512] bf16, lse [B,H] f32, plan);
     with quant=True through the fused entry point, returning (out or None, lse, plan, codes [B,H,512] u8,
     scales [B,H,16] u8)."""
@@ -128,9 +145,7 @@ def attention(cache, layer, q, table, seq_lens, scale, max_seq_len=None, want_ls
     batch, heads = q.shape[0], q.shape[1]
     lens = seq_lens.cpu().numpy()
     max_seq_len = max(int(lens.max()), 1) if max_seq_len is None else max_seq_len
-    plan = ffi.AttnPlan()
-    ffi.check(lib.mlakvAttnPlanInit(batch, heads, max_seq_len, cache.block_size,
-                                    ffi.DTYPE_FP8_E4M3 if cache.fp8 else ffi.DTYPE_BF16, C.byref(plan)))
+    plan = make_plan(batch, heads, max_seq_len, cache.block_size, cache.fp8, **plan_options)
     workspace = torch.empty(max(int(plan.workspace_bytes), 16), dtype=torch.uint8, device="cuda")
     out = torch.full((batch, heads, LATENT), float("nan"), dtype=torch.bfloat16, device="cuda") if want_out else None
     lse = torch.full((batch, heads), float("nan"), dtype=torch.float32, device="cuda") if want_lse else None
@@ -151,13 +166,11 @@ def attention(cache, layer, q, table, seq_lens, scale, max_seq_len=None, want_ls
     return out, lse, plan, codes, scales
 
 
-def sparse_attention(cache, layer, q, table, seq_lens, selection, scale, want_lse=True):
+def sparse_attention(cache, layer, q, table, seq_lens, selection, scale, want_lse=True, **plan_options):
     """Selected-token attention: `selection` int32 cuda [B, k]. Returns (out, lse, plan)."""
     lib = ffi.load()
     batch, heads = q.shape[0], q.shape[1]
-    plan = ffi.AttnPlan()
-    ffi.check(lib.mlakvAttnSparsePlanInit(batch, heads, selection.shape[1], cache.block_size,
-                                          ffi.DTYPE_FP8_E4M3 if cache.fp8 else ffi.DTYPE_BF16, C.byref(plan)))
+    plan = make_plan(batch, heads, selection.shape[1], cache.block_size, cache.fp8, selection=True, **plan_options)
     workspace = torch.empty(max(int(plan.workspace_bytes), 16), dtype=torch.uint8, device="cuda")
     out = torch.full((batch, heads, LATENT), float("nan"), dtype=torch.bfloat16, device="cuda")
     lse = torch.full((batch, heads), float("nan"), dtype=torch.float32, device="cuda") if want_lse else None

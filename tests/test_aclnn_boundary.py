@@ -170,7 +170,7 @@ def test_attention_plan_contract_workspace_and_ir_indices():
     assert status == 0 and executor, acl.last_error()
     plan = ffi.AttnPlan()
     ffi.check(ffi.load().mlakvAttnPlanInit(1, 64, 8192, 64, ffi.DTYPE_BF16, C.byref(plan)))
-    assert plan.max_chunks > 1 and workspace >= plan.workspace_bytes + 4  # split-KV partials + the lengths
+    assert plan.max_units >= 1 and workspace >= plan.workspace_bytes + 4  # partials of split sequences + the lengths
     assert lib.aclSetAclOpExecutorRepeatable(executor) == 0
     layer_latent, layer_rope = FAKE + 0x3000000, FAKE + 0xB000000
     assert lib.aclSetDynamicTensorAddr(executor, 1, 0, e.key_list, layer_latent) == 0    # kFiaKeyList
@@ -209,8 +209,26 @@ def test_thin_abi_argument_validation_without_a_device():
     lib = ffi.load()
     plan = ffi.AttnPlan()
     assert lib.mlakvAttnPlanInit(32, 64, 2048, 64, ffi.DTYPE_BF16, C.byref(plan)) == 0
-    assert (plan.chunk_tiles, plan.max_chunks) == (8, 8)  # 32-token tiles; 256 CUs / 32 sequences
-    assert plan.workspace_bytes == 32 * 8 * 64 * 512 * 2 + 32 * 8 * 64 * 4  # bf16 partial outputs + fp32 partial LSEs
+    # without a device the plan assumes 256 CUs: one workgroup each, units cut from the live lengths at launch
+    assert (plan.chunk_tiles, plan.work_groups, plan.max_units) == (0, 256, 256)
+    assert (plan.merge_mode, plan.merge_spin_us) == (ffi.ATTN_MERGE_SECOND_LAUNCH, 50)
+    # one partial slot per unit and one per sequence: bf16 partial outputs + fp32 partial LSEs
+    assert plan.workspace_bytes == (256 + 32) * 64 * 512 * 2 + (256 + 32) * 64 * 4
+    options = ffi.AttnPlanOptions(chunk_tiles=2, work_groups=0, merge_mode=ffi.ATTN_MERGE_IN_LAUNCH, merge_spin_us=-5)
+    forced = ffi.AttnPlan()
+    assert lib.mlakvAttnPlanInitEx(32, 128, 2048, 64, ffi.DTYPE_BF16, C.byref(options), C.byref(forced)) == 0
+    assert (forced.chunk_tiles, forced.work_groups, forced.max_units) == (2, 128, 32 * 64 // 2)
+    assert (forced.merge_mode, forced.merge_spin_us) == (ffi.ATTN_MERGE_IN_LAUNCH, -1)
+    assert forced.workspace_bytes == 2 * (1024 + 32) * 64 * (1024 + 4)
+    options.chunk_tiles = 1 << 20  # clamped to what a segment's staged table entries can address
+    assert lib.mlakvAttnPlanInitEx(1, 64, 1 << 20, 16, ffi.DTYPE_BF16, C.byref(options), C.byref(forced)) == 0
+    assert forced.chunk_tiles == (510 * 16 + 2) // 32
+    options.merge_mode = 3
+    assert lib.mlakvAttnPlanInitEx(32, 64, 2048, 64, ffi.DTYPE_BF16, C.byref(options), C.byref(forced)) == ffi.ERR_PARAM_INVALID
+    # more (head group, sequence) pairs than the library keeps counters for: the merge stays a second launch
+    options.merge_mode = ffi.ATTN_MERGE_IN_LAUNCH
+    assert lib.mlakvAttnPlanInitEx(4097, 64, 64, 64, ffi.DTYPE_BF16, C.byref(options), C.byref(forced)) == 0
+    assert forced.merge_mode == ffi.ATTN_MERGE_SECOND_LAUNCH
     assert lib.mlakvAttnPlanInit(32, 60, 2048, 64, ffi.DTYPE_BF16, C.byref(plan)) == ffi.ERR_PARAM_INVALID
     assert lib.mlakvAttnPlanInit(32, 64, 2048, 64, 7, C.byref(plan)) == ffi.ERR_PARAM_INVALID
     assert lib.mlakvAttnPlanInit(32, 64, 2048, 64, ffi.DTYPE_BF16, None) == ffi.ERR_PARAM_NULLPTR
@@ -239,15 +257,15 @@ def test_thin_abi_argument_validation_without_a_device():
                                    0.07, FAKE, 64 * 1024, 1024, None, None, 0, None)
 
     assert decode(plan) == ffi.ERR_PARAM_NULLPTR          # everything fine up to the missing workspace
-    for field, value in (("chunk_tiles", 4096), ("chunk_tiles", 0), ("max_chunks", 9), ("heads", 60), ("workspace_bytes", 16),
-                         ("reserved", 2), ("batch", 0)):
+    for field, value in (("chunk_tiles", 4096), ("chunk_tiles", -1), ("max_units", 9), ("heads", 60), ("workspace_bytes", 16),
+                         ("reserved", 2), ("batch", 0), ("work_groups", 0), ("merge_mode", 0), ("merge_spin_us", 0)):
         altered = ffi.AttnPlan.from_buffer_copy(plan)
         setattr(altered, field, value)
         assert decode(altered) == ffi.ERR_PARAM_INVALID, field
         assert "not one made by" in ffi.last_error()
     sparse = ffi.AttnPlan()
     assert lib.mlakvAttnSparsePlanInit(32, 64, 512, 64, ffi.DTYPE_BF16, C.byref(sparse)) == 0
-    assert sparse.reserved == 1 and sparse.max_seq_len == 512 and sparse.chunk_tiles * 32 <= 1024
+    assert sparse.reserved == 1 and sparse.max_seq_len == 512 and sparse.chunk_tiles == 0
     assert decode(sparse) == ffi.ERR_PARAM_INVALID        # a selection plan handed to the whole-context entry
 
 

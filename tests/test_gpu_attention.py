@@ -9,6 +9,7 @@ import pytest
 import torch
 
 import kv_testing as kt
+import mlakv_ffi as ffi
 import oracle_ffi as orc
 
 pytestmark = pytest.mark.gpu
@@ -39,7 +40,7 @@ def _assert_close(got_bf16, expected_f32, tol):
 
 @pytest.mark.parametrize("bs", [16, 64, 128])
 @pytest.mark.parametrize("heads", [16, 64, 128])
-def test_attention_matches_oracle_ragged(bs, heads, monkeypatch):
+def test_attention_matches_oracle_ragged(bs, heads):
     ctxs = [1, 63, 64, 65, 200, 333]
     blocks = sum(-(-c // bs) for c in ctxs) + 4
     pool = kt.build_tables(ctxs, bs, blocks, seed=31)
@@ -48,14 +49,20 @@ def test_attention_matches_oracle_ragged(bs, heads, monkeypatch):
     _fill_cache(cache, ctxs, table, seed=40)
     q = kt.randn_bf16((len(ctxs), heads, LATENT + ROPE), seed=50).cuda()
     expected, expected_lse = kt.oracle_attention(cache, 1, q, table, ctxs, SCALE)
-    for chunk_tiles in (None, 1, 2, 100):  # planner's choice, many chunks, single chunk (direct path)
-        if chunk_tiles is None:
-            monkeypatch.delenv("MLAKV_ATTN_CHUNK_TILES", raising=False)
-        else:
-            monkeypatch.setenv("MLAKV_ATTN_CHUNK_TILES", str(chunk_tiles))
-        out, lse, plan = kt.attention(cache, 1, q, kt.dev_i32(table), kt.dev_i32(ctxs), SCALE)
+    # the planner's choice; units of one tile (every sequence split, several units per workgroup
+    # when there are fewer workgroups than units); two tiles; units that each hold whole sequences
+    # (written without partials); then the merge inside the launch: contributors that wait for each
+    # other, a merge that never waits (the contributor that arrives last does all of it), a wait
+    # that mostly gives up (two workgroups take turns over many units)
+    in_launch = ffi.ATTN_MERGE_IN_LAUNCH
+    for options in ({}, {"chunk_tiles": 1}, {"chunk_tiles": 1, "work_groups": 3}, {"chunk_tiles": 2}, {"chunk_tiles": 100},
+                    {"chunk_tiles": 1, "merge_mode": in_launch}, {"merge_mode": in_launch},
+                    {"chunk_tiles": 2, "merge_mode": in_launch, "merge_spin_us": -1},
+                    {"chunk_tiles": 1, "work_groups": 3, "merge_mode": in_launch},
+                    {"chunk_tiles": 3, "work_groups": 2, "merge_mode": in_launch, "merge_spin_us": 1}):
+        out, lse, plan = kt.attention(cache, 1, q, kt.dev_i32(table), kt.dev_i32(ctxs), SCALE, **options)
         _assert_close(out, expected, TOL_BF16)
-        assert np.abs(lse.cpu().numpy() - expected_lse).max() <= 2e-2
+        assert np.abs(lse.cpu().numpy() - expected_lse).max() <= 2e-2, options
 
 
 def test_attention_special_cases():
@@ -109,7 +116,7 @@ def test_attention_invariant_under_physical_block_permutation():
     assert torch.equal(outs[0][1], outs[1][1])
 
 
-def test_attention_empty_sequence_gives_zeros(monkeypatch):
+def test_attention_empty_sequence_gives_zeros():
     bs, heads = 64, 64
     ctxs = [0, 70, 0]
     blocks = 4
@@ -118,9 +125,8 @@ def test_attention_empty_sequence_gives_zeros(monkeypatch):
     cache = kt.PagedCache(1, blocks, bs)
     _fill_cache(cache, ctxs, table, seed=80)
     q = kt.randn_bf16((3, heads, LATENT + ROPE), seed=81).cuda()
-    for chunk_tiles in ("1", "100"):
-        monkeypatch.setenv("MLAKV_ATTN_CHUNK_TILES", chunk_tiles)
-        out, lse, _ = kt.attention(cache, 0, q, kt.dev_i32(table), kt.dev_i32(ctxs), SCALE, max_seq_len=128)
+    for chunk_tiles in (1, 100):
+        out, lse, _ = kt.attention(cache, 0, q, kt.dev_i32(table), kt.dev_i32(ctxs), SCALE, max_seq_len=128, chunk_tiles=chunk_tiles)
         assert (out[0] == 0).all() and (out[2] == 0).all()
         assert torch.isinf(lse[0]).all() and (lse[0] < 0).all()
         expected, _ = kt.oracle_attention(cache, 0, q, table, ctxs, SCALE)
@@ -173,10 +179,10 @@ def test_config3_full_size_against_oracle_sample_and_torch():
 
 @pytest.mark.parametrize("fp8", [False, True])
 def test_maximum_context_single_sequence_many_chunks(fp8):
-    """BASELINE's largest context (32768 tokens) for one sequence: the plan splits it into hundreds
-    of chunks, so the merge runs over many groups of partials. The whole sequence is checked
+    """BASELINE's largest context (32768 tokens) for one sequence: the launch cuts it into one unit per
+    CU, so the merge runs over many groups of partials. The whole sequence is checked
     against a float32 torch evaluation on the GPU (library routine), 16 heads of it against the
-    float64 oracle; a second, short sequence in the same batch leaves most chunks empty."""
+    float64 oracle; a second, short sequence in the same batch shares the last unit."""
     heads, bs = 64, 128
     ctxs = [32768, 200]
     blocks = sum(-(-c // bs) for c in ctxs) + 8
@@ -190,7 +196,7 @@ def test_maximum_context_single_sequence_many_chunks(fp8):
     kt.append(cache, latent_src, rope_src, kt.dev_i32(kt.slots_for(table, ctxs, bs)))
     q = torch.randn(len(ctxs), heads, LATENT + ROPE, generator=gen, device="cuda").to(torch.bfloat16)
     out, lse, plan = kt.attention(cache, 0, q, kt.dev_i32(table), kt.dev_i32(ctxs), SCALE)
-    assert plan.max_chunks >= 64
+    assert plan.work_groups >= 64  # the long sequence is cut over (nearly) all of them
     tol = TOL_FP8 if fp8 else TOL_BF16
     if fp8:  # compare against the values the cache really holds
         lat_rows, rope_rows = kt.gather(cache, kt.dev_i32(table), kt.dev_i32(ctxs))

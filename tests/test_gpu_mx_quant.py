@@ -80,8 +80,8 @@ def test_standalone_strided_rows_ragged_row_count_and_argument_checks():
 
 
 @pytest.mark.parametrize("fp8", [False, True])
-@pytest.mark.parametrize("chunk_tiles", [None, 2, 100])
-def test_attention_epilogue_equals_quantising_the_bf16_output(fp8, chunk_tiles, monkeypatch):
+@pytest.mark.parametrize("options", [{}, {"chunk_tiles": 2}, {"chunk_tiles": 100}, {"chunk_tiles": 1, "merge_mode": 1}])
+def test_attention_epilogue_equals_quantising_the_bf16_output(fp8, options):
     bs, heads = 64, 64
     ctxs = [1, 0, 65, 200, 333, 32]   # one empty sequence: zero codes under scale byte 0
     blocks = sum(-(-c // bs) for c in ctxs) + 3
@@ -93,14 +93,11 @@ def test_attention_epilogue_equals_quantising_the_bf16_output(fp8, chunk_tiles, 
     rope = kt.randn_bf16((1, total, ROPE), seed=75).cuda()
     kt.append(cache, latent, rope, kt.dev_i32(kt.slots_for(table, ctxs, bs)))
     q = kt.randn_bf16((len(ctxs), heads, LATENT + ROPE), seed=76).cuda()
-    if chunk_tiles is None:
-        monkeypatch.delenv("MLAKV_ATTN_CHUNK_TILES", raising=False)
-    else:
-        monkeypatch.setenv("MLAKV_ATTN_CHUNK_TILES", str(chunk_tiles))
+    # planner's choice; sequences split over units (the merge quantises); whole sequences per unit
+    # (the kernel's own epilogue quantises); the merge inside the launch
     table_d, lens_d = kt.dev_i32(table), kt.dev_i32(ctxs)
-    out, lse, plan = kt.attention(cache, 0, q, table_d, lens_d, SCALE)
-    assert (plan.max_chunks == 1) == (chunk_tiles == 100)
-    out_q, lse_q, _, codes, scales = kt.attention(cache, 0, q, table_d, lens_d, SCALE, quant=True)
+    out, lse, plan = kt.attention(cache, 0, q, table_d, lens_d, SCALE, **options)
+    out_q, lse_q, _, codes, scales = kt.attention(cache, 0, q, table_d, lens_d, SCALE, quant=True, **options)
     assert torch.equal(out_q, out) and torch.equal(lse_q, lse)       # the bf16 output is unchanged by the epilogue
     want_codes, want_scales = orc.mx_quant_rows(kt.bits16(out).reshape(-1, LATENT))
     assert np.array_equal(scales.cpu().numpy().reshape(-1, LATENT // 32), want_scales)
@@ -110,7 +107,8 @@ def test_attention_epilogue_equals_quantising_the_bf16_output(fp8, chunk_tiles, 
     alone_codes, alone_scales = _quant(out.reshape(-1, LATENT))
     assert np.array_equal(alone_codes, want_codes) and np.array_equal(alone_scales, want_scales)
     # without the bf16 output
-    none_out, _, _, codes2, scales2 = kt.attention(cache, 0, q, table_d, lens_d, SCALE, quant=True, want_out=False, want_lse=False)
+    none_out, _, _, codes2, scales2 = kt.attention(cache, 0, q, table_d, lens_d, SCALE, quant=True, want_out=False, want_lse=False,
+                                                   **options)
     assert none_out is None and torch.equal(codes2, codes) and torch.equal(scales2, scales)
 
 

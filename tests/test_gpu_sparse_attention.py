@@ -41,7 +41,7 @@ def _close(got_bf16, expected, tol):
 
 @pytest.mark.parametrize("fp8", [False, True])
 @pytest.mark.parametrize("bs,k", [(64, 512), (16, 100), (128, 2048)])
-def test_selected_tokens_match_oracle(fp8, bs, k, monkeypatch):
+def test_selected_tokens_match_oracle(fp8, bs, k):
     heads = 64
     ctxs = [3000, 700, 1, 0, 2049, 130]
     cache, table = _setup(ctxs, bs, fp8, seed=80)
@@ -55,13 +55,9 @@ def test_selected_tokens_match_oracle(fp8, bs, k, monkeypatch):
     q = kt.randn_bf16((len(ctxs), heads, LATENT + ROPE), seed=82).cuda()
     expected, expected_lse = kt.oracle_attention(cache, 0, q, table, ctxs, SCALE, sparse_indices=selection)
     table_d, lens_d, sel_d = kt.dev_i32(table), kt.dev_i32(ctxs), kt.dev_i32(selection)
-    for chunk_tiles in (None, 1, 100):
-        if chunk_tiles is None:
-            monkeypatch.delenv("MLAKV_ATTN_CHUNK_TILES", raising=False)
-        else:
-            monkeypatch.setenv("MLAKV_ATTN_CHUNK_TILES", str(chunk_tiles))
-        out, lse, plan = kt.sparse_attention(cache, 0, q, table_d, lens_d, sel_d, SCALE)
-        assert plan.chunk_tiles * 32 <= 1024
+    for options in ({}, {"chunk_tiles": 1}, {"chunk_tiles": 100}, {"chunk_tiles": 3, "merge_mode": 1}):
+        out, lse, plan = kt.sparse_attention(cache, 0, q, table_d, lens_d, sel_d, SCALE, **options)
+        assert plan.chunk_tiles * 32 <= 512  # a unit's selected tokens are staged in LDS, one entry each
         _close(out, expected, 6e-2 if fp8 else 2e-2)
         live = np.array([min(n, k) > 0 for n in ctxs])
         assert np.abs(lse.cpu().numpy()[live] - expected_lse[live]).max() <= (6e-2 if fp8 else 2e-2)
