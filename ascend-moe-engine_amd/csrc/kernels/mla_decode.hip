@@ -501,6 +501,21 @@ struct SeqWindow {
   __device__ __forceinline__ int Incl(int seq) const { return __builtin_amdgcn_readlane(incl, seq - base); }
 };
 
+// Tiles per work unit for a launch whose sequences add up to `total_tiles`: an equal share per
+// workgroup, not below what amortises a query load and not above what a segment's staged
+// block-table entries can address (or the plan's fixed value).
+__device__ __forceinline__ int TilesPerUnit(const AttnArgs& a, int total_tiles, int work_groups) {
+  int share;
+  if (a.forced_unit_tiles > 0) {
+    share = a.forced_unit_tiles;
+  } else if ((work_groups & (work_groups - 1)) == 0) {  // the usual case, without a division
+    share = (total_tiles + work_groups - 1) >> __builtin_ctz(work_groups);
+  } else {
+    share = (total_tiles + work_groups - 1) / work_groups;
+  }
+  return min(max(share, a.forced_unit_tiles > 0 ? 1 : a.min_unit_tiles), a.cap_unit_tiles);
+}
+
 // Stores and loads that other CUs' accesses of the same kind see without a cache write-back or
 // invalidate in between (agent scope: the sc1 bit): the partials and the counters travel through
 // these. The 16-byte forms have no builtin; a load's result is ready after WaitAgentLoads on it.
@@ -676,10 +691,10 @@ __global__ __launch_bounds__(kThreads) void MlaDecodeKernel(AttnArgs a) {
     win.Load(a, lane0, win.base + 64, win.End());
   }
   const int total_tiles = win.End();
-  int tiles_per_unit = a.forced_unit_tiles > 0 ? a.forced_unit_tiles : max(a.min_unit_tiles, (total_tiles + work_groups - 1) / work_groups);
-  tiles_per_unit = min(tiles_per_unit, a.cap_unit_tiles);
-  const int units = (total_tiles + tiles_per_unit - 1) / tiles_per_unit;  // <= a.max_units, ensured by the plan
-  if (wg >= units) return;
+  const int tiles_per_unit = TilesPerUnit(a, total_tiles, work_groups);
+  // unit u covers flat tiles [u, u + 1) * tiles_per_unit; there are ceil(total / tiles_per_unit)
+  // units, at most a.max_units (ensured by the plan)
+  if (static_cast<int64_t>(wg) * tiles_per_unit >= total_tiles) return;
   if (win.base != 0) win.Load(a, lane0, 0, 0);
 
   // Q fragments (score waves): lane (head i16, k-group g) holds, for k-step ks, the eight query
@@ -763,7 +778,8 @@ __global__ __launch_bounds__(kThreads) void MlaDecodeKernel(AttnArgs a) {
     duties = 0;
   };
 
-  for (int unit = wg; unit < units; unit += work_groups) {
+  bool first_segment = true;
+  for (int unit = wg; static_cast<int64_t>(unit) * tiles_per_unit < total_tiles; unit += work_groups) {
     const int flat_end = min(total_tiles, (unit + 1) * tiles_per_unit);
     int flat = unit * tiles_per_unit;
     while (win.End() <= flat) win.Load(a, lane0, win.base + 64, win.End());
@@ -779,7 +795,8 @@ __global__ __launch_bounds__(kThreads) void MlaDecodeKernel(AttnArgs a) {
       const int slot = holds_first ? a.max_units + seq : unit;
       int seq_len = win.Tok(seq);
 
-      __syncthreads();  // the previous segment's staging rows, table entries and P slots are free
+      if (!first_segment) __syncthreads();  // the previous segment's staging rows, table entries and P slots are free
+      first_segment = false;
 
       // Everything that depends on the thread id alone is formed here, per segment, from a copy
       // of the id that the compiler cannot see through: hoisted out of the segment loop, these
@@ -1353,8 +1370,18 @@ __global__ __launch_bounds__(kThreads) void MlaDecodeKernel(AttnArgs a) {
 template <bool MXQ, bool SPARSE>
 __global__ __launch_bounds__(kMergeHeads * 64) void MlaMergeKernel(AttnArgs a) {
   const int lane = threadIdx.x & 63, wave = Uniform(threadIdx.x >> 6);
-  const int seq = blockIdx.y, z = blockIdx.z;
-  const int h = blockIdx.x * kMergeHeads + wave;
+  // Workgroups go to the XCDs round-robin by linear id. The main launch put the units of XCD x's
+  // share of the flat tile axis on XCD x; with equal lengths that is the x-th eighth of the
+  // sequences, whose partials are most likely still in that L2.
+  int seq = blockIdx.y, group = blockIdx.x;
+  const int z = blockIdx.z;
+  if ((gridDim.y & (kXcds - 1)) == 0) {
+    const int linear = blockIdx.y * gridDim.x + blockIdx.x;
+    const int within = linear / kXcds;
+    seq = (linear & (kXcds - 1)) * (gridDim.y / kXcds) + within / static_cast<int>(gridDim.x);
+    group = within % static_cast<int>(gridDim.x);
+  }
+  const int h = group * kMergeHeads + wave;
   if (h >= min(64, a.heads - 64 * z)) return;
   SeqWindow<SPARSE> win;
   win.Load(a, lane, 0, 0);
@@ -1369,8 +1396,7 @@ __global__ __launch_bounds__(kMergeHeads * 64) void MlaMergeKernel(AttnArgs a) {
   }
   const int total_tiles = win.End();
   if (seq_tiles == 0) return;
-  int tiles_per_unit = a.forced_unit_tiles > 0 ? a.forced_unit_tiles : max(a.min_unit_tiles, (total_tiles + a.work_groups - 1) / a.work_groups);
-  tiles_per_unit = min(tiles_per_unit, a.cap_unit_tiles);
+  const int tiles_per_unit = TilesPerUnit(a, total_tiles, a.work_groups);
   const int first_unit = (seq_end - seq_tiles) / tiles_per_unit;
   const int partials = (seq_end - 1) / tiles_per_unit - first_unit + 1;
   if (partials == 1) return;  // written by the workgroup that held the whole sequence
