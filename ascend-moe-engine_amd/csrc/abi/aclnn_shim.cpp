@@ -6,6 +6,7 @@
 
 #include <hip/hip_runtime.h>
 
+#include <algorithm>
 #include <chrono>
 #include <cstring>
 #include <mutex>
@@ -14,6 +15,7 @@
 #include <unordered_set>
 #include <vector>
 
+#include "../kernels/kernels.h"
 #include "abi_common.h"
 #include "mlakv.h"
 
@@ -75,7 +77,9 @@ struct aclTensor {
   }
 };
 struct aclTensorList { std::vector<aclTensor*> items; };
-struct aclIntArray { const int64_t* values = nullptr; uint64_t size = 0; };
+// The values are copied at creation, as the reference's own implementation of the call does
+// (mock/mock_descriptor.cpp:249-256): callers build arrays from temporaries.
+struct aclIntArray { std::vector<int64_t> storage; const int64_t* values = nullptr; uint64_t size = 0; };
 struct aclScalar { void* value = nullptr; aclDataType dtype = ACL_DT_UNDEFINED; };
 
 namespace {
@@ -138,9 +142,8 @@ struct aclOpExecutor {
   int32_t sparse_count = 0;
   uint64_t workspace_bytes = 0;
   uint64_t lens_offset = 0;  // attention: where the int32 lengths live inside the workspace
-  const aclIntArray* host_lens = nullptr;
   const int32_t* bound_lens = nullptr;
-  std::vector<int32_t> lens_staging;  // pageable on purpose: hipMemcpyAsync snapshots it before returning
+  std::vector<int32_t> host_lens;  // plan-time kv lengths, or those of the latest aclnnMlaKvSetSeqLens
 };
 
 namespace {
@@ -489,7 +492,8 @@ aclIntArray* aclCreateIntArray(const int64_t* value, uint64_t size) {
     return nullptr;
   }
   auto* array = new aclIntArray();
-  array->values = value;
+  array->storage.assign(value, value + size);
+  array->values = array->storage.data();
   array->size = size;
   Register(array);
   return array;
@@ -864,6 +868,11 @@ aclnnStatus aclnnFusedInferAttentionScoreV5GetWorkspaceSize(
   }
   const int64_t width = block_table->dims[1];
   SHIM_REQUIRE(tokens <= 65535 && width * bs <= INT32_MAX && blocks <= INT32_MAX / bs, ACLNN_ERR_PARAM_INVALID, "%s: sizes exceed the launch limits", who);
+  for (int64_t b = 0; b < tokens; ++b) {
+    const int64_t len = actual_seq_lengths_kv->values[b];
+    SHIM_REQUIRE(len >= 0 && len <= width * bs, ACLNN_ERR_PARAM_INVALID, "%s: kv length %lld of sequence %lld outside [0, %lld]", who,
+                 static_cast<long long>(len), static_cast<long long>(b), static_cast<long long>(width * bs));
+  }
   mlakvAttnPlan plan;
   if (mlakvStatus s = mlakvAttnPlanInit(static_cast<int32_t>(tokens), static_cast<int32_t>(heads), static_cast<int32_t>(width * bs),
                                         static_cast<int32_t>(bs), MLAKV_DTYPE_BF16, &plan)) {
@@ -900,8 +909,8 @@ aclnnStatus aclnnFusedInferAttentionScoreV5GetWorkspaceSize(
   e->plan = plan;
   e->lens_offset = (plan.workspace_bytes + 255) & ~255ull;
   e->workspace_bytes = e->lens_offset + ((static_cast<uint64_t>(tokens) * sizeof(int32_t) + 255) & ~255ull);
-  e->host_lens = actual_seq_lengths_kv;
-  e->lens_staging.resize(static_cast<size_t>(tokens));
+  e->host_lens.resize(static_cast<size_t>(tokens));
+  for (int64_t b = 0; b < tokens; ++b) e->host_lens[static_cast<size_t>(b)] = static_cast<int32_t>(actual_seq_lengths_kv->values[b]);
   *workspace_size = e->workspace_bytes;
   *executor = e;
   return ACLNN_SUCCESS;
@@ -946,17 +955,14 @@ aclnnStatus aclnnFusedInferAttentionScoreV5(void* workspace, uint64_t workspace_
                "%s: the value tensor must alias the key tensor (absorbed MLA reads the latent cache as K and V)", who);
   const int32_t* device_lens = e->bound_lens;
   if (device_lens == nullptr) {
-    SHIM_REQUIRE(IsLive(e->host_lens), ACLNN_ERR_PARAM_INVALID, "%s: the kv-length array was destroyed before the launch", who);
-    for (int32_t b = 0; b < e->batch; ++b) {
-      const int64_t len = e->host_lens->values[b];
-      SHIM_REQUIRE(len >= 0 && len <= e->max_seq_len, ACLNN_ERR_PARAM_INVALID, "%s: kv length %lld of sequence %d outside [0, %d]", who,
-                   static_cast<long long>(len), b, e->max_seq_len);
-      e->lens_staging[static_cast<size_t>(b)] = static_cast<int32_t>(len);
-    }
+    // The lengths travel in the argument block of a one-workgroup kernel: the host vector is free
+    // again when the call returns, and nothing is staged or waited for.
     int32_t* staged = reinterpret_cast<int32_t*>(static_cast<char*>(workspace) + e->lens_offset);
-    const hipError_t status = hipMemcpyAsync(staged, e->lens_staging.data(), sizeof(int32_t) * static_cast<size_t>(e->batch),
-                                             hipMemcpyHostToDevice, static_cast<hipStream_t>(stream));
-    SHIM_REQUIRE(status == hipSuccess, ACLNN_ERR_RUNTIME_ERROR, "%s: length upload failed: %s", who, hipGetErrorString(status));
+    for (int32_t first = 0; first < e->batch; first += mlakv::kMaxStoreWords) {
+      const int count = std::min<int32_t>(mlakv::kMaxStoreWords, e->batch - first);
+      const hipError_t status = mlakv::LaunchStoreWords(e->host_lens.data() + first, count, staged + first, static_cast<hipStream_t>(stream));
+      SHIM_REQUIRE(status == hipSuccess, ACLNN_ERR_RUNTIME_ERROR, "%s: length upload failed: %s", who, hipGetErrorString(status));
+    }
     device_lens = staged;
   }
   mlakvCacheView view;
@@ -968,6 +974,21 @@ aclnnStatus aclnnFusedInferAttentionScoreV5(void* workspace, uint64_t workspace_
       e->slots[31].addresses[0], e->out_token_stride, e->out_head_stride, lse, workspace, e->plan.workspace_bytes, stream);
   if (status == MLAKV_SUCCESS) e->launched = true;
   return status;
+}
+
+aclnnStatus aclnnMlaKvSetSeqLens(aclOpExecutor* executor, const int64_t* seq_lens, uint64_t count) {
+  const char* who = "aclnnMlaKvSetSeqLens";
+  SHIM_REQUIRE(executor && seq_lens, ACLNN_ERR_PARAM_NULLPTR, "%s: null executor or lengths", who);
+  SHIM_REQUIRE(AsExecutor(executor) && executor->kind == OpKind::kAttention, ACLNN_ERR_PARAM_INVALID, "%s: not an attention executor", who);
+  SHIM_REQUIRE(count == static_cast<uint64_t>(executor->batch), ACLNN_ERR_PARAM_INVALID, "%s: %llu lengths for %d sequences", who,
+               static_cast<unsigned long long>(count), executor->batch);
+  for (uint64_t b = 0; b < count; ++b) {
+    SHIM_REQUIRE(seq_lens[b] >= 0 && seq_lens[b] <= executor->max_seq_len, ACLNN_ERR_PARAM_INVALID,
+                 "%s: kv length %lld of sequence %llu outside [0, %d]", who, static_cast<long long>(seq_lens[b]),
+                 static_cast<unsigned long long>(b), executor->max_seq_len);
+  }
+  for (uint64_t b = 0; b < count; ++b) executor->host_lens[b] = static_cast<int32_t>(seq_lens[b]);
+  return ACLNN_SUCCESS;
 }
 
 aclnnStatus aclnnMlaKvBindSeqLens(aclOpExecutor* executor, const int32_t* device_seq_lens) {

@@ -764,6 +764,10 @@ mlakvStatus mlakvDynamicMxQuant(const void* x, int64_t x_row_stride, int64_t row
 struct mlakvArena {
   std::unique_ptr<moe_hip::IDeviceBackend> backend;
   std::unique_ptr<moe_hip::StaticMemoryArena> arena;
+  // Caches hold a reference to the arena: destroying the arena while some are alive only marks
+  // it, and the last cache to go takes the arena with it.
+  int live_caches = 0;
+  bool destroy_requested = false;
 };
 
 struct mlakvKvCache {
@@ -807,6 +811,10 @@ mlakvStatus mlakvArenaCreate(int32_t backend, mlakvArena** arena) {
 
 void mlakvArenaDestroy(mlakvArena* arena) {
   if (arena == nullptr) return;
+  if (arena->live_caches > 0) {
+    arena->destroy_requested = true;
+    return;
+  }
   arena->arena.reset();
   arena->backend.reset();
   delete arena;
@@ -922,11 +930,17 @@ mlakvStatus mlakvKvCacheCreate(mlakvArena* arena, const mlakvKvConfig* config, m
     handle->manager = std::make_unique<moe_hip::KvCacheManager>(*arena->arena, c);
   });
   if (status != MLAKV_SUCCESS) return status;
+  ++arena->live_caches;
   *cache = handle.release();
   return MLAKV_SUCCESS;
 }
 
-void mlakvKvCacheDestroy(mlakvKvCache* cache) { delete cache; }
+void mlakvKvCacheDestroy(mlakvKvCache* cache) {
+  if (cache == nullptr) return;
+  mlakvArena* owner = cache->owner;
+  delete cache;
+  if (owner != nullptr && --owner->live_caches == 0 && owner->destroy_requested) mlakvArenaDestroy(owner);
+}
 
 mlakvStatus mlakvKvCacheBind(mlakvKvCache* cache) {
   MLAKV_NEED(cache, "mlakvKvCacheBind");
@@ -971,6 +985,14 @@ mlakvStatus mlakvKvCacheAppendToken(mlakvKvCache* cache, int64_t seq, int32_t* s
   return Guard("mlakvKvCacheAppendToken", [&] {
     const int32_t s = cache->manager->AppendToken(seq);
     if (slot != nullptr) *slot = s;
+  });
+}
+
+mlakvStatus mlakvKvCacheAppendTokenAll(mlakvKvCache* cache, int32_t* slots, int64_t* appended) {
+  MLAKV_NEED(cache, "mlakvKvCacheAppendTokenAll");
+  return Guard("mlakvKvCacheAppendTokenAll", [&] {
+    const int64_t n = cache->manager->AppendTokenAll(slots);
+    if (appended != nullptr) *appended = n;
   });
 }
 

@@ -229,14 +229,22 @@ KvCacheManager::KvCacheManager(StaticMemoryArena& arena, const KvCacheConfig& co
 
 KvCacheManager::~KvCacheManager() {
   IDeviceBackend& backend = arena_.backend();
+  // A destructor reports nothing: after a device error the waits below may fail, and the
+  // staging memory is then released without them.
+  const auto quietly = [](auto&& body) {
+    try {
+      body();
+    } catch (...) {
+    }
+  };
   for (int k = 0; k < 2; ++k) {
-    if (staging_busy_[k]) backend.SynchronizeEvent(staging_event_[k]);
-    backend.DestroyEvent(staging_event_[k]);
-    backend.HostPinnedFree(staging_[k]);
+    if (staging_busy_[k]) quietly([&] { backend.SynchronizeEvent(staging_event_[k]); });
+    quietly([&] { backend.DestroyEvent(staging_event_[k]); });
+    quietly([&] { backend.HostPinnedFree(staging_[k]); });
   }
-  if (moves_busy_) backend.SynchronizeEvent(moves_event_);
-  backend.DestroyEvent(moves_event_);
-  backend.HostPinnedFree(moves_staging_);
+  if (moves_busy_) quietly([&] { backend.SynchronizeEvent(moves_event_); });
+  quietly([&] { backend.DestroyEvent(moves_event_); });
+  quietly([&] { backend.HostPinnedFree(moves_staging_); });
 }
 
 void KvCacheManager::Bind() {
@@ -299,6 +307,20 @@ int32_t KvCacheManager::AppendToken(int64_t seq) {
   return slot;
 }
 
+int64_t KvCacheManager::AppendTokenAll(int32_t* slots) {
+  int64_t appended = 0;
+  for (int64_t seq = 0; seq < config_.max_batch; ++seq) {
+    if (pool_->seq_len(seq) < 0) {
+      if (slots != nullptr) slots[seq] = -1;
+      continue;
+    }
+    const int32_t slot = AppendToken(seq);
+    if (slots != nullptr) slots[seq] = slot;
+    ++appended;
+  }
+  return appended;
+}
+
 void KvCacheManager::FreeSequence(int64_t seq) {
   pool_->FreeSequence(seq);
   host_small_[static_cast<size_t>(seq)] = -1;
@@ -355,6 +377,23 @@ void KvCacheManager::UploadStep(void* stream) {
 std::vector<std::pair<int32_t, int32_t>> KvCacheManager::Compact(void* stream) {
   std::vector<std::pair<int32_t, int32_t>> moves = pool_->Compact();
   table_dirty_ = true;
+  // Tokens appended since the last UploadStep have their slots waiting in the mirror: a slot
+  // inside a block that moves follows the block (the append kernel, which runs after the copy
+  // in stream order, then writes the row where attention will look for it).
+  if (!moves.empty()) {
+    const int32_t bs = static_cast<int32_t>(config_.block_size);
+    for (int64_t seq = 0; seq < config_.max_batch; ++seq) {
+      int32_t& slot = host_small_[static_cast<size_t>(seq)];
+      if (slot < 0) continue;
+      const int32_t block = slot / bs;
+      for (const auto& move : moves) {
+        if (move.first == block) {
+          slot = move.second * bs + slot % bs;
+          break;
+        }
+      }
+    }
+  }
   if (moves.empty() || !bound_) return moves;
   IDeviceBackend& backend = arena_.backend();
   if (moves_busy_) backend.SynchronizeEvent(moves_event_);

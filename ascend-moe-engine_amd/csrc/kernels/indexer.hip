@@ -202,8 +202,14 @@ __global__ __launch_bounds__(kScoreThreads) void IndexerScoreKernel(IndexerArgs 
     my_scale = a.key_scale_base[block * a.key_scale_block_stride + slot];
   }
   // Loads return in issue order: query, keys (two loads per group of 16 tokens), the scale. A
-  // group is scored while the later ones are still on their way.
-  asm volatile("s_waitcnt vmcnt(7)" ::: "memory");
+  // group is scored while the later ones are still on their way: a wave that asked for keys has
+  // nine newer loads behind its query rows, so all but seven of them done means the query landed.
+  // A wave past the end of its sequence asked for no keys and waits for everything it issued.
+  if (wave_in_range && token0 < seq_len) {
+    asm volatile("s_waitcnt vmcnt(7)" ::: "memory");
+  } else {
+    asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+  }
   __syncthreads();  // the query rows the other waves fetched
   if (token0 >= seq_len) return;
 

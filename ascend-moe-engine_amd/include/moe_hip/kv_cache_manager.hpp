@@ -116,7 +116,13 @@ class KvCacheManager {
   size_t rope_layer_stride() const { return rope_layer_stride_; }
 
   void AddSequence(int64_t seq, int64_t context_len);
+  // Bookkeeping of one token of one sequence; returns its slot. The slot mapping that UploadStep
+  // sends holds one entry per sequence, the slot of its latest token: a caller that appends
+  // several tokens of a sequence between uploads (a prefill) keeps the returned slots itself.
   int32_t AppendToken(int64_t seq);
+  // The same for every live sequence in one call; slots (optional, max_batch entries) receives
+  // each sequence's slot, -1 for an unused entry. Returns the number of tokens appended.
+  int64_t AppendTokenAll(int32_t* slots);
   void FreeSequence(int64_t seq);
   // Plans and (on a kernel-capable backend) enqueues the defragmentation copy.
   std::vector<std::pair<int32_t, int32_t>> Compact(void* stream);

@@ -140,6 +140,7 @@ PROTOTYPES = {
     "mlakvKvCachePoolBlocks": (_i64, [_vp]),
     "mlakvKvCacheAddSequence": (_i32, [_vp, _i64, _i64]),
     "mlakvKvCacheAppendToken": (_i32, [_vp, _i64, _P(_i32)]),
+    "mlakvKvCacheAppendTokenAll": (_i32, [_vp, _P(_i32), _P(_i64)]),
     "mlakvKvCacheFreeSequence": (_i32, [_vp, _i64]),
     "mlakvKvCacheCompact": (_i32, [_vp, _P(_i32), _P(_i64), _vp]),
     "mlakvKvCacheUploadStep": (_i32, [_vp, _vp]),
@@ -343,6 +344,12 @@ class KvCache:
         out = _i32()
         check(self.lib.mlakvKvCacheAppendToken(self.handle, seq, C.byref(out)))
         return out.value
+
+    def append_token_all(self):
+        """One token for every live sequence; returns the number appended."""
+        appended = C.c_int64()
+        check(self.lib.mlakvKvCacheAppendTokenAll(self.handle, None, C.byref(appended)))
+        return appended.value
 
     def free_sequence(self, seq):
         check(self.lib.mlakvKvCacheFreeSequence(self.handle, seq))

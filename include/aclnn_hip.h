@@ -160,11 +160,11 @@ aclnnStatus aclnnScatterPaKvCache(void* workspace, uint64_t workspace_size, aclO
  * bf16 views (any element strides), one key tensor and one value tensor that alias the same
  * paged latent cache [blocks, block, 1, 512], key_rope [blocks, block, 1, 64], block_table
  * int32 [T, W], one query token per sequence, layout "TND", num_key_value_heads 1, no masks,
- * no quantisation arguments. actual_seq_lengths_kv holds one length per sequence and is read
- * at every launch through the pointer given to aclCreateIntArray (the reference keeps that
- * storage alive for the arena's lifetime, include/moe/memory/static_arena.hpp:169-174), so the
- * caller may update the live lengths in place between launches; aclnnMlaKvBindSeqLens
- * replaces it by a device array. The workspace covers the split-KV partials. */
+ * no quantisation arguments. actual_seq_lengths_kv holds one length per sequence; its values
+ * are copied at plan time (the reference fixes them there, src/memory/static_arena_manager.cpp:
+ * 584-588). A caller that attends over the live context, not the reserved one, updates them
+ * with aclnnMlaKvSetSeqLens (host values) or aclnnMlaKvBindSeqLens (a device array). The
+ * workspace covers the partials of sequences split over several workgroups and the lengths. */
 aclnnStatus aclnnFusedInferAttentionScoreV5GetWorkspaceSize(
     const aclTensor* query, const aclTensorList* key, const aclTensorList* value, const aclTensor* pse_shift,
     const aclTensor* atten_mask, const aclIntArray* actual_seq_lengths, const aclIntArray* actual_seq_lengths_kv,
@@ -214,7 +214,8 @@ aclnnStatus aclnnQuantLightningIndexerGetWorkspaceSize(const aclTensor* query, c
                                                        uint64_t* workspace_size, aclOpExecutor** executor);
 aclnnStatus aclnnQuantLightningIndexer(void* workspace, uint64_t workspace_size, aclOpExecutor* executor, aclrtStream stream);
 
-/* Block-table gather as a two-phase operator, for callers that want the paged read the
+/* EXTENSION (the reference has no such operator: its paged read is implicit in the attention
+ * operator). Block-table gather as a two-phase operator, for callers that want the paged read the
  * reference leaves inside its attention operator (addressing as in third_party/ops_transformer/
  * attention/quant_lightning_indexer/op_kernel/arch35/quant_lightning_indexer_service_cube.h:243-270).
  * key_cache / value_cache [blocks, block, 1, dim] bf16; block_table int32 [B, W]; seq_lens and
@@ -227,10 +228,14 @@ aclnnStatus aclnnGatherPaKvCacheGetWorkspaceSize(const aclTensor* key_cache, con
                                                  int64_t max_seq_len, uint64_t* workspace_size, aclOpExecutor** executor);
 aclnnStatus aclnnGatherPaKvCache(void* workspace, uint64_t workspace_size, aclOpExecutor* executor, aclrtStream stream);
 
-/* Binds a device int32 array [T] of live context lengths to a planned attention executor; it
- * then replaces the plan-time host array, with no per-launch copy. NULL unbinds. No reference
- * counterpart: the reference fixes the length at build time
- * (src/memory/static_arena_manager.cpp:584-588). */
+/* EXTENSION (no reference counterpart: the reference fixes the length at build time,
+ * src/memory/static_arena_manager.cpp:584-588). Replaces the kv lengths of a planned attention
+ * executor by `count` = T host values, each in [0, table width * block size]; they are copied, and
+ * every later launch sends them to the device in the argument block of a small kernel. */
+aclnnStatus aclnnMlaKvSetSeqLens(aclOpExecutor* executor, const int64_t* seq_lens, uint64_t count);
+/* EXTENSION (no reference counterpart, as above). Binds a device int32 array [T] of live context
+ * lengths to a planned attention executor; it then replaces the host values, with no per-launch
+ * copy. NULL unbinds. */
 aclnnStatus aclnnMlaKvBindSeqLens(aclOpExecutor* executor, const int32_t* device_seq_lens);
 
 #ifdef __cplusplus

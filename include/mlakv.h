@@ -397,10 +397,18 @@ mlakvStatus mlakvKvCacheAddSequence(mlakvKvCache* cache, int64_t seq, int64_t co
  * (slot = table[pos / bs] * bs + pos % bs; identity paging gives slot = position,
  * src/pipeline/pipeline.cpp:517). */
 mlakvStatus mlakvKvCacheAppendToken(mlakvKvCache* cache, int64_t seq, int32_t* slot);
+/* The same for every live sequence in one call (the batched decode step): slots, when not NULL,
+ * receives max_batch entries, -1 for an unused sequence; appended receives the count. The slot
+ * mapping that mlakvKvCacheUploadStep sends holds one entry per sequence, the slot of its latest
+ * token: a caller that appends several tokens of one sequence between uploads (a prefill) keeps
+ * the slots these calls return and passes them to mlakvAppend itself. */
+mlakvStatus mlakvKvCacheAppendTokenAll(mlakvKvCache* cache, int32_t* slots, int64_t* appended);
 mlakvStatus mlakvKvCacheFreeSequence(mlakvKvCache* cache, int64_t seq);
 /* Plans the defragmentation (live blocks to ids [0, n_live)), rewrites the host tables and
  * free list, writes the (src, dst) pairs to `moves` (capacity 2 * pool_blocks, may be NULL)
- * and, when the arena is on the HIP backend, uploads them and enqueues the copy kernel. */
+ * and, when the arena is on the HIP backend, uploads them and enqueues the copy kernel. May be
+ * called between mlakvKvCacheAppendToken and mlakvKvCacheUploadStep: the slots of tokens that
+ * wait for the upload follow their blocks. */
 mlakvStatus mlakvKvCacheCompact(mlakvKvCache* cache, int32_t* moves, int64_t* num_moves, void* stream);
 /* Enqueues the H2D copy of this step's metadata (block table, slot mapping, seq_lens,
  * cu_seq_lens) from the pinned mirror; the batched form of the reference's 4-byte

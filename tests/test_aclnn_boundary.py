@@ -181,6 +181,12 @@ def test_attention_plan_contract_workspace_and_ir_indices():
     assert lib.aclSetDynamicTensorAddr(executor, 1, 1, e.key_list, layer_latent) == 161002
     assert lib.aclSetDynamicTensorAddr(executor, 1, 0, e.value_list, layer_latent) == 161002
     assert lib.aclnnMlaKvBindSeqLens(executor, FAKE) == 0 and lib.aclnnMlaKvBindSeqLens(executor, None) == 0
+    one = (C.c_int64 * 1)(17)
+    assert lib.aclnnMlaKvSetSeqLens(executor, one, 1) == 0
+    assert lib.aclnnMlaKvSetSeqLens(executor, one, 2) == 161002          # one length per sequence
+    assert lib.aclnnMlaKvSetSeqLens(executor, (C.c_int64 * 1)(-1), 1) == 161002
+    assert lib.aclnnMlaKvSetSeqLens(executor, (C.c_int64 * 1)(1 << 40), 1) == 161002
+    assert lib.aclnnMlaKvSetSeqLens(executor, None, 1) == 161001
     assert lib.aclDestroyAclOpExecutor(executor) == 0
     # refusals, each naming the contract it breaks
     assert e.plan_attention(heads=32)[0] == 161002

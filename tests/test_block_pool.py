@@ -3,6 +3,8 @@ brute force; the product's pool (KV cache manager, host backend, bookkeeping onl
 agree with the oracle bit for bit on tables, slots, free lists and compaction moves."""
 import random
 
+import ctypes as C
+
 import numpy as np
 import pytest
 
@@ -222,3 +224,56 @@ def test_upload_step_refreshes_lengths_and_resets_slot_mapping():
     assert list(table) == list(cache.host_block_table().reshape(-1))
     cache.close()
     arena.close()
+
+
+def test_compaction_between_append_and_upload_moves_the_pending_slots():
+    """A token whose slot waits for the upload sits in a block that compaction moves: the slot
+    has to follow the block, or the append kernel would write the row into a freed block. The
+    oracle pool, driven through the same operations, gives the expected slots."""
+    bs, blocks = 16, 12
+    arena = ffi.Arena(ffi.BACKEND_HOST)
+    cache = ffi.KvCache(arena, num_layers=1, block_size=bs, max_context_len=64, max_batch=4, pool_blocks=blocks, seed=5, shuffle=1)
+    arena.commit()
+    cache.bind()
+    pool = orc.Pool(blocks, bs, 4, 4, seed=5, shuffle=True)
+    for s, n in enumerate([20, 33, 16, 47]):
+        cache.add_sequence(s, n)
+        assert pool.add_sequence(s, n) == orc.OK
+    cache.upload_step(None)
+    cache.free_sequence(0)
+    cache.free_sequence(2)
+    pool.free_sequence(0)
+    pool.free_sequence(2)
+    assert cache.append_token_all() == 2          # sequences 1 and 3 (3 opens a new block: 48 tokens)
+    want_before = {s: pool.append_token(s)[1] for s in (1, 3)}
+    assert [int(v) for v in cache.host_slot_mapping()] == [-1, want_before[1], -1, want_before[3]]
+    moves = cache.compact(None)
+    want_moves = pool.compact()
+    assert [tuple(m) for m in moves] == [tuple(m) for m in want_moves] and len(moves) > 0
+    table = pool.table()
+    expected = [-1, -1, -1, -1]
+    for s in (1, 3):
+        pos = pool.seq_len(s) - 1
+        expected[s] = int(table[s, pos // bs]) * bs + pos % bs
+    assert [int(v) for v in cache.host_slot_mapping()] == expected
+    assert expected != [-1, want_before[1], -1, want_before[3]]   # at least one pending slot did move
+    assert np.array_equal(cache.host_block_table(), table)
+    cache.close()
+    arena.close()
+
+
+def test_arena_outlives_its_caches_whatever_the_order_of_destruction():
+    arena = ffi.Arena(ffi.BACKEND_HOST)
+    cache = ffi.KvCache(arena, num_layers=1, block_size=16, max_context_len=64, max_batch=2)
+    arena.commit()
+    cache.bind()
+    cache.add_sequence(0, 3)
+    lib = ffi.load()
+    handle, arena_handle = cache.handle, arena.handle
+    arena.handle = None                     # the wrapper must not destroy it a second time
+    lib.mlakvArenaDestroy(arena_handle)     # deferred: the cache still refers to the arena
+    slot = C.c_int32()
+    assert lib.mlakvKvCacheAppendToken(handle, 0, C.byref(slot)) == 0 and slot.value >= 0
+    assert lib.mlakvKvCacheUploadStep(handle, None) == 0
+    cache.handle = None
+    lib.mlakvKvCacheDestroy(handle)         # the last cache takes the arena with it

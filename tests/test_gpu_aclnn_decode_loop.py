@@ -86,7 +86,9 @@ def test_reference_shaped_decode_loop_matches_oracle():
     for position in range(steps):
         C.cast(mailbox, C.POINTER(C.c_int32))[position] = position  # a fresh mailbox word per step: no reuse while in flight
         _ok(lib.aclrtMemcpyAsync(slot_dev, 4, mailbox.value + 4 * position, 4, H2D, stream))
-        seq_kv_storage[0] = position + 1  # live length, read through the int-array's storage at launch
+        seq_kv_storage[0] = -7  # the array's values were copied when it was created: the caller's storage is its own again
+        live = (C.c_int64 * 1)(position + 1)
+        _ok(lib.aclnnMlaKvSetSeqLens(ex_attn, live, 1))  # the live length, copied; `live` may go out of scope
         for layer in range(layers):
             latent, rope = latent_base + layer * latent_stride, rope_base + layer * rope_stride
             _ok(lib.aclSetTensorAddr(ex_scatter, 1, t_latent_cache, latent))
