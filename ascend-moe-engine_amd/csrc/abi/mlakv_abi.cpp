@@ -321,7 +321,8 @@ PlanShape ShapeOf(int32_t batch, int32_t heads, int32_t max_seq_len, int32_t blo
   shape.max_tiles = (static_cast<int64_t>(max_seq_len) + mlakv::kTileTokens - 1) / mlakv::kTileTokens;
   shape.head_groups = (heads + 63) / 64;
   shape.cap = CapUnitTiles(block_size, sparse);
-  const int64_t total = static_cast<int64_t>(batch) * shape.max_tiles;
+  // the longest flat axis a launch can see: every sequence full, each with its idle positions in front
+  const int64_t total = static_cast<int64_t>(batch) * (shape.max_tiles + mlakv::kAttnBoundaryTiles);
   if (chunk_tiles > 0) {
     shape.units = (total + chunk_tiles - 1) / chunk_tiles;
   } else {

@@ -165,6 +165,7 @@ constexpr int kLatentDim = 512;
 constexpr int kRopeDim = 64;
 constexpr int kTileTokens = 32;
 constexpr int kAttnTableEntries = 512;     // block-table entries (or selected tokens) of one segment staged in LDS
+constexpr int kAttnBoundaryTiles = 4;      // what entering a sequence inside a work unit costs, in tiles (see MakeCut)
 constexpr int kAttnSyncSequences = 4096;   // (head group, sequence) pairs a launch can merge in place
 
 hipError_t LaunchAppend(const AppendArgs& args, hipStream_t stream);

@@ -473,14 +473,15 @@ __device__ __forceinline__ int WaveInclusiveScan(int v) {
   return v;
 }
 
-// 64 consecutive sequences, one per lane: tokens that count, tiles, and the running tile total
-// up to and including the lane's sequence. Windows are visited in increasing order.
+// 64 consecutive sequences, one per lane: tokens that count, tiles, and the running totals of
+// tiles and of sequences that have tiles, up to and including the lane's sequence. Windows are
+// visited in increasing order.
 template <bool SPARSE>
 struct SeqWindow {
   int base;   // first sequence of the window; uniform
-  int tok, tiles, incl;
+  int tok, tiles, incl_tiles, incl_live;
 
-  __device__ __forceinline__ void Load(const AttnArgs& a, int lane, int new_base, int carry) {
+  __device__ __forceinline__ void Load(const AttnArgs& a, int lane, int new_base, int carry_tiles, int carry_live) {
     base = new_base;
     const int seq = base + lane;
     int n = 0;
@@ -493,12 +494,26 @@ struct SeqWindow {
     }
     tok = n;
     tiles = (n + kTileTokens - 1) / kTileTokens;
-    incl = carry + WaveInclusiveScan(tiles);
+    incl_tiles = carry_tiles + WaveInclusiveScan(tiles);
+    incl_live = carry_live + WaveInclusiveScan(tiles != 0 ? 1 : 0);
   }
-  __device__ __forceinline__ int End() const { return __builtin_amdgcn_readlane(incl, 63); }
+  __device__ __forceinline__ void Next(const AttnArgs& a, int lane) { Load(a, lane, base + 64, EndTiles(), EndLive()); }
+  __device__ __forceinline__ int EndTiles() const { return __builtin_amdgcn_readlane(incl_tiles, 63); }
+  __device__ __forceinline__ int EndLive() const { return __builtin_amdgcn_readlane(incl_live, 63); }
   __device__ __forceinline__ int Tok(int seq) const { return __builtin_amdgcn_readlane(tok, seq - base); }
   __device__ __forceinline__ int Tiles(int seq) const { return __builtin_amdgcn_readlane(tiles, seq - base); }
-  __device__ __forceinline__ int Incl(int seq) const { return __builtin_amdgcn_readlane(incl, seq - base); }
+  // End of sequence `seq` on the flat axis on which every sequence with tiles is preceded by `pad` idle positions.
+  __device__ __forceinline__ int End(int seq, int pad) const {
+    return __builtin_amdgcn_readlane(incl_tiles, seq - base) + pad * __builtin_amdgcn_readlane(incl_live, seq - base);
+  }
+  __device__ __forceinline__ int EndOfLane(int pad) const { return incl_tiles + pad * incl_live; }
+  // The tile count shared by every sequence of the window that has tiles (0: none has, -1: they differ).
+  __device__ __forceinline__ int CommonTiles() const {
+    const u64 live = __builtin_amdgcn_ballot_w64(tiles != 0);
+    if (live == 0) return 0;
+    const int first = __builtin_amdgcn_readlane(tiles, __builtin_ctzll(live));
+    return __builtin_amdgcn_ballot_w64(tiles != 0 && tiles != first) == 0 ? first : -1;
+  }
 };
 
 // Tiles per work unit for a launch whose sequences add up to `total_tiles`: an equal share per
@@ -514,6 +529,33 @@ __device__ __forceinline__ int TilesPerUnit(const AttnArgs& a, int total_tiles, 
     share = (total_tiles + work_groups - 1) / work_groups;
   }
   return min(max(share, a.forced_unit_tiles > 0 ? 1 : a.min_unit_tiles), a.cap_unit_tiles);
+}
+
+// How a launch cuts its work. Entering a sequence in the middle of a unit costs a workgroup about
+// as much as kBoundaryTiles tiles (the query, the table entries and the first tiles of the new
+// sequence arrive while nothing is computed), and the launch lasts as long as its slowest
+// workgroup. So the flat axis gives every sequence with tiles kBoundaryTiles idle positions in
+// front of its tiles: units are equal on that axis, and one that enters sequences on its way
+// gets that many fewer tiles. When every sequence has the same number of tiles and units divide
+// it, unit and sequence boundaries coincide anyway and the axis stays unpadded.
+constexpr int kBoundaryTiles = kAttnBoundaryTiles;
+struct Cut {
+  int pad;             // idle positions in front of every sequence that has tiles
+  int total;           // length of the flat axis
+  int tiles_per_unit;  // positions per unit
+};
+__device__ __forceinline__ Cut MakeCut(const AttnArgs& a, int total_tiles, int live_sequences, int common_tiles, int work_groups) {
+  Cut cut;
+  cut.pad = 0;
+  cut.total = total_tiles;
+  cut.tiles_per_unit = TilesPerUnit(a, total_tiles, work_groups);
+  const bool coincide = live_sequences <= 1 || (common_tiles > 0 && common_tiles % cut.tiles_per_unit == 0);
+  if (!coincide) {
+    cut.pad = kBoundaryTiles;
+    cut.total = total_tiles + kBoundaryTiles * live_sequences;
+    cut.tiles_per_unit = TilesPerUnit(a, cut.total, work_groups);
+  }
+  return cut;
 }
 
 // Stores and loads that other CUs' accesses of the same kind see without a cache write-back or
@@ -677,7 +719,8 @@ __global__ __launch_bounds__(kThreads) void MlaDecodeKernel(AttnArgs a) {
   // Every wave walks the batch itself: the total number of tiles fixes the cut of the flat axis.
   // On the way the empty sequences (no tile, so no unit) get their zeros, spread over the workgroups.
   SeqWindow<SPARSE> win;
-  win.Load(a, lane0, 0, 0);
+  win.Load(a, lane0, 0, 0, 0);
+  int common_tiles = 0;  // the tile count all sequences with tiles share; -1 when they differ
   for (;;) {
     if constexpr (!SPARSE) {
       u64 empties = __builtin_amdgcn_ballot_w64(win.base + lane0 < a.batch && win.tiles == 0);
@@ -687,15 +730,17 @@ __global__ __launch_bounds__(kThreads) void MlaDecodeKernel(AttnArgs a) {
         empties &= empties - 1;
       }
     }
+    const int here = win.CommonTiles();
+    if (here != 0) common_tiles = common_tiles == 0 || common_tiles == here ? here : -1;
     if (win.base + 64 >= a.batch) break;
-    win.Load(a, lane0, win.base + 64, win.End());
+    win.Next(a, lane0);
   }
-  const int total_tiles = win.End();
-  const int tiles_per_unit = TilesPerUnit(a, total_tiles, work_groups);
-  // unit u covers flat tiles [u, u + 1) * tiles_per_unit; there are ceil(total / tiles_per_unit)
-  // units, at most a.max_units (ensured by the plan)
+  const Cut cut = MakeCut(a, win.EndTiles(), win.EndLive(), common_tiles, work_groups);
+  const int tiles_per_unit = cut.tiles_per_unit, total_tiles = cut.total, pad = cut.pad;
+  // unit u covers positions [u, u + 1) * tiles_per_unit of the flat axis; there are
+  // ceil(total / tiles_per_unit) units, at most a.max_units (ensured by the plan)
   if (static_cast<int64_t>(wg) * tiles_per_unit >= total_tiles) return;
-  if (win.base != 0) win.Load(a, lane0, 0, 0);
+  if (win.base != 0) win.Load(a, lane0, 0, 0, 0);
 
   // Q fragments (score waves): lane (head i16, k-group g) holds, for k-step ks, the eight query
   // elements that meet the lane's K fragment of that step: Q[head][32 ks + 8g .. +7] for bf16
@@ -782,581 +827,586 @@ __global__ __launch_bounds__(kThreads) void MlaDecodeKernel(AttnArgs a) {
   for (int unit = wg; static_cast<int64_t>(unit) * tiles_per_unit < total_tiles; unit += work_groups) {
     const int flat_end = min(total_tiles, (unit + 1) * tiles_per_unit);
     int flat = unit * tiles_per_unit;
-    while (win.End() <= flat) win.Load(a, lane0, win.base + 64, win.End());
-    int seq = win.base + __builtin_ctzll(__builtin_amdgcn_ballot_w64(win.incl > flat));
+    while (win.End(win.base + 63, pad) <= flat) win.Next(a, lane0);
+    int seq = win.base + __builtin_ctzll(__builtin_amdgcn_ballot_w64(win.EndOfLane(pad) > flat));
     while (flat < flat_end) {
-      // Segment: tiles [flat, segment_end) of the flat axis, inside sequence `seq`.
-      const int seq_end = win.Incl(seq), seq_begin = seq_end - win.Tiles(seq);
-      const int segment_end = min(flat_end, seq_end);
-      const int tile_begin = flat - seq_begin;          // first tile of the segment inside its sequence
-      const int segment_tiles = segment_end - flat;     // >= 1
-      const bool holds_first = flat == seq_begin, holds_last = segment_end == seq_end;
-      const bool direct = holds_first && holds_last;    // the whole sequence: write the final output here
-      const int slot = holds_first ? a.max_units + seq : unit;
-      int seq_len = win.Tok(seq);
-
-      if (!first_segment) __syncthreads();  // the previous segment's staging rows, table entries and P slots are free
-      first_segment = false;
-
-      // Everything that depends on the thread id alone is formed here, per segment, from a copy
-      // of the id that the compiler cannot see through: hoisted out of the segment loop, these
-      // values would stay live through both roles' tile loops, where no register is to spare.
-      int tid = tid0;
-      asm volatile("" : "+v"(tid));
-      const int lane = tid & 63, wave = Uniform(tid >> 6);
-      const bool score_wave = wave < kScoreWaves;   // wave-uniform role
-      const int hw = wave & (kScoreWaves - 1);      // which 16 heads of the 64
-      const int g = lane >> 4, i16 = lane & 15;
-      const int head_base = z * 64 + hw * 16;
-      const bool active = head_base < a.heads;  // wave-uniform
-      const int head = head_base + i16;
-      const int per_tile = FP8 ? LoadsPerTile8(wave) : LoadsPerTile(wave);
-      // Direct loads: lane L of a latent row fetches chunk L ^ swizzle(row); rows of this wave.
-      IssueLane il;
-      IssueLane8 il8;
-      if (FP8) {
-    #pragma unroll
-        for (int j = 0; j < 2; ++j) {
-          const int row = 2 * wave + 16 * j + (lane >> 5);
-          il8.lat[j] = (lane >> 5) * static_cast<int>(a.latent.row_stride) + (((lane & 31) ^ SwizzleLat8(row)) << 4);
-        }
-        const int rope_row = 16 * (wave & 1) + (lane >> 2);
-        il8.rope = (lane >> 2) * static_cast<int>(a.rope.row_stride) + (((lane & 3) ^ SwizzleRope8(rope_row)) << 4);
-      } else {
-    #pragma unroll
-        for (int j = 0; j < 2; ++j) {
-          il.lat[j] = (lane ^ SwizzleLat(wave + kWaves * j)) << 4;
-          il.partner_lat[j] = (lane ^ SwizzleLat((wave & (kScoreWaves - 1)) + kWaves * j)) << 4;
-        }
-        il.rope_chunk = ((lane & 7) ^ SwizzleRope(8 * (wave - kScoreWaves) + (lane >> 3))) << 4;
-        il.rope = (lane >> 3) * static_cast<int>(a.rope.row_stride) + il.rope_chunk;
-      }
-
-      unsigned char* p_lds = lds + G::kPOff + (hw * 64 + lane) * 16;           // + parity * kScoreWaves * 64 * 16
-      float* alpha_lds = reinterpret_cast<float*>(lds + G::kAlphaOff) + hw * 64 + lane;  // + parity * kScoreWaves * 64
-      float* inv_lds = reinterpret_cast<float*>(lds + G::kInvOff) + hw * 64 + lane;
-      int* flag_lds = reinterpret_cast<int*>(lds + G::kFlagOff) + hw;          // + parity * kScoreWaves
-
-      // Stage this segment's block-table entries in LDS.
-      TileMap<ALIGNED> map;
-      map.entries = table_lds;
-      map.block_size = a.block_size;
-      map.sparse = SPARSE;
-      map.first_pos = tile_begin * kTileTokens;
-      map.first_block = 0;
-      map.next_entry = 0;
-      map.next_slot0 = 0;
-      map.tile_block = 0;
-      map.tile_slot0 = 0;
-      int staged[kTableEntries / 64];  // kSoloPrologue: this lane's table entries on their way to LDS
-      int staged_count = 0;
-      const auto write_table = [&]() __attribute__((always_inline)) {
-        if constexpr (kSoloPrologue) {
-#pragma unroll
-          for (int j = 0; j < kTableEntries / 64; ++j) {
-            const int i = lane + 64 * j;
-            if (i < staged_count) table_lds[i] = static_cast<unsigned>(staged[j]) < static_cast<unsigned>(a.num_blocks) ? staged[j] : -1;
-          }
-        }
-      };
-      if constexpr (!SPARSE) {
-        const int first_pos = tile_begin * kTileTokens;
-        const int last_pos = first_pos + segment_tiles * kTileTokens - 1;
-        map.first_block = first_pos / a.block_size;
-        map.next_slot0 = first_pos - map.first_block * a.block_size;
-        int count = last_pos / a.block_size - map.first_block + 1;  // <= kTableEntries, ensured by the plan's cap
-        count = min(count, a.table_stride - map.first_block);
-        const int32_t* table_row = a.block_table + static_cast<int64_t>(seq) * a.table_stride + map.first_block;
-        if constexpr (kSoloPrologue) {
-          // Every wave stages all entries itself (the same values to the same addresses), so that it
-          // can read them back without waiting for the other waves. Here they are only asked for;
-          // each role writes them to LDS where it first needs them (write_table below).
-          staged_count = count;
-#pragma unroll
-          for (int j = 0; j < kTableEntries / 64; ++j) {
-            const int i = lane + 64 * j;
-            staged[j] = i < count ? table_row[i] : -1;
-          }
-        } else {
-          for (int i = tid; i < count; i += kThreads) {
-            const int entry = table_row[i];
-            table_lds[i] = static_cast<unsigned>(entry) < static_cast<unsigned>(a.num_blocks) ? entry : -1;
-          }
-        }
-      } else {
-        // The selection ends at its first entry that is negative or not inside the context. Then
-        // this segment's part of it is resolved to pool slots through the block table.
-        const int context = static_cast<int>(
-            min(static_cast<int64_t>(max(Uniform(a.seq_lens[seq]), 0)), static_cast<int64_t>(a.table_stride) * a.block_size));
-        const int32_t* selection = a.sparse_indices + static_cast<int64_t>(seq) * a.sparse_seq_stride;
-        if (tid == 0) scalar_lds[0] = a.sparse_count;
-        __syncthreads();
-        for (int i = tid; i < a.sparse_count; i += kThreads) {
-          const int index = selection[i];
-          if (index < 0 || index >= context) atomicMin(scalar_lds, i);
-        }
-        __syncthreads();
-        seq_len = Uniform(scalar_lds[0]);
-        const int32_t* table_row = a.block_table + static_cast<int64_t>(seq) * a.table_stride;
-        const int segment_tokens = min(segment_tiles * kTileTokens, seq_len - map.first_pos);  // <= kTableEntries, ensured by the plan's cap
-        for (int i = tid; i < segment_tokens; i += kThreads) {
-          const int index = selection[map.first_pos + i];  // inside [0, context): before the end of the selection
-          const int logical = index / a.block_size;
-          const int entry = table_row[logical];
-          table_lds[i] = static_cast<unsigned>(entry) < static_cast<unsigned>(a.num_blocks)
-                             ? entry * a.block_size + (index - logical * a.block_size)
-                             : -1;
-        }
-      }
-      map.seq_len = seq_len;
-      const int num_tiles = (seq_len + kTileTokens - 1) / kTileTokens;
-      // tiles of this segment that exist (a selection may end before the list does)
-      const int ntiles = min(segment_tiles, num_tiles - tile_begin);
-      if (SPARSE && ntiles <= 0) {
-        if (direct) {
-          ZeroFill<MXQ>(a, z, seq, wave, lane);
-        } else if (active && score_wave && g == 0) {  // empty partial: the merge reads every partial's LSE
-          StoreAgentF32(a.partial_lse + PartialRow(a, z, slot, hw * 16 + i16), -__builtin_inff());
-        }
-      } else {
-        const auto issue = [&](int t) __attribute__((always_inline)) {
-          if constexpr (FP8) {
-            return IssueTileFp8(a, map, il8, tile_begin + t, lds_base + ring(t), lds + ring(t), tid);
-          } else {
-            return IssueTileBf16(a, map, il, tile_begin + t, lds_base + ring(t), lds + ring(t), tid);
-          }
-        };
-        // Prologue (each role runs its own copy, below): tiles 0 .. kRing-2 on their way, tile 0
-        // landed and published. A tile whose load count is not known (rare path) makes every wait
-        // up to and including its own a full one.
-        int last_unknown = -1;  // newest tile issued with an unknown number of loads
-        int issued = 0;         // tiles issued so far
-        // Loads this wave has in flight that are newer than those of tile t: the first `solo_tiles`
-        // tiles carry `solo_loads` each, the later ones `per_tile`.
-        const int solo_tiles = kSoloPrologue ? min(G::kRing - 1, ntiles) : 0;
-        const int solo_loads = score_wave ? 0 : per_tile + kRowsPerWave;
-        const auto newer_than = [&](int t) __attribute__((always_inline)) {
-          const int solo = max(0, min(issued, solo_tiles) - (t + 1));
-          const int shared = max(0, issued - max(t + 1, solo_tiles));
-          return solo * solo_loads + shared * per_tile;
-        };
-        // Top of iteration i, both roles: tile i+1 must have landed (later tiles may still be in
-        // flight); the barrier publishes it together with P(i) and retires every wave's reads of
-        // tile i-1, whose ring slot the next tile to be issued reuses.
-        const auto publish = [&](int i) __attribute__((always_inline)) {
-          if (i + 1 < ntiles) WaitLoads(last_unknown >= i + 1 ? 0 : newer_than(i + 1));
-          __syncthreads();
-        };
-        // Issues the next tile of the ring (tile i + kRing - 1 during iteration i).
-        const auto issue_next = [&](int i) __attribute__((always_inline)) {
-          if (issued < ntiles) {
-            if (!issue(issued)) last_unknown = issued;
-            ++issued;
-          }
-        };
-
-        if (score_wave) {
-          // ---------------------------------------------------------------- score waves
-          // Vector memory requests of a CU are served in order: the query (72 KB per workgroup) is
-          // asked for behind the few bytes of table entries that the first tile addresses depend on.
-          // It lives in this role's branch only; the output waves' prologue has no room for it.
-          bf16x8 q[kKSteps];
-          if (active) {
-            const char* q_latent = a.q_latent + seq * a.q_latent_seq_stride + head * a.q_latent_head_stride;
-            const char* q_rope = a.q_rope + seq * a.q_rope_seq_stride + head * a.q_rope_head_stride;
-#pragma unroll
-            for (int ks = 0; ks < kKSteps; ++ks) {
-              const int d0 = FP8 ? 64 * (ks >> 1) + 16 * g + 8 * (ks & 1) : 32 * ks + 8 * g;
-              const char* p = d0 < kLatentDim ? q_latent + d0 * 2 : q_rope + (d0 - kLatentDim) * 2;
-              q[ks] = __builtin_bit_cast(bf16x8, GlobalLoad16(p));
-            }
-          } else {
-#pragma unroll
-            for (int ks = 0; ks < kKSteps; ++ks) q[ks] = __builtin_bit_cast(bf16x8, u32x4{0u, 0u, 0u, 0u});
-          }
-          write_table();  // asked for before the query, so it is here first
-          // The query must have arrived before this wave issues tile loads: the compiler's own wait
-          // for it would otherwise also wait for every tile load issued in between. Both paths above
-          // pass through the statement: were it skipped on one, the compiler would have to assume the
-          // query still in flight where they meet again, and would wait for it -- with counts that
-          // know nothing of the tile loads, so in effect for every tile in flight -- inside the
-          // score loop, at every use.
-#pragma unroll
-          for (int ks = 0; ks < kKSteps; ++ks) asm volatile("" ::"v"(q[ks]));
-          if constexpr (!kSoloPrologue) __syncthreads();  // table entries visible
-          for (; issued < G::kRing - 1 && issued < ntiles; ++issued) {
-            if constexpr (kSoloPrologue) {
-              map.Begin(issued);  // keeps the cursor in step with the tiles this wave does not issue
-            } else {
-              if (!issue(issued)) last_unknown = issued;
-            }
-          }
-          WaitLoads(last_unknown >= 0 ? 0 : newer_than(0));
-          __syncthreads();
-
-          // bf16 K reads: token = 16t + i16, chunk = 4 ks + g (latent, ks < 16) or 4 (ks - 16) + g (rope).
-          const int k_lat = i16 * Geom<false>::kLatRow, k_rope = Geom<false>::kLatRegion + i16 * Geom<false>::kRopeRow;
-          int k_e[4], kr_e[2];
-#pragma unroll
-          for (int j = 0; j < 4; ++j) k_e[j] = ((4 * j + g) ^ SwizzleLat(i16)) << 4;
-#pragma unroll
-          for (int j = 0; j < 2; ++j) kr_e[j] = ((4 * j + g) ^ SwizzleRope(i16)) << 4;
-          // K fragment of pipeline step `step` (k-step step/2, token subtile step&1) of the tile at `buf`.
-          const auto k_frag = [&](const unsigned char* buf, int step) __attribute__((always_inline)) {
-            const int ks = step >> 1, t = step & 1;
-            const int offset = ks < 16 ? k_lat + (ks >> 2) * 256 + k_e[ks & 3] + t * 16 * Geom<false>::kLatRow
-                                       : k_rope + kr_e[ks & 1] + t * 16 * Geom<false>::kRopeRow;
-            return *reinterpret_cast<const bf16x8*>(buf + offset);
-          };
-          // FP8 K reads: read u = 2 kp + t fetches the 16 codes k = 64 kp + 16 g .. +15 of token 16t + i16
-          // (k-steps 2kp and 2kp+1): chunk (4 kp + g) ^ swizzle(token) of the 512-byte row; kp = 8 is the
-          // rope row (chunk g ^ swizzle). The tile base is a multiple of 512, so the XOR with kp << 6 is
-          // applied to the lane-constant part.
-          int k8_lat[2];
-#pragma unroll
-          for (int t = 0; t < 2; ++t) k8_lat[t] = (16 * t + i16) * Geom<true>::kLatRow + ((g ^ SwizzleLat8(16 * t + i16)) << 4);
-          const int k8_rope = Geom<true>::kLatRegion + i16 * Geom<true>::kRopeRow + ((g ^ SwizzleRope8(i16)) << 4);
-          const auto k8_read = [&](const unsigned char* buf, int u) __attribute__((always_inline)) {
-            const int kp = u >> 1, t = u & 1;
-            const int offset = kp < 8 ? (k8_lat[t] ^ (kp << 6)) : k8_rope + t * 16 * Geom<true>::kRopeRow;
-            return *reinterpret_cast<const u32x4*>(buf + offset);
-          };
-
-          float m_ref = -__builtin_inff();  // reference maximum of the exponentials, log2 domain
-          float l_run = 0.0f;               // this lane's share of the running denominator
-
-          // S^T of tile `tile_rel`, its softmax against the running reference, P and the rescale
-          // request into the LDS slots of the tile's parity.
-          const auto score_tile = [&](int tile_rel, int issue_iteration) __attribute__((always_inline)) {
-            const unsigned char* buf = lds + ring(tile_rel);
-            f32x4 acc[4];
-#pragma unroll
-            for (int j = 0; j < 4; ++j) acc[j] = f32x4{0.f, 0.f, 0.f, 0.f};
-            f32x4 row_scale[2];  // FP8: scales of tokens 4g+j and 16+4g+j
-            if constexpr (FP8) {
-              const float* scales = reinterpret_cast<const float*>(buf + G::kScaleOff);
-              row_scale[0] = *reinterpret_cast<const f32x4*>(scales + 4 * g);
-              row_scale[1] = *reinterpret_cast<const f32x4*>(scales + 16 + 4 * g);
-              u32x4 kr[kKAhead8];
-#pragma unroll
-              for (int d = 0; d < kKAhead8; ++d) kr[d] = k8_read(buf, d);
-              __builtin_amdgcn_sched_barrier(0);
-              StaticFor<kKSteps>([&](auto u_c) __attribute__((always_inline)) {
-                constexpr int u = decltype(u_c)::value;  // kp = u / 2, token subtile t = u & 1
-                const u32x4 codes = kr[u % kKAhead8];
-                if constexpr (u + kKAhead8 < kKSteps) kr[u % kKAhead8] = k8_read(buf, u + kKAhead8);
-                constexpr int t = u & 1, kp = u >> 1;
-                acc[2 * t] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(CodesToBf16(codes.x, codes.y), q[2 * kp], acc[2 * t], 0, 0, 0);
-                acc[2 * t + 1] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(CodesToBf16(codes.z, codes.w), q[2 * kp + 1], acc[2 * t + 1], 0, 0, 0);
-                __builtin_amdgcn_sched_barrier(0);
-              });
-            } else {
-              bf16x8 kf[kKAhead];
-#pragma unroll
-              for (int d = 0; d < kKAhead; ++d) kf[d] = k_frag(buf, d);
-              __builtin_amdgcn_sched_barrier(0);
-              StaticFor<kQkSteps>([&](auto step_c) __attribute__((always_inline)) {
-                constexpr int step = decltype(step_c)::value;
-                constexpr int slot_acc = (step & 1) * 2 + ((step >> 1) & 1);  // two accumulators per token subtile
-                acc[slot_acc] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(kf[step % kKAhead], q[step >> 1], acc[slot_acc], 0, 0, 0);
-                if constexpr (step + kKAhead < kQkSteps) kf[step % kKAhead] = k_frag(buf, step + kKAhead);
-                __builtin_amdgcn_sched_barrier(0);
-              });
-            }
-            // the score waves ask for their rows of the next ring tile behind the QK phase
-            if (kLateIssue && issue_iteration >= 0) issue_next(issue_iteration);
-            // lane holds tokens 4g+j (x[0..3]) and 16+4g+j (x[4..7]) of head i16
-            float x[8];
-#pragma unroll
-            for (int j = 0; j < 4; ++j) {
-              x[j] = (acc[0][j] + acc[1][j]) * a.scale_log2;
-              x[4 + j] = (acc[2][j] + acc[3][j]) * a.scale_log2;
-              if constexpr (FP8) {  // the codes were multiplied unscaled
-                x[j] *= row_scale[0][j];
-                x[4 + j] *= row_scale[1][j];
-              }
-            }
-            const int valid = seq_len - (tile_begin + tile_rel) * kTileTokens;  // >= 1
-            if (valid < kTileTokens) {  // wave-uniform: only the last tile of a sequence
-#pragma unroll
-              for (int j = 0; j < 8; ++j) {
-                if (16 * (j >> 2) + 4 * g + (j & 3) >= valid) x[j] = -__builtin_inff();
-              }
-            }
-            float tile_max = fmaxf(fmaxf(fmaxf(x[0], x[1]), fmaxf(x[2], x[3])), fmaxf(fmaxf(x[4], x[5]), fmaxf(x[6], x[7])));
-            tile_max = MaxAcrossHalves(MaxAcrossRows16(tile_max));
-            const int parity = tile_rel & 1;
-            // Move the reference only when some head's maximum outgrew it by more than the threshold.
-            const bool moved = __builtin_amdgcn_ballot_w64(tile_max > m_ref + kRescaleThreshold) != 0;
-            if (moved) {
-              const float m_new = fmaxf(m_ref, tile_max);  // finite: token 0 of the tile is valid
-              const float alpha = __builtin_amdgcn_exp2f(m_ref - m_new);
-              l_run *= alpha;
-              m_ref = m_new;
-              alpha_lds[parity * kScoreWaves * 64] = alpha;
-            }
-            if (lane == 0) flag_lds[parity * kScoreWaves] = moved && tile_rel != 0 ? 1 : 0;  // O is still zero on the first tile
-            bf16x8 p;
-            float sum = 0.0f;
-#pragma unroll
-            for (int j = 0; j < 8; ++j) {
-              const float e = __builtin_amdgcn_exp2f(x[j] - m_ref);
-              sum += e;
-              p[j] = static_cast<__bf16>(FP8 ? e * row_scale[j >> 2][j & 3] : e);  // FP8: V is multiplied unscaled as well
-            }
-            l_run += sum;
-            *reinterpret_cast<bf16x8*>(p_lds + parity * kScoreWaves * 64 * 16) = p;
-          };
-
-          if (active) score_tile(0, -1);
-          for (int i = 0; i < ntiles; ++i) {
-            publish(i);
-            const bool scores = active && i + 1 < ntiles;
-            if (!kLateIssue || !scores) issue_next(i);
-            if (scores) score_tile(i + 1, i);
-          }
-          if (active) {
-            const float l_total = SumAcrossHeadLanes(l_run);
-            *inv_lds = 1.0f / l_total;
-            const float lse2 = m_ref + __builtin_amdgcn_logf(l_total);  // v_log_f32 is log2
-            if (g == 0) {
-              if (direct) {
-                if (a.lse != nullptr) a.lse[seq * a.heads + head] = lse2 * 0.6931471805599453f;
-              } else {
-                StoreAgentF32(a.partial_lse + PartialRow(a, z, slot, hw * 16 + i16), lse2);
-              }
-            }
-          }
-          __syncthreads();  // 1/denominator visible to the output waves
-        } else {
-          // ---------------------------------------------------------------- output waves
-          write_table();
-          if constexpr (!kSoloPrologue) __syncthreads();  // table entries visible
-          for (; issued < G::kRing - 1 && issued < ntiles; ++issued) {
-            if constexpr (kSoloPrologue) {
-              // bf16 tiles: these waves have no query to wait for and issue the first tiles of the ring
-              // alone, their own rows and those of their partner score waves
-              if (!IssueTileBf16<ALIGNED, true>(a, map, il, tile_begin + issued, lds_base + ring(issued), lds + ring(issued), tid)) {
-                last_unknown = issued;
-              }
-            } else {
-              if (!issue(issued)) last_unknown = issued;
-            }
-          }
-          WaitLoads(last_unknown >= 0 ? 0 : newer_than(0));
-          __syncthreads();
-
-          // bf16 V reads: token = (16 +) 4g + i16/4, chunk = 2n + (i16 & 3) / 2, 8-byte half i16 & 1.
-          const int v_row = 4 * g + (i16 >> 2);
-          const int v_lane = v_row * Geom<false>::kLatRow + (i16 & 1) * 8;
-          int v_e[8];
-#pragma unroll
-          for (int j = 0; j < 8; ++j) v_e[j] = ((2 * j + ((i16 & 3) >> 1)) ^ SwizzleLat(v_row)) << 4;
-          // FP8 V reads (ds_read_b64_tr_b8: output lane i of a 16-lane group, element e <- byte i & 7 of
-          // the 8 bytes addressed by lane 2e + (i >> 3)): as a source, lane j addresses bytes
-          // 16n + 8 (j & 1) .. +7 of the row of token kappa = j >> 1 (tokens 4g + kappa, 16 + 4g + kappa - 4).
-          const int v8_token = 4 * g + ((i16 >> 1) & 3) + 16 * (i16 >> 3);
-          const int v8_base = v8_token * Geom<true>::kLatRow + (SwizzleLat8(v8_token) << 4) + 8 * (i16 & 1);
-          // Raw V^T fragment of output tile n (dv 16n..16n+15) over the 32 tokens of the tile at `buf`:
-          // eight bf16 for bf16 tiles, eight codes in the low two dwords for FP8 tiles.
-          const auto v_fetch = [&](const unsigned char* buf, int n) __attribute__((always_inline)) {
-            if constexpr (FP8) {
-              const i32x2 codes = __builtin_amdgcn_ds_read_tr8_b64_v2i32((__attribute__((address_space(3))) i32x2*)(buf + (v8_base ^ (n << 4))));
-              return u32x4{static_cast<unsigned>(codes.x), static_cast<unsigned>(codes.y), 0u, 0u};
-            } else {
-              const unsigned char* addr = buf + v_lane + (n >> 3) * 256 + v_e[n & 7];
-              const s16x4 lo = __builtin_amdgcn_ds_read_tr16_b64_v4i16((__attribute__((address_space(3))) s16x4*)(addr));
-              const s16x4 hi = __builtin_amdgcn_ds_read_tr16_b64_v4i16((__attribute__((address_space(3))) s16x4*)(addr + 16 * Geom<false>::kLatRow));
-              return __builtin_bit_cast(u32x4, __builtin_shufflevector(lo, hi, 0, 1, 2, 3, 4, 5, 6, 7));
-            }
-          };
-          const auto v_operand = [&](const u32x4& raw) __attribute__((always_inline)) {
-            if constexpr (FP8) {
-              return CodesToBf16(raw.x, raw.y);
-            } else {
-              return __builtin_bit_cast(bf16x8, raw);
-            }
-          };
-
-          // Output wave w owns the 128 output columns [128 w, 128 w + 128) of all 64 heads of the group:
-          // every V^T fragment is then fetched (and, for FP8, converted) by one wave only, and meets the
-          // P fragments of the four score waves. Head blocks past the group's heads are computed on
-          // whatever their LDS slots hold and never written.
-          constexpr int kDvPerWave = kDvTiles / (kWaves - kScoreWaves);
-          const unsigned char* p_all = lds + G::kPOff + lane * 16;                                   // + (parity * 4 + hb) * 64 * 16
-          const float* alpha_all = reinterpret_cast<const float*>(lds + G::kAlphaOff) + lane;      // + (parity * 4 + hb) * 64
-          const float* inv_all = reinterpret_cast<const float*>(lds + G::kInvOff) + lane;          // + hb * 64
-          const int* flag_all = reinterpret_cast<const int*>(lds + G::kFlagOff);                   // [parity * 4 + hb]
-          f32x4 o[kScoreWaves][kDvPerWave];
-#pragma unroll
-          for (int hb = 0; hb < kScoreWaves; ++hb) {
-#pragma unroll
-            for (int n = 0; n < kDvPerWave; ++n) o[hb][n] = f32x4{0.f, 0.f, 0.f, 0.f};
-          }
-
-          for (int i = 0; i < ntiles; ++i) {
-            publish(i);
-            issue_next(i);
-            {
-              const unsigned char* buf = lds + ring(i);
-              const int parity = i & 1;
-              // the four rescale flags of the tile in one read; a moved reference maximum is the exception
-              const i32x4 flags = *reinterpret_cast<const i32x4*>(flag_all + parity * kScoreWaves);
-              if (Uniform(flags.x | flags.y | flags.z | flags.w) != 0) {
-                const int moved[kScoreWaves] = {flags.x, flags.y, flags.z, flags.w};
-#pragma unroll
-                for (int hb = 0; hb < kScoreWaves; ++hb) {
-                  if (Uniform(moved[hb]) != 0) {  // that block's reference maximum moved: rescale its O first
-                    const float alpha = alpha_all[(parity * kScoreWaves + hb) * 64];
-#pragma unroll
-                    for (int n = 0; n < kDvPerWave; ++n) o[hb][n] *= alpha;
-                  }
-                }
-              }
-              u32x4 vf[kVAhead];
-#pragma unroll
-              for (int d = 0; d < kVAhead; ++d) vf[d] = v_fetch(buf, kDvPerWave * hw + d);
-              bf16x8 p[kScoreWaves];
-#pragma unroll
-              for (int hb = 0; hb < kScoreWaves; ++hb) p[hb] = *reinterpret_cast<const bf16x8*>(p_all + (parity * kScoreWaves + hb) * 64 * 16);
-              __builtin_amdgcn_sched_barrier(0);
-              if constexpr (FP8) {
-                // the next fragment is converted while this one's four MFMAs run
-                bf16x8 v = v_operand(vf[0]);
-                if constexpr (kVAhead < kDvPerWave) vf[0] = v_fetch(buf, kDvPerWave * hw + kVAhead);
-                StaticFor<kDvPerWave>([&](auto n_c) __attribute__((always_inline)) {
-                  constexpr int n = decltype(n_c)::value;
-                  bf16x8 v_next = v;
-                  if constexpr (n + 1 < kDvPerWave) v_next = v_operand(vf[(n + 1) % kVAhead]);
-#pragma unroll
-                  for (int hb = 0; hb < kScoreWaves; ++hb) o[hb][n] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(v, p[hb], o[hb][n], 0, 0, 0);
-                  if constexpr (n + 1 + kVAhead < kDvPerWave) vf[(n + 1) % kVAhead] = v_fetch(buf, kDvPerWave * hw + n + 1 + kVAhead);
-                  v = v_next;
-                  __builtin_amdgcn_sched_barrier(0);
-                });
-              } else {
-                StaticFor<kDvPerWave>([&](auto n_c) __attribute__((always_inline)) {
-                  constexpr int n = decltype(n_c)::value;
-                  const bf16x8 v = v_operand(vf[n % kVAhead]);
-#pragma unroll
-                  for (int hb = 0; hb < kScoreWaves; ++hb) o[hb][n] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(v, p[hb], o[hb][n], 0, 0, 0);
-                  if constexpr (n + kVAhead < kDvPerWave) vf[n % kVAhead] = v_fetch(buf, kDvPerWave * hw + n + kVAhead);
-                  __builtin_amdgcn_sched_barrier(0);
-                });
-              }
-            }
-          }
-          __syncthreads();  // 1/denominator from the score waves
-          if (MXQ && direct) {
-            // Quantising epilogue of a whole sequence: a block of 32 columns is a pair of this
-            // wave's column tiles over the four lanes that share a head; the wave covers blocks
-            // 4 w .. 4 w + 3 of every head.
-#pragma unroll
-            for (int hb = 0; hb < kScoreWaves; ++hb) {
-              if (hb >= hba) continue;
-              const int h = 16 * hb + i16;
-              const float inv = inv_all[hb * 64];
-              char* codes_row = a.out_codes + seq * a.out_codes_seq_stride + (group_head0 + h) * a.out_codes_head_stride;
-              char* out_row = a.out == nullptr ? nullptr : a.out + seq * a.out_seq_stride + (group_head0 + h) * a.out_head_stride;
-              unsigned scale_codes = 0u;
-#pragma unroll
-              for (int k = 0; k < kDvPerWave / 2; ++k) {
-                u32x2 packed[2];
-                unsigned magnitude = 0u;
-#pragma unroll
-                for (int half = 0; half < 2; ++half) {
-                  const int n = 2 * k + half;
-                  packed[half].x = PackBf16(o[hb][n][0] * inv, o[hb][n][1] * inv);
-                  packed[half].y = PackBf16(o[hb][n][2] * inv, o[hb][n][3] * inv);
-                  magnitude = MxMagnitudeMax(packed[half].y, MxMagnitudeMax(packed[half].x, magnitude));
-                  if (out_row != nullptr) {
-                    __builtin_nontemporal_store(packed[half], reinterpret_cast<u32x2*>(out_row + (16 * (kDvPerWave * hw + n) + 4 * g) * 2));
-                  }
-                }
-                magnitude = UMaxAcrossHeadLanes(magnitude);
-                const MxScale s = MxScaleFromMaxBits(magnitude);
-#pragma unroll
-                for (int half = 0; half < 2; ++half) {
-                  const unsigned four = MxEncodeWord(packed[half].x, s) | (MxEncodeWord(packed[half].y, s) << 16);
-                  __builtin_nontemporal_store(four, reinterpret_cast<unsigned*>(codes_row + 16 * (kDvPerWave * hw + 2 * k + half) + 4 * g));
-                }
-                scale_codes |= s.code << (8 * k);
-              }
-              if (g == 0) {
-                *reinterpret_cast<unsigned*>(a.out_scales + seq * a.out_scales_seq_stride + (group_head0 + h) * a.out_scales_head_stride +
-                                             (kDvPerWave / 2) * hw) = scale_codes;
-              }
-            }
-          } else {
-            // The accumulators hold O^T (lane = head i16 of a block, four columns per 16-column tile),
-            // which stored as it is would write 8-byte pieces of sixteen different rows per
-            // instruction. The tile ring is dead after the last barrier: each output wave transposes
-            // its 256-byte slices of the 64 rows through its own part of it and writes them 16 bytes per
-            // lane, four whole slices per instruction. A row stride of 272 bytes (= 4 banks mod 64)
-            // spreads the 8-byte writes of a half-wave over all banks.
-            constexpr int kSliceBytes = kDvPerWave * 16 * 2;  // 256
-            constexpr int kStageRow = kSliceBytes + 16;
-            static_assert((kWaves - kScoreWaves) * 64 * kStageRow <= G::kRing * G::kTileBytes, "the staging rows fit in the ring");
-            unsigned char* stage = lds + G::Slot(0) + hw * (64 * kStageRow);
-#pragma unroll
-            for (int hb = 0; hb < kScoreWaves; ++hb) {
-              const float inv = inv_all[hb * 64];
-#pragma unroll
-              for (int n = 0; n < kDvPerWave; ++n) {
-                u32x2 packed;
-                packed.x = PackBf16(o[hb][n][0] * inv, o[hb][n][1] * inv);
-                packed.y = PackBf16(o[hb][n][2] * inv, o[hb][n][3] * inv);
-                *reinterpret_cast<u32x2*>(stage + (16 * hb + i16) * kStageRow + (16 * n + 4 * g) * 2) = packed;
-              }
-            }
-            // Same wave wrote and reads: the LDS queue is in order, no barrier needed.
-            const int piece = lane & 15, sub = lane >> 4;
-            if (direct) {
-              char* out0 = a.out + seq * a.out_seq_stride + group_head0 * a.out_head_stride + kSliceBytes * hw + piece * 16;
-#pragma unroll
-              for (int it = 0; it < 16; ++it) {
-                const int h = 4 * it + sub;
-                if (h < 16 * hba) {
-                  const u32x4 v = *reinterpret_cast<const u32x4*>(stage + h * kStageRow + piece * 16);
-                  __builtin_nontemporal_store(v, reinterpret_cast<u32x4*>(out0 + h * a.out_head_stride));
-                }
-              }
-            } else {
-              char* out0 = a.partial_out + PartialRow(a, z, slot, 0) * (kLatentDim * 2) + kSliceBytes * hw + piece * 16;
-#pragma unroll
-              for (int it = 0; it < 16; ++it) {
-                const int h = 4 * it + sub;
-                if (h < 16 * hba) {
-                  const u32x4 v = *reinterpret_cast<const u32x4*>(stage + h * kStageRow + piece * 16);
-                  if (sync_group != nullptr) {
-                    StoreAgent16(out0 + h * (kLatentDim * 2), v);
-                  } else {
-                    __builtin_nontemporal_store(v, reinterpret_cast<u32x4*>(out0 + h * (kLatentDim * 2)));
-                  }
-                }
-              }
-            }
-          }
-        }
-      }
-
-      if (!direct && sync_group != nullptr) {
-        // A merge to take part in once this workgroup's units are done (all its partials are
-        // announced together then: nothing waits in between).
-        if (tid == 0) {
-          const int first_unit = seq_begin / tiles_per_unit;
-          const int partials = (seq_end - 1) / tiles_per_unit - first_unit + 1;
-          duty_lds[duties] = i32x4{seq, first_unit, partials, unit - first_unit};
-        }
-        ++duties;
-        if (duties == kMaxDuties) flush_duties();
-      }
-
+      // Sequence `seq` holds positions [seq_begin - pad, seq_end) of the flat axis, its tiles the
+      // last Tiles(seq) of them; the unit's part of those tiles is the segment.
+      const int seq_end = win.End(seq, pad), seq_begin = seq_end - win.Tiles(seq);
+      const int segment_begin = max(flat, seq_begin), segment_end = min(flat_end, seq_end);
       flat = segment_end;
+      if (segment_begin >= segment_end) {
+        flat = min(flat_end, seq_end);  // only idle positions of this sequence fall into the unit
+      } else {
+        const int tile_begin = segment_begin - seq_begin;          // first tile of the segment inside its sequence
+        const int segment_tiles = segment_end - segment_begin;     // >= 1
+        const bool holds_first = tile_begin == 0, holds_last = segment_end == seq_end;
+        const bool direct = holds_first && holds_last;    // the whole sequence: write the final output here
+        const int slot = holds_first ? a.max_units + seq : unit;
+        int seq_len = win.Tok(seq);
+
+        if (!first_segment) __syncthreads();  // the previous segment's staging rows, table entries and P slots are free
+        first_segment = false;
+
+        // Everything that depends on the thread id alone is formed here, per segment, from a copy
+        // of the id that the compiler cannot see through: hoisted out of the segment loop, these
+        // values would stay live through both roles' tile loops, where no register is to spare.
+        int tid = tid0;
+        asm volatile("" : "+v"(tid));
+        const int lane = tid & 63, wave = Uniform(tid >> 6);
+        const bool score_wave = wave < kScoreWaves;   // wave-uniform role
+        const int hw = wave & (kScoreWaves - 1);      // which 16 heads of the 64
+        const int g = lane >> 4, i16 = lane & 15;
+        const int head_base = z * 64 + hw * 16;
+        const bool active = head_base < a.heads;  // wave-uniform
+        const int head = head_base + i16;
+        const int per_tile = FP8 ? LoadsPerTile8(wave) : LoadsPerTile(wave);
+        // Direct loads: lane L of a latent row fetches chunk L ^ swizzle(row); rows of this wave.
+        IssueLane il;
+        IssueLane8 il8;
+        if (FP8) {
+      #pragma unroll
+          for (int j = 0; j < 2; ++j) {
+            const int row = 2 * wave + 16 * j + (lane >> 5);
+            il8.lat[j] = (lane >> 5) * static_cast<int>(a.latent.row_stride) + (((lane & 31) ^ SwizzleLat8(row)) << 4);
+          }
+          const int rope_row = 16 * (wave & 1) + (lane >> 2);
+          il8.rope = (lane >> 2) * static_cast<int>(a.rope.row_stride) + (((lane & 3) ^ SwizzleRope8(rope_row)) << 4);
+        } else {
+      #pragma unroll
+          for (int j = 0; j < 2; ++j) {
+            il.lat[j] = (lane ^ SwizzleLat(wave + kWaves * j)) << 4;
+            il.partner_lat[j] = (lane ^ SwizzleLat((wave & (kScoreWaves - 1)) + kWaves * j)) << 4;
+          }
+          il.rope_chunk = ((lane & 7) ^ SwizzleRope(8 * (wave - kScoreWaves) + (lane >> 3))) << 4;
+          il.rope = (lane >> 3) * static_cast<int>(a.rope.row_stride) + il.rope_chunk;
+        }
+
+        unsigned char* p_lds = lds + G::kPOff + (hw * 64 + lane) * 16;           // + parity * kScoreWaves * 64 * 16
+        float* alpha_lds = reinterpret_cast<float*>(lds + G::kAlphaOff) + hw * 64 + lane;  // + parity * kScoreWaves * 64
+        float* inv_lds = reinterpret_cast<float*>(lds + G::kInvOff) + hw * 64 + lane;
+        int* flag_lds = reinterpret_cast<int*>(lds + G::kFlagOff) + hw;          // + parity * kScoreWaves
+
+        // Stage this segment's block-table entries in LDS.
+        TileMap<ALIGNED> map;
+        map.entries = table_lds;
+        map.block_size = a.block_size;
+        map.sparse = SPARSE;
+        map.first_pos = tile_begin * kTileTokens;
+        map.first_block = 0;
+        map.next_entry = 0;
+        map.next_slot0 = 0;
+        map.tile_block = 0;
+        map.tile_slot0 = 0;
+        int staged[kTableEntries / 64];  // kSoloPrologue: this lane's table entries on their way to LDS
+        int staged_count = 0;
+        const auto write_table = [&]() __attribute__((always_inline)) {
+          if constexpr (kSoloPrologue) {
+  #pragma unroll
+            for (int j = 0; j < kTableEntries / 64; ++j) {
+              const int i = lane + 64 * j;
+              if (i < staged_count) table_lds[i] = static_cast<unsigned>(staged[j]) < static_cast<unsigned>(a.num_blocks) ? staged[j] : -1;
+            }
+          }
+        };
+        if constexpr (!SPARSE) {
+          const int first_pos = tile_begin * kTileTokens;
+          const int last_pos = first_pos + segment_tiles * kTileTokens - 1;
+          map.first_block = first_pos / a.block_size;
+          map.next_slot0 = first_pos - map.first_block * a.block_size;
+          int count = last_pos / a.block_size - map.first_block + 1;  // <= kTableEntries, ensured by the plan's cap
+          count = min(count, a.table_stride - map.first_block);
+          const int32_t* table_row = a.block_table + static_cast<int64_t>(seq) * a.table_stride + map.first_block;
+          if constexpr (kSoloPrologue) {
+            // Every wave stages all entries itself (the same values to the same addresses), so that it
+            // can read them back without waiting for the other waves. Here they are only asked for;
+            // each role writes them to LDS where it first needs them (write_table below).
+            staged_count = count;
+  #pragma unroll
+            for (int j = 0; j < kTableEntries / 64; ++j) {
+              const int i = lane + 64 * j;
+              staged[j] = i < count ? table_row[i] : -1;
+            }
+          } else {
+            for (int i = tid; i < count; i += kThreads) {
+              const int entry = table_row[i];
+              table_lds[i] = static_cast<unsigned>(entry) < static_cast<unsigned>(a.num_blocks) ? entry : -1;
+            }
+          }
+        } else {
+          // The selection ends at its first entry that is negative or not inside the context. Then
+          // this segment's part of it is resolved to pool slots through the block table.
+          const int context = static_cast<int>(
+              min(static_cast<int64_t>(max(Uniform(a.seq_lens[seq]), 0)), static_cast<int64_t>(a.table_stride) * a.block_size));
+          const int32_t* selection = a.sparse_indices + static_cast<int64_t>(seq) * a.sparse_seq_stride;
+          if (tid == 0) scalar_lds[0] = a.sparse_count;
+          __syncthreads();
+          for (int i = tid; i < a.sparse_count; i += kThreads) {
+            const int index = selection[i];
+            if (index < 0 || index >= context) atomicMin(scalar_lds, i);
+          }
+          __syncthreads();
+          seq_len = Uniform(scalar_lds[0]);
+          const int32_t* table_row = a.block_table + static_cast<int64_t>(seq) * a.table_stride;
+          const int segment_tokens = min(segment_tiles * kTileTokens, seq_len - map.first_pos);  // <= kTableEntries, ensured by the plan's cap
+          for (int i = tid; i < segment_tokens; i += kThreads) {
+            const int index = selection[map.first_pos + i];  // inside [0, context): before the end of the selection
+            const int logical = index / a.block_size;
+            const int entry = table_row[logical];
+            table_lds[i] = static_cast<unsigned>(entry) < static_cast<unsigned>(a.num_blocks)
+                               ? entry * a.block_size + (index - logical * a.block_size)
+                               : -1;
+          }
+        }
+        map.seq_len = seq_len;
+        const int num_tiles = (seq_len + kTileTokens - 1) / kTileTokens;
+        // tiles of this segment that exist (a selection may end before the list does)
+        const int ntiles = min(segment_tiles, num_tiles - tile_begin);
+        if (SPARSE && ntiles <= 0) {
+          if (direct) {
+            ZeroFill<MXQ>(a, z, seq, wave, lane);
+          } else if (active && score_wave && g == 0) {  // empty partial: the merge reads every partial's LSE
+            StoreAgentF32(a.partial_lse + PartialRow(a, z, slot, hw * 16 + i16), -__builtin_inff());
+          }
+        } else {
+          const auto issue = [&](int t) __attribute__((always_inline)) {
+            if constexpr (FP8) {
+              return IssueTileFp8(a, map, il8, tile_begin + t, lds_base + ring(t), lds + ring(t), tid);
+            } else {
+              return IssueTileBf16(a, map, il, tile_begin + t, lds_base + ring(t), lds + ring(t), tid);
+            }
+          };
+          // Prologue (each role runs its own copy, below): tiles 0 .. kRing-2 on their way, tile 0
+          // landed and published. A tile whose load count is not known (rare path) makes every wait
+          // up to and including its own a full one.
+          int last_unknown = -1;  // newest tile issued with an unknown number of loads
+          int issued = 0;         // tiles issued so far
+          // Loads this wave has in flight that are newer than those of tile t: the first `solo_tiles`
+          // tiles carry `solo_loads` each, the later ones `per_tile`.
+          const int solo_tiles = kSoloPrologue ? min(G::kRing - 1, ntiles) : 0;
+          const int solo_loads = score_wave ? 0 : per_tile + kRowsPerWave;
+          const auto newer_than = [&](int t) __attribute__((always_inline)) {
+            const int solo = max(0, min(issued, solo_tiles) - (t + 1));
+            const int shared = max(0, issued - max(t + 1, solo_tiles));
+            return solo * solo_loads + shared * per_tile;
+          };
+          // Top of iteration i, both roles: tile i+1 must have landed (later tiles may still be in
+          // flight); the barrier publishes it together with P(i) and retires every wave's reads of
+          // tile i-1, whose ring slot the next tile to be issued reuses.
+          const auto publish = [&](int i) __attribute__((always_inline)) {
+            if (i + 1 < ntiles) WaitLoads(last_unknown >= i + 1 ? 0 : newer_than(i + 1));
+            __syncthreads();
+          };
+          // Issues the next tile of the ring (tile i + kRing - 1 during iteration i).
+          const auto issue_next = [&](int i) __attribute__((always_inline)) {
+            if (issued < ntiles) {
+              if (!issue(issued)) last_unknown = issued;
+              ++issued;
+            }
+          };
+
+          if (score_wave) {
+            // ---------------------------------------------------------------- score waves
+            // Vector memory requests of a CU are served in order: the query (72 KB per workgroup) is
+            // asked for behind the few bytes of table entries that the first tile addresses depend on.
+            // It lives in this role's branch only; the output waves' prologue has no room for it.
+            bf16x8 q[kKSteps];
+            if (active) {
+              const char* q_latent = a.q_latent + seq * a.q_latent_seq_stride + head * a.q_latent_head_stride;
+              const char* q_rope = a.q_rope + seq * a.q_rope_seq_stride + head * a.q_rope_head_stride;
+  #pragma unroll
+              for (int ks = 0; ks < kKSteps; ++ks) {
+                const int d0 = FP8 ? 64 * (ks >> 1) + 16 * g + 8 * (ks & 1) : 32 * ks + 8 * g;
+                const char* p = d0 < kLatentDim ? q_latent + d0 * 2 : q_rope + (d0 - kLatentDim) * 2;
+                q[ks] = __builtin_bit_cast(bf16x8, GlobalLoad16(p));
+              }
+            } else {
+  #pragma unroll
+              for (int ks = 0; ks < kKSteps; ++ks) q[ks] = __builtin_bit_cast(bf16x8, u32x4{0u, 0u, 0u, 0u});
+            }
+            write_table();  // asked for before the query, so it is here first
+            // The query must have arrived before this wave issues tile loads: the compiler's own wait
+            // for it would otherwise also wait for every tile load issued in between. Both paths above
+            // pass through the statement: were it skipped on one, the compiler would have to assume the
+            // query still in flight where they meet again, and would wait for it -- with counts that
+            // know nothing of the tile loads, so in effect for every tile in flight -- inside the
+            // score loop, at every use.
+  #pragma unroll
+            for (int ks = 0; ks < kKSteps; ++ks) asm volatile("" ::"v"(q[ks]));
+            if constexpr (!kSoloPrologue) __syncthreads();  // table entries visible
+            for (; issued < G::kRing - 1 && issued < ntiles; ++issued) {
+              if constexpr (kSoloPrologue) {
+                map.Begin(issued);  // keeps the cursor in step with the tiles this wave does not issue
+              } else {
+                if (!issue(issued)) last_unknown = issued;
+              }
+            }
+            WaitLoads(last_unknown >= 0 ? 0 : newer_than(0));
+            __syncthreads();
+
+            // bf16 K reads: token = 16t + i16, chunk = 4 ks + g (latent, ks < 16) or 4 (ks - 16) + g (rope).
+            const int k_lat = i16 * Geom<false>::kLatRow, k_rope = Geom<false>::kLatRegion + i16 * Geom<false>::kRopeRow;
+            int k_e[4], kr_e[2];
+  #pragma unroll
+            for (int j = 0; j < 4; ++j) k_e[j] = ((4 * j + g) ^ SwizzleLat(i16)) << 4;
+  #pragma unroll
+            for (int j = 0; j < 2; ++j) kr_e[j] = ((4 * j + g) ^ SwizzleRope(i16)) << 4;
+            // K fragment of pipeline step `step` (k-step step/2, token subtile step&1) of the tile at `buf`.
+            const auto k_frag = [&](const unsigned char* buf, int step) __attribute__((always_inline)) {
+              const int ks = step >> 1, t = step & 1;
+              const int offset = ks < 16 ? k_lat + (ks >> 2) * 256 + k_e[ks & 3] + t * 16 * Geom<false>::kLatRow
+                                         : k_rope + kr_e[ks & 1] + t * 16 * Geom<false>::kRopeRow;
+              return *reinterpret_cast<const bf16x8*>(buf + offset);
+            };
+            // FP8 K reads: read u = 2 kp + t fetches the 16 codes k = 64 kp + 16 g .. +15 of token 16t + i16
+            // (k-steps 2kp and 2kp+1): chunk (4 kp + g) ^ swizzle(token) of the 512-byte row; kp = 8 is the
+            // rope row (chunk g ^ swizzle). The tile base is a multiple of 512, so the XOR with kp << 6 is
+            // applied to the lane-constant part.
+            int k8_lat[2];
+  #pragma unroll
+            for (int t = 0; t < 2; ++t) k8_lat[t] = (16 * t + i16) * Geom<true>::kLatRow + ((g ^ SwizzleLat8(16 * t + i16)) << 4);
+            const int k8_rope = Geom<true>::kLatRegion + i16 * Geom<true>::kRopeRow + ((g ^ SwizzleRope8(i16)) << 4);
+            const auto k8_read = [&](const unsigned char* buf, int u) __attribute__((always_inline)) {
+              const int kp = u >> 1, t = u & 1;
+              const int offset = kp < 8 ? (k8_lat[t] ^ (kp << 6)) : k8_rope + t * 16 * Geom<true>::kRopeRow;
+              return *reinterpret_cast<const u32x4*>(buf + offset);
+            };
+
+            float m_ref = -__builtin_inff();  // reference maximum of the exponentials, log2 domain
+            float l_run = 0.0f;               // this lane's share of the running denominator
+
+            // S^T of tile `tile_rel`, its softmax against the running reference, P and the rescale
+            // request into the LDS slots of the tile's parity.
+            const auto score_tile = [&](int tile_rel, int issue_iteration) __attribute__((always_inline)) {
+              const unsigned char* buf = lds + ring(tile_rel);
+              f32x4 acc[4];
+  #pragma unroll
+              for (int j = 0; j < 4; ++j) acc[j] = f32x4{0.f, 0.f, 0.f, 0.f};
+              f32x4 row_scale[2];  // FP8: scales of tokens 4g+j and 16+4g+j
+              if constexpr (FP8) {
+                const float* scales = reinterpret_cast<const float*>(buf + G::kScaleOff);
+                row_scale[0] = *reinterpret_cast<const f32x4*>(scales + 4 * g);
+                row_scale[1] = *reinterpret_cast<const f32x4*>(scales + 16 + 4 * g);
+                u32x4 kr[kKAhead8];
+  #pragma unroll
+                for (int d = 0; d < kKAhead8; ++d) kr[d] = k8_read(buf, d);
+                __builtin_amdgcn_sched_barrier(0);
+                StaticFor<kKSteps>([&](auto u_c) __attribute__((always_inline)) {
+                  constexpr int u = decltype(u_c)::value;  // kp = u / 2, token subtile t = u & 1
+                  const u32x4 codes = kr[u % kKAhead8];
+                  if constexpr (u + kKAhead8 < kKSteps) kr[u % kKAhead8] = k8_read(buf, u + kKAhead8);
+                  constexpr int t = u & 1, kp = u >> 1;
+                  acc[2 * t] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(CodesToBf16(codes.x, codes.y), q[2 * kp], acc[2 * t], 0, 0, 0);
+                  acc[2 * t + 1] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(CodesToBf16(codes.z, codes.w), q[2 * kp + 1], acc[2 * t + 1], 0, 0, 0);
+                  __builtin_amdgcn_sched_barrier(0);
+                });
+              } else {
+                bf16x8 kf[kKAhead];
+  #pragma unroll
+                for (int d = 0; d < kKAhead; ++d) kf[d] = k_frag(buf, d);
+                __builtin_amdgcn_sched_barrier(0);
+                StaticFor<kQkSteps>([&](auto step_c) __attribute__((always_inline)) {
+                  constexpr int step = decltype(step_c)::value;
+                  constexpr int slot_acc = (step & 1) * 2 + ((step >> 1) & 1);  // two accumulators per token subtile
+                  acc[slot_acc] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(kf[step % kKAhead], q[step >> 1], acc[slot_acc], 0, 0, 0);
+                  if constexpr (step + kKAhead < kQkSteps) kf[step % kKAhead] = k_frag(buf, step + kKAhead);
+                  __builtin_amdgcn_sched_barrier(0);
+                });
+              }
+              // the score waves ask for their rows of the next ring tile behind the QK phase
+              if (kLateIssue && issue_iteration >= 0) issue_next(issue_iteration);
+              // lane holds tokens 4g+j (x[0..3]) and 16+4g+j (x[4..7]) of head i16
+              float x[8];
+  #pragma unroll
+              for (int j = 0; j < 4; ++j) {
+                x[j] = (acc[0][j] + acc[1][j]) * a.scale_log2;
+                x[4 + j] = (acc[2][j] + acc[3][j]) * a.scale_log2;
+                if constexpr (FP8) {  // the codes were multiplied unscaled
+                  x[j] *= row_scale[0][j];
+                  x[4 + j] *= row_scale[1][j];
+                }
+              }
+              const int valid = seq_len - (tile_begin + tile_rel) * kTileTokens;  // >= 1
+              if (valid < kTileTokens) {  // wave-uniform: only the last tile of a sequence
+  #pragma unroll
+                for (int j = 0; j < 8; ++j) {
+                  if (16 * (j >> 2) + 4 * g + (j & 3) >= valid) x[j] = -__builtin_inff();
+                }
+              }
+              float tile_max = fmaxf(fmaxf(fmaxf(x[0], x[1]), fmaxf(x[2], x[3])), fmaxf(fmaxf(x[4], x[5]), fmaxf(x[6], x[7])));
+              tile_max = MaxAcrossHalves(MaxAcrossRows16(tile_max));
+              const int parity = tile_rel & 1;
+              // Move the reference only when some head's maximum outgrew it by more than the threshold.
+              const bool moved = __builtin_amdgcn_ballot_w64(tile_max > m_ref + kRescaleThreshold) != 0;
+              if (moved) {
+                const float m_new = fmaxf(m_ref, tile_max);  // finite: token 0 of the tile is valid
+                const float alpha = __builtin_amdgcn_exp2f(m_ref - m_new);
+                l_run *= alpha;
+                m_ref = m_new;
+                alpha_lds[parity * kScoreWaves * 64] = alpha;
+              }
+              if (lane == 0) flag_lds[parity * kScoreWaves] = moved && tile_rel != 0 ? 1 : 0;  // O is still zero on the first tile
+              bf16x8 p;
+              float sum = 0.0f;
+  #pragma unroll
+              for (int j = 0; j < 8; ++j) {
+                const float e = __builtin_amdgcn_exp2f(x[j] - m_ref);
+                sum += e;
+                p[j] = static_cast<__bf16>(FP8 ? e * row_scale[j >> 2][j & 3] : e);  // FP8: V is multiplied unscaled as well
+              }
+              l_run += sum;
+              *reinterpret_cast<bf16x8*>(p_lds + parity * kScoreWaves * 64 * 16) = p;
+            };
+
+            if (active) score_tile(0, -1);
+            for (int i = 0; i < ntiles; ++i) {
+              publish(i);
+              const bool scores = active && i + 1 < ntiles;
+              if (!kLateIssue || !scores) issue_next(i);
+              if (scores) score_tile(i + 1, i);
+            }
+            if (active) {
+              const float l_total = SumAcrossHeadLanes(l_run);
+              *inv_lds = 1.0f / l_total;
+              const float lse2 = m_ref + __builtin_amdgcn_logf(l_total);  // v_log_f32 is log2
+              if (g == 0) {
+                if (direct) {
+                  if (a.lse != nullptr) a.lse[seq * a.heads + head] = lse2 * 0.6931471805599453f;
+                } else {
+                  StoreAgentF32(a.partial_lse + PartialRow(a, z, slot, hw * 16 + i16), lse2);
+                }
+              }
+            }
+            __syncthreads();  // 1/denominator visible to the output waves
+          } else {
+            // ---------------------------------------------------------------- output waves
+            write_table();
+            if constexpr (!kSoloPrologue) __syncthreads();  // table entries visible
+            for (; issued < G::kRing - 1 && issued < ntiles; ++issued) {
+              if constexpr (kSoloPrologue) {
+                // bf16 tiles: these waves have no query to wait for and issue the first tiles of the ring
+                // alone, their own rows and those of their partner score waves
+                if (!IssueTileBf16<ALIGNED, true>(a, map, il, tile_begin + issued, lds_base + ring(issued), lds + ring(issued), tid)) {
+                  last_unknown = issued;
+                }
+              } else {
+                if (!issue(issued)) last_unknown = issued;
+              }
+            }
+            WaitLoads(last_unknown >= 0 ? 0 : newer_than(0));
+            __syncthreads();
+
+            // bf16 V reads: token = (16 +) 4g + i16/4, chunk = 2n + (i16 & 3) / 2, 8-byte half i16 & 1.
+            const int v_row = 4 * g + (i16 >> 2);
+            const int v_lane = v_row * Geom<false>::kLatRow + (i16 & 1) * 8;
+            int v_e[8];
+  #pragma unroll
+            for (int j = 0; j < 8; ++j) v_e[j] = ((2 * j + ((i16 & 3) >> 1)) ^ SwizzleLat(v_row)) << 4;
+            // FP8 V reads (ds_read_b64_tr_b8: output lane i of a 16-lane group, element e <- byte i & 7 of
+            // the 8 bytes addressed by lane 2e + (i >> 3)): as a source, lane j addresses bytes
+            // 16n + 8 (j & 1) .. +7 of the row of token kappa = j >> 1 (tokens 4g + kappa, 16 + 4g + kappa - 4).
+            const int v8_token = 4 * g + ((i16 >> 1) & 3) + 16 * (i16 >> 3);
+            const int v8_base = v8_token * Geom<true>::kLatRow + (SwizzleLat8(v8_token) << 4) + 8 * (i16 & 1);
+            // Raw V^T fragment of output tile n (dv 16n..16n+15) over the 32 tokens of the tile at `buf`:
+            // eight bf16 for bf16 tiles, eight codes in the low two dwords for FP8 tiles.
+            const auto v_fetch = [&](const unsigned char* buf, int n) __attribute__((always_inline)) {
+              if constexpr (FP8) {
+                const i32x2 codes = __builtin_amdgcn_ds_read_tr8_b64_v2i32((__attribute__((address_space(3))) i32x2*)(buf + (v8_base ^ (n << 4))));
+                return u32x4{static_cast<unsigned>(codes.x), static_cast<unsigned>(codes.y), 0u, 0u};
+              } else {
+                const unsigned char* addr = buf + v_lane + (n >> 3) * 256 + v_e[n & 7];
+                const s16x4 lo = __builtin_amdgcn_ds_read_tr16_b64_v4i16((__attribute__((address_space(3))) s16x4*)(addr));
+                const s16x4 hi = __builtin_amdgcn_ds_read_tr16_b64_v4i16((__attribute__((address_space(3))) s16x4*)(addr + 16 * Geom<false>::kLatRow));
+                return __builtin_bit_cast(u32x4, __builtin_shufflevector(lo, hi, 0, 1, 2, 3, 4, 5, 6, 7));
+              }
+            };
+            const auto v_operand = [&](const u32x4& raw) __attribute__((always_inline)) {
+              if constexpr (FP8) {
+                return CodesToBf16(raw.x, raw.y);
+              } else {
+                return __builtin_bit_cast(bf16x8, raw);
+              }
+            };
+
+            // Output wave w owns the 128 output columns [128 w, 128 w + 128) of all 64 heads of the group:
+            // every V^T fragment is then fetched (and, for FP8, converted) by one wave only, and meets the
+            // P fragments of the four score waves. Head blocks past the group's heads are computed on
+            // whatever their LDS slots hold and never written.
+            constexpr int kDvPerWave = kDvTiles / (kWaves - kScoreWaves);
+            const unsigned char* p_all = lds + G::kPOff + lane * 16;                                   // + (parity * 4 + hb) * 64 * 16
+            const float* alpha_all = reinterpret_cast<const float*>(lds + G::kAlphaOff) + lane;      // + (parity * 4 + hb) * 64
+            const float* inv_all = reinterpret_cast<const float*>(lds + G::kInvOff) + lane;          // + hb * 64
+            const int* flag_all = reinterpret_cast<const int*>(lds + G::kFlagOff);                   // [parity * 4 + hb]
+            f32x4 o[kScoreWaves][kDvPerWave];
+  #pragma unroll
+            for (int hb = 0; hb < kScoreWaves; ++hb) {
+  #pragma unroll
+              for (int n = 0; n < kDvPerWave; ++n) o[hb][n] = f32x4{0.f, 0.f, 0.f, 0.f};
+            }
+
+            for (int i = 0; i < ntiles; ++i) {
+              publish(i);
+              issue_next(i);
+              {
+                const unsigned char* buf = lds + ring(i);
+                const int parity = i & 1;
+                // the four rescale flags of the tile in one read; a moved reference maximum is the exception
+                const i32x4 flags = *reinterpret_cast<const i32x4*>(flag_all + parity * kScoreWaves);
+                if (Uniform(flags.x | flags.y | flags.z | flags.w) != 0) {
+                  const int moved[kScoreWaves] = {flags.x, flags.y, flags.z, flags.w};
+  #pragma unroll
+                  for (int hb = 0; hb < kScoreWaves; ++hb) {
+                    if (Uniform(moved[hb]) != 0) {  // that block's reference maximum moved: rescale its O first
+                      const float alpha = alpha_all[(parity * kScoreWaves + hb) * 64];
+  #pragma unroll
+                      for (int n = 0; n < kDvPerWave; ++n) o[hb][n] *= alpha;
+                    }
+                  }
+                }
+                u32x4 vf[kVAhead];
+  #pragma unroll
+                for (int d = 0; d < kVAhead; ++d) vf[d] = v_fetch(buf, kDvPerWave * hw + d);
+                bf16x8 p[kScoreWaves];
+  #pragma unroll
+                for (int hb = 0; hb < kScoreWaves; ++hb) p[hb] = *reinterpret_cast<const bf16x8*>(p_all + (parity * kScoreWaves + hb) * 64 * 16);
+                __builtin_amdgcn_sched_barrier(0);
+                if constexpr (FP8) {
+                  // the next fragment is converted while this one's four MFMAs run
+                  bf16x8 v = v_operand(vf[0]);
+                  if constexpr (kVAhead < kDvPerWave) vf[0] = v_fetch(buf, kDvPerWave * hw + kVAhead);
+                  StaticFor<kDvPerWave>([&](auto n_c) __attribute__((always_inline)) {
+                    constexpr int n = decltype(n_c)::value;
+                    bf16x8 v_next = v;
+                    if constexpr (n + 1 < kDvPerWave) v_next = v_operand(vf[(n + 1) % kVAhead]);
+  #pragma unroll
+                    for (int hb = 0; hb < kScoreWaves; ++hb) o[hb][n] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(v, p[hb], o[hb][n], 0, 0, 0);
+                    if constexpr (n + 1 + kVAhead < kDvPerWave) vf[(n + 1) % kVAhead] = v_fetch(buf, kDvPerWave * hw + n + 1 + kVAhead);
+                    v = v_next;
+                    __builtin_amdgcn_sched_barrier(0);
+                  });
+                } else {
+                  StaticFor<kDvPerWave>([&](auto n_c) __attribute__((always_inline)) {
+                    constexpr int n = decltype(n_c)::value;
+                    const bf16x8 v = v_operand(vf[n % kVAhead]);
+  #pragma unroll
+                    for (int hb = 0; hb < kScoreWaves; ++hb) o[hb][n] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(v, p[hb], o[hb][n], 0, 0, 0);
+                    if constexpr (n + kVAhead < kDvPerWave) vf[n % kVAhead] = v_fetch(buf, kDvPerWave * hw + n + kVAhead);
+                    __builtin_amdgcn_sched_barrier(0);
+                  });
+                }
+              }
+            }
+            __syncthreads();  // 1/denominator from the score waves
+            if (MXQ && direct) {
+              // Quantising epilogue of a whole sequence: a block of 32 columns is a pair of this
+              // wave's column tiles over the four lanes that share a head; the wave covers blocks
+              // 4 w .. 4 w + 3 of every head.
+  #pragma unroll
+              for (int hb = 0; hb < kScoreWaves; ++hb) {
+                if (hb >= hba) continue;
+                const int h = 16 * hb + i16;
+                const float inv = inv_all[hb * 64];
+                char* codes_row = a.out_codes + seq * a.out_codes_seq_stride + (group_head0 + h) * a.out_codes_head_stride;
+                char* out_row = a.out == nullptr ? nullptr : a.out + seq * a.out_seq_stride + (group_head0 + h) * a.out_head_stride;
+                unsigned scale_codes = 0u;
+  #pragma unroll
+                for (int k = 0; k < kDvPerWave / 2; ++k) {
+                  u32x2 packed[2];
+                  unsigned magnitude = 0u;
+  #pragma unroll
+                  for (int half = 0; half < 2; ++half) {
+                    const int n = 2 * k + half;
+                    packed[half].x = PackBf16(o[hb][n][0] * inv, o[hb][n][1] * inv);
+                    packed[half].y = PackBf16(o[hb][n][2] * inv, o[hb][n][3] * inv);
+                    magnitude = MxMagnitudeMax(packed[half].y, MxMagnitudeMax(packed[half].x, magnitude));
+                    if (out_row != nullptr) {
+                      __builtin_nontemporal_store(packed[half], reinterpret_cast<u32x2*>(out_row + (16 * (kDvPerWave * hw + n) + 4 * g) * 2));
+                    }
+                  }
+                  magnitude = UMaxAcrossHeadLanes(magnitude);
+                  const MxScale s = MxScaleFromMaxBits(magnitude);
+  #pragma unroll
+                  for (int half = 0; half < 2; ++half) {
+                    const unsigned four = MxEncodeWord(packed[half].x, s) | (MxEncodeWord(packed[half].y, s) << 16);
+                    __builtin_nontemporal_store(four, reinterpret_cast<unsigned*>(codes_row + 16 * (kDvPerWave * hw + 2 * k + half) + 4 * g));
+                  }
+                  scale_codes |= s.code << (8 * k);
+                }
+                if (g == 0) {
+                  *reinterpret_cast<unsigned*>(a.out_scales + seq * a.out_scales_seq_stride + (group_head0 + h) * a.out_scales_head_stride +
+                                               (kDvPerWave / 2) * hw) = scale_codes;
+                }
+              }
+            } else {
+              // The accumulators hold O^T (lane = head i16 of a block, four columns per 16-column tile),
+              // which stored as it is would write 8-byte pieces of sixteen different rows per
+              // instruction. The tile ring is dead after the last barrier: each output wave transposes
+              // its 256-byte slices of the 64 rows through its own part of it and writes them 16 bytes per
+              // lane, four whole slices per instruction. A row stride of 272 bytes (= 4 banks mod 64)
+              // spreads the 8-byte writes of a half-wave over all banks.
+              constexpr int kSliceBytes = kDvPerWave * 16 * 2;  // 256
+              constexpr int kStageRow = kSliceBytes + 16;
+              static_assert((kWaves - kScoreWaves) * 64 * kStageRow <= G::kRing * G::kTileBytes, "the staging rows fit in the ring");
+              unsigned char* stage = lds + G::Slot(0) + hw * (64 * kStageRow);
+  #pragma unroll
+              for (int hb = 0; hb < kScoreWaves; ++hb) {
+                const float inv = inv_all[hb * 64];
+  #pragma unroll
+                for (int n = 0; n < kDvPerWave; ++n) {
+                  u32x2 packed;
+                  packed.x = PackBf16(o[hb][n][0] * inv, o[hb][n][1] * inv);
+                  packed.y = PackBf16(o[hb][n][2] * inv, o[hb][n][3] * inv);
+                  *reinterpret_cast<u32x2*>(stage + (16 * hb + i16) * kStageRow + (16 * n + 4 * g) * 2) = packed;
+                }
+              }
+              // Same wave wrote and reads: the LDS queue is in order, no barrier needed.
+              const int piece = lane & 15, sub = lane >> 4;
+              if (direct) {
+                char* out0 = a.out + seq * a.out_seq_stride + group_head0 * a.out_head_stride + kSliceBytes * hw + piece * 16;
+  #pragma unroll
+                for (int it = 0; it < 16; ++it) {
+                  const int h = 4 * it + sub;
+                  if (h < 16 * hba) {
+                    const u32x4 v = *reinterpret_cast<const u32x4*>(stage + h * kStageRow + piece * 16);
+                    __builtin_nontemporal_store(v, reinterpret_cast<u32x4*>(out0 + h * a.out_head_stride));
+                  }
+                }
+              } else {
+                char* out0 = a.partial_out + PartialRow(a, z, slot, 0) * (kLatentDim * 2) + kSliceBytes * hw + piece * 16;
+  #pragma unroll
+                for (int it = 0; it < 16; ++it) {
+                  const int h = 4 * it + sub;
+                  if (h < 16 * hba) {
+                    const u32x4 v = *reinterpret_cast<const u32x4*>(stage + h * kStageRow + piece * 16);
+                    if (sync_group != nullptr) {
+                      StoreAgent16(out0 + h * (kLatentDim * 2), v);
+                    } else {
+                      __builtin_nontemporal_store(v, reinterpret_cast<u32x4*>(out0 + h * (kLatentDim * 2)));
+                    }
+                  }
+                }
+              }
+            }
+          }
+        }
+
+        if (!direct && sync_group != nullptr) {
+          // A merge to take part in once this workgroup's units are done (all its partials are
+          // announced together then: nothing waits in between).
+          if (tid == 0) {
+            const int first_unit = seq_begin / tiles_per_unit;
+            const int partials = (seq_end - 1) / tiles_per_unit - first_unit + 1;
+            duty_lds[duties] = i32x4{seq, first_unit, partials, unit - first_unit};
+          }
+          ++duties;
+          if (duties == kMaxDuties) flush_duties();
+        }
+
+      }
       if (flat < flat_end) {  // the next sequence that has tiles
         do {
           ++seq;
-          if (seq >= win.base + 64) win.Load(a, lane0, win.base + 64, win.End());
+          if (seq >= win.base + 64) win.Next(a, lane0);
         } while (win.Tiles(seq) == 0);
       }
     }
@@ -1384,21 +1434,24 @@ __global__ __launch_bounds__(kMergeHeads * 64) void MlaMergeKernel(AttnArgs a) {
   const int h = group * kMergeHeads + wave;
   if (h >= min(64, a.heads - 64 * z)) return;
   SeqWindow<SPARSE> win;
-  win.Load(a, lane, 0, 0);
-  int seq_end = 0, seq_tiles = 0;
+  win.Load(a, lane, 0, 0, 0);
+  int end_tiles = 0, end_live = 0, seq_tiles = 0, common_tiles = 0;
   for (;;) {
     if (seq >= win.base && seq < win.base + 64) {
-      seq_end = win.Incl(seq);
+      end_tiles = win.End(seq, 0);
+      end_live = win.End(seq, 1) - end_tiles;
       seq_tiles = win.Tiles(seq);
     }
+    const int here = win.CommonTiles();
+    if (here != 0) common_tiles = common_tiles == 0 || common_tiles == here ? here : -1;
     if (win.base + 64 >= a.batch) break;
-    win.Load(a, lane, win.base + 64, win.End());
+    win.Next(a, lane);
   }
-  const int total_tiles = win.End();
   if (seq_tiles == 0) return;
-  const int tiles_per_unit = TilesPerUnit(a, total_tiles, a.work_groups);
-  const int first_unit = (seq_end - seq_tiles) / tiles_per_unit;
-  const int partials = (seq_end - 1) / tiles_per_unit - first_unit + 1;
+  const Cut cut = MakeCut(a, win.EndTiles(), win.EndLive(), common_tiles, a.work_groups);
+  const int seq_end = end_tiles + cut.pad * end_live;
+  const int first_unit = (seq_end - seq_tiles) / cut.tiles_per_unit;
+  const int partials = (seq_end - 1) / cut.tiles_per_unit - first_unit + 1;
   if (partials == 1) return;  // written by the workgroup that held the whole sequence
   MergeHead<MXQ, false>(a, z, seq, h, a.max_units + seq, first_unit, partials, lane);
 }

@@ -35,6 +35,20 @@ HBM_PEAK_GBPS = 8000.0      # MI355X HBM3E, published
 MFMA_BF16_PEAK_TFLOPS = 2500.0
 LATENT, ROPE, ROW = 512, 64, 576
 ROW_BYTES = ROW * 2
+CONTEXT_SEED = 20251125
+# HBM bytes per algorithmic byte of the attention launches (decode + merge kernel), from the
+# rocprofv3 --pmc runs summarised in profiles/attention_hbm_counters.md (FETCH_SIZE x2.000,
+# WRITE_SIZE x1.000 as for the gather): the excess is the partials of sequences split over
+# several workgroups, written once and read once.
+ATTENTION_TRAFFIC = {
+    "attention": {"ratio": None, "source": None},
+    "attention_fp8": {"ratio": None, "source": None},
+    "attention_long": {"ratio": None, "source": None},
+}
+# Host orchestration of the reference's own 43-layer decode step (its mock build: every operator
+# launch is a no-op), measured in the build container on 8 cores: 128 steps, 132,480 launches,
+# 48.9 ms.
+REFERENCE_HOST_PLUMBING_MS_PER_STEP = 0.38
 
 
 def sustained_us(torch, fn, min_iters, warm_ms=250.0, timed_ms=100.0):
@@ -64,6 +78,8 @@ def parse_args():
     p.add_argument("--no-attention", action="store_true")
     p.add_argument("--side-only", action="store_true", help="development aid: time only the FP8 append/gather and compaction kernels")
     p.add_argument("--attention-only", action="store_true", help="development aid: time only the attention configurations")
+    p.add_argument("--config5-only", action="store_true", help="development aid: run only the continuous-batching loop of configs[4]")
+    p.add_argument("--config5-pool-gb", type=float, default=200.0, help="KV pool of the configs[4] loop, in GB (clamped to free memory)")
     p.add_argument("--split-out", action="store_true", help="gather into separate latent/rope planes instead of 576-wide rows")
     return p.parse_args()
 
@@ -116,8 +132,7 @@ def bench_append_gather(args, torch, np, ffi):
     gather_events = []
 
     def step(timed):
-        for s in range(batch):
-            cache.append_token(s)
+        cache.append_token_all()
         cache.upload_step(stream_ptr(torch))
         # events bracket the gather only: every record is a barrier packet in the queue, and a third
         # one in front of the 4-us append cost more than the append itself
@@ -190,42 +205,64 @@ def bench_append_gather(args, torch, np, ffi):
     return result
 
 
-def bench_attention(args, torch, np, ffi, fp8=False, batch=32, ctx=2048, heads=64, slices=8, iters=None, label=None,
-                    mx_quant=False, sparse_k=None):
+def draw_contexts(np, kind, batch, seed):
+    """Context lengths of the attention configurations, from a seeded numpy Generator (PCG64)."""
+    rng = np.random.default_rng(seed)
+    if kind == "uniform_512_8192":      # configs[3]
+        return [int(v) for v in rng.integers(512, 8193, size=batch)]
+    if kind == "lognormal_4096_cap_32768":  # configs[4]: median 4096, sigma 1.0
+        return [int(min(32768, max(1, round(v)))) for v in np.exp(rng.normal(math.log(4096.0), 1.0, size=batch))]
+    raise ValueError(kind)
+
+
+def fill_cache(torch, np, ffi, lib, cache, view, ctxs, layers, bs, seed, outlier_fraction=0.0):
+    """Every live slot of `layers` layer slices gets N(0,1) rows (optionally with outliers x20) through
+    the append kernel (an FP8 cache quantizes on the way), in pieces of at most 128k rows."""
+    table = cache.host_block_table()
+    slots = np.concatenate([table[s, np.arange(n) // bs].astype(np.int64) * bs + np.arange(n) % bs
+                            for s, n in enumerate(ctxs)]).astype(np.int32)
+    slots_dev = torch.as_tensor(slots, device="cuda")
+    gen = torch.Generator(device="cuda").manual_seed(seed)
+    piece = 128 * 1024
+    for layer in range(layers):
+        for start in range(0, len(slots), piece):
+            rows = min(piece, len(slots) - start)
+            x = torch.randn(rows, ROW, generator=gen, device="cuda")
+            if outlier_fraction > 0:
+                x = torch.where(torch.rand(rows, ROW, generator=gen, device="cuda") < outlier_fraction, x * 20.0, x)
+            x = x.to(torch.bfloat16)
+            ffi.check(lib.mlakvAppend(C.byref(view), layer, 1, x.data_ptr(), 0, ROW_BYTES, x.data_ptr() + LATENT * 2, 0, ROW_BYTES,
+                                      slots_dev.data_ptr() + 4 * start, rows, stream_ptr(torch)))
+            torch.cuda.synchronize()
+
+
+def bench_attention(args, torch, np, ffi, ctxs, fp8=False, heads=64, slices=8, iters=None, label=None, distribution=None,
+                    outlier_fraction=0.0, mx_quant=False, sparse_k=None, traffic_ratio=None):
     lib = ffi.load()
     bs = 64
-    slices = int(os.environ.get("MLAKV_BENCH_SLICES", slices))  # development aid: 1 keeps the KV cache-resident
-    blocks_per_seq = -(-ctx // bs)
-    pool_blocks = batch * blocks_per_seq + 8
+    batch = len(ctxs)
+    max_ctx = max(ctxs)
+    blocks = sum(-(-c // bs) for c in ctxs)
+    pool_blocks = blocks + 8
     arena = ffi.Arena(ffi.BACKEND_HIP)
-    cache = ffi.KvCache(arena, num_layers=slices, block_size=bs, max_context_len=ctx, max_batch=batch,
-                        pool_blocks=pool_blocks, seed=7, shuffle=int(os.environ.get("MLAKV_BENCH_SHUFFLE", "1")),
-                        dtype=ffi.DTYPE_FP8_E4M3 if fp8 else ffi.DTYPE_BF16)
+    cache = ffi.KvCache(arena, num_layers=slices, block_size=bs, max_context_len=max_ctx, max_batch=batch,
+                        pool_blocks=pool_blocks, seed=7, shuffle=1, dtype=ffi.DTYPE_FP8_E4M3 if fp8 else ffi.DTYPE_BF16)
     plan = ffi.AttnPlan()
     if sparse_k:
         ffi.check(lib.mlakvAttnSparsePlanInit(batch, heads, sparse_k, bs, cache.config.dtype, C.byref(plan)))
     else:
-        ffi.check(lib.mlakvAttnPlanInit(batch, heads, ctx, bs, cache.config.dtype, C.byref(plan)))
+        ffi.check(lib.mlakvAttnPlanInit(batch, heads, max_ctx, bs, cache.config.dtype, C.byref(plan)))
     arena.note_workspace(int(plan.workspace_bytes))
     arena.commit()
     arena.commit_workspace()
     cache.bind()
     arena.seal()
     view = cache.view()
-    for s in range(batch):
-        cache.add_sequence(s, ctx)
+    for s, n in enumerate(ctxs):
+        cache.add_sequence(s, n)
     cache.upload_step(stream_ptr(torch))
-    table = cache.host_block_table()
-    slots = np.concatenate([table[s, np.arange(ctx) // bs].astype(np.int64) * bs + np.arange(ctx) % bs
-                            for s in range(batch)]).astype(np.int32)
-    slots_dev = torch.as_tensor(slots, device="cuda")
-    gen = torch.Generator(device="cuda").manual_seed(2)
-    for layer in range(slices):
-        lat = torch.randn(batch * ctx, LATENT, generator=gen, device="cuda").to(torch.bfloat16)
-        rop = torch.randn(batch * ctx, ROPE, generator=gen, device="cuda").to(torch.bfloat16)
-        ffi.check(lib.mlakvAppend(C.byref(view), layer, 1, lat.data_ptr(), 0, LATENT * 2, rop.data_ptr(), 0, ROPE * 2,
-                                  slots_dev.data_ptr(), batch * ctx, stream_ptr(torch)))
-        torch.cuda.synchronize()
+    fill_cache(torch, np, ffi, lib, cache, view, ctxs, slices, bs, seed=2, outlier_fraction=outlier_fraction)
+    gen = torch.Generator(device="cuda").manual_seed(3)
     q = torch.randn(slices, batch, heads, ROW, generator=gen, device="cuda").to(torch.bfloat16)
     out = torch.empty(slices, batch, heads, LATENT, dtype=torch.bfloat16, device="cuda")
 
@@ -234,7 +271,7 @@ def bench_attention(args, torch, np, ffi, fp8=False, batch=32, ctx=2048, heads=6
         # every sequence attends to sparse_k distinct random positions of its context (what a
         # top-k selection looks like to the memory system), a fresh draw per layer slice
         rng = np.random.default_rng(5)
-        selection = torch.as_tensor(np.stack([np.stack([rng.permutation(ctx)[:sparse_k] for _ in range(batch)])
+        selection = torch.as_tensor(np.stack([np.stack([rng.permutation(n)[:sparse_k] for n in ctxs])
                                               for _ in range(slices)]).astype(np.int32), device="cuda")
 
     def launch_sparse(i):
@@ -287,18 +324,23 @@ def bench_attention(args, torch, np, ffi, fp8=False, batch=32, ctx=2048, heads=6
 
         mx = {"us_fused_epilogue": timed_us(fused), "us_attention_then_quant": timed_us(unfused)}
     kv_row = 580 if fp8 else ROW_BYTES
-    attended = sparse_k or ctx
-    algorithmic = batch * attended * kv_row + batch * heads * ROW * 2 + batch * heads * LATENT * 2 + 4 * batch * blocks_per_seq
+    attended = batch * sparse_k if sparse_k else sum(ctxs)
+    algorithmic = attended * kv_row + batch * heads * ROW * 2 + batch * heads * LATENT * 2 + 4 * blocks
     if sparse_k:
         algorithmic += 4 * batch * sparse_k
-    flops = 2.0 * batch * heads * attended * (ROW + LATENT)
+    flops = 2.0 * heads * attended * (ROW + LATENT)
+    lengths = (f"ctx {ctxs[0]}" if min(ctxs) == max(ctxs)
+               else f"ctx {distribution} (min {min(ctxs)}, mean {sum(ctxs) / batch:.0f}, max {max(ctxs)})")
     result = {
         "us_per_step": us,
-        "workload": f"{label or ('configs[3]-shape' if fp8 else 'configs[2]-shape')}: 1 layer per launch, batch {batch}, {heads} heads, ctx {ctx}, block 64, "
-                    f"{'fp8 e4m3 + fp32 row scale' if fp8 else 'bf16'} KV, shuffled table, {slices} rotating layer slices"
+        "workload": f"{label}: 1 layer per launch, batch {batch}, {heads} heads, {lengths}, block 64, "
+                    f"{'fp8 e4m3 + fp32 row scale' if fp8 else 'bf16'} KV"
+                    + (", N(0,1) rows with 1% of the elements x20" if outlier_fraction else ", N(0,1) rows")
+                    + f", shuffled table, {slices} rotating layer slices"
                     + (f", {sparse_k} selected tokens per sequence" if sparse_k else ""),
         "roofline": {"bound": "hbm", "achieved": algorithmic / (us * 1e-6) / 1e9, "peak": HBM_PEAK_GBPS, "unit": "GB/s",
-                     "frac": algorithmic / (us * 1e-6) / 1e9 / HBM_PEAK_GBPS, "traffic": None},
+                     "frac": algorithmic / (us * 1e-6) / 1e9 / HBM_PEAK_GBPS,
+                     "traffic": algorithmic * traffic_ratio["ratio"] if traffic_ratio else None},
         "algorithmic_bytes": algorithmic,
         "mfma_tflops": flops / (us * 1e-6) / 1e12,
         "mfma_frac_of_bf16_peak": flops / (us * 1e-6) / 1e12 / MFMA_BF16_PEAK_TFLOPS,
@@ -306,6 +348,11 @@ def bench_attention(args, torch, np, ffi, fp8=False, batch=32, ctx=2048, heads=6
         "merge": "in launch" if plan.merge_mode == ffi.ATTN_MERGE_IN_LAUNCH else "second launch",
         "workspace_bytes": int(plan.workspace_bytes), "timing": "250 ms of back-to-back launches untimed, then at least 100 ms of them timed",
     }
+    if traffic_ratio:
+        result["roofline"]["traffic_source"] = traffic_ratio["source"]
+    if min(ctxs) != max(ctxs):
+        result["context_seed"] = CONTEXT_SEED
+        result["total_tokens"] = sum(ctxs)
     if mx is not None:
         result["mx_quant_output"] = mx
     cache.close()
@@ -458,9 +505,151 @@ def bench_side_kernels(args, torch, np, ffi):
     return out
 
 
+def bench_config5(args, torch, np, ffi, batch=128, heads=64, steps=6, warmup=2):
+    """configs[4]: reservation pressure over all 43 layers. A pool of about 200 GB (clamped to what
+    the device has free), 128 sequences with lognormal contexts, seeded finish times; a finished
+    sequence frees its blocks and a new one (fresh lognormal context) takes its place from the
+    recycled free list; after every step in which something finished the pool is compacted (the
+    copy kernel moves the displaced blocks in all 43 layers). Every step appends one token per
+    sequence and layer and runs the decode attention of all 43 layers."""
+    lib = ffi.load()
+    bs, layers = 64, 43
+    block_bytes = bs * ROW_BYTES
+    free_bytes, _ = torch.cuda.mem_get_info()
+    pool_bytes = min(args.config5_pool_gb * 1e9, free_bytes - 24e9)
+    pool_blocks = int(pool_bytes // (layers * block_bytes))
+    rng = np.random.default_rng(CONTEXT_SEED + 5)
+
+    def draw():
+        return int(min(32768, max(1, round(float(np.exp(rng.normal(math.log(4096.0), 1.0)))))))
+
+    ctxs = [draw() for _ in range(batch)]
+    total_steps = steps + warmup
+    max_ctx = 32768 + total_steps
+    need_blocks = sum(-(-(c + total_steps) // bs) for c in ctxs)
+    if pool_blocks < need_blocks + need_blocks // 4:
+        return {"skipped": f"only {free_bytes / 1e9:.0f} GB free: a pool of {pool_blocks} blocks per layer is too small"}
+    arena = ffi.Arena(ffi.BACKEND_HIP)
+    cache = ffi.KvCache(arena, num_layers=layers, block_size=bs, max_context_len=max_ctx, max_batch=batch,
+                        pool_blocks=pool_blocks, seed=CONTEXT_SEED, shuffle=1)
+    plan = ffi.AttnPlan()
+    ffi.check(lib.mlakvAttnPlanInit(batch, heads, max_ctx, bs, ffi.DTYPE_BF16, C.byref(plan)))
+    arena.note_workspace(int(plan.workspace_bytes))
+    torch.cuda.synchronize()
+    t0 = time.perf_counter()
+    arena.commit()   # one allocation, zero-filled
+    torch.cuda.synchronize()
+    commit_seconds = time.perf_counter() - t0
+    arena.commit_workspace()
+    cache.bind()
+    arena.seal()
+    view = cache.view()
+    # every slot of the pool gets N(0,1) rows, the same rows in every layer (one append call
+    # writes a piece of slots into all 43 layers from one source): recycled blocks then hold data
+    gen = torch.Generator(device="cuda").manual_seed(11)
+    piece = 64 * 1024
+    for start in range(0, pool_blocks * bs, piece):
+        rows = min(piece, pool_blocks * bs - start)
+        x = torch.randn(rows, ROW, generator=gen, device="cuda").to(torch.bfloat16)
+        slots = torch.arange(start, start + rows, dtype=torch.int32, device="cuda")
+        ffi.check(lib.mlakvAppend(C.byref(view), 0, layers, x.data_ptr(), 0, ROW_BYTES, x.data_ptr() + LATENT * 2, 0, ROW_BYTES,
+                                  slots.data_ptr(), rows, stream_ptr(torch)))
+        torch.cuda.synchronize()
+    for s, n in enumerate(ctxs):
+        cache.add_sequence(s, n)
+    remaining = [int(v) for v in rng.integers(1, 2 * total_steps, size=batch)]  # steps until the sequence finishes
+    qslices = 4
+    q = torch.randn(qslices, batch, heads, ROW, generator=gen, device="cuda").to(torch.bfloat16)
+    out = torch.empty(batch, heads, LATENT, dtype=torch.bfloat16, device="cuda")
+    step_latent = torch.randn(layers, batch, LATENT, generator=gen, device="cuda").to(torch.bfloat16)
+    step_rope = torch.randn(layers, batch, ROPE, generator=gen, device="cuda").to(torch.bfloat16)
+    allocations_before = arena.device_allocations
+    records = []
+    for step in range(total_steps):
+        finished = [s for s in range(batch) if remaining[s] == 0]
+        for s in finished:
+            cache.free_sequence(s)
+        for s in finished:
+            cache.add_sequence(s, draw())
+            remaining[s] = int(rng.integers(1, 2 * total_steps))
+        ev = [torch.cuda.Event(enable_timing=True) for _ in range(4)]
+        ev[0].record()
+        moved = len(cache.compact(stream_ptr(torch))) if finished else 0
+        ev[1].record()
+        cache.append_token_all()
+        cache.upload_step(stream_ptr(torch))
+        ffi.check(lib.mlakvAppend(C.byref(view), 0, layers, step_latent.data_ptr(), batch * LATENT * 2, LATENT * 2,
+                                  step_rope.data_ptr(), batch * ROPE * 2, ROPE * 2, cache.device_slot_mapping, batch,
+                                  stream_ptr(torch)))
+        ev[2].record()
+        for layer in range(layers):
+            k = layer % qslices
+            ffi.check(lib.mlakvAttnDecode(C.byref(plan), C.byref(view), layer, q[k].data_ptr(), heads * ROW_BYTES, ROW_BYTES,
+                                          q[k].data_ptr() + LATENT * 2, heads * ROW_BYTES, ROW_BYTES, cache.device_block_table,
+                                          cache.num_blocks, cache.device_seq_lens, 1.0 / math.sqrt(192.0), out.data_ptr(),
+                                          heads * LATENT * 2, LATENT * 2, None, arena.workspace, arena.workspace_bytes,
+                                          stream_ptr(torch)))
+        ev[3].record()
+        torch.cuda.synchronize()
+        lens = [int(v) for v in cache.host_seq_lens()]
+        tokens = sum(lens)
+        attention_bytes = layers * (tokens * ROW_BYTES + batch * heads * (ROW + LATENT) * 2 + 4 * sum(-(-n // bs) for n in lens))
+        records.append({"finished": len(finished), "moved_blocks": moved, "tokens": tokens,
+                        "compaction_ms": ev[0].elapsed_time(ev[1]), "append_ms": ev[1].elapsed_time(ev[2]),
+                        "attention_ms": ev[2].elapsed_time(ev[3]), "step_ms": ev[0].elapsed_time(ev[3]),
+                        "attention_bytes": attention_bytes, "compaction_bytes": 2 * moved * block_bytes * layers,
+                        "append_bytes": layers * batch * (2 * ROW_BYTES + 4)})
+        for s in range(batch):
+            remaining[s] -= 1
+    assert arena.device_allocations == allocations_before, "a step allocated device memory"
+    timed = records[warmup:]
+    step_ms = sum(r["step_ms"] for r in timed) / len(timed)
+    attention_ms = sum(r["attention_ms"] for r in timed) / len(timed)
+    attention_bytes = sum(r["attention_bytes"] for r in timed) / len(timed)
+    all_bytes = sum(r["attention_bytes"] + r["compaction_bytes"] + r["append_bytes"] for r in timed) / len(timed)
+    compactions = [r for r in timed if r["moved_blocks"] > 0]
+    stats = cache.stats()
+    result = {
+        "workload": f"configs[4]: {layers} layers, batch {batch}, ctx lognormal (median 4096, sigma 1.0, cap 32768), block 64, bf16, "
+                    f"pool {pool_blocks} blocks per layer = {pool_blocks * layers * block_bytes / 1e9:.1f} GB, seeded finish times, "
+                    "recycled blocks, compaction after every step that finished a sequence, decode attention of every layer each step",
+        "seed": CONTEXT_SEED + 5, "steps": steps, "warmup": warmup,
+        "ms_per_step": step_ms, "attention_ms_per_step": attention_ms, "attention_us_per_layer": attention_ms * 1e3 / layers,
+        "gbps": all_bytes / (step_ms * 1e-3) / 1e9,
+        "roofline": {"bound": "hbm", "achieved": attention_bytes / (attention_ms * 1e-3) / 1e9, "peak": HBM_PEAK_GBPS, "unit": "GB/s",
+                     "frac": attention_bytes / (attention_ms * 1e-3) / 1e9 / HBM_PEAK_GBPS, "traffic": None,
+                     "what": "the 43 attention launches of a step, algorithmic bytes over HIP-event time"},
+        "mean_tokens": sum(r["tokens"] for r in timed) / len(timed),
+        "finished_sequences": sum(r["finished"] for r in timed),
+        "compaction": {"steps_with_compaction": len(compactions),
+                       "moved_blocks": sum(r["moved_blocks"] for r in compactions),
+                       "bytes": sum(r["compaction_bytes"] for r in compactions),
+                       "ms": sum(r["compaction_ms"] for r in compactions),
+                       "gbps": (sum(r["compaction_bytes"] for r in compactions) / (sum(r["compaction_ms"] for r in compactions) * 1e-3) / 1e9
+                                if compactions else None),
+                       "note": "ms covers the host-side plan, the move-list upload and the copy kernel"},
+        "arena_commit_seconds": commit_seconds, "arena_bytes": arena.total_bytes,
+        "kv_cache_utilization": stats.kv_cache_utilization,
+    }
+    cache.close()
+    arena.close()
+    return result
+
+
+def _threads():
+    """One thread per core this process may use, at most 16 (a one-GPU box's CPU share)."""
+    try:
+        return max(1, min(16, len(os.sched_getaffinity(0))))
+    except AttributeError:
+        return max(1, min(16, os.cpu_count() or 1))
+
+
 def cpu_baseline(np, ag):
-    """The CPU oracle (a port: the reference has no CPU numerics for this path) on one core, on a
-    bounded sample of the same workload: the append+gather step of all 43 layers, 12 times."""
+    """The CPU oracle (a port: the reference has no CPU numerics for this path) on a bounded sample
+    of the same workload: the append+gather step of all 43 layers, on one core and with one thread
+    per core (layers are independent; the C routines run outside the interpreter lock)."""
+    from concurrent.futures import ThreadPoolExecutor
+
     import oracle_ffi as orc
     bs, batch = 64, len(ag["ctxs"])
     sample_layers = 43
@@ -474,39 +663,89 @@ def cpu_baseline(np, ag):
     planes = [plane0.copy() for _ in range(sample_layers)]  # distinct memory per layer, same bytes
     rows = rng.integers(0, 255, size=(sample_layers, batch * ROW_BYTES), dtype=np.uint8)
     slots = np.array([int(table[s, (n - 1) // bs]) * bs + (n - 1) % bs for s, n in enumerate(ctxs)], dtype=np.int32)
-    times = []
-    for rep in range(13):
-        t0 = time.perf_counter()
-        for layer in range(sample_layers):
-            orc.append_rows(planes[layer], bs * ROW_BYTES, ROW_BYTES, bs, rows[layer], ROW_BYTES, ROW_BYTES, slots)
-            orc.gather_rows(planes[layer], bs * ROW_BYTES, ROW_BYTES, bs, table, ctxs, ROW_BYTES)
-        times.append(time.perf_counter() - t0)
-    times = sorted(times[1:])
-    median = times[len(times) // 2]
+
+    def one_layer(layer):
+        orc.append_rows(planes[layer], bs * ROW_BYTES, ROW_BYTES, bs, rows[layer], ROW_BYTES, ROW_BYTES, slots)
+        orc.gather_rows(planes[layer], bs * ROW_BYTES, ROW_BYTES, bs, table, ctxs, ROW_BYTES)
+
+    def median_seconds(step, reps):
+        times = []
+        for _ in range(reps + 1):
+            t0 = time.perf_counter()
+            step()
+            times.append(time.perf_counter() - t0)
+        times = sorted(times[1:])
+        return times[len(times) // 2]
+
     nbytes = sample_layers * (2 * sum(ctxs) * ROW_BYTES + 2 * batch * ROW_BYTES)
-    return {"value": nbytes / median / 1e9, "unit": "GB/s", "cores": 1, "kind": "port",
+    single = median_seconds(lambda: [one_layer(layer) for layer in range(sample_layers)], 8)
+    threads = _threads()
+    with ThreadPoolExecutor(max_workers=threads) as workers:
+        multi = median_seconds(lambda: list(workers.map(one_layer, range(sample_layers))), 8)
+    return {"value": nbytes / single / 1e9, "unit": "GB/s", "cores": 1, "kind": "port",
             "sample": f"append+gather of {sample_layers} of 43 layers of the same workload (fused 576-element rows), "
-                      f"median of 12 runs after one warm-up, host cores visible: {os.cpu_count()}"}
+                      f"median of 8 runs after one warm-up, host cores visible: {os.cpu_count()}",
+            "all_cores": {"value": nbytes / multi / 1e9, "unit": "GB/s", "cores": threads,
+                          "sample": "the same step, layers spread over one thread per core"},
+            "reference_host_plumbing": {"ms_per_step": REFERENCE_HOST_PLUMBING_MS_PER_STEP,
+                                        "what": "host orchestration of the reference's own 43-layer decode step in its mock build "
+                                                "(operator launches are no-ops; no KV byte moves), 8 cores of the build container; "
+                                                "the reference has no CPU numerics for this path to time"}}
 
 
 def cpu_attention_baseline(np):
+    """Config-3 attention by the CPU oracle (fp32 accumulate): every one of the 32 sequences, on one
+    core and with one thread per core (sequences are independent)."""
+    from concurrent.futures import ThreadPoolExecutor
+
     import oracle_ffi as orc
-    bs, heads, ctx, batch = 64, 64, 2048, 1
-    sample = 32  # every sequence, one after the other (about 10 s on one core)
+    bs, heads, ctx, batch = 64, 64, 2048, 32
     rng = np.random.default_rng(4)
     blocks = ctx // bs
-    latent = orc.bf16_to_f32(np.zeros(1, np.uint16))  # warm the library
+    orc.bf16_to_f32(np.zeros(1, np.uint16))  # warm the library
     latent_plane = (rng.standard_normal(blocks * bs * LATENT).astype(np.float32).view(np.uint32) >> 16).astype(np.uint16)
     rope_plane = (rng.standard_normal(blocks * bs * ROPE).astype(np.float32).view(np.uint32) >> 16).astype(np.uint16)
-    q_lat = (rng.standard_normal((batch, heads, LATENT)).astype(np.float32).view(np.uint32) >> 16).astype(np.uint16)
-    q_rope = (rng.standard_normal((batch, heads, ROPE)).astype(np.float32).view(np.uint32) >> 16).astype(np.uint16)
+    q_lat = (rng.standard_normal((1, heads, LATENT)).astype(np.float32).view(np.uint32) >> 16).astype(np.uint16)
+    q_rope = (rng.standard_normal((1, heads, ROPE)).astype(np.float32).view(np.uint32) >> 16).astype(np.uint16)
     table = np.arange(blocks, dtype=np.int32).reshape(1, blocks)
-    t0 = time.perf_counter()
-    for _ in range(sample):
+
+    def one_sequence(_):
         orc.mla_decode(q_lat, q_rope, latent_plane, rope_plane, bs, table, [ctx], 1 / math.sqrt(192.0), accum_f32=True)
-    seconds = time.perf_counter() - t0
-    return {"value": seconds * 32 / sample * 1e6, "unit": "us/step", "cores": 1, "kind": "port",
-            "sample": f"{sample} of 32 sequences (64 heads, ctx 2048, fp32 accumulate), time scaled by {32 // sample}"}
+
+    t0 = time.perf_counter()
+    for b in range(batch):
+        one_sequence(b)
+    single = time.perf_counter() - t0
+    threads = _threads()
+    with ThreadPoolExecutor(max_workers=threads) as workers:
+        t0 = time.perf_counter()
+        list(workers.map(one_sequence, range(batch)))
+        multi = time.perf_counter() - t0
+    return {"value": single * 1e6, "unit": "us/step", "cores": 1, "kind": "port",
+            "sample": "all 32 sequences (64 heads, ctx 2048, fp32 accumulate), one after the other",
+            "all_cores": {"value": multi * 1e6, "unit": "us/step", "cores": threads,
+                          "sample": "the same 32 sequences spread over one thread per core"}}
+
+
+def attention_suite(args, torch, np, ffi):
+    """The attention configurations: configs[2] (the target shape), configs[3] (FP8 KV, ragged
+    contexts with outliers), configs[4]'s decode step for one layer (lognormal contexts), the
+    selected-token decode and the indexer that feeds it."""
+    out = {}
+    out["attention"] = bench_attention(args, torch, np, ffi, [2048] * 32, mx_quant=True, label="configs[2]",
+                                       traffic_ratio=ATTENTION_TRAFFIC["attention"] if ATTENTION_TRAFFIC["attention"]["ratio"] else None)
+    out["attention_fp8"] = bench_attention(
+        args, torch, np, ffi, draw_contexts(np, "uniform_512_8192", 64, CONTEXT_SEED), fp8=True, iters=64, label="configs[3]",
+        distribution="uniform in [512, 8192]", outlier_fraction=0.01,
+        traffic_ratio=ATTENTION_TRAFFIC["attention_fp8"] if ATTENTION_TRAFFIC["attention_fp8"]["ratio"] else None)
+    out["attention_long"] = bench_attention(
+        args, torch, np, ffi, draw_contexts(np, "lognormal_4096_cap_32768", 128, CONTEXT_SEED), slices=2, iters=16,
+        label="configs[4] decode attention of one layer", distribution="lognormal (median 4096, sigma 1.0, cap 32768)",
+        traffic_ratio=ATTENTION_TRAFFIC["attention_long"] if ATTENTION_TRAFFIC["attention_long"]["ratio"] else None)
+    out["attention_sparse"] = bench_attention(args, torch, np, ffi, [8192] * 32, slices=4, sparse_k=512,
+                                              label="selected-token decode (index_topk 512 of 8192)")
+    out["indexer"] = bench_indexer(args, torch, np, ffi)
+    return out
 
 
 def main():
@@ -534,13 +773,10 @@ def main():
         print(json.dumps({"side_kernels": bench_side_kernels(args, torch, np, ffi)}))
         return 0
     if args.attention_only:
-        print(json.dumps({"attention": bench_attention(args, torch, np, ffi, mx_quant=True),
-                          "attention_fp8": bench_attention(args, torch, np, ffi, fp8=True, batch=64, ctx=4352, iters=64),
-                          "attention_long": bench_attention(args, torch, np, ffi, batch=128, ctx=8192, slices=2, iters=16,
-                                                            label="configs[4]-scale decode shape (one workgroup per sequence)"),
-                          "attention_sparse": bench_attention(args, torch, np, ffi, batch=32, ctx=8192, slices=4, sparse_k=512,
-                                                              label="selected-token decode (index_topk 512 of 8192)"),
-                          "indexer": bench_indexer(args, torch, np, ffi)}))
+        print(json.dumps(attention_suite(args, torch, np, ffi)))
+        return 0
+    if args.config5_only:
+        print(json.dumps({"config5": bench_config5(args, torch, np, ffi)}))
         return 0
     ag = bench_append_gather(args, torch, np, ffi)
     line = {
@@ -565,14 +801,9 @@ def main():
                            "bound by the launch rate, the kernel itself runs about 4 us in the rocprofv3 trace"},
     }
     if not args.no_attention:
-        line["attention"] = bench_attention(args, torch, np, ffi, mx_quant=True)
-        line["attention_fp8"] = bench_attention(args, torch, np, ffi, fp8=True, batch=64, ctx=4352, iters=64)
-        line["attention_long"] = bench_attention(args, torch, np, ffi, batch=128, ctx=8192, slices=2, iters=16,
-                                                 label="configs[4]-scale decode shape (one workgroup per sequence)")
-        line["attention_sparse"] = bench_attention(args, torch, np, ffi, batch=32, ctx=8192, slices=4, sparse_k=512,
-                                                   label="selected-token decode (index_topk 512 of 8192)")
-        line["indexer"] = bench_indexer(args, torch, np, ffi)
+        line.update(attention_suite(args, torch, np, ffi))
         line["side_kernels"] = bench_side_kernels(args, torch, np, ffi)
+        line["config5"] = bench_config5(args, torch, np, ffi)
     if not args.no_cpu_baseline:
         line["cpu_baseline"] = cpu_baseline(np, ag)
         if not args.no_attention:

@@ -223,9 +223,9 @@ def test_thin_abi_argument_validation_without_a_device():
     options = ffi.AttnPlanOptions(chunk_tiles=2, work_groups=0, merge_mode=ffi.ATTN_MERGE_IN_LAUNCH, merge_spin_us=-5)
     forced = ffi.AttnPlan()
     assert lib.mlakvAttnPlanInitEx(32, 128, 2048, 64, ffi.DTYPE_BF16, C.byref(options), C.byref(forced)) == 0
-    assert (forced.chunk_tiles, forced.work_groups, forced.max_units) == (2, 128, 32 * 64 // 2)
+    assert (forced.chunk_tiles, forced.work_groups, forced.max_units) == (2, 128, 32 * (64 + 4) // 2)
     assert (forced.merge_mode, forced.merge_spin_us) == (ffi.ATTN_MERGE_IN_LAUNCH, -1)
-    assert forced.workspace_bytes == 2 * (1024 + 32) * 64 * (1024 + 4)
+    assert forced.workspace_bytes == 2 * (1088 + 32) * 64 * (1024 + 4)
     options.chunk_tiles = 1 << 20  # clamped to what a segment's staged table entries can address
     assert lib.mlakvAttnPlanInitEx(1, 64, 1 << 20, 16, ffi.DTYPE_BF16, C.byref(options), C.byref(forced)) == 0
     assert forced.chunk_tiles == (510 * 16 + 2) // 32
