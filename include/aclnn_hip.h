@@ -124,7 +124,7 @@ aclnnStatus aclGetRawTensorAddr(const aclTensor* tensor, void** address);
 aclnnStatus aclGetViewOffset(const aclTensor* tensor, int64_t* offset);
 aclTensorList* aclCreateTensorList(const aclTensor* const* tensors, uint64_t size);
 aclnnStatus aclDestroyTensorList(const aclTensorList* tensor_list);
-aclIntArray* aclCreateIntArray(const int64_t* value, uint64_t size); /* keeps the pointer; the caller keeps the storage */
+aclIntArray* aclCreateIntArray(const int64_t* value, uint64_t size); /* copies the values */
 aclnnStatus aclDestroyIntArray(const aclIntArray* array);
 aclScalar* aclCreateScalar(void* value, aclDataType dtype);
 aclnnStatus aclDestroyScalar(const aclScalar* scalar);
