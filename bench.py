@@ -37,13 +37,17 @@ LATENT, ROPE, ROW = 512, 64, 576
 ROW_BYTES = ROW * 2
 CONTEXT_SEED = 20251125
 # HBM bytes per algorithmic byte of the attention launches (decode + merge kernel), from the
-# rocprofv3 --pmc runs summarised in profiles/attention_hbm_counters.md (FETCH_SIZE x2.000,
-# WRITE_SIZE x1.000 as for the gather): the excess is the partials of sequences split over
-# several workgroups, written once and read once.
+# rocprofv3 --pmc runs of this file summarised in profiles/bench_hbm_counters.md (FETCH_SIZE
+# x2.000, WRITE_SIZE x1.000 as for the gather): the excess is the partials of sequences split
+# over several workgroups, written once and read once.
+_TRAFFIC_SOURCE = ("rocprofv3 --pmc FETCH_SIZE x2.000 + WRITE_SIZE x1.000 per decode + merge dispatch pair of this command, "
+                   "applied as a ratio to the algorithmic bytes of the timed launches")
 ATTENTION_TRAFFIC = {
-    "attention": {"ratio": None, "source": None},
-    "attention_fp8": {"ratio": None, "source": None},
-    "attention_long": {"ratio": None, "source": None},
+    "attention": {"ratio": 1.429, "source": _TRAFFIC_SOURCE},        # 114.27 MB against 79.96 MB
+    "attention_fp8": {"ratio": 1.254, "source": _TRAFFIC_SOURCE},    # 221.43 MB against 176.52 MB
+    "attention_long": {"ratio": 1.060, "source": _TRAFFIC_SOURCE},   # 952.84 MB against 898.64 MB
+    "attention_sparse": {"ratio": 2.465, "source": _TRAFFIC_SOURCE}, # 57.70 MB against 23.41 MB
+    "indexer": {"ratio": 1.094, "source": _TRAFFIC_SOURCE},          # 38.26 MB against 34.96 MB
 }
 # Host orchestration of the reference's own 43-layer decode step (its mock build: every operator
 # launch is a no-op), measured in the build container on 8 cores: 128 steps, 132,480 launches,
@@ -389,7 +393,9 @@ def bench_indexer(args, torch, np, ffi, batch=32, ctx=8192, heads=64, k=512, bs=
             "workload": f"batch {batch}, ctx {ctx}, {heads} index heads x 128, top-{k}, block {bs}, e4m3 keys + fp32 row scale, "
                         f"shuffled table, {slices} rotating key pools",
             "roofline": {"bound": "hbm", "achieved": algorithmic / (us * 1e-6) / 1e9, "peak": HBM_PEAK_GBPS, "unit": "GB/s",
-                         "frac": algorithmic / (us * 1e-6) / 1e9 / HBM_PEAK_GBPS, "traffic": None},
+                         "frac": algorithmic / (us * 1e-6) / 1e9 / HBM_PEAK_GBPS,
+                         "traffic": algorithmic * ATTENTION_TRAFFIC["indexer"]["ratio"],
+                         "traffic_source": ATTENTION_TRAFFIC["indexer"]["source"]},
             "algorithmic_bytes": algorithmic, "timing": "250 ms of back-to-back launches untimed, then at least 100 ms of them timed"}
 
 
@@ -617,7 +623,9 @@ def bench_config5(args, torch, np, ffi, batch=128, heads=64, steps=6, warmup=2):
         "ms_per_step": step_ms, "attention_ms_per_step": attention_ms, "attention_us_per_layer": attention_ms * 1e3 / layers,
         "gbps": all_bytes / (step_ms * 1e-3) / 1e9,
         "roofline": {"bound": "hbm", "achieved": attention_bytes / (attention_ms * 1e-3) / 1e9, "peak": HBM_PEAK_GBPS, "unit": "GB/s",
-                     "frac": attention_bytes / (attention_ms * 1e-3) / 1e9 / HBM_PEAK_GBPS, "traffic": None,
+                     "frac": attention_bytes / (attention_ms * 1e-3) / 1e9 / HBM_PEAK_GBPS,
+                     "traffic": attention_bytes * ATTENTION_TRAFFIC["attention_long"]["ratio"],
+                     "traffic_source": "the ratio measured for the attention_long launches (same kernel, same context distribution)",
                      "what": "the 43 attention launches of a step, algorithmic bytes over HIP-event time"},
         "mean_tokens": sum(r["tokens"] for r in timed) / len(timed),
         "finished_sequences": sum(r["finished"] for r in timed),
@@ -733,17 +741,18 @@ def attention_suite(args, torch, np, ffi):
     selected-token decode and the indexer that feeds it."""
     out = {}
     out["attention"] = bench_attention(args, torch, np, ffi, [2048] * 32, mx_quant=True, label="configs[2]",
-                                       traffic_ratio=ATTENTION_TRAFFIC["attention"] if ATTENTION_TRAFFIC["attention"]["ratio"] else None)
+                                       traffic_ratio=ATTENTION_TRAFFIC["attention"])
     out["attention_fp8"] = bench_attention(
         args, torch, np, ffi, draw_contexts(np, "uniform_512_8192", 64, CONTEXT_SEED), fp8=True, iters=64, label="configs[3]",
         distribution="uniform in [512, 8192]", outlier_fraction=0.01,
-        traffic_ratio=ATTENTION_TRAFFIC["attention_fp8"] if ATTENTION_TRAFFIC["attention_fp8"]["ratio"] else None)
+        traffic_ratio=ATTENTION_TRAFFIC["attention_fp8"])
     out["attention_long"] = bench_attention(
         args, torch, np, ffi, draw_contexts(np, "lognormal_4096_cap_32768", 128, CONTEXT_SEED), slices=2, iters=16,
         label="configs[4] decode attention of one layer", distribution="lognormal (median 4096, sigma 1.0, cap 32768)",
-        traffic_ratio=ATTENTION_TRAFFIC["attention_long"] if ATTENTION_TRAFFIC["attention_long"]["ratio"] else None)
+        traffic_ratio=ATTENTION_TRAFFIC["attention_long"])
     out["attention_sparse"] = bench_attention(args, torch, np, ffi, [8192] * 32, slices=4, sparse_k=512,
-                                              label="selected-token decode (index_topk 512 of 8192)")
+                                              label="selected-token decode (index_topk 512 of 8192)",
+                                              traffic_ratio=ATTENTION_TRAFFIC["attention_sparse"])
     out["indexer"] = bench_indexer(args, torch, np, ffi)
     return out
 
