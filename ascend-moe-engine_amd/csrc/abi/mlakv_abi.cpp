@@ -1021,6 +1021,22 @@ mlakvStatus mlakvKvCacheUploadStep(mlakvKvCache* cache, void* stream) {
   return Guard("mlakvKvCacheUploadStep", [&] { cache->manager->UploadStep(stream); });
 }
 
+mlakvStatus mlakvKvCacheUploadStepAndAppend(mlakvKvCache* cache, int32_t layer_begin, int32_t layer_count, const void* latent_src,
+                                            int64_t latent_src_layer_stride, int64_t latent_src_row_stride, const void* rope_src,
+                                            int64_t rope_src_layer_stride, int64_t rope_src_row_stride, void* stream) {
+  MLAKV_NEED(cache, "mlakvKvCacheUploadStepAndAppend");
+  const char* who = "mlakvKvCacheUploadStepAndAppend";
+  if (latent_src == nullptr || rope_src == nullptr) return Fail(MLAKV_ERR_PARAM_NULLPTR, "%s: source rows are required", who);
+  if (!Aligned16(latent_src) || !Aligned16(rope_src) || latent_src_row_stride % 16 != 0 || rope_src_row_stride % 16 != 0 ||
+      latent_src_layer_stride % 16 != 0 || rope_src_layer_stride % 16 != 0) {
+    return Fail(MLAKV_ERR_PARAM_INVALID, "%s: source rows must be 16-byte aligned with 16-byte-multiple strides", who);
+  }
+  return Guard(who, [&] {
+    cache->manager->UploadStepAndAppend(latent_src, latent_src_layer_stride, latent_src_row_stride, rope_src, rope_src_layer_stride,
+                                        rope_src_row_stride, layer_begin, layer_count, stream);
+  });
+}
+
 mlakvStatus mlakvKvCacheGetStats(const mlakvKvCache* cache, mlakvKvStats* stats) {
   MLAKV_NEED(cache, "mlakvKvCacheGetStats");
   MLAKV_NEED(stats, "mlakvKvCacheGetStats");

@@ -302,7 +302,9 @@ void KvCacheManager::AddSequence(int64_t seq, int64_t context_len) {
 int32_t KvCacheManager::AppendToken(int64_t seq) {
   const int64_t blocks_before = seq >= 0 && seq < config_.max_batch ? pool_->seq_blocks(seq) : 0;
   const int32_t slot = pool_->AppendToken(seq);
-  if (pool_->seq_blocks(seq) != blocks_before) table_dirty_ = true;
+  // A token that opened a block changed one table entry: it is remembered and sent with the
+  // step's small arrays instead of marking the whole table for a copy.
+  if (pool_->seq_blocks(seq) != blocks_before) pending_entries_.push_back(static_cast<int32_t>(seq * num_blocks_ + blocks_before));
   host_small_[static_cast<size_t>(seq)] = slot;
   return slot;
 }
@@ -351,12 +353,20 @@ void KvCacheManager::UploadStep(void* stream) {
   // a device that runs kernels they ride in the argument block of a one-workgroup kernel: no
   // pinned staging, no copy engine and no event per step, which together cost more stream time
   // than the append itself.
-  const bool by_kernel = backend.runs_kernels() && !table_dirty_ && host_small_.size() <= static_cast<size_t>(mlakv::kMaxStoreWords);
+  const bool by_kernel = StepFitsOneLaunch();
   if (by_kernel) {
+    entry_words_.clear();
+    for (const int32_t index : pending_entries_) {
+      entry_words_.push_back(index);
+      entry_words_.push_back(host_table_[static_cast<size_t>(index)]);
+    }
     const hipError_t e = mlakv::LaunchStoreWords(host_small_.data(), static_cast<int>(host_small_.size()),
-                                                 static_cast<int32_t*>(d_small_), static_cast<hipStream_t>(stream));
+                                                 static_cast<int32_t*>(d_small_), entry_words_.data(),
+                                                 static_cast<int>(pending_entries_.size()), d_table_,
+                                                 static_cast<hipStream_t>(stream));
     MOE_HIP_REQUIRE(e == hipSuccess, "UploadStep: metadata kernel launch failed");
   } else {
+    if (!pending_entries_.empty()) table_dirty_ = true;  // too many for one argument block
     const int k = staging_next_;
     staging_next_ ^= 1;
     if (staging_busy_[k]) backend.SynchronizeEvent(staging_event_[k]);  // copy from two steps ago
@@ -371,7 +381,62 @@ void KvCacheManager::UploadStep(void* stream) {
     backend.RecordEvent(staging_event_[k], stream);
     staging_busy_[k] = true;
   }
+  FinishStep();
+}
+
+// Whether the step's small arrays and the table entries opened since the last upload ((index,
+// value) pairs) fit the argument block of one kernel.
+bool KvCacheManager::StepFitsOneLaunch() const {
+  return arena_.backend().runs_kernels() && !table_dirty_ &&
+         host_small_.size() + 2 * pending_entries_.size() <= static_cast<size_t>(mlakv::kMaxStoreWords);
+}
+
+void KvCacheManager::FinishStep() {
+  pending_entries_.clear();
   for (int64_t s = 0; s < config_.max_batch; ++s) host_small_[static_cast<size_t>(s)] = -1;
+}
+
+void KvCacheManager::UploadStepAndAppend(const void* latent_src, int64_t latent_layer_stride, int64_t latent_row_stride,
+                                         const void* rope_src, int64_t rope_layer_stride, int64_t rope_row_stride,
+                                         int32_t layer_begin, int32_t layer_count, void* stream) {
+  MOE_HIP_REQUIRE(bound_, "UploadStepAndAppend before Bind");
+  MOE_HIP_REQUIRE(arena_.backend().runs_kernels(), "UploadStepAndAppend needs a backend that runs kernels");
+  MOE_HIP_REQUIRE(latent_src != nullptr && rope_src != nullptr, "UploadStepAndAppend: source rows are required");
+  MOE_HIP_REQUIRE(layer_begin >= 0 && layer_count >= 0 && layer_begin + layer_count <= view_.num_layers,
+                  "UploadStepAndAppend: layers [" << layer_begin << ", " << layer_begin + layer_count << ") outside the cache");
+  mlakv::AppendArgs args{};
+  const auto plane = [&](const KvPlane& p) {
+    char* base = static_cast<char*>(p.base);
+    return mlakv::Plane{base == nullptr ? nullptr : base + layer_begin * p.layer_stride, p.layer_stride, p.block_stride, p.row_stride};
+  };
+  args.latent = plane(view_.latent);
+  args.rope = plane(view_.rope);
+  args.scale = plane(view_.scale);
+  args.latent_src = {const_cast<char*>(static_cast<const char*>(latent_src)), latent_layer_stride, latent_row_stride};
+  args.rope_src = {const_cast<char*>(static_cast<const char*>(rope_src)), rope_layer_stride, rope_row_stride};
+  args.slots = d_small_;
+  args.num_tokens = static_cast<int32_t>(config_.max_batch);
+  args.num_layers = layer_count;
+  args.num_blocks = view_.num_blocks;
+  args.block_size = view_.block_size;
+  args.fp8 = config_.dtype == KvDtype::kFp8E4m3;
+  if (layer_count == 0 || !StepFitsOneLaunch()) {
+    UploadStep(stream);
+    const hipError_t e = mlakv::LaunchAppend(args, static_cast<hipStream_t>(stream));
+    MOE_HIP_REQUIRE(e == hipSuccess, "UploadStepAndAppend: append launch failed: " << hipGetErrorString(e));
+    return;
+  }
+  RefreshSeqLens();
+  entry_words_.clear();
+  for (const int32_t index : pending_entries_) {
+    entry_words_.push_back(index);
+    entry_words_.push_back(host_table_[static_cast<size_t>(index)]);
+  }
+  const hipError_t e = mlakv::LaunchAppendWithWords(args, host_small_.data(), static_cast<int>(host_small_.size()), d_small_,
+                                                    entry_words_.data(), static_cast<int>(pending_entries_.size()), d_table_,
+                                                    static_cast<hipStream_t>(stream));
+  MOE_HIP_REQUIRE(e == hipSuccess, "UploadStepAndAppend: launch failed: " << hipGetErrorString(e));
+  FinishStep();
 }
 
 std::vector<std::pair<int32_t, int32_t>> KvCacheManager::Compact(void* stream) {

@@ -177,6 +177,15 @@ hipError_t LaunchCopyBlocks(const CopyBlocksArgs& args, hipStream_t stream);
 // buffer is free again on return, with no staging buffer, copy engine or event involved.
 constexpr int kMaxStoreWords = 960;
 hipError_t LaunchStoreWords(const int32_t* host_words, int count, int32_t* dst, hipStream_t stream);
+// The same with `pairs` scattered words behind them: host_pairs holds (index, value) couples and
+// the kernel also writes scatter_dst[index] = value; count + 2 * pairs <= kMaxStoreWords.
+hipError_t LaunchStoreWords(const int32_t* host_words, int count, int32_t* dst, const int32_t* host_pairs, int pairs,
+                            int32_t* scatter_dst, hipStream_t stream);
+// One launch for a step's metadata and its append: the words of LaunchStoreWords travel in the
+// append kernel's argument block, its first workgroup stores them, and every workgroup takes its
+// slots from the block (host_words[0 .. num_tokens) is the slot mapping) instead of from memory.
+hipError_t LaunchAppendWithWords(const AppendArgs& args, const int32_t* host_words, int count, int32_t* dst, const int32_t* host_pairs,
+                                 int pairs, int32_t* scatter_dst, hipStream_t stream);
 hipError_t LaunchAttnDecode(const AttnArgs& args, hipStream_t stream);
 hipError_t LaunchMxQuant(const MxQuantArgs& args, hipStream_t stream);
 hipError_t LaunchIndexer(const IndexerArgs& args, hipStream_t stream);

@@ -9,6 +9,8 @@
 // wave-uniform, so the address arithmetic stays in scalar registers.
 #include "kernels.h"
 
+#include <type_traits>
+
 namespace mlakv {
 namespace {
 
@@ -102,16 +104,51 @@ __device__ __forceinline__ u32x4 Dequant8(u32x2 codes, float scale) {
 // and rows) are issued together: with the row fetched only after its slot had arrived, a
 // prefill-sized append was bound by two memory latencies per row. The quantising kernel, which has
 // a shuffle reduction and a division per row to hide, takes four rows per wavefront.
+struct StoreWordsArgs {
+  int32_t words[kMaxStoreWords];
+};
+// The step's metadata riding in the argument block of an append launch: `count` words for `dst`
+// (the slot mapping comes first in them), then `pairs` (index, value) couples for `scatter_dst`.
+struct StepWords {
+  StoreWordsArgs args;
+  int32_t count, pairs;
+  int32_t* dst;
+  int32_t* scatter_dst;
+};
+struct NoStepWords {};
+
+// Slot of `token`: from the argument block when the launch carries the step's words (the copy in
+// memory is being written by the first workgroup of this very launch), else from memory.
+template <typename WORDS>
+__device__ __forceinline__ int SlotOf(const AppendArgs& a, const WORDS& w, int token) {
+  if constexpr (std::is_same<WORDS, StepWords>::value) {
+    return w.args.words[token];
+  } else {
+    return a.slots[token];
+  }
+}
+template <typename WORDS>
+__device__ __forceinline__ void StoreStepWords(const WORDS& w) {
+  if constexpr (std::is_same<WORDS, StepWords>::value) {
+    if (blockIdx.x == 0 && blockIdx.y == 0) {
+      for (int i = threadIdx.x; i < w.count; i += kThreads) w.dst[i] = w.args.words[i];
+      for (int i = threadIdx.x; i < w.pairs; i += kThreads) w.scatter_dst[w.args.words[w.count + 2 * i]] = w.args.words[w.count + 2 * i + 1];
+    }
+  }
+}
+
 constexpr int kAppendRows = 4;      // FP8: rows per wavefront
 constexpr int kAppendRowsBf16 = 1;  // bf16: a pure copy ran fastest with one row per wavefront (8 layers x 311k rows: 984 us, 1081 with two, 1106 with four)
 
-__global__ __launch_bounds__(kThreads) void AppendBf16Kernel(AppendArgs a) {
+template <typename WORDS>
+__global__ __launch_bounds__(kThreads) void AppendBf16Kernel(AppendArgs a, WORDS w) {
+  StoreStepWords(w);
   const int lane = threadIdx.x & (kWave - 1);
   const int token0 = Uniform((blockIdx.x * kWavesPerGroup + (threadIdx.x >> 6)) * kAppendRowsBf16);
   const int layer = blockIdx.y;
   if (token0 >= a.num_tokens) return;
   int my_slot = -1;
-  if (lane < kAppendRowsBf16 && token0 + lane < a.num_tokens) my_slot = a.slots[token0 + lane];
+  if (lane < kAppendRowsBf16 && token0 + lane < a.num_tokens) my_slot = SlotOf(a, w, token0 + lane);
   static_assert(kLatentDim * 2 / 16 == kWave, "one latent row is one wave access");
   const bool rope_lane = lane < kRopeDim * 2 / 16;
   const char* latent_src = a.latent_src.base + layer * a.latent_src.layer_stride;
@@ -213,14 +250,16 @@ __device__ __forceinline__ void QuantizeRowAndStore(const AppendArgs& a, int lay
 // Quantize-on-append: per-row absmax over latent+rope by wave shuffles, scale = absmax/448,
 // code = e4m3(x / scale) with the correctly rounded quotient. Each lane quantizes the 8 latent
 // values it loaded (8-byte store) and one of the 64 rope values (1-byte store).
-__global__ __launch_bounds__(kThreads) void AppendFp8Kernel(AppendArgs a) {
+template <typename WORDS>
+__global__ __launch_bounds__(kThreads) void AppendFp8Kernel(AppendArgs a, WORDS w) {
   static_assert(kRopeDim == kWave, "one rope element per lane");
+  StoreStepWords(w);
   const int lane = threadIdx.x & (kWave - 1);
   const int token0 = Uniform((blockIdx.x * kWavesPerGroup + (threadIdx.x >> 6)) * kAppendRows);
   const int layer = blockIdx.y;
   if (token0 >= a.num_tokens) return;
   int my_slot = -1;
-  if (lane < kAppendRows && token0 + lane < a.num_tokens) my_slot = a.slots[token0 + lane];
+  if (lane < kAppendRows && token0 + lane < a.num_tokens) my_slot = SlotOf(a, w, token0 + lane);
   u32x4 lv[kAppendRows];
   unsigned short rv[kAppendRows];
 #pragma unroll
@@ -552,12 +591,10 @@ int DivUp(int a, int b) { return (a + b - 1) / b; }
 
 // ---- per-step metadata ---------------------------------------------------------
 
-struct StoreWordsArgs {
-  int32_t words[kMaxStoreWords];
-};
-
-__global__ __launch_bounds__(kThreads) void StoreWordsKernel(StoreWordsArgs args, int count, int32_t* dst) {
+__global__ __launch_bounds__(kThreads) void StoreWordsKernel(StoreWordsArgs args, int count, int32_t* dst, int pairs,
+                                                             int32_t* scatter_dst) {
   for (int i = threadIdx.x; i < count; i += kThreads) dst[i] = args.words[i];
+  for (int i = threadIdx.x; i < pairs; i += kThreads) scatter_dst[args.words[count + 2 * i]] = args.words[count + 2 * i + 1];
 }
 
 }  // namespace
@@ -566,10 +603,33 @@ hipError_t LaunchAppend(const AppendArgs& args, hipStream_t stream) {
   if (args.num_tokens <= 0 || args.num_layers <= 0) return hipSuccess;
   if (args.fp8) {
     const dim3 grid(DivUp(args.num_tokens, kWavesPerGroup * kAppendRows), args.num_layers);
-    hipLaunchKernelGGL(AppendFp8Kernel, grid, dim3(kThreads), 0, stream, args);
+    hipLaunchKernelGGL(AppendFp8Kernel<NoStepWords>, grid, dim3(kThreads), 0, stream, args, NoStepWords{});
   } else {
     const dim3 grid(DivUp(args.num_tokens, kWavesPerGroup * kAppendRowsBf16), args.num_layers);
-    hipLaunchKernelGGL(AppendBf16Kernel, grid, dim3(kThreads), 0, stream, args);
+    hipLaunchKernelGGL(AppendBf16Kernel<NoStepWords>, grid, dim3(kThreads), 0, stream, args, NoStepWords{});
+  }
+  return hipGetLastError();
+}
+
+hipError_t LaunchAppendWithWords(const AppendArgs& args, const int32_t* host_words, int count, int32_t* dst, const int32_t* host_pairs,
+                                 int pairs, int32_t* scatter_dst, hipStream_t stream) {
+  if (args.num_tokens <= 0 || args.num_layers <= 0 || count < args.num_tokens || pairs < 0 || count + 2 * pairs > kMaxStoreWords ||
+      host_words == nullptr || dst == nullptr || (pairs > 0 && (host_pairs == nullptr || scatter_dst == nullptr))) {
+    return hipErrorInvalidValue;
+  }
+  StepWords words;
+  for (int i = 0; i < count; ++i) words.args.words[i] = host_words[i];
+  for (int i = 0; i < 2 * pairs; ++i) words.args.words[count + i] = host_pairs[i];
+  words.count = count;
+  words.pairs = pairs;
+  words.dst = dst;
+  words.scatter_dst = scatter_dst;
+  if (args.fp8) {
+    const dim3 grid(DivUp(args.num_tokens, kWavesPerGroup * kAppendRows), args.num_layers);
+    hipLaunchKernelGGL(AppendFp8Kernel<StepWords>, grid, dim3(kThreads), 0, stream, args, words);
+  } else {
+    const dim3 grid(DivUp(args.num_tokens, kWavesPerGroup * kAppendRowsBf16), args.num_layers);
+    hipLaunchKernelGGL(AppendBf16Kernel<StepWords>, grid, dim3(kThreads), 0, stream, args, words);
   }
   return hipGetLastError();
 }
@@ -616,11 +676,20 @@ hipError_t LaunchGather(const GatherArgs& args, hipStream_t stream) {
 }
 
 hipError_t LaunchStoreWords(const int32_t* host_words, int count, int32_t* dst, hipStream_t stream) {
-  if (count <= 0) return hipSuccess;
-  if (count > kMaxStoreWords || host_words == nullptr || dst == nullptr) return hipErrorInvalidValue;
+  return LaunchStoreWords(host_words, count, dst, nullptr, 0, nullptr, stream);
+}
+
+hipError_t LaunchStoreWords(const int32_t* host_words, int count, int32_t* dst, const int32_t* host_pairs, int pairs,
+                            int32_t* scatter_dst, hipStream_t stream) {
+  if (count <= 0 && pairs <= 0) return hipSuccess;
+  if (count < 0 || pairs < 0 || count + 2 * pairs > kMaxStoreWords) return hipErrorInvalidValue;
+  if ((count > 0 && (host_words == nullptr || dst == nullptr)) || (pairs > 0 && (host_pairs == nullptr || scatter_dst == nullptr))) {
+    return hipErrorInvalidValue;
+  }
   StoreWordsArgs args;
   for (int i = 0; i < count; ++i) args.words[i] = host_words[i];
-  hipLaunchKernelGGL(StoreWordsKernel, dim3(1), dim3(kThreads), 0, stream, args, count, dst);
+  for (int i = 0; i < 2 * pairs; ++i) args.words[count + i] = host_pairs[i];
+  hipLaunchKernelGGL(StoreWordsKernel, dim3(1), dim3(kThreads), 0, stream, args, count, dst, pairs, scatter_dst);
   return hipGetLastError();
 }
 

@@ -129,6 +129,14 @@ class KvCacheManager {
   // Enqueues the H2D copies of this step's metadata; afterwards the host slot mapping is
   // reset to -1 for the next step.
   void UploadStep(void* stream);
+  // UploadStep followed by the append of one row per sequence (the rows of sequence s of layer l
+  // at latent_src + l * layer stride + s * row stride, bf16; sequences without a token this step
+  // are skipped) into layers [layer_begin, layer_begin + layer_count). When the step's metadata
+  // fits one argument block both happen in a single launch: the append kernel carries the words,
+  // its first workgroup stores them, and the rows take their slots from the block. Kernel-capable
+  // backends only.
+  void UploadStepAndAppend(const void* latent_src, int64_t latent_layer_stride, int64_t latent_row_stride, const void* rope_src,
+                           int64_t rope_layer_stride, int64_t rope_row_stride, int32_t layer_begin, int32_t layer_count, void* stream);
 
   PagedAttentionStats stats() const;
   const BlockPool& pool() const { return *pool_; }
@@ -150,6 +158,8 @@ class KvCacheManager {
 
  private:
   void RefreshSeqLens();
+  bool StepFitsOneLaunch() const;
+  void FinishStep();
 
   StaticMemoryArena& arena_;
   KvCacheConfig config_;
@@ -164,6 +174,8 @@ class KvCacheManager {
   std::vector<int32_t> host_small_;
   size_t small_seq_lens_ = 0, small_cu_ = 0;  // int32 offsets inside host_small_
   bool table_dirty_ = true;
+  std::vector<int32_t> pending_entries_;  // table entries (flat indices) opened by AppendToken since the last upload
+  std::vector<int32_t> entry_words_;      // their (index, value) pairs, rebuilt per upload
   std::unique_ptr<BlockPool> pool_;
   // Device addresses and pinned staging (two slots, reused only after their copy drained).
   int32_t* d_table_ = nullptr;

@@ -144,6 +144,7 @@ PROTOTYPES = {
     "mlakvKvCacheFreeSequence": (_i32, [_vp, _i64]),
     "mlakvKvCacheCompact": (_i32, [_vp, _P(_i32), _P(_i64), _vp]),
     "mlakvKvCacheUploadStep": (_i32, [_vp, _vp]),
+    "mlakvKvCacheUploadStepAndAppend": (_i32, [_vp, _i32, _i32, _vp, _i64, _i64, _vp, _i64, _i64, _vp]),
     "mlakvKvCacheGetStats": (_i32, [_vp, _P(KvStats)]),
     "mlakvKvStatsFormatJson": (_i64, [_P(KvStats), C.c_char_p, _sz]),
     "mlakvKvCacheHostBlockTable": (_P(_i32), [_vp]),
@@ -362,6 +363,11 @@ class KvCache:
 
     def upload_step(self, stream=None):
         check(self.lib.mlakvKvCacheUploadStep(self.handle, stream))
+
+    def upload_step_and_append(self, layer_begin, layer_count, latent_ptr, latent_layer_stride, latent_row_stride, rope_ptr,
+                               rope_layer_stride, rope_row_stride, stream=None):
+        check(self.lib.mlakvKvCacheUploadStepAndAppend(self.handle, layer_begin, layer_count, latent_ptr, latent_layer_stride,
+                                                       latent_row_stride, rope_ptr, rope_layer_stride, rope_row_stride, stream))
 
     def stats(self):
         out = KvStats()

@@ -137,13 +137,12 @@ def bench_append_gather(args, torch, np, ffi):
 
     def step(timed):
         cache.append_token_all()
-        cache.upload_step(stream_ptr(torch))
         # events bracket the gather only: every record is a barrier packet in the queue, and a third
         # one in front of the 4-us append cost more than the append itself
         ev = [torch.cuda.Event(enable_timing=True) for _ in range(2)] if timed else None
-        ffi.check(lib.mlakvAppend(C.byref(view), 0, layers, step_latent.data_ptr(), batch * LATENT * 2, LATENT * 2,
-                                  step_rope.data_ptr(), batch * ROPE * 2, ROPE * 2, cache.device_slot_mapping, batch,
-                                  stream_ptr(torch)))
+        # the step's metadata and its 32 x 43 rows in one launch
+        cache.upload_step_and_append(0, layers, step_latent.data_ptr(), batch * LATENT * 2, LATENT * 2, step_rope.data_ptr(),
+                                     batch * ROPE * 2, ROPE * 2, stream_ptr(torch))
         if timed:
             ev[0].record()
         ffi.check(lib.mlakvGather(C.byref(view), 0, layers, cache.device_block_table, cache.num_blocks,

@@ -414,6 +414,16 @@ mlakvStatus mlakvKvCacheCompact(mlakvKvCache* cache, int32_t* moves, int64_t* nu
  * cu_seq_lens) from the pinned mirror; the batched form of the reference's 4-byte
  * slot mailbox copy (src/pipeline/pipeline.cpp:515-519). On the host backend it is a memcpy. */
 mlakvStatus mlakvKvCacheUploadStep(mlakvKvCache* cache, void* stream);
+/* mlakvKvCacheUploadStep followed by mlakvAppend of one row per sequence with the cache's own slot
+ * mapping (the per-step pair of src/pipeline/pipeline.cpp:515-519 and :399-404, for all layers
+ * [layer_begin, layer_begin + layer_count) at once): the row of sequence s of layer l is at
+ * src + l * layer_stride + s * row_stride (bf16, 16-byte aligned, strides multiples of 16);
+ * sequences without a token this step are skipped. When the step's metadata fits the argument
+ * block of one kernel (the usual decode step) both happen in ONE launch; otherwise it is the
+ * two calls. HIP backend only. */
+mlakvStatus mlakvKvCacheUploadStepAndAppend(mlakvKvCache* cache, int32_t layer_begin, int32_t layer_count, const void* latent_src,
+                                            int64_t latent_src_layer_stride, int64_t latent_src_row_stride, const void* rope_src,
+                                            int64_t rope_src_layer_stride, int64_t rope_src_row_stride, void* stream);
 mlakvStatus mlakvKvCacheGetStats(const mlakvKvCache* cache, mlakvKvStats* stats);
 /* The "paged_attention" member of the reference's --diag-json file, byte for byte as
  * InferenceDiagnostics::DumpJson writes it (src/diagnostics/inference_stats.cpp:42-47: two-space

@@ -314,3 +314,93 @@ def test_config2_full_size_round_trip():
     pool_sum = cache.latent.view(torch.int16).to(torch.int64).sum().item()
     src_sum = latent_src.view(torch.int16).to(torch.int64).sum().item() + step_latent.view(torch.int16).to(torch.int64).sum().item()
     assert pool_sum == src_sum
+
+
+_HIP = None
+
+
+def _device_i32(pointer, count):
+    """`count` int32 values at a raw device address (the C ABI hands out addresses, not tensors)."""
+    global _HIP
+    if _HIP is None:
+        _HIP = C.CDLL("libamdhip64.so")
+        _HIP.hipMemcpy.argtypes = [C.c_void_p, C.c_void_p, C.c_size_t, C.c_int]
+        _HIP.hipMemcpy.restype = C.c_int
+    out = np.empty(count, dtype=np.int32)
+    torch.cuda.synchronize()
+    assert _HIP.hipMemcpy(out.ctypes.data, pointer, count * 4, 2) == 0  # hipMemcpyDeviceToHost
+    return out
+
+
+@pytest.mark.parametrize("fp8", [False, True])
+def test_one_launch_step_equals_upload_then_append(fp8):
+    """mlakvKvCacheUploadStepAndAppend against mlakvKvCacheUploadStep + mlakvAppend on a twin cache:
+    the same planes, and the device metadata equal to the host mirrors, over steps that open
+    blocks (entries sent as pairs), steps after a sequence left or joined (whole table copied:
+    the two-call fallback) and steps where some sequences have no token."""
+    bs, layers, batch, max_ctx = 16, 3, 6, 160
+    lib = ffi.load()
+    twins = []
+    for _ in range(2):
+        arena = ffi.Arena(ffi.BACKEND_HIP)
+        cache = ffi.KvCache(arena, num_layers=layers, block_size=bs, max_context_len=max_ctx, max_batch=batch, pool_blocks=48,
+                            seed=9, shuffle=1, dtype=ffi.DTYPE_FP8_E4M3 if fp8 else ffi.DTYPE_BF16)
+        arena.commit()
+        cache.bind()
+        arena.seal()
+        twins.append((arena, cache, cache.view()))
+    for _, cache, _ in twins:
+        for seq, n in enumerate([5, 15, 16, 0, 31]):  # sequence 5 stays unused
+            cache.add_sequence(seq, n)
+        cache.upload_step(kt.stream_ptr())
+    width = twins[0][1].num_blocks
+    for step in range(40):
+        latent = kt.randn_bf16((layers, batch, LATENT), seed=1000 + 2 * step, outlier_fraction=0.01 if fp8 else 0.0).cuda()
+        rope = kt.randn_bf16((layers, batch, ROPE), seed=1001 + 2 * step).cuda()
+        for which, (_, cache, view) in enumerate(twins):
+            if step == 12:
+                cache.free_sequence(1)
+            if step == 20:
+                cache.add_sequence(1, 7)
+            if step % 5 == 3:   # only some sequences get a token
+                for seq in (0, 4):
+                    cache.append_token(seq)
+            else:
+                cache.append_token_all()
+            if which == 0:
+                cache.upload_step(kt.stream_ptr())
+                ffi.check(lib.mlakvAppend(C.byref(view), 0, layers, latent.data_ptr(), batch * LATENT * 2, LATENT * 2, rope.data_ptr(),
+                                          batch * ROPE * 2, ROPE * 2, cache.device_slot_mapping, batch, kt.stream_ptr()))
+            else:
+                cache.upload_step_and_append(0, layers, latent.data_ptr(), batch * LATENT * 2, LATENT * 2, rope.data_ptr(),
+                                             batch * ROPE * 2, ROPE * 2, kt.stream_ptr())
+        torch.cuda.synchronize()
+        fused = twins[1][1]
+        assert np.array_equal(_device_i32(fused.device_block_table, batch * width).reshape(batch, width), fused.host_block_table())
+        assert np.array_equal(_device_i32(fused.device_seq_lens, batch), fused.host_seq_lens())
+        lens = fused.host_seq_lens()
+        assert np.array_equal(_device_i32(fused.device_cu_seq_lens, batch + 1), np.concatenate([[0], np.cumsum(lens)]))
+        assert np.array_equal(_device_i32(fused.device_slot_mapping, batch), _device_i32(twins[0][1].device_slot_mapping, batch))
+    # the planes of the twins hold the same bytes
+    for name in ("latent", "rope", "scale"):
+        pointers = [getattr(view, name) for _, _, view in twins]
+        if not pointers[0]:
+            continue
+        stride = getattr(twins[0][2], name + "_layer_stride")
+        a, b = (_device_i32(p, layers * stride // 4) for p in pointers)
+        assert np.array_equal(a, b)
+    # a layer window, and refusals
+    _, cache, view = twins[1]
+    cache.append_token_all()
+    cache.upload_step_and_append(1, 2, latent.data_ptr(), batch * LATENT * 2, LATENT * 2, rope.data_ptr(), batch * ROPE * 2, ROPE * 2,
+                                 kt.stream_ptr())
+    torch.cuda.synchronize()
+    assert lib.mlakvKvCacheUploadStepAndAppend(cache.handle, 2, 2, latent.data_ptr(), 0, LATENT * 2, rope.data_ptr(), 0, ROPE * 2,
+                                               None) == ffi.ERR_CONTRACT  # layers outside the cache: the manager refuses
+    assert lib.mlakvKvCacheUploadStepAndAppend(cache.handle, 0, 1, None, 0, LATENT * 2, rope.data_ptr(), 0, ROPE * 2,
+                                               None) == ffi.ERR_PARAM_NULLPTR
+    assert lib.mlakvKvCacheUploadStepAndAppend(cache.handle, 0, 1, latent.data_ptr() + 2, 0, LATENT * 2, rope.data_ptr(), 0, ROPE * 2,
+                                               None) == ffi.ERR_PARAM_INVALID
+    for arena, cache, _ in twins:
+        cache.close()
+        arena.close()
