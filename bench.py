@@ -753,6 +753,16 @@ def attention_suite(args, torch, np, ffi):
                                               label="selected-token decode (index_topk 512 of 8192)",
                                               traffic_ratio=ATTENTION_TRAFFIC["attention_sparse"])
     out["indexer"] = bench_indexer(args, torch, np, ffi)
+    # The pair as a decode step would run it (indexer, then attention over its selection), against
+    # the bytes the pair has to move: B * ctx * 132 of index keys and scales, B * k * 1152 of selected rows.
+    pair_us = out["indexer"]["us_per_step"] + out["attention_sparse"]["us_per_step"]
+    pair_bytes = 32 * 8192 * 132 + 32 * 512 * ROW_BYTES
+    out["indexer_then_attention_sparse"] = {
+        "us_per_step": pair_us, "algorithmic_bytes": pair_bytes,
+        "roofline": {"bound": "hbm", "achieved": pair_bytes / (pair_us * 1e-6) / 1e9, "peak": HBM_PEAK_GBPS, "unit": "GB/s",
+                     "frac": pair_bytes / (pair_us * 1e-6) / 1e9 / HBM_PEAK_GBPS, "traffic": None},
+        "what": "sum of the two launches above (each timed back to back on its own), batch 32, ctx 8192, top-512",
+    }
     return out
 
 
