@@ -222,6 +222,19 @@ def test_upload_step_refreshes_lengths_and_resets_slot_mapping():
     assert list(lens) == [6, 0, 17] and list(cu) == [0, 6, 6, 23] and list(slots) == [s0, -1, s2]
     table = (C.c_int32 * 12).from_address(cache.device_block_table)
     assert list(table) == list(cache.host_block_table().reshape(-1))
+    # a later step that opens a block (position 16 of sequence 0 after ten more tokens) reaches the table too
+    for _ in range(10):
+        cache.append_token(0)
+        cache.upload_step(None)
+    assert list(cache.host_seq_lens()) == [16, 0, 17]
+    cache.append_token(0)
+    cache.upload_step(None)
+    assert list(table) == list(cache.host_block_table().reshape(-1)) and table[1] == cache.host_block_table()[0, 1]
+    # the one-launch step needs kernels: the bookkeeping backend refuses it and says why
+    lib = ffi.load()
+    rows = (C.c_uint16 * (3 * 576))()
+    status = lib.mlakvKvCacheUploadStepAndAppend(cache.handle, 0, 1, C.addressof(rows), 0, 1152, C.addressof(rows), 0, 1152, None)
+    assert status == ffi.ERR_CONTRACT and b"kernels" in lib.mlakvGetLastError()
     cache.close()
     arena.close()
 
