@@ -954,7 +954,8 @@ aclnnStatus aclnnFusedInferAttentionScoreV5(void* workspace, uint64_t workspace_
   SHIM_REQUIRE(e->slots[2].addresses[0] == latent, ACLNN_ERR_PARAM_INVALID,
                "%s: the value tensor must alias the key tensor (absorbed MLA reads the latent cache as K and V)", who);
   const int32_t* device_lens = e->bound_lens;
-  if (device_lens == nullptr) {
+  const bool inline_lens = device_lens == nullptr && e->batch <= MLAKV_ATTN_HOST_LENS_MAX;
+  if (device_lens == nullptr && !inline_lens) {
     // The lengths travel in the argument block of a one-workgroup kernel: the host vector is free
     // again when the call returns, and nothing is staged or waited for.
     int32_t* staged = reinterpret_cast<int32_t*>(static_cast<char*>(workspace) + e->lens_offset);
@@ -968,10 +969,19 @@ aclnnStatus aclnnFusedInferAttentionScoreV5(void* workspace, uint64_t workspace_
   mlakvCacheView view;
   FillView(&view, e, latent, e->slots[25].addresses[0]);
   float* lse = e->want_lse ? static_cast<float*>(e->slots[32].addresses[0]) : nullptr;
-  const mlakvStatus status = mlakvAttnDecode(
-      &e->plan, &view, 0, e->slots[0].addresses[0], e->q_token_stride, e->q_head_stride, e->slots[24].addresses[0], e->qr_token_stride,
-      e->qr_head_stride, static_cast<const int32_t*>(e->slots[14].addresses[0]), e->table_width, device_lens, e->scale,
-      e->slots[31].addresses[0], e->out_token_stride, e->out_head_stride, lse, workspace, e->plan.workspace_bytes, stream);
+  // Up to MLAKV_ATTN_HOST_LENS_MAX sequences (the reference has one): the lengths ride in the
+  // attention kernels' own argument block, no launch is spent on them.
+  const mlakvStatus status =
+      inline_lens ? mlakvAttnDecodeHostLens(&e->plan, &view, 0, e->slots[0].addresses[0], e->q_token_stride, e->q_head_stride,
+                                            e->slots[24].addresses[0], e->qr_token_stride, e->qr_head_stride,
+                                            static_cast<const int32_t*>(e->slots[14].addresses[0]), e->table_width, e->host_lens.data(),
+                                            e->scale, e->slots[31].addresses[0], e->out_token_stride, e->out_head_stride, lse, workspace,
+                                            e->plan.workspace_bytes, stream)
+                  : mlakvAttnDecode(&e->plan, &view, 0, e->slots[0].addresses[0], e->q_token_stride, e->q_head_stride,
+                                    e->slots[24].addresses[0], e->qr_token_stride, e->qr_head_stride,
+                                    static_cast<const int32_t*>(e->slots[14].addresses[0]), e->table_width, device_lens, e->scale,
+                                    e->slots[31].addresses[0], e->out_token_stride, e->out_head_stride, lse, workspace,
+                                    e->plan.workspace_bytes, stream);
   if (status == MLAKV_SUCCESS) e->launched = true;
   return status;
 }

@@ -426,8 +426,15 @@ mlakvStatus AttnDecodeImpl(const char* who, const mlakvAttnPlan* plan, const mla
                            int32_t table_stride, const int32_t* seq_lens, double scale, void* out, int64_t out_seq_stride,
                            int64_t out_head_stride, const mlakvMxQuantOut* quant, const int32_t* sparse_indices,
                            int64_t sparse_indices_seq_stride, float* lse, void* workspace, uint64_t workspace_bytes,
-                           void* stream) {
+                           void* stream, const int32_t* host_lens = nullptr) {
   if (plan == nullptr) return Fail(MLAKV_ERR_PARAM_NULLPTR, "%s: plan is null", who);
+  if (host_lens != nullptr) {
+    if (plan->batch > mlakv::kAttnInlineLens) {
+      return Fail(MLAKV_ERR_PARAM_INVALID, "%s: host lengths ride in the argument block for up to %d sequences, the plan has %d", who,
+                  mlakv::kAttnInlineLens, plan->batch);
+    }
+    seq_lens = host_lens;  // (only its being non-null matters below)
+  }
   if (mlakvStatus s = CheckView(cache, who)) return s;
   if (mlakvStatus s = CheckLayers(cache, layer, 1, who)) return s;
   if (q_latent == nullptr || q_rope == nullptr || block_table == nullptr || seq_lens == nullptr) {
@@ -513,7 +520,11 @@ mlakvStatus AttnDecodeImpl(const char* who, const mlakvAttnPlan* plan, const mla
   args.q_rope_head_stride = q_rope_head_stride;
   args.block_table = block_table;
   args.table_stride = table_stride;
-  args.seq_lens = seq_lens;
+  args.seq_lens = host_lens != nullptr ? nullptr : seq_lens;
+  if (host_lens != nullptr) {
+    args.inline_count = plan->batch;
+    for (int32_t i = 0; i < plan->batch; ++i) args.inline_lens[i] = host_lens[i];
+  }
   args.out = static_cast<char*>(out);
   args.out_seq_stride = out_seq_stride;
   args.out_head_stride = out_head_stride;
@@ -568,6 +579,20 @@ mlakvStatus mlakvAttnDecode(const mlakvAttnPlan* plan, const mlakvCacheView* cac
   return AttnDecodeImpl("mlakvAttnDecode", plan, cache, layer, q_latent, q_latent_seq_stride, q_latent_head_stride, q_rope,
                         q_rope_seq_stride, q_rope_head_stride, block_table, table_stride, seq_lens, scale, out, out_seq_stride,
                         out_head_stride, nullptr, nullptr, 0, lse, workspace, workspace_bytes, stream);
+}
+
+mlakvStatus mlakvAttnDecodeHostLens(const mlakvAttnPlan* plan, const mlakvCacheView* cache, int32_t layer, const void* q_latent,
+                                    int64_t q_latent_seq_stride, int64_t q_latent_head_stride, const void* q_rope,
+                                    int64_t q_rope_seq_stride, int64_t q_rope_head_stride, const int32_t* block_table,
+                                    int32_t table_stride, const int32_t* host_seq_lens, double scale, void* out,
+                                    int64_t out_seq_stride, int64_t out_head_stride, float* lse, void* workspace,
+                                    uint64_t workspace_bytes, void* stream) {
+  const char* who = "mlakvAttnDecodeHostLens";
+  if (out == nullptr) return Fail(MLAKV_ERR_PARAM_NULLPTR, "%s: the output is required", who);
+  if (host_seq_lens == nullptr) return Fail(MLAKV_ERR_PARAM_NULLPTR, "%s: the lengths are required", who);
+  return AttnDecodeImpl(who, plan, cache, layer, q_latent, q_latent_seq_stride, q_latent_head_stride, q_rope, q_rope_seq_stride,
+                        q_rope_head_stride, block_table, table_stride, nullptr, scale, out, out_seq_stride, out_head_stride, nullptr,
+                        nullptr, 0, lse, workspace, workspace_bytes, stream, host_seq_lens);
 }
 
 mlakvStatus mlakvAttnDecodeNoAlloc(const mlakvAttnPlan* plan, const mlakvCacheView* cache, int32_t layer, const void* q_latent,

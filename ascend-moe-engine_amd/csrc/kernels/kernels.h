@@ -84,6 +84,8 @@ struct CopyBlocksArgs {
   bool has_scale;
 };
 
+constexpr int kAttnInlineLens = 64;
+
 struct AttnArgs {
   Plane latent, rope, scale;  // offset to the layer of the launch; layer_stride unused
   const char* q_latent;
@@ -92,7 +94,7 @@ struct AttnArgs {
   int64_t q_rope_seq_stride, q_rope_head_stride;
   const int32_t* block_table;
   int32_t table_stride;
-  const int32_t* seq_lens;
+  const int32_t* seq_lens;   // device array, unless the lengths ride in the argument block (below)
   char* out;
   int64_t out_seq_stride, out_head_stride;
   float* lse;            // optional
@@ -126,6 +128,10 @@ struct AttnArgs {
   bool merge_in_launch;       // false: the merge is a second launch
   bool fp8;
   unsigned* sync;             // set by the launcher: this launch's counters, null for a second-launch merge
+  // Host-known lengths of a small batch travel here instead of through device memory: no upload,
+  // no launch for it, and the kernels' first dependent load is gone. inline_count = 0: unused.
+  int32_t inline_count;
+  int32_t inline_lens[kAttnInlineLens];
 };
 
 struct MxQuantArgs {

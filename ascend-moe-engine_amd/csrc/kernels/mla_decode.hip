@@ -476,6 +476,11 @@ __device__ __forceinline__ int WaveInclusiveScan(int v) {
 // 64 consecutive sequences, one per lane: tokens that count, tiles, and the running totals of
 // tiles and of sequences that have tiles, up to and including the lane's sequence. Windows are
 // visited in increasing order.
+// The live length of a sequence: from the argument block when the caller knew it on the host.
+__device__ __forceinline__ int LiveLength(const AttnArgs& a, int seq) {
+  return a.inline_count > 0 ? a.inline_lens[seq] : a.seq_lens[seq];
+}
+
 template <bool SPARSE>
 struct SeqWindow {
   int base;   // first sequence of the window; uniform
@@ -489,7 +494,7 @@ struct SeqWindow {
       if (SPARSE) {
         n = a.sparse_count;
       } else {
-        n = min(max(a.seq_lens[seq], 0), a.max_tokens);
+        n = min(max(LiveLength(a, seq), 0), a.max_tokens);
       }
     }
     tok = n;
@@ -937,7 +942,7 @@ __global__ __launch_bounds__(kThreads) void MlaDecodeKernel(AttnArgs a) {
           // The selection ends at its first entry that is negative or not inside the context. Then
           // this segment's part of it is resolved to pool slots through the block table.
           const int context = static_cast<int>(
-              min(static_cast<int64_t>(max(Uniform(a.seq_lens[seq]), 0)), static_cast<int64_t>(a.table_stride) * a.block_size));
+              min(static_cast<int64_t>(max(Uniform(LiveLength(a, seq)), 0)), static_cast<int64_t>(a.table_stride) * a.block_size));
           const int32_t* selection = a.sparse_indices + static_cast<int64_t>(seq) * a.sparse_seq_stride;
           if (tid == 0) scalar_lds[0] = a.sparse_count;
           __syncthreads();

@@ -100,6 +100,8 @@ PROTOTYPES = {
     "mlakvAttnPlanInitEx": (_i32, [_i32, _i32, _i32, _i32, _i32, _P(AttnPlanOptions), _P(AttnPlan)]),
     "mlakvAttnDecode": (_i32, [_P(AttnPlan), _P(CacheView), _i32, _vp, _i64, _i64, _vp, _i64, _i64, _vp, _i32, _vp,
                                C.c_double, _vp, _i64, _i64, _vp, _vp, _u64, _vp]),
+    "mlakvAttnDecodeHostLens": (_i32, [_P(AttnPlan), _P(CacheView), _i32, _vp, _i64, _i64, _vp, _i64, _i64, _vp, _i32, _vp,
+                                       C.c_double, _vp, _i64, _i64, _vp, _vp, _u64, _vp]),
     "mlakvAttnDecodeNoAlloc": (_i32, [_P(AttnPlan), _P(CacheView), _i32, _vp, _i64, _i64, _vp, _i64, _i64, _vp, _i32, _vp,
                                       C.c_double, _vp, _i64, _i64, _vp, _vp]),
     "mlakvAttnDecodeMxQuant": (_i32, [_P(AttnPlan), _P(CacheView), _i32, _vp, _i64, _i64, _vp, _i64, _i64, _vp, _i32, _vp,

@@ -191,6 +191,19 @@ mlakvStatus mlakvAttnDecode(const mlakvAttnPlan* plan, const mlakvCacheView* cac
                             void* out, int64_t out_seq_stride, int64_t out_head_stride, float* lse, void* workspace,
                             uint64_t workspace_bytes, void* stream);
 
+/* mlakvAttnDecode for a caller that knows the live lengths on the host (the engine's decode loop
+ * does: src/pipeline/pipeline.cpp:515-519 derives the position on the host): host_seq_lens holds
+ * plan->batch values, at most MLAKV_ATTN_HOST_LENS_MAX; they are copied into the kernels' argument
+ * block, so nothing is uploaded and the buffer is free again on return. A larger batch is refused
+ * with MLAKV_ERR_PARAM_INVALID: upload the lengths and call mlakvAttnDecode. */
+#define MLAKV_ATTN_HOST_LENS_MAX 64
+mlakvStatus mlakvAttnDecodeHostLens(const mlakvAttnPlan* plan, const mlakvCacheView* cache, int32_t layer,
+                                    const void* q_latent, int64_t q_latent_seq_stride, int64_t q_latent_head_stride,
+                                    const void* q_rope, int64_t q_rope_seq_stride, int64_t q_rope_head_stride,
+                                    const int32_t* block_table, int32_t table_stride, const int32_t* host_seq_lens,
+                                    double scale, void* out, int64_t out_seq_stride, int64_t out_head_stride, float* lse,
+                                    void* workspace, uint64_t workspace_bytes, void* stream);
+
 /* mlakvAttnDecode for callers that cannot allocate device memory and have no workspace to pass
  * (code under HIP graph capture, tight serving loops, harnesses that forbid hipMalloc). It has no
  * counterpart in the reference, whose operators always receive the arena's shared workspace

@@ -215,3 +215,40 @@ def test_maximum_context_single_sequence_many_chunks(fp8):
     if not fp8:
         expected, _ = kt.oracle_attention(cache, 0, q[:1, :16].contiguous(), table[:1], ctxs[:1], SCALE)
         _assert_close(out[:1, :16], expected, TOL_BF16)
+
+
+def test_host_lengths_in_the_argument_block_give_the_same_bits():
+    """mlakvAttnDecodeHostLens against mlakvAttnDecode with the same lengths in device memory: the
+    kernels only read the lengths from another place, so every output bit agrees; split and
+    unsplit sequences, an empty one, bf16 and FP8; more than 64 sequences are refused."""
+    import ctypes as C
+    lib = ffi.load()
+    for fp8 in (False, True):
+        bs, heads = 64, 64
+        ctxs = [1, 0, 700, 64, 333, 2048, 65]
+        blocks = sum(-(-c // bs) for c in ctxs) + 4
+        pool = kt.build_tables(ctxs, bs, blocks, seed=77)
+        table = pool.table()
+        cache = kt.PagedCache(1, blocks, bs, fp8=fp8)
+        _fill_cache(cache, ctxs, table, seed=78, outliers=0.01 if fp8 else 0.0)
+        q = kt.randn_bf16((len(ctxs), heads, LATENT + ROPE), seed=79).cuda()
+        tab = kt.dev_i32(table)
+        for options in ({}, {"chunk_tiles": 1}, {"chunk_tiles": 3, "merge_mode": ffi.ATTN_MERGE_IN_LAUNCH}):
+            want, want_lse, plan = kt.attention(cache, 0, q, tab, kt.dev_i32(ctxs), SCALE, **options)
+            ws = torch.empty(int(plan.workspace_bytes), dtype=torch.uint8, device="cuda")
+            out = torch.full_like(want, float("nan"))
+            lse = torch.full_like(want_lse, float("nan"))
+            host = (C.c_int32 * len(ctxs))(*ctxs)
+            row = (LATENT + ROPE) * 2
+            ffi.check(lib.mlakvAttnDecodeHostLens(C.byref(plan), C.byref(cache.view), 0, q.data_ptr(), heads * row, row,
+                                                  q.data_ptr() + LATENT * 2, heads * row, row, tab.data_ptr(), tab.shape[1],
+                                                  C.cast(host, C.c_void_p), SCALE, out.data_ptr(), heads * LATENT * 2, LATENT * 2,
+                                                  lse.data_ptr(), ws.data_ptr(), ws.numel(), kt.stream_ptr()))
+            host[2] = 5  # the values were copied: changing the buffer after the call changes nothing
+            torch.cuda.synchronize()
+            assert torch.equal(out.view(torch.int16), want.view(torch.int16)), (fp8, options)
+            assert torch.equal(lse, want_lse)
+    many = kt.make_plan(65, 64, 64, 64, False)
+    assert lib.mlakvAttnDecodeHostLens(C.byref(many), C.byref(cache.view), 0, q.data_ptr(), 1, 1, q.data_ptr(), 1, 1, tab.data_ptr(), 1,
+                                       C.cast(host, C.c_void_p), SCALE, out.data_ptr(), 1, 1, None, ws.data_ptr(), ws.numel(),
+                                       None) == ffi.ERR_PARAM_INVALID
