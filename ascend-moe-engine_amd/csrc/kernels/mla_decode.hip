@@ -56,6 +56,8 @@
 #include <utility>
 
 #include "kernels.h"
+
+#include <cstddef>
 #include "mx_quant_device.h"
 
 #pragma clang diagnostic ignored "-Winline-asm"
@@ -477,8 +479,16 @@ __device__ __forceinline__ int WaveInclusiveScan(int v) {
 // tiles and of sequences that have tiles, up to and including the lane's sequence. Windows are
 // visited in increasing order.
 // The live length of a sequence: from the argument block when the caller knew it on the host.
+// One load either way: the source is chosen as an address (AttnArgs is the kernels' only explicit
+// argument, so it starts the kernel-argument segment); a select between two loaded values cost the
+// launch pair 1 to 3 us.
 __device__ __forceinline__ int LiveLength(const AttnArgs& a, int seq) {
-  return a.inline_count > 0 ? a.inline_lens[seq] : a.seq_lens[seq];
+  const int32_t* lengths = a.seq_lens;
+  if (a.inline_count > 0) {
+    const char* segment = (const char*)__builtin_amdgcn_kernarg_segment_ptr();  // (constant -> generic address space)
+    lengths = reinterpret_cast<const int32_t*>(segment + offsetof(AttnArgs, inline_lens));
+  }
+  return lengths[seq];
 }
 
 template <bool SPARSE>
