@@ -231,7 +231,8 @@ aclnnStatus aclnnGatherPaKvCache(void* workspace, uint64_t workspace_size, aclOp
 /* EXTENSION (no reference counterpart: the reference fixes the length at build time,
  * src/memory/static_arena_manager.cpp:584-588). Replaces the kv lengths of a planned attention
  * executor by `count` = T host values, each in [0, table width * block size]; they are copied, and
- * every later launch sends them to the device in the argument block of a small kernel. */
+ * every later launch carries them in the attention kernels' own argument block (T <= 64) or sends
+ * them to the device in the argument block of a small kernel in front of it. */
 aclnnStatus aclnnMlaKvSetSeqLens(aclOpExecutor* executor, const int64_t* seq_lens, uint64_t count);
 /* EXTENSION (no reference counterpart, as above). Binds a device int32 array [T] of live context
  * lengths to a planned attention executor; it then replaces the host values, with no per-launch
