@@ -487,6 +487,15 @@ mlakvStatus AttnDecodeImpl(const char* who, const mlakvAttnPlan* plan, const mla
   if (sparse && (sparse_indices_seq_stride < plan->max_seq_len || reinterpret_cast<uintptr_t>(sparse_indices) % 4 != 0)) {
     return Fail(MLAKV_ERR_PARAM_INVALID, "%s: a row of the selection holds %d int32 entries", who, plan->max_seq_len);
   }
+  if (sparse) {
+    // The kernel stages a selected token as (block << ceil(log2(block_size))) | slot in 31 bits.
+    int slot_bits = 0;
+    while ((int64_t{1} << slot_bits) < cache->block_size) ++slot_bits;
+    if ((static_cast<int64_t>(cache->num_blocks) << slot_bits) > (int64_t{1} << 31)) {
+      return Fail(MLAKV_ERR_PARAM_INVALID, "%s: %d blocks of %d slots exceed the 2^31 pool slots selected-token attention addresses", who,
+                  cache->num_blocks, cache->block_size);
+    }
+  }
   if (table_stride <= 0) return Fail(MLAKV_ERR_PARAM_INVALID, "%s: the block table needs at least one column", who);
   if (!sparse && static_cast<int64_t>(table_stride) * cache->block_size < plan->max_seq_len) {
     return Fail(MLAKV_ERR_PARAM_INVALID, "%s: a table row of %d blocks cannot address %d tokens", who, table_stride,

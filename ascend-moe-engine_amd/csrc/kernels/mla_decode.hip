@@ -237,10 +237,12 @@ struct TileMap {
   const int* entries;  // LDS
   int first_block, block_size, seq_len;
   // Selected-token mode (never ALIGNED): `entries` holds, for each of the chunk's selected tokens
-  // from position `first_pos` of the selection on, the linear pool slot of that token (-1: behind
-  // a bad table entry), and `seq_len` is the number of selected tokens.
+  // from position `first_pos` of the selection on, the physical block and the slot inside it as
+  // (block << slot_bits) | slot (-1: behind a bad table entry), so that a row is located without a
+  // division; `seq_len` is the number of selected tokens.
   bool sparse;
   int first_pos;
+  int slot_bits;  // ceil(log2(block_size))
   int tile_block, tile_slot0;  // ALIGNED only: where the tile of the last Begin() sits
   int next_entry, next_slot0;  // ALIGNED only: cursor of the next tile (tiles are begun in order)
 
@@ -267,11 +269,11 @@ struct TileMap {
       return pos < seq_len && tile_block >= 0;
     }
     if (sparse) {
-      const int linear = pos < seq_len ? entries[pos - first_pos] : -1;
-      const int usable = linear < 0 ? 0 : linear;
-      *block = usable / block_size;
-      *slot = usable - *block * block_size;
-      return linear >= 0;
+      const int packed = pos < seq_len ? entries[pos - first_pos] : -1;
+      const int usable = packed < 0 ? 0 : packed;
+      *block = usable >> slot_bits;
+      *slot = usable & ((1 << slot_bits) - 1);
+      return packed >= 0;
     }
     const int clamped = pos < seq_len ? pos : seq_len - 1;
     const int logical = clamped / block_size;
@@ -331,18 +333,38 @@ __device__ __forceinline__ bool IssueTileBf16(const AttnArgs& a, TileMap<ALIGNED
   // Rare path (last tile of a sequence, unaligned block sizes, bad table entries): one row at a
   // time, kept as a loop so that it costs little code.
   bool all_real = true;
+  if constexpr (!ALIGNED && !WITH_PARTNER) {
+    // Every row is located first (the LDS reads of the staged entries go out together; the loads
+    // below are opaque to the compiler and would otherwise keep each read behind the load before it).
+    int blocks[kRowsPerWave], slots[kRowsPerWave];
+    bool reals[kRowsPerWave];
+#pragma unroll
+    for (int i = 0; i < kRowsPerWave; ++i) reals[i] = map.Row(tile, wave + kWaves * i, &blocks[i], &slots[i]);
+#pragma unroll
+    for (int i = 0; i < kRowsPerWave; ++i) {
+      const int row = wave + kWaves * i;  // wave-uniform
+      all_real = all_real && reals[i];
+      if (reals[i]) {
+        const char* src = a.latent.base + Uniform(blocks[i]) * a.latent.block_stride + Uniform(slots[i]) * a.latent.row_stride;
+        DirectLoad16(src, (lane ^ SwizzleLat(row)) << 4, buf + row * G::kLatRow);
+      } else {
+        *reinterpret_cast<u32x4*>(buf_ptr + row * G::kLatRow + lane * 16) = u32x4{0u, 0u, 0u, 0u};
+      }
+    }
+  } else {
 #pragma nounroll
-  for (int i = 0; i < (WITH_PARTNER ? 2 : 1) * kRowsPerWave; ++i) {
-    // wave-uniform; with a partner the wave walks rows (wave - 4) + 4 i, its partner's and its own in turn
-    const int row = WITH_PARTNER ? wave - kScoreWaves + kScoreWaves * i : wave + kWaves * i;
-    int block, slot;
-    const bool real = map.Row(tile, row, &block, &slot);
-    all_real = all_real && real;
-    if (real) {
-      const char* src = a.latent.base + Uniform(block) * a.latent.block_stride + Uniform(slot) * a.latent.row_stride;
-      DirectLoad16(src, (lane ^ SwizzleLat(row)) << 4, buf + row * G::kLatRow);
-    } else {
-      *reinterpret_cast<u32x4*>(buf_ptr + row * G::kLatRow + lane * 16) = u32x4{0u, 0u, 0u, 0u};
+    for (int i = 0; i < (WITH_PARTNER ? 2 : 1) * kRowsPerWave; ++i) {
+      // wave-uniform; with a partner the wave walks rows (wave - 4) + 4 i, its partner's and its own in turn
+      const int row = WITH_PARTNER ? wave - kScoreWaves + kScoreWaves * i : wave + kWaves * i;
+      int block, slot;
+      const bool real = map.Row(tile, row, &block, &slot);
+      all_real = all_real && real;
+      if (real) {
+        const char* src = a.latent.base + Uniform(block) * a.latent.block_stride + Uniform(slot) * a.latent.row_stride;
+        DirectLoad16(src, (lane ^ SwizzleLat(row)) << 4, buf + row * G::kLatRow);
+      } else {
+        *reinterpret_cast<u32x4*>(buf_ptr + row * G::kLatRow + lane * 16) = u32x4{0u, 0u, 0u, 0u};
+      }
     }
   }
   if (!rope_wave) return all_real;
@@ -908,6 +930,7 @@ __global__ __launch_bounds__(kThreads) void MlaDecodeKernel(AttnArgs a) {
         map.block_size = a.block_size;
         map.sparse = SPARSE;
         map.first_pos = tile_begin * kTileTokens;
+        map.slot_bits = a.block_size > 1 ? 32 - __builtin_clz(static_cast<unsigned>(a.block_size - 1)) : 0;
         map.first_block = 0;
         map.next_entry = 0;
         map.next_slot0 = 0;
@@ -969,7 +992,7 @@ __global__ __launch_bounds__(kThreads) void MlaDecodeKernel(AttnArgs a) {
             const int logical = index / a.block_size;
             const int entry = table_row[logical];
             table_lds[i] = static_cast<unsigned>(entry) < static_cast<unsigned>(a.num_blocks)
-                               ? entry * a.block_size + (index - logical * a.block_size)
+                               ? (entry << map.slot_bits) | (index - logical * a.block_size)
                                : -1;
           }
         }
@@ -1040,6 +1063,9 @@ __global__ __launch_bounds__(kThreads) void MlaDecodeKernel(AttnArgs a) {
               for (int ks = 0; ks < kKSteps; ++ks) q[ks] = __builtin_bit_cast(bf16x8, u32x4{0u, 0u, 0u, 0u});
             }
             write_table();  // asked for before the query, so it is here first
+            // Shared prologue: the table entries become visible here, before this wave waits for its
+            // query, so that the output waves start their tile loads a query latency earlier.
+            if constexpr (!kSoloPrologue) __syncthreads();
             // The query must have arrived before this wave issues tile loads: the compiler's own wait
             // for it would otherwise also wait for every tile load issued in between. Both paths above
             // pass through the statement: were it skipped on one, the compiler would have to assume the
@@ -1048,7 +1074,6 @@ __global__ __launch_bounds__(kThreads) void MlaDecodeKernel(AttnArgs a) {
             // score loop, at every use.
   #pragma unroll
             for (int ks = 0; ks < kKSteps; ++ks) asm volatile("" ::"v"(q[ks]));
-            if constexpr (!kSoloPrologue) __syncthreads();  // table entries visible
             for (; issued < G::kRing - 1 && issued < ntiles; ++issued) {
               if constexpr (kSoloPrologue) {
                 map.Begin(issued);  // keeps the cursor in step with the tiles this wave does not issue
@@ -1532,6 +1557,10 @@ hipError_t LaunchAttnDecode(const AttnArgs& args_in, hipStream_t stream) {
   hipError_t e;
   if (sparse) {
     if (quantise) return hipErrorInvalidValue;
+    // a selected token is staged as (block << ceil(log2(block_size))) | slot in 31 bits
+    int slot_bits = 0;
+    while ((int64_t{1} << slot_bits) < args.block_size) ++slot_bits;
+    if ((static_cast<int64_t>(args.num_blocks) << slot_bits) > (int64_t{1} << 31)) return hipErrorInvalidValue;
     e = args.fp8 ? Launch<true, false, false, true>(args, grid, stream) : Launch<false, false, false, true>(args, grid, stream);
   } else {
     e = quantise ? LaunchByCache<true>(args, grid, stream) : LaunchByCache<false>(args, grid, stream);

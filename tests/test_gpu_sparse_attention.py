@@ -40,7 +40,7 @@ def _close(got_bf16, expected, tol):
 
 
 @pytest.mark.parametrize("fp8", [False, True])
-@pytest.mark.parametrize("bs,k", [(64, 512), (16, 100), (128, 2048)])
+@pytest.mark.parametrize("bs,k", [(64, 512), (16, 100), (128, 2048), (48, 200)])  # 48: slots packed behind six bits, not all used
 def test_selected_tokens_match_oracle(fp8, bs, k):
     heads = 64
     ctxs = [3000, 700, 1, 0, 2049, 130]
@@ -124,6 +124,14 @@ def test_selection_ends_at_first_invalid_entry_and_argument_checks():
     assert sparse_call(plan, sel=None) == ffi.ERR_PARAM_NULLPTR
     assert sparse_call(plan, stride=k - 1) == ffi.ERR_PARAM_INVALID
     assert sparse_call(plan, out_ptr=None) == ffi.ERR_PARAM_NULLPTR
+    # a selected token is staged as (block, slot) in 31 bits: a pool beyond that is refused before any launch
+    huge = type(cache.view).from_buffer_copy(cache.view)
+    huge.num_blocks = 1 << 26
+    refused = lib.mlakvAttnDecodeSparse(C.byref(plan), C.byref(huge), 0, q.data_ptr(), heads * row, row, q.data_ptr() + LATENT * 2,
+                                        heads * row, row, table_d.data_ptr(), table_d.shape[1], lens_d.data_ptr(), sel_d.data_ptr(), k,
+                                        SCALE, out_t.data_ptr(), heads * LATENT * 2, LATENT * 2, None, workspace.data_ptr(),
+                                        workspace.numel(), kt.stream_ptr())
+    assert refused == ffi.ERR_PARAM_INVALID and b"2^31" in lib.mlakvGetLastError()
     dense_with_sparse_plan = lib.mlakvAttnDecode(C.byref(plan), C.byref(cache.view), 0, q.data_ptr(), heads * row, row,
                                                  q.data_ptr() + LATENT * 2, heads * row, row, table_d.data_ptr(), table_d.shape[1],
                                                  lens_d.data_ptr(), SCALE, out_t.data_ptr(), heads * LATENT * 2, LATENT * 2, None,
