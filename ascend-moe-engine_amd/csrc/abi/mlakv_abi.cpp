@@ -233,11 +233,11 @@ mlakvStatus mlakvNormRopeAppend(const mlakvCacheView* cache, int32_t layer, cons
   return status == hipSuccess ? MLAKV_SUCCESS : HipFail(status, who);
 }
 
-mlakvStatus mlakvGather(const mlakvCacheView* cache, int32_t layer_begin, int32_t layer_count, const int32_t* block_table,
-                        int32_t table_stride, const int32_t* seq_lens, const int32_t* cu_seq_lens, int32_t batch,
-                        int32_t max_seq_len, void* latent_dst, int64_t latent_dst_layer_stride,
-                        int64_t latent_dst_row_stride, void* rope_dst, int64_t rope_dst_layer_stride,
-                        int64_t rope_dst_row_stride, void* stream) {
+static mlakvStatus GatherImpl(const mlakvCacheView* cache, int32_t layer_begin, int32_t layer_count, const int32_t* block_table,
+                              int32_t table_stride, const int32_t* seq_lens, const int32_t* cu_seq_lens, int32_t batch,
+                              int32_t max_seq_len, void* latent_dst, int64_t latent_dst_layer_stride,
+                              int64_t latent_dst_row_stride, void* rope_dst, int64_t rope_dst_layer_stride,
+                              int64_t rope_dst_row_stride, void* stream, void* start_event, void* stop_event) {
   if (mlakvStatus s = CheckView(cache, "mlakvGather")) return s;
   if (mlakvStatus s = CheckLayers(cache, layer_begin, layer_count, "mlakvGather")) return s;
   if (batch < 0 || max_seq_len < 0 || table_stride < 0) return Fail(MLAKV_ERR_PARAM_INVALID, "mlakvGather: negative size");
@@ -267,8 +267,35 @@ mlakvStatus mlakvGather(const mlakvCacheView* cache, int32_t layer_begin, int32_
   args.num_blocks = cache->num_blocks;
   args.block_size = cache->block_size;
   args.fp8 = cache->dtype == MLAKV_DTYPE_FP8_E4M3;
-  const hipError_t status = mlakv::LaunchGather(args, static_cast<hipStream_t>(stream));
+  const hipError_t status = mlakv::LaunchGather(args, static_cast<hipStream_t>(stream), static_cast<hipEvent_t>(start_event),
+                                                static_cast<hipEvent_t>(stop_event));
   return status == hipSuccess ? MLAKV_SUCCESS : HipFail(status, "mlakvGather");
+}
+
+mlakvStatus mlakvGather(const mlakvCacheView* cache, int32_t layer_begin, int32_t layer_count, const int32_t* block_table,
+                        int32_t table_stride, const int32_t* seq_lens, const int32_t* cu_seq_lens, int32_t batch,
+                        int32_t max_seq_len, void* latent_dst, int64_t latent_dst_layer_stride,
+                        int64_t latent_dst_row_stride, void* rope_dst, int64_t rope_dst_layer_stride,
+                        int64_t rope_dst_row_stride, void* stream) {
+  return GatherImpl(cache, layer_begin, layer_count, block_table, table_stride, seq_lens, cu_seq_lens, batch, max_seq_len, latent_dst,
+                    latent_dst_layer_stride, latent_dst_row_stride, rope_dst, rope_dst_layer_stride, rope_dst_row_stride, stream,
+                    nullptr, nullptr);
+}
+
+mlakvStatus mlakvGatherTimed(const mlakvCacheView* cache, int32_t layer_begin, int32_t layer_count, const int32_t* block_table,
+                             int32_t table_stride, const int32_t* seq_lens, const int32_t* cu_seq_lens, int32_t batch,
+                             int32_t max_seq_len, void* latent_dst, int64_t latent_dst_layer_stride,
+                             int64_t latent_dst_row_stride, void* rope_dst, int64_t rope_dst_layer_stride,
+                             int64_t rope_dst_row_stride, void* stream, void* start_event, void* stop_event) {
+  if (start_event == nullptr || stop_event == nullptr) {
+    return Fail(MLAKV_ERR_PARAM_NULLPTR, "mlakvGatherTimed: both events are required");
+  }
+  if (batch == 0 || layer_count == 0 || max_seq_len == 0) {
+    return Fail(MLAKV_ERR_PARAM_INVALID, "mlakvGatherTimed: an empty gather launches nothing, so there is nothing to time");
+  }
+  return GatherImpl(cache, layer_begin, layer_count, block_table, table_stride, seq_lens, cu_seq_lens, batch, max_seq_len, latent_dst,
+                    latent_dst_layer_stride, latent_dst_row_stride, rope_dst, rope_dst_layer_stride, rope_dst_row_stride, stream,
+                    start_event, stop_event);
 }
 
 mlakvStatus mlakvCopyBlocks(const mlakvCacheView* cache, int32_t layer_begin, int32_t layer_count, const int32_t* moves,

@@ -176,7 +176,9 @@ constexpr int kAttnSyncSequences = 4096;   // (head group, sequence) pairs a lau
 
 hipError_t LaunchAppend(const AppendArgs& args, hipStream_t stream);
 hipError_t LaunchNormRopeAppend(const NormRopeAppendArgs& args, hipStream_t stream);
-hipError_t LaunchGather(const GatherArgs& args, hipStream_t stream);
+// With both events the launch records its own start and end in them (the dispatch's timestamps:
+// no marker packets of their own in the queue, unlike hipEventRecord around the launch).
+hipError_t LaunchGather(const GatherArgs& args, hipStream_t stream, hipEvent_t start = nullptr, hipEvent_t stop = nullptr);
 hipError_t LaunchCopyBlocks(const CopyBlocksArgs& args, hipStream_t stream);
 // Writes `count` (<= kMaxStoreWords) 32-bit words to device memory at `dst`. The words travel in
 // the kernel's argument block, which the runtime copies when the launch is queued: the caller's

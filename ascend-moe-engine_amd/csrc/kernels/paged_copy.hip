@@ -9,6 +9,8 @@
 // wave-uniform, so the address arithmetic stays in scalar registers.
 #include "kernels.h"
 
+#include <hip/hip_ext.h>
+
 #include <type_traits>
 
 namespace mlakv {
@@ -653,14 +655,27 @@ hipError_t LaunchNormRopeAppend(const NormRopeAppendArgs& args, hipStream_t stre
   return hipGetLastError();
 }
 
-hipError_t LaunchGather(const GatherArgs& args, hipStream_t stream) {
+namespace {
+// The plain launch, or the one that stamps the dispatch's own start and end into two events.
+template <typename Kernel, typename... Args>
+void LaunchMaybeTimed(Kernel kernel, const dim3& grid, const dim3& block, unsigned lds_bytes, hipStream_t stream, hipEvent_t start,
+                      hipEvent_t stop, Args... args) {
+  if (start != nullptr && stop != nullptr) {
+    hipExtLaunchKernelGGL(kernel, grid, block, lds_bytes, stream, start, stop, 0, args...);
+  } else {
+    hipLaunchKernelGGL(kernel, grid, block, lds_bytes, stream, args...);
+  }
+}
+}  // namespace
+
+hipError_t LaunchGather(const GatherArgs& args, hipStream_t stream, hipEvent_t start, hipEvent_t stop) {
   if (args.batch <= 0 || args.num_layers <= 0 || args.max_seq_len <= 0) return hipSuccess;
   const int blocks = DivUp(args.max_seq_len, args.block_size);
   if (!args.fp8 && args.block_size % kGatherTileRows == 0) {
     const int per_block = args.block_size / kGatherTileRows;
     const dim3 tile_grid(blocks * per_block, args.batch, args.num_layers);
-    hipLaunchKernelGGL(GatherBf16TileKernel<kGatherTileRows>, tile_grid, dim3(kThreads), kGatherLdsReserve, stream, args,
-                       per_block);
+    LaunchMaybeTimed(GatherBf16TileKernel<kGatherTileRows>, tile_grid, dim3(kThreads), kGatherLdsReserve, stream, start, stop, args,
+                     per_block);
     return hipGetLastError();
   }
   // Two-row items measured fastest for the generic kernels as well (more, shorter waves).
@@ -668,9 +683,9 @@ hipError_t LaunchGather(const GatherArgs& args, hipStream_t stream) {
   const int items_per_block = args.block_size / rows_per_item;
   const dim3 grid(DivUp(blocks * items_per_block, kWavesPerGroup), args.batch, args.num_layers);
   if (args.fp8) {
-    hipLaunchKernelGGL(GatherFp8Kernel, grid, dim3(kThreads), 0, stream, args, rows_per_item);
+    LaunchMaybeTimed(GatherFp8Kernel, grid, dim3(kThreads), 0, stream, start, stop, args, rows_per_item);
   } else {
-    hipLaunchKernelGGL(GatherBf16Kernel, grid, dim3(kThreads), 0, stream, args, rows_per_item);
+    LaunchMaybeTimed(GatherBf16Kernel, grid, dim3(kThreads), 0, stream, start, stop, args, rows_per_item);
   }
   return hipGetLastError();
 }

@@ -95,6 +95,8 @@ PROTOTYPES = {
     "mlakvNormRopeAppend": (_i32, [_P(CacheView), _i32, _vp, _i64, _vp, C.c_double, _vp, _vp, _i64, _vp, _vp, _i32, _vp, _i64,
                                    _vp, _i64, _vp, _i64, _i64, _i32, _vp]),
     "mlakvGather": (_i32, [_P(CacheView), _i32, _i32, _vp, _i32, _vp, _vp, _i32, _i32, _vp, _i64, _i64, _vp, _i64, _i64, _vp]),
+    "mlakvGatherTimed": (_i32, [_P(CacheView), _i32, _i32, _vp, _i32, _vp, _vp, _i32, _i32, _vp, _i64, _i64, _vp, _i64, _i64, _vp,
+                                _vp, _vp]),
     "mlakvCopyBlocks": (_i32, [_P(CacheView), _i32, _i32, _vp, _i32, _vp]),
     "mlakvAttnPlanInit": (_i32, [_i32, _i32, _i32, _i32, _i32, _P(AttnPlan)]),
     "mlakvAttnPlanInitEx": (_i32, [_i32, _i32, _i32, _i32, _i32, _P(AttnPlanOptions), _P(AttnPlan)]),

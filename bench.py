@@ -133,24 +133,26 @@ def bench_append_gather(args, torch, np, ffi):
         out = torch.empty(layers, rows_cap, ROW, dtype=torch.bfloat16, device="cuda")
         dst = (out.data_ptr(), rows_cap * ROW_BYTES, ROW_BYTES, out.data_ptr() + LATENT * 2, rows_cap * ROW_BYTES, ROW_BYTES)
     allocations_before = arena.device_allocations
-    gather_events = []
+    # The gather of every timed step stamps its own start and end into a pair of HIP events
+    # (mlakvGatherTimed): events recorded around it would each put a marker packet into the queue,
+    # which cost the step 4 to 5 us.
+    hip = HipEvents()
+    gather_events = [(hip.create(), hip.create()) for _ in range(args.steps)]
+    timed_steps = []
 
     def step(timed):
         cache.append_token_all()
-        # events bracket the gather only: every record is a barrier packet in the queue, and a third
-        # one in front of the 4-us append cost more than the append itself
-        ev = [torch.cuda.Event(enable_timing=True) for _ in range(2)] if timed else None
         # the step's metadata and its 32 x 43 rows in one launch
         cache.upload_step_and_append(0, layers, step_latent.data_ptr(), batch * LATENT * 2, LATENT * 2, step_rope.data_ptr(),
                                      batch * ROPE * 2, ROPE * 2, stream_ptr(torch))
+        gather_args = (C.byref(view), 0, layers, cache.device_block_table, cache.num_blocks, cache.device_seq_lens,
+                       cache.device_cu_seq_lens, batch, max_ctx, dst[0], dst[1], dst[2], dst[3], dst[4], dst[5], stream_ptr(torch))
         if timed:
-            ev[0].record()
-        ffi.check(lib.mlakvGather(C.byref(view), 0, layers, cache.device_block_table, cache.num_blocks,
-                                  cache.device_seq_lens, cache.device_cu_seq_lens, batch, max_ctx, dst[0], dst[1], dst[2],
-                                  dst[3], dst[4], dst[5], stream_ptr(torch)))
-        if timed:
-            ev[1].record()
-            gather_events.append((ev[0], ev[1]))
+            pair = gather_events[len(timed_steps)]
+            timed_steps.append(pair)
+            ffi.check(lib.mlakvGatherTimed(*gather_args, pair[0], pair[1]))
+        else:
+            ffi.check(lib.mlakvGather(*gather_args))
 
     for _ in range(args.warmup):
         step(False)
@@ -173,7 +175,10 @@ def bench_append_gather(args, torch, np, ffi):
     append_bytes = layers * (2 * batch * ROW_BYTES + 4 * batch)
     g_bytes = [gather_bytes(rows_per_step[i], lens, args.steps - 1 - i) for i in range(args.steps)]
     total_bytes = sum(g_bytes) + append_bytes * args.steps
-    gather_ms = [a.elapsed_time(b) for a, b in gather_events]
+    gather_ms = [hip.elapsed_ms(a, b) for a, b in timed_steps]
+    for a, b in gather_events:
+        hip.destroy(a)
+        hip.destroy(b)
     # the append launch on its own, after the timed region: the same rows to the same slots again,
     # 64 launches back to back between two events (one launch between two events times the events)
     def append_again():
@@ -206,6 +211,34 @@ def bench_append_gather(args, torch, np, ffi):
     cache.close()
     arena.close()
     return result
+
+
+class HipEvents:
+    """HIP events through the runtime's C interface (the library torch has loaded), for the entry
+    point that takes hipEvent_t handles."""
+
+    def __init__(self):
+        self.hip = C.CDLL("libamdhip64.so")
+        self.hip.hipEventCreate.argtypes = [C.POINTER(C.c_void_p)]
+        self.hip.hipEventDestroy.argtypes = [C.c_void_p]
+        self.hip.hipEventElapsedTime.argtypes = [C.POINTER(C.c_float), C.c_void_p, C.c_void_p]
+
+    def create(self):
+        event = C.c_void_p()
+        status = self.hip.hipEventCreate(C.byref(event))
+        if status != 0:
+            raise RuntimeError(f"hipEventCreate failed with {status}")
+        return event
+
+    def elapsed_ms(self, start, stop):
+        ms = C.c_float()
+        status = self.hip.hipEventElapsedTime(C.byref(ms), start, stop)
+        if status != 0:
+            raise RuntimeError(f"hipEventElapsedTime failed with {status}")
+        return float(ms.value)
+
+    def destroy(self, event):
+        self.hip.hipEventDestroy(event)
 
 
 def draw_contexts(np, kind, batch, seed):

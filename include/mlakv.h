@@ -121,6 +121,19 @@ mlakvStatus mlakvGather(const mlakvCacheView* cache, int32_t layer_begin, int32_
                         int64_t latent_dst_layer_stride, int64_t latent_dst_row_stride, void* rope_dst,
                         int64_t rope_dst_layer_stride, int64_t rope_dst_row_stride, void* stream);
 
+/* mlakvGather that also times itself: the launch stamps its own start and end into the two
+ * hipEvent_t (created by the caller with timing enabled); hipEventElapsedTime(start, stop) after
+ * the stream has passed the launch is the kernel's duration. Unlike events recorded around a launch
+ * these put no marker packets into the queue (measured: two recorded events cost a 0.7 ms step
+ * 4 to 5 us). No counterpart in the reference; it is for benchmarks and profilers. An empty gather
+ * launches nothing and is refused. */
+mlakvStatus mlakvGatherTimed(const mlakvCacheView* cache, int32_t layer_begin, int32_t layer_count,
+                             const int32_t* block_table, int32_t table_stride, const int32_t* seq_lens,
+                             const int32_t* cu_seq_lens, int32_t batch, int32_t max_seq_len, void* latent_dst,
+                             int64_t latent_dst_layer_stride, int64_t latent_dst_row_stride, void* rope_dst,
+                             int64_t rope_dst_layer_stride, int64_t rope_dst_row_stride, void* stream,
+                             void* start_event, void* stop_event);
+
 /* Compaction copy: cache[l][dst_block] = cache[l][src_block] for every (src, dst) pair
  * in `moves` (device int32[2 * num_moves]) and every layer. Sources and destinations must
  * be disjoint sets, which the block pool's plan guarantees. No reference counterpart

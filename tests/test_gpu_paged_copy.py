@@ -404,3 +404,49 @@ def test_one_launch_step_equals_upload_then_append(fp8):
     for arena, cache, _ in twins:
         cache.close()
         arena.close()
+
+
+@pytest.mark.parametrize("fp8,bs", [(False, 64), (False, 12), (True, 64)])  # the tiled, the generic and the FP8 kernel
+def test_gather_that_times_itself_moves_the_same_bytes(fp8, bs):
+    """mlakvGatherTimed: the plain gather's bytes, and a kernel duration in the caller's two events."""
+    layers = 4
+    ctxs = [300, 0, 77, 1000]
+    blocks = sum(-(-c // bs) for c in ctxs) + 3
+    table = kt.build_tables(ctxs, bs, blocks, seed=11).table()
+    total = sum(ctxs)
+    cache = kt.PagedCache(layers, blocks, bs, fp8=fp8)
+    kt.append(cache, kt.randn_bf16((layers, total, LATENT), seed=12).cuda(), kt.randn_bf16((layers, total, ROPE), seed=13).cuda(),
+              kt.dev_i32(kt.slots_for(table, ctxs, bs)))
+    table_d, lens_d = kt.dev_i32(table), kt.dev_i32(ctxs)
+    want_latent, want_rope = kt.gather(cache, table_d, lens_d)
+
+    hip = C.CDLL("libamdhip64.so")
+    hip.hipEventCreate.argtypes = [C.POINTER(C.c_void_p)]
+    hip.hipEventDestroy.argtypes = [C.c_void_p]
+    hip.hipEventElapsedTime.argtypes = [C.POINTER(C.c_float), C.c_void_p, C.c_void_p]
+    start, stop = C.c_void_p(), C.c_void_p()
+    assert hip.hipEventCreate(C.byref(start)) == 0 and hip.hipEventCreate(C.byref(stop)) == 0
+    lib = ffi.load()
+    cu = kt.dev_i32(np.concatenate([[0], np.cumsum(ctxs)]))
+    latent = torch.zeros(layers, total, LATENT, dtype=torch.bfloat16, device="cuda")
+    rope = torch.zeros(layers, total, ROPE, dtype=torch.bfloat16, device="cuda")
+
+    def timed(first, second, batch=len(ctxs)):
+        return lib.mlakvGatherTimed(C.byref(cache.view), 0, layers, table_d.data_ptr(), table_d.shape[1], lens_d.data_ptr(),
+                                    cu.data_ptr(), batch, max(ctxs), latent.data_ptr(), total * LATENT * 2, LATENT * 2,
+                                    rope.data_ptr(), total * ROPE * 2, ROPE * 2, kt.stream_ptr(), first, second)
+
+    outer = [torch.cuda.Event(enable_timing=True) for _ in range(2)]
+    outer[0].record()
+    assert timed(start, stop) == 0
+    outer[1].record()
+    torch.cuda.synchronize()
+    assert torch.equal(latent, want_latent) and torch.equal(rope, want_rope)
+    ms = C.c_float(-1.0)
+    assert hip.hipEventElapsedTime(C.byref(ms), start, stop) == 0
+    # the kernel's own duration: positive, and inside the interval that recorded events bracket
+    assert 0.0 < ms.value <= outer[0].elapsed_time(outer[1]) + 1e-3, (ms.value, outer[0].elapsed_time(outer[1]))
+    assert timed(None, stop) == ffi.ERR_PARAM_NULLPTR and timed(start, None) == ffi.ERR_PARAM_NULLPTR
+    assert timed(start, stop, batch=0) == ffi.ERR_PARAM_INVALID  # nothing would be launched, so nothing to time
+    hip.hipEventDestroy(start)
+    hip.hipEventDestroy(stop)
