@@ -252,3 +252,48 @@ def test_host_lengths_in_the_argument_block_give_the_same_bits():
     assert lib.mlakvAttnDecodeHostLens(C.byref(many), C.byref(cache.view), 0, q.data_ptr(), 1, 1, q.data_ptr(), 1, 1, tab.data_ptr(), 1,
                                        C.cast(host, C.c_void_p), SCALE, out.data_ptr(), 1, 1, None, ws.data_ptr(), ws.numel(),
                                        None) == ffi.ERR_PARAM_INVALID
+
+
+@pytest.mark.parametrize("seed", range(10))
+def test_attention_on_drawn_shapes(seed):
+    """Shapes, block sizes (multiples of the 32-token tile and not), cache types, plan options and a
+    selection drawn from a seeded generator: dense and selected-token attention against the oracle."""
+    rng = np.random.default_rng(1000 + seed)
+    bs = int(rng.choice([16, 24, 32, 48, 64, 96, 128]))
+    heads = int(rng.choice([16, 32, 48, 64, 80, 128]))
+    fp8 = bool(rng.integers(0, 2))
+    batch = int(rng.integers(1, 13))
+    ctxs = [int(v) for v in rng.integers(0, 600, size=batch)]
+    if batch > 2:
+        ctxs[int(rng.integers(0, batch))] = 0          # an empty sequence among the others
+    ctxs[int(rng.integers(0, batch))] = int(rng.integers(600, 1400))  # and a long one
+    blocks = sum(-(-c // bs) for c in ctxs) + 5
+    table = kt.build_tables(ctxs, bs, blocks, seed=seed).table()
+    cache = kt.PagedCache(1, blocks, bs, fp8=fp8)
+    _fill_cache(cache, ctxs, table, seed=2000 + seed, outliers=0.01 if fp8 else 0.0)
+    q = kt.randn_bf16((batch, heads, LATENT + ROPE), seed=3000 + seed).cuda()
+    tol = TOL_FP8 if fp8 else TOL_BF16
+    options = {}
+    if rng.integers(0, 2):
+        options["chunk_tiles"] = int(rng.choice([1, 2, 5, 40]))
+    if rng.integers(0, 2):
+        options["work_groups"] = int(rng.choice([1, 7, 300]))
+    if rng.integers(0, 3) == 0:
+        options["merge_mode"] = ffi.ATTN_MERGE_IN_LAUNCH
+    table_d, lens_d = kt.dev_i32(table), kt.dev_i32(ctxs)
+    expected, expected_lse = kt.oracle_attention(cache, 0, q, table, ctxs, SCALE)
+    out, lse, _ = kt.attention(cache, 0, q, table_d, lens_d, SCALE, **options)
+    case = dict(bs=bs, heads=heads, fp8=fp8, ctxs=ctxs, options=options)
+    live = np.array(ctxs) > 0
+    assert np.abs(out.float().cpu().numpy()[~live]).max(initial=0.0) == 0.0, case   # nothing to attend to: zeros
+    _assert_close(out[torch.as_tensor(live)], expected[live], tol)
+    assert np.abs(lse.cpu().numpy()[live] - expected_lse[live]).max() <= (6e-2 if fp8 else 2e-2), case
+    # a selection of up to k positions per sequence, shorter lists ended by -1
+    k = int(rng.choice([32, 100, 256]))
+    selection = np.full((batch, k), -1, dtype=np.int32)
+    for b, n in enumerate(ctxs):
+        take = min(n, k, int(rng.integers(1, k + 1)))
+        selection[b, :take] = rng.permutation(n)[:take]
+    expected_s, _ = kt.oracle_attention(cache, 0, q, table, ctxs, SCALE, sparse_indices=selection)
+    out_s, _, _ = kt.sparse_attention(cache, 0, q, table_d, lens_d, kt.dev_i32(selection), SCALE)
+    _assert_close(out_s[torch.as_tensor(live)], expected_s[live], tol)
