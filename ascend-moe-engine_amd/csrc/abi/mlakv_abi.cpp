@@ -1143,7 +1143,7 @@ int64_t mlakvKvCacheFreeBlocks(const mlakvKvCache* cache) { return cache ? cache
 int64_t mlakvKvCacheFreeList(const mlakvKvCache* cache, int32_t* out) {
   if (cache == nullptr) return 0;
   const std::vector<int32_t> list = cache->manager->pool().FreeList();
-  if (out != nullptr) std::memcpy(out, list.data(), list.size() * sizeof(int32_t));
+  if (out != nullptr && !list.empty()) std::memcpy(out, list.data(), list.size() * sizeof(int32_t));
   return static_cast<int64_t>(list.size());
 }
 
