@@ -450,3 +450,57 @@ def test_gather_that_times_itself_moves_the_same_bytes(fp8, bs):
     assert timed(start, stop, batch=0) == ffi.ERR_PARAM_INVALID  # nothing would be launched, so nothing to time
     hip.hipEventDestroy(start)
     hip.hipEventDestroy(stop)
+
+
+@pytest.mark.parametrize("seed", range(8))
+def test_append_and_gather_on_drawn_shapes(seed):
+    """Layers, block sizes (with and without the 8-row tile), context lengths, cache type and plane
+    layout drawn from a seeded generator: the cache planes and the gathered rows, bit for bit."""
+    rng = np.random.default_rng(500 + seed)
+    fp8 = bool(rng.integers(0, 2))
+    bs = int(rng.choice([4, 8, 12, 16, 40, 64, 128]))
+    layers = int(rng.integers(1, 6))
+    batch = int(rng.integers(1, 10))
+    ctxs = [int(v) for v in rng.integers(0, 5 * bs + 9, size=batch)]
+    ctxs[int(rng.integers(0, batch))] = 0
+    blocks = sum(-(-c // bs) for c in ctxs) + int(rng.integers(1, 6))
+    table = kt.build_tables(ctxs, bs, blocks, seed=seed).table()
+    total = sum(ctxs)
+    fused = (not fp8) and bool(rng.integers(0, 2))
+    cache = kt.PagedCache(layers, blocks, bs, fp8=fp8, fused=fused) if not fp8 else kt.PagedCache(layers, blocks, bs, fp8=True)
+    latent_src = kt.randn_bf16((layers, max(total, 1), LATENT), seed=600 + seed, outlier_fraction=0.01)[:, :total].contiguous().cuda()
+    rope_src = kt.randn_bf16((layers, max(total, 1), ROPE), seed=700 + seed, outlier_fraction=0.01)[:, :total].contiguous().cuda()
+    slots = kt.slots_for(table, ctxs, bs)
+    case = dict(fp8=fp8, bs=bs, layers=layers, ctxs=ctxs, fused=fused)
+    if total:
+        kt.append(cache, latent_src, rope_src, kt.dev_i32(slots))
+    torch.cuda.synchronize()
+    lat, rop, scl = _oracle_planes(layers, blocks, bs, fp8=fp8)
+    if fp8:
+        for layer in range(layers):
+            if total:
+                orc.append_rows_fp8(lat[layer], rop[layer], scl[layer], bs, kt.bits16(latent_src[layer]), kt.bits16(rope_src[layer]), slots)
+            assert cache.scale_np(layer).tobytes() == scl[layer].tobytes(), case
+            assert cache.latent_np(layer).tobytes() == lat[layer].tobytes(), case
+            assert cache.rope_np(layer).tobytes() == rop[layer].tobytes(), case
+    else:
+        if total:
+            _oracle_append_bf16(lat, rop, bs, latent_src, rope_src, slots)
+        for layer in range(layers):
+            assert kt.u8(cache.latent[layer].contiguous()).reshape(-1).tobytes() == lat[layer].tobytes(), case
+            assert kt.u8(cache.rope[layer].contiguous()).reshape(-1).tobytes() == rop[layer].tobytes(), case
+    if total == 0:
+        return
+    first = int(rng.integers(0, layers))
+    count = int(rng.integers(1, layers - first + 1))
+    got_latent, got_rope = kt.gather(cache, kt.dev_i32(table), kt.dev_i32(ctxs), fused_out=bool(rng.integers(0, 2)),
+                                     layer_begin=first, layer_count=count)
+    for i in range(count):
+        layer = first + i
+        if fp8:
+            exp_latent, exp_rope = orc.gather_rows_fp8(lat[layer], rop[layer], scl[layer], bs, table, ctxs)
+            assert kt.bits16(got_latent[i]).tobytes() == exp_latent.tobytes(), case
+            assert kt.bits16(got_rope[i]).tobytes() == exp_rope.tobytes(), case
+        else:
+            assert torch.equal(got_latent[i].contiguous(), latent_src[layer]), case
+            assert torch.equal(got_rope[i].contiguous(), rope_src[layer]), case
