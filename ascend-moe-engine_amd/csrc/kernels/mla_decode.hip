@@ -556,7 +556,7 @@ struct SeqWindow {
 // Tiles per work unit for a launch whose sequences add up to `total_tiles`: an equal share per
 // workgroup, not below what amortises a query load and not above what a segment's staged
 // block-table entries can address (or the plan's fixed value).
-__device__ __forceinline__ int TilesPerUnit(const AttnArgs& a, int total_tiles, int work_groups) {
+__host__ __device__ __forceinline__ int TilesPerUnit(const AttnArgs& a, int total_tiles, int work_groups) {
   int share;
   if (a.forced_unit_tiles > 0) {
     share = a.forced_unit_tiles;
@@ -565,7 +565,9 @@ __device__ __forceinline__ int TilesPerUnit(const AttnArgs& a, int total_tiles, 
   } else {
     share = (total_tiles + work_groups - 1) / work_groups;
   }
-  return min(max(share, a.forced_unit_tiles > 0 ? 1 : a.min_unit_tiles), a.cap_unit_tiles);
+  const int least = a.forced_unit_tiles > 0 ? 1 : a.min_unit_tiles;
+  const int raised = share > least ? share : least;
+  return raised < a.cap_unit_tiles ? raised : a.cap_unit_tiles;
 }
 
 // How a launch cuts its work. Entering a sequence in the middle of a unit costs a workgroup about
@@ -581,7 +583,7 @@ struct Cut {
   int total;           // length of the flat axis
   int tiles_per_unit;  // positions per unit
 };
-__device__ __forceinline__ Cut MakeCut(const AttnArgs& a, int total_tiles, int live_sequences, int common_tiles, int work_groups) {
+__host__ __device__ __forceinline__ Cut MakeCut(const AttnArgs& a, int total_tiles, int live_sequences, int common_tiles, int work_groups) {
   Cut cut;
   cut.pad = 0;
   cut.total = total_tiles;
@@ -1542,6 +1544,39 @@ hipError_t SyncRegion(unsigned** region) {
 
 hipError_t PrepareAttnKernels() { return hipSuccess; }
 
+// Whether any sequence of the launch is cut into several work units, i.e. whether partials will be
+// written that the merge has to put together. The host can tell when it knows the token counts:
+// a selection has the same count for every sequence, and lengths that ride in the argument block
+// are here; it then makes the cut the kernels make (same functions). Lengths in device memory: yes.
+bool AnySequenceSplit(const AttnArgs& a) {
+  const bool sparse = a.sparse_indices != nullptr;
+  if (!sparse && a.inline_count <= 0) return true;
+  const auto tiles_of = [&](int seq) {
+    const int tokens = sparse ? a.sparse_count : std::min(std::max(a.inline_lens[seq], 0), a.max_tokens);
+    return (tokens + kTileTokens - 1) / kTileTokens;
+  };
+  int total = 0, live = 0, common = 0;  // as SeqWindow accumulates them
+  for (int seq = 0; seq < a.batch; ++seq) {
+    const int tiles = tiles_of(seq);
+    if (tiles == 0) continue;
+    total += tiles;
+    ++live;
+    common = common == 0 || common == tiles ? tiles : -1;
+  }
+  if (live == 0) return false;
+  const Cut cut = MakeCut(a, total, live, common, a.work_groups);
+  int end_tiles = 0, end_live = 0;
+  for (int seq = 0; seq < a.batch; ++seq) {
+    const int tiles = tiles_of(seq);
+    if (tiles == 0) continue;
+    end_tiles += tiles;
+    ++end_live;
+    const int seq_end = end_tiles + cut.pad * end_live;
+    if ((seq_end - 1) / cut.tiles_per_unit != (seq_end - tiles) / cut.tiles_per_unit) return true;
+  }
+  return false;
+}
+
 hipError_t LaunchAttnDecode(const AttnArgs& args_in, hipStream_t stream) {
   AttnArgs args = args_in;
   if (args.batch <= 0) return hipSuccess;
@@ -1566,6 +1601,7 @@ hipError_t LaunchAttnDecode(const AttnArgs& args_in, hipStream_t stream) {
     e = quantise ? LaunchByCache<true>(args, grid, stream) : LaunchByCache<false>(args, grid, stream);
   }
   if (e != hipSuccess || merge_in_launch) return e;
+  if (!AnySequenceSplit(args)) return hipSuccess;  // every sequence is written by the one unit that holds it
   const dim3 merge_grid((std::min(64, args.heads) + kMergeHeads - 1) / kMergeHeads, args.batch, head_groups);
   if (sparse) {
     hipLaunchKernelGGL((MlaMergeKernel<false, true>), merge_grid, dim3(kMergeHeads * 64), 0, stream, args);

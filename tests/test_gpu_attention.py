@@ -223,9 +223,11 @@ def test_host_lengths_in_the_argument_block_give_the_same_bits():
     unsplit sequences, an empty one, bf16 and FP8; more than 64 sequences are refused."""
     import ctypes as C
     lib = ffi.load()
-    for fp8 in (False, True):
+    # the second list leaves every sequence inside one work unit: with the lengths on the host the
+    # launcher sees that and does not launch the merge at all
+    for fp8, ctxs in ((False, [1, 0, 700, 64, 333, 2048, 65]), (True, [1, 0, 700, 64, 333, 2048, 65]),
+                      (False, [100, 0, 128, 64, 1]), (True, [100, 0, 128, 64, 1])):
         bs, heads = 64, 64
-        ctxs = [1, 0, 700, 64, 333, 2048, 65]
         blocks = sum(-(-c // bs) for c in ctxs) + 4
         pool = kt.build_tables(ctxs, bs, blocks, seed=77)
         table = pool.table()
@@ -286,6 +288,20 @@ def test_attention_on_drawn_shapes(seed):
     case = dict(bs=bs, heads=heads, fp8=fp8, ctxs=ctxs, options=options)
     live = np.array(ctxs) > 0
     assert np.abs(out.float().cpu().numpy()[~live]).max(initial=0.0) == 0.0, case   # nothing to attend to: zeros
+    # the same launch with the lengths in the argument block (the merge is then only launched when
+    # the host-side cut splits a sequence): the same bits
+    import ctypes as C
+    plan = kt.make_plan(batch, heads, max(max(ctxs), 1), bs, fp8, **options)
+    ws = torch.empty(max(int(plan.workspace_bytes), 16), dtype=torch.uint8, device="cuda")
+    out_h = torch.full_like(out, float("nan"))
+    host = (C.c_int32 * batch)(*ctxs)
+    row = (LATENT + ROPE) * 2
+    ffi.check(ffi.load().mlakvAttnDecodeHostLens(C.byref(plan), C.byref(cache.view), 0, q.data_ptr(), heads * row, row,
+                                                 q.data_ptr() + LATENT * 2, heads * row, row, table_d.data_ptr(), table_d.shape[1],
+                                                 C.cast(host, C.c_void_p), SCALE, out_h.data_ptr(), heads * LATENT * 2, LATENT * 2,
+                                                 None, ws.data_ptr(), ws.numel(), kt.stream_ptr()))
+    torch.cuda.synchronize()
+    assert torch.equal(out_h.view(torch.int16), out.view(torch.int16)), case
     _assert_close(out[torch.as_tensor(live)], expected[live], tol)
     assert np.abs(lse.cpu().numpy()[live] - expected_lse[live]).max() <= (6e-2 if fp8 else 2e-2), case
     # a selection of up to k positions per sequence, shorter lists ended by -1
