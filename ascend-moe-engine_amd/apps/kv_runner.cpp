@@ -35,14 +35,18 @@ constexpr int64_t kHeads = 64, kLatent = 512, kRope = 64, kRow = kLatent + kRope
 struct Options {
   int64_t block_size = 128;      // RuntimeConfig defaults, include/moe/core/config.hpp:271-308
   int64_t max_context = 8192;
-  int64_t prompt_tokens = 128;
+  int64_t prompt_tokens = 128;   // when neither --prompt-tokens nor --prompt-ids is given
   int64_t max_new_tokens = 1;
   int64_t layers = 43;
+  int64_t qk_nope_head_dim = 128;  // only the softmax scale depends on it: 1 / sqrt(nope + rope), pipeline.cpp:238
   int32_t device = 0;
   uint64_t seed = 20251125;
-  std::string diag_json, stats_json;
+  std::string diag_json, stats_json, report_path;
+  std::vector<std::string> ignored;  // flags of stages this runner does not have, accepted for the reference's harness
+  bool prompt_from_ids = false;
   bool verbose = false;
   bool dry_run = false;
+  bool help = false;
 };
 
 [[noreturn]] void Die(const std::string& what) { throw std::runtime_error(what); }
@@ -56,31 +60,112 @@ void Check(int status, const char* call) {
 }
 #define RUNNER_CHECK(call) Check((call), #call)
 
+// Strict decimal integer, as the reference's ParseInt (apps/moe_runner.cpp:108-113).
+int64_t Integer(const std::string& text, const std::string& flag) {
+  char* end = nullptr;
+  const long long parsed = std::strtoll(text.c_str(), &end, 10);
+  if (text.empty() || end == nullptr || *end != '\0') Die(flag + " expects an integer, got '" + text + "'");
+  return static_cast<int64_t>(parsed);
+}
+
+void PrintUsage() {
+  std::printf(
+      "kv_runner -- the KV-cache path of the decode loop (append + decode attention per layer) on one GPU\n"
+      "\n"
+      "  --prompt-ids a,b,c        prompt token ids: their count is the prompt length (the ids themselves\n"
+      "                            feed an embedding this runner does not have and are otherwise unused)\n"
+      "  --prompt-tokens <n>       prompt length without ids (default 128; not together with --prompt-ids)\n"
+      "  --max-new-tokens <n>      tokens to generate (default 1)\n"
+      "  --block-size <n>          paged KV block size (default 128)\n"
+      "  --max-context <n>         reserved context length (default 8192)\n"
+      "  --kv-lora-rank <n>        must be 512, --qk-rope-head-dim <n> must be 64, --v-head-dim <n> must be 128:\n"
+      "                            the kernels are compiled for that geometry\n"
+      "  --qk-nope-head-dim <n>    enters the softmax scale 1/sqrt(nope + rope) only (default 128)\n"
+      "  --layers <n>              layers per step (default 43)\n"
+      "  --device <id>             GPU (default 0)\n"
+      "  --seed <n>                seed of the synthetic stage outputs\n"
+      "  --dry-run                 size and report, decode nothing\n"
+      "  --report <path>           write the report there as well as to stdout\n"
+      "  --diag-json <path>        structured diagnostics (also for dry runs)\n"
+      "  --stats-json <path>       machine-readable run stats after a decode\n"
+      "  --verbose\n"
+      "  --synthetic-weights       accepted: the only kind of input this runner has\n"
+      "  --weights --config --prompt --vram-slots --moe-path --moe-backend --gating-norm-type\n"
+      "  --dense-group-size --routed-coverage <value>\n"
+      "                            accepted and ignored: they configure stages (weights, MoE, GEMMs)\n"
+      "                            that are not part of the KV path; the report lists them\n");
+}
+
+// The reference runner's command line (apps/moe_runner.cpp:137-218), so that a driver written for it
+// (python/benchmarks/bench_runner.py:55-71 always passes --prompt-ids, --max-new-tokens, --stats-json
+// and --synthetic-weights or --weights, optionally --config) starts this binary unchanged.
 Options Parse(int argc, char** argv) {
   Options o;
+  bool prompt_tokens_given = false;
   for (int i = 1; i < argc; ++i) {
     const std::string flag = argv[i];
     const auto value = [&]() -> std::string {
       if (i + 1 >= argc) Die(flag + " needs a value");
       return argv[++i];
     };
-    if (flag == "--block-size") o.block_size = std::stoll(value());
-    else if (flag == "--max-context") o.max_context = std::stoll(value());
-    else if (flag == "--prompt-tokens") o.prompt_tokens = std::stoll(value());
-    else if (flag == "--max-new-tokens") o.max_new_tokens = std::stoll(value());
-    else if (flag == "--layers") o.layers = std::stoll(value());
-    else if (flag == "--device") o.device = static_cast<int32_t>(std::stol(value()));
+    const auto geometry = [&](int64_t compiled) {
+      const int64_t asked = Integer(value(), flag);
+      if (asked != compiled) {
+        Die(flag + " " + std::to_string(asked) + " refused: the kernels are compiled for kv_lora_rank 512, qk_rope_head_dim 64, "
+            "v_head_dim 128 (" + flag + " must be " + std::to_string(compiled) + ")");
+      }
+    };
+    if (flag == "--help" || flag == "-h") o.help = true;
+    else if (flag == "--block-size") o.block_size = Integer(value(), flag);
+    else if (flag == "--max-context") o.max_context = Integer(value(), flag);
+    else if (flag == "--prompt-tokens") {
+      o.prompt_tokens = Integer(value(), flag);
+      if (o.prompt_tokens <= 0) Die("--prompt-tokens must be positive");
+      prompt_tokens_given = true;
+    } else if (flag == "--prompt-ids") {
+      // ParseIdList (apps/moe_runner.cpp:115-125): comma-separated integers, empty pieces skipped
+      const std::string list = value();
+      int64_t count = 0;
+      std::stringstream pieces(list);
+      std::string piece;
+      while (std::getline(pieces, piece, ',')) {
+        if (piece.empty()) continue;
+        Integer(piece, flag);
+        ++count;
+      }
+      o.prompt_tokens = count;
+      o.prompt_from_ids = true;
+    }
+    else if (flag == "--max-new-tokens") o.max_new_tokens = Integer(value(), flag);
+    else if (flag == "--layers") o.layers = Integer(value(), flag);
+    else if (flag == "--device") o.device = static_cast<int32_t>(Integer(value(), flag));
     else if (flag == "--seed") o.seed = std::stoull(value());
+    else if (flag == "--kv-lora-rank") geometry(kLatent);
+    else if (flag == "--qk-rope-head-dim") geometry(kRope);
+    else if (flag == "--v-head-dim") geometry(128);
+    else if (flag == "--qk-nope-head-dim") {
+      o.qk_nope_head_dim = Integer(value(), flag);
+      if (o.qk_nope_head_dim <= 0) Die("--qk-nope-head-dim must be positive");
+    }
     else if (flag == "--diag-json") o.diag_json = value();
     else if (flag == "--stats-json") o.stats_json = value();
+    else if (flag == "--report") o.report_path = value();
     else if (flag == "--verbose") o.verbose = true;
     else if (flag == "--dry-run") o.dry_run = true;
     else if (flag == "--synthetic-weights") {}  // the only kind of input this runner has
-    else Die("unknown flag " + flag + " (flags: --block-size --max-context --prompt-tokens --max-new-tokens --layers --device "
-             "--seed --diag-json --stats-json --dry-run --verbose)");
+    else if (flag == "--weights" || flag == "--config" || flag == "--prompt" || flag == "--vram-slots" || flag == "--moe-path" ||
+             flag == "--moe-backend" || flag == "--gating-norm-type" || flag == "--dense-group-size" || flag == "--routed-coverage") {
+      o.ignored.push_back(flag + " " + value());
+    }
+    else Die("unknown flag: " + flag + " (--help lists the flags)");
   }
-  if (o.block_size <= 0 || o.max_context < o.block_size) Die("block size must be positive and not above the context");
-  if (o.prompt_tokens < 1 || o.max_new_tokens < 1 || o.layers < 1) Die("prompt tokens, new tokens and layers must be at least 1");
+  if (prompt_tokens_given && o.prompt_from_ids) Die("--prompt-tokens cannot be combined with --prompt-ids");
+  if (o.block_size <= 0 || o.max_context <= 0) Die("context length and block size must be positive");
+  if (o.max_context < o.block_size) Die("block size must not be above the context");
+  if (o.max_new_tokens <= 0) Die("--max-new-tokens must be positive");
+  if (o.layers < 1) Die("--layers must be at least 1");
+  if (o.prompt_from_ids && o.prompt_tokens == 0 && !o.dry_run) Die("--prompt-ids is empty: there is nothing to decode");
+  if (o.prompt_tokens > o.max_context) Die("prompt exceeds context capacity");
   return o;
 }
 
@@ -143,6 +228,10 @@ void DumpDiagJson(const std::string& path, const Options& o, const Diagnostics& 
 
 int Run(int argc, char** argv) {
   const Options o = Parse(argc, argv);
+  if (o.help) {
+    PrintUsage();
+    return 0;
+  }
   const int64_t num_blocks = (o.max_context + o.block_size - 1) / o.block_size;  // static_arena_manager.cpp:192-201
   const int64_t steps = std::min(o.prompt_tokens + o.max_new_tokens - 1, o.max_context);
   Diagnostics diag;
@@ -152,9 +241,20 @@ int Run(int argc, char** argv) {
   std::ostringstream report;
   report << "kv_runner: " << o.layers << " layers, block " << o.block_size << ", context " << o.max_context << " (" << num_blocks
          << " blocks per layer), " << o.prompt_tokens << " prompt + " << o.max_new_tokens << " new tokens = " << steps << " steps\n";
+  if (o.prompt_from_ids) report << "prompt length taken from --prompt-ids (" << o.prompt_tokens << " ids; their values are not used)\n";
+  for (const std::string& flag : o.ignored) report << "ignored (not a flag of the KV path): " << flag << "\n";
+  const auto emit_report = [&]() {
+    std::cout << report.str();
+    if (!o.report_path.empty()) {
+      std::ofstream file(o.report_path);
+      if (!file.is_open()) Die("cannot write the report to " + o.report_path);
+      file << report.str();
+    }
+  };
   if (o.dry_run) {
     if (!o.diag_json.empty()) DumpDiagJson(o.diag_json, o, diag);
-    std::cout << report.str();
+    report << "--dry-run: sized and reported; no token was decoded.\n";
+    emit_report();
     return 0;
   }
 
@@ -247,7 +347,7 @@ int Run(int argc, char** argv) {
   RUNNER_CHECK(aclnnFusedInferAttentionScoreV5GetWorkspaceSize(
       q_latent, key_list, value_list, nullptr, nullptr, actual_seq_q, actual_seq_kv, nullptr, nullptr, nullptr, nullptr, nullptr, nullptr,
       nullptr, block_table, nullptr, nullptr, nullptr, nullptr, nullptr, nullptr, nullptr, nullptr, nullptr, q_rope, rope_cache_view,
-      nullptr, nullptr, nullptr, nullptr, nullptr, kHeads, 1.0 / std::sqrt(192.0), 65536, 0, layout, 1, 3, 0, o.block_size, 0, false, 0, 0,
+      nullptr, nullptr, nullptr, nullptr, nullptr, kHeads, 1.0 / std::sqrt(static_cast<double>(o.qk_nope_head_dim + kRope)), 65536, 0, layout, 1, 3, 0, o.block_size, 0, false, 0, 0,
       0, 0, attn_out, nullptr, &ws_attention, &ex_attention));
   RUNNER_CHECK(aclnnGatherPaKvCacheGetWorkspaceSize(latent_cache, rope_cache, block_table, seq_lens, cu_seq_lens, gather_latent, gather_rope,
                                                     o.max_context, &ws_gather, &ex_gather));
@@ -401,7 +501,7 @@ int Run(int argc, char** argv) {
     DumpDiagJson(o.diag_json, o, diag);
     report << "diagnostics written to " << o.diag_json << "\n";
   }
-  std::cout << report.str();
+  emit_report();
 
   // Teardown in the reference's order: executors after the streams drain and before descriptors
   // and buffers (include/moe/core/op_table.hpp:131-134; src/memory/static_arena.cpp:50-69).

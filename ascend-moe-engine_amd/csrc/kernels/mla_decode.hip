@@ -600,8 +600,10 @@ __host__ __device__ __forceinline__ Cut MakeCut(const AttnArgs& a, int total_til
 // Stores and loads that other CUs' accesses of the same kind see without a cache write-back or
 // invalidate in between (agent scope: the sc1 bit): the partials and the counters travel through
 // these. The 16-byte forms have no builtin; a load's result is ready after WaitAgentLoads on it.
+// (The compiler does not know that the statement reads `v` for a few cycles after issue, as a
+// store of more than 8 bytes does: the s_nop keeps a following write of those registers away.)
 __device__ __forceinline__ void StoreAgent16(char* p, const u32x4& v) {
-  asm volatile("global_store_dwordx4 %0, %1, off sc1" : : "v"(p), "v"(v) : "memory");
+  asm volatile("global_store_dwordx4 %0, %1, off sc1\n\ts_nop 1" : : "v"(p), "v"(v) : "memory");
 }
 __device__ __forceinline__ u32x4 LoadAgent16(const char* p) {
   u32x4 v;

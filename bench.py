@@ -84,6 +84,10 @@ def parse_args():
     p.add_argument("--attention-only", action="store_true", help="development aid: time only the attention configurations")
     p.add_argument("--config5-only", action="store_true", help="development aid: run only the continuous-batching loop of configs[4]")
     p.add_argument("--config5-pool-gb", type=float, default=200.0, help="KV pool of the configs[4] loop, in GB (clamped to free memory)")
+    p.add_argument("--attn-merge", choices=["auto", "in", "second"], default="auto",
+                   help="development aid: how the attention launches merge their partials (default: the planner's choice)")
+    p.add_argument("--attn-host-lens", action="store_true",
+                   help="development aid: pass the lengths from the host (mlakvAttnDecodeHostLens) where the batch allows")
     p.add_argument("--split-out", action="store_true", help="gather into separate latent/rope planes instead of 576-wide rows")
     return p.parse_args()
 
@@ -284,7 +288,11 @@ def bench_attention(args, torch, np, ffi, ctxs, fp8=False, heads=64, slices=8, i
     cache = ffi.KvCache(arena, num_layers=slices, block_size=bs, max_context_len=max_ctx, max_batch=batch,
                         pool_blocks=pool_blocks, seed=7, shuffle=1, dtype=ffi.DTYPE_FP8_E4M3 if fp8 else ffi.DTYPE_BF16)
     plan = ffi.AttnPlan()
-    if sparse_k:
+    merge_mode = {"auto": ffi.ATTN_MERGE_AUTO, "in": ffi.ATTN_MERGE_IN_LAUNCH, "second": ffi.ATTN_MERGE_SECOND_LAUNCH}[args.attn_merge]
+    if merge_mode != ffi.ATTN_MERGE_AUTO:
+        options = ffi.AttnPlanOptions(0, 0, merge_mode, 0, 1 if sparse_k else 0)
+        ffi.check(lib.mlakvAttnPlanInitEx(batch, heads, sparse_k or max_ctx, bs, cache.config.dtype, C.byref(options), C.byref(plan)))
+    elif sparse_k:
         ffi.check(lib.mlakvAttnSparsePlanInit(batch, heads, sparse_k, bs, cache.config.dtype, C.byref(plan)))
     else:
         ffi.check(lib.mlakvAttnPlanInit(batch, heads, max_ctx, bs, cache.config.dtype, C.byref(plan)))
@@ -319,9 +327,21 @@ def bench_attention(args, torch, np, ffi, ctxs, fp8=False, heads=64, slices=8, i
                                             heads * LATENT * 2, LATENT * 2, None, arena.workspace, arena.workspace_bytes,
                                             stream_ptr(torch)))
 
+    host_lens = (C.c_int32 * batch)(*ctxs)
+
+    def launch_host_lens(i):
+        k = i % slices
+        ffi.check(lib.mlakvAttnDecodeHostLens(C.byref(plan), C.byref(view), k, q[k].data_ptr(), heads * ROW_BYTES, ROW_BYTES,
+                                              q[k].data_ptr() + LATENT * 2, heads * ROW_BYTES, ROW_BYTES,
+                                              cache.device_block_table, cache.num_blocks, host_lens,
+                                              1.0 / math.sqrt(192.0), out[k].data_ptr(), heads * LATENT * 2, LATENT * 2, None,
+                                              arena.workspace, arena.workspace_bytes, stream_ptr(torch)))
+
     def launch(i):
         if sparse_k:
             return launch_sparse(i)
+        if args.attn_host_lens and batch <= 64:
+            return launch_host_lens(i)
         k = i % slices
         ffi.check(lib.mlakvAttnDecode(C.byref(plan), C.byref(view), k, q[k].data_ptr(), heads * ROW_BYTES, ROW_BYTES,
                                       q[k].data_ptr() + LATENT * 2, heads * ROW_BYTES, ROW_BYTES,

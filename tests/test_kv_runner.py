@@ -60,6 +60,59 @@ def test_flags_are_checked_and_a_missing_device_is_an_error(tmp_path):
         assert done.returncode == 2 and "aclrtSetDevice" in done.stderr  # no CPU path behind the boundary
 
 
+def harness_argv(prompt_ids, new_tokens, stats_path, weights=None, config=None):
+    """The command line the reference's benchmark driver starts its runner with
+    (python/benchmarks/bench_runner.py:55-63 and :120-126): --prompt-ids <csv>, --max-new-tokens,
+    --stats-json, then --weights <dir> or --synthetic-weights, then --config <file> when given."""
+    argv = ["--prompt-ids", ",".join(str(t) for t in prompt_ids), "--max-new-tokens", str(new_tokens), "--stats-json", str(stats_path)]
+    argv += ["--weights", weights] if weights else ["--synthetic-weights"]
+    if config:
+        argv += ["--config", config]
+    return argv
+
+
+def test_the_reference_harness_command_line_is_accepted(tmp_path):
+    """What bench_runner.py passes, plus --dry-run so that no device is needed: the prompt length is
+    the number of ids; --weights / --config are taken and reported as ignored; the MLA geometry
+    flags of apps/moe_runner.cpp:170-181 are accepted at the compiled geometry and refused elsewhere."""
+    ids = [(7919 * i + 13) % 129280 for i in range(37)]
+    stats, diag = tmp_path / "stats.json", tmp_path / "diag.json"
+    done = run(*harness_argv(ids, 32, stats), "--dry-run", "--diag-json", diag)
+    assert "37 prompt + 32 new tokens = 68 steps" in done.stdout
+    parsed = json.loads(diag.read_text())
+    assert parsed["prompt_tokens"] == 37 and parsed["dry_run"] is True and parsed["generated_tokens"] == 0
+    assert not stats.exists()                                    # written after a decode only, as the reference does
+    done = run(*harness_argv(ids, 4, stats, weights="/models/ckpt", config="/models/ckpt/config.json"), "--dry-run")
+    assert "ignored (not a flag of the KV path): --weights /models/ckpt" in done.stdout
+    assert "ignored (not a flag of the KV path): --config /models/ckpt/config.json" in done.stdout
+    run("--dry-run", "--kv-lora-rank", 512, "--qk-rope-head-dim", 64, "--qk-nope-head-dim", 128, "--v-head-dim", 128, "--prompt-tokens", 8)
+    refused = run("--dry-run", "--kv-lora-rank", 256, check=False)
+    assert refused.returncode == 2 and "compiled for kv_lora_rank 512, qk_rope_head_dim 64" in refused.stderr
+    assert run("--dry-run", "--qk-rope-head-dim", 32, check=False).returncode == 2
+    assert run("--dry-run", "--prompt-ids", "1,2", "--prompt-tokens", 2, check=False).returncode == 2   # apps/moe_runner.cpp:281-283
+    assert run("--dry-run", "--prompt-ids", "1,x", check=False).returncode == 2
+    assert run("--prompt-ids", "", check=False).returncode == 2                                         # nothing to decode
+    report = tmp_path / "report.txt"
+    done = run("--dry-run", "--prompt-tokens", 5, "--report", report, "--moe-path", "fused", "--vram-slots", 3)
+    assert report.read_text() == done.stdout
+    assert run("--help").stdout.startswith("kv_runner --")
+
+
+@pytest.mark.gpu
+def test_the_reference_harness_command_line_decodes(tmp_path):
+    """The same command line for real: 24 prompt ids + 3 new tokens; the fields the driver reads
+    from --stats-json (bench_runner.py:66-69, :74-94) are there and sensible."""
+    ids = [(7919 * i + 13) % 129280 for i in range(24)]
+    stats = tmp_path / "stats.json"
+    run(*harness_argv(ids, 3, stats), "--block-size", 64, "--max-context", 256)
+    report = json.loads(stats.read_text())
+    assert list(report.keys())[:len(STATS_FIELDS)] == STATS_FIELDS
+    assert report["prompt_tokens"] == 24 and report["generated_tokens"] == 3 and report["steps"] == 26
+    assert report["ttft_seconds"] > 0 and report["tpot_seconds"] > 0
+    assert report["total_seconds"] >= report["ttft_seconds"] + report["decode_span_seconds"] - 1e-6
+    assert report["backbone_bytes"] > 43 * 256 * 1152 and report["gathered_rows_mismatched"] == 0
+
+
 @pytest.mark.gpu
 def test_configs0_through_the_operator_boundary(tmp_path):
     """128-token prompt, one more decode token, 43 layers, block 64, context 8192: every row of
