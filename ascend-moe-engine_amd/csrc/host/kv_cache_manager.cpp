@@ -461,16 +461,33 @@ std::vector<std::pair<int32_t, int32_t>> KvCacheManager::Compact(void* stream) {
   }
   if (moves.empty() || !bound_) return moves;
   IDeviceBackend& backend = arena_.backend();
-  if (moves_busy_) backend.SynchronizeEvent(moves_event_);
-  int32_t* staging = static_cast<int32_t*>(moves_staging_);
-  for (size_t i = 0; i < moves.size(); ++i) {
-    staging[2 * i] = moves[i].first;
-    staging[2 * i + 1] = moves[i].second;
+  if (backend.runs_kernels()) {
+    // The (source, destination) pairs travel in the argument blocks of small launches, 480 pairs
+    // each: the runtime copies an argument block when the launch is queued, so there is no staging
+    // buffer to keep alive until an event fires and no copy engine between two kernels of the stream.
+    move_words_.resize(moves.size() * 2);
+    for (size_t i = 0; i < moves.size(); ++i) {
+      move_words_[2 * i] = moves[i].first;
+      move_words_[2 * i + 1] = moves[i].second;
+    }
+    for (size_t done = 0; done < move_words_.size(); done += mlakv::kMaxStoreWords) {
+      const size_t count = std::min(move_words_.size() - done, static_cast<size_t>(mlakv::kMaxStoreWords));
+      const hipError_t e = mlakv::LaunchStoreWords(move_words_.data() + done, static_cast<int>(count), d_moves_ + done,
+                                                   static_cast<hipStream_t>(stream));
+      MOE_HIP_REQUIRE(e == hipSuccess, "compaction move upload failed: " << hipGetErrorString(e));
+    }
+  } else {
+    if (moves_busy_) backend.SynchronizeEvent(moves_event_);
+    int32_t* staging = static_cast<int32_t*>(moves_staging_);
+    for (size_t i = 0; i < moves.size(); ++i) {
+      staging[2 * i] = moves[i].first;
+      staging[2 * i + 1] = moves[i].second;
+    }
+    const size_t bytes = moves.size() * 2 * sizeof(int32_t);
+    backend.MemcpyAsync(d_moves_, arena_.Bytes(h_moves_), staging, bytes, CopyKind::kHostToDevice, stream);
+    backend.RecordEvent(moves_event_, stream);
+    moves_busy_ = true;
   }
-  const size_t bytes = moves.size() * 2 * sizeof(int32_t);
-  backend.MemcpyAsync(d_moves_, arena_.Bytes(h_moves_), staging, bytes, CopyKind::kHostToDevice, stream);
-  backend.RecordEvent(moves_event_, stream);
-  moves_busy_ = true;
   if (backend.runs_kernels()) {
     mlakv::CopyBlocksArgs args{};
     const auto plane = [](const KvPlane& p) {

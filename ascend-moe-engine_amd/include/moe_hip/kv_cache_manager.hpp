@@ -187,6 +187,7 @@ class KvCacheManager {
   void* staging_event_[2] = {nullptr, nullptr};
   bool staging_busy_[2] = {false, false};
   void* moves_staging_ = nullptr;
+  std::vector<int32_t> move_words_;  // the pairs of the last compaction, as they were sent
   void* moves_event_ = nullptr;
   bool moves_busy_ = false;
   KvCacheView view_;

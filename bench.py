@@ -17,6 +17,7 @@ used only for the cpu_baseline leg.
 """
 import argparse
 import ctypes as C
+import gc
 import json
 import math
 import os
@@ -36,6 +37,11 @@ MFMA_BF16_PEAK_TFLOPS = 2500.0
 LATENT, ROPE, ROW = 512, 64, 576
 ROW_BYTES = ROW * 2
 CONTEXT_SEED = 20251125
+# Context draws of the headline workload (numpy default_rng(seed).integers(128, 2049, 32)): the first
+# has the distribution's own mean (1088.0 against (128 + 2048) / 2 = 1088); the others are the three
+# seeds from CONTEXT_SEED on, whatever their means are (1231, 1136, 981). The reported value is the
+# lowest of the four runs.
+HEADLINE_SEEDS = (20251176, 20251125, 20251126, 20251127)
 # HBM bytes per algorithmic byte of the attention launches (decode + merge kernel), from the
 # rocprofv3 --pmc runs of this file summarised in profiles/bench_hbm_counters.md (FETCH_SIZE
 # x2.000, WRITE_SIZE x1.000 as for the gather): the excess is the partials of sequences split
@@ -96,17 +102,18 @@ def stream_ptr(torch):
     return C.c_void_p(torch.cuda.current_stream().cuda_stream)
 
 
-def bench_append_gather(args, torch, np, ffi):
+def bench_append_gather(args, torch, np, ffi, seed):
+    gc.collect()
     lib = ffi.load()
     layers, batch, bs = 43, 32, 64
-    rng = np.random.default_rng(20251125)
+    rng = np.random.default_rng(seed)
     ctxs = [int(v) for v in rng.integers(128, 2049, size=batch)]
     total_steps = args.warmup + args.steps
     max_ctx = 2048 + max(128, -(-total_steps // bs) * bs)  # every sequence grows by one token per step
     pool_blocks = sum(-(-(c + total_steps) // bs) for c in ctxs) + 32
     arena = ffi.Arena(ffi.BACKEND_HIP)
     cache = ffi.KvCache(arena, num_layers=layers, block_size=bs, max_context_len=max_ctx, max_batch=batch,
-                        pool_blocks=pool_blocks, seed=20251125, shuffle=1)
+                        pool_blocks=pool_blocks, seed=seed, shuffle=1)
     arena.commit()
     cache.bind()
     arena.seal()
@@ -210,7 +217,7 @@ def bench_append_gather(args, torch, np, ffi):
         "bytes_per_step": total_bytes / args.steps,
         "gather_bytes_per_launch": sum(g_bytes) / args.steps,
         "mean_ctx": sum(rows_per_step) / len(rows_per_step) / batch,
-        "ctxs": ctxs, "pool_blocks": pool_blocks, "seed": 20251125,
+        "ctxs": ctxs, "pool_blocks": pool_blocks, "seed": seed, "initial_mean_ctx": sum(ctxs) / batch,
     }
     cache.close()
     arena.close()
@@ -278,6 +285,7 @@ def fill_cache(torch, np, ffi, lib, cache, view, ctxs, layers, bs, seed, outlier
 
 def bench_attention(args, torch, np, ffi, ctxs, fp8=False, heads=64, slices=8, iters=None, label=None, distribution=None,
                     outlier_fraction=0.0, mx_quant=False, sparse_k=None, traffic_ratio=None):
+    gc.collect()
     lib = ffi.load()
     bs = 64
     batch = len(ctxs)
@@ -420,6 +428,7 @@ def bench_indexer(args, torch, np, ffi, batch=32, ctx=8192, heads=64, k=512, bs=
     """Lightning Indexer at the shape the selected-token attention is timed on: FP8 index keys
     (128 + 4 bytes per cached token) scored against one query token per sequence, top-k selected.
     HIP-event time of the operator (score kernel + selection kernel) over rotating key pools."""
+    gc.collect()
     lib = ffi.load()
     blocks = batch * (ctx // bs)
     rng = np.random.default_rng(9)
@@ -455,6 +464,7 @@ def bench_side_kernels(args, torch, np, ffi):
     """The other data-movement kernels of the path at configs[3]/[4]-like sizes (8 layers to bound
     memory): FP8 quantize-on-append, FP8 dequantising gather, bf16 compaction copy. HIP-event
     time per launch against algorithmic bytes."""
+    gc.collect()
     lib = ffi.load()
     bs, layers, batch, max_ctx = 64, 8, 64, 8192
     rng = np.random.default_rng(11)
@@ -542,12 +552,16 @@ def bench_side_kernels(args, torch, np, ffi):
             for s in range(0, batch, 2):
                 cache.free_sequence(s)
             torch.cuda.synchronize()
+            # (the C call alone between the events: building a Python list of the moves inside the
+            # bracket once triggered a 36 ms garbage collection that was then read as the library's time)
             start, stop = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+            moves_out, moves_count = (C.c_int32 * (2 * cache.pool_blocks))(), C.c_int64()
             start.record()
-            moves = cache.compact(stream_ptr(torch))
+            ffi.check(lib.mlakvKvCacheCompact(cache.handle, moves_out, C.byref(moves_count), stream_ptr(torch)))
             stop.record()
             torch.cuda.synchronize()
             whole_ms = start.elapsed_time(stop)
+            moves = [(moves_out[2 * i], moves_out[2 * i + 1]) for i in range(moves_count.value)]
             # the copy kernel alone, replaying the same move list from device memory
             moves_dev = torch.as_tensor(np.asarray(moves, dtype=np.int32).reshape(-1), device="cuda")
 
@@ -570,6 +584,7 @@ def bench_config5(args, torch, np, ffi, batch=128, heads=64, steps=6, warmup=2):
     recycled free list; after every step in which something finished the pool is compacted (the
     copy kernel moves the displaced blocks in all 43 layers). Every step appends one token per
     sequence and layer and runs the decode attention of all 43 layers."""
+    gc.collect()
     lib = ffi.load()
     bs, layers = 64, 43
     block_bytes = bs * ROW_BYTES
@@ -833,6 +848,10 @@ def main():
         sys.stderr.write("bench.py needs a GPU: the HIP library has no CPU fallback\n")
         return 3
     torch.cuda.set_device(0)
+    # The interpreter's cycle collector stays out of the timed regions (a full collection takes
+    # tens of milliseconds with torch loaded and falls wherever an allocation count happens to
+    # cross its threshold); it runs between the sections instead.
+    gc.disable()
     # A plain 1 GiB device copy of known size: the reference point that scales rocprofv3's
     # FETCH_SIZE / WRITE_SIZE readings for the kernels below.
     calib_src = torch.ones(1 << 30, dtype=torch.uint8, device="cuda")
@@ -849,7 +868,8 @@ def main():
     if args.config5_only:
         print(json.dumps({"config5": bench_config5(args, torch, np, ffi)}))
         return 0
-    ag = bench_append_gather(args, torch, np, ffi)
+    draws = [bench_append_gather(args, torch, np, ffi, seed) for seed in HEADLINE_SEEDS]
+    ag = min(draws, key=lambda d: d["value"])   # the slowest draw is the one reported
     line = {
         "metric": "paged-KV append+gather GB/s; MLA decode attn us/step (% HBM roofline)",
         "value": ag["value"], "unit": "GB/s", "n_gpus": 1, "steps": args.steps, "warmup": args.warmup,
@@ -859,7 +879,13 @@ def main():
                                f"(mean {ag['mean_ctx']:.0f} in the timed steps), block 64, seeded-shuffled free list, bf16 rows "
                                "of 576 elements, 1 row appended per sequence per layer then full-context gather into "
                                + ("separate latent/rope planes" if args.split_out else "contiguous 576-element rows"),
-                   "bytes_per_step": ag["bytes_per_step"], "frac_of_hbm_peak": ag["value"] / HBM_PEAK_GBPS},
+                   "bytes_per_step": ag["bytes_per_step"], "frac_of_hbm_peak": ag["value"] / HBM_PEAK_GBPS,
+                   "context_seed": ag["seed"],
+                   "context_draws": [{"seed": d["seed"], "initial_mean_ctx": d["initial_mean_ctx"], "mean_ctx_timed": d["mean_ctx"],
+                                      "value_gbps": d["value"], "frac_of_hbm_peak": d["value"] / HBM_PEAK_GBPS,
+                                      "ms_per_step": d["ms_per_step"], "gather_kernel_frac": d["gather_gbps"] / HBM_PEAK_GBPS}
+                                     for d in draws],
+                   "value_is": "the lowest of the context draws listed (each: W warm-up steps, then K timed steps)"},
         "roofline": {"bound": "hbm", "achieved": ag["gather_gbps"], "peak": HBM_PEAK_GBPS, "unit": "GB/s",
                      "frac": ag["gather_gbps"] / HBM_PEAK_GBPS,
                      "traffic": ag["gather_bytes_per_launch"] * GATHER_TRAFFIC_PER_ALGORITHMIC_BYTE,
