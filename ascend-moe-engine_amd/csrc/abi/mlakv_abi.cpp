@@ -124,6 +124,14 @@ extern "C" {
 
 const char* mlakvGetLastError(void) { return LastError(); }
 
+mlakvStatus mlakvPrepare(void) {
+  for (hipError_t (*prepare)() : {mlakv::PrepareAttnKernels, mlakv::PreparePagedCopyKernels, mlakv::PrepareIndexerKernels,
+                                   mlakv::PrepareMxQuantKernels}) {
+    if (const hipError_t status = prepare(); status != hipSuccess) return HipFail(status, "mlakvPrepare");
+  }
+  return MLAKV_SUCCESS;
+}
+
 int32_t mlakvDeviceCount(void) {
   int count = 0;
   if (hipGetDeviceCount(&count) != hipSuccess) return 0;
@@ -541,11 +549,6 @@ mlakvStatus AttnDecodeImpl(const char* who, const mlakvAttnPlan* plan, const mla
     return Fail(MLAKV_ERR_PARAM_INVALID, "%s: workspace of %llu bytes (16-byte aligned) needed, %llu given", who,
                 static_cast<unsigned long long>(plan->workspace_bytes), static_cast<unsigned long long>(workspace_bytes));
   }
-  static std::once_flag prepared;
-  static hipError_t prepare_status = hipSuccess;
-  std::call_once(prepared, [] { prepare_status = mlakv::PrepareAttnKernels(); });
-  if (prepare_status != hipSuccess) return HipFail(prepare_status, who);
-
   mlakv::AttnArgs args{};
   FillPlanes(cache, layer, &args.latent, &args.rope, &args.scale);
   args.q_latent = static_cast<const char*>(q_latent);

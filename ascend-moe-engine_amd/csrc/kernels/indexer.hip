@@ -14,6 +14,8 @@
 // E4M3 -> bf16 conversion: the FP8 MFMA of this part does not keep full fp32 precision while it
 // accumulates (scores came out about 1e-4 off, enough to move 3 % of the bf16 keys by one step),
 // and both forms take 16 cycles for 32 elements.
+#include <mutex>
+
 #include "kernels.h"
 
 namespace mlakv {
@@ -450,18 +452,41 @@ __global__ __launch_bounds__(256) void IndexKeyAppendKernel(IndexKeyAppendArgs a
   if (piece == 0) a.key_scale_base[block * a.key_scale_block_stride + in_block] = scale;
 }
 
+// Dynamic LDS above 64 KB needs the attribute per kernel and device (PrepareIndexerKernels).
+template <int HB>
+hipError_t PrepareScore() {
+  constexpr int kLdsBytes = HB * 16 * kIndexDim + kTokensPerGroup * kIndexDim;
+  return hipFuncSetAttribute(reinterpret_cast<const void*>(&IndexerScoreKernel<HB>), hipFuncAttributeMaxDynamicSharedMemorySize, kLdsBytes);
+}
+
 template <int HB>
 hipError_t LaunchScore(const IndexerArgs& args, const dim3& grid, hipStream_t stream) {
   constexpr int kLdsBytes = HB * 16 * kIndexDim + kTokensPerGroup * kIndexDim;  // query codes + the keys of eight waves
-  // Dynamic LDS above 64 KB needs the attribute once per kernel and process.
-  static const hipError_t prepared = hipFuncSetAttribute(reinterpret_cast<const void*>(&IndexerScoreKernel<HB>),
-                                                         hipFuncAttributeMaxDynamicSharedMemorySize, kLdsBytes);
-  if (prepared != hipSuccess) return prepared;
   hipLaunchKernelGGL(IndexerScoreKernel<HB>, grid, dim3(kScoreThreads), kLdsBytes, stream, args);
   return hipGetLastError();
 }
 
 }  // namespace
+
+hipError_t PrepareIndexerKernels() {
+  static std::mutex guard;
+  static PerDeviceOnce once;
+  int device = 0;
+  if (hipError_t e = hipGetDevice(&device); e != hipSuccess) return e;
+  if (device < 0 || device >= PerDeviceOnce::kMaxDevices) return hipErrorInvalidDevice;
+  std::lock_guard<std::mutex> lock(guard);
+  if (once.state[device] == 1) return hipSuccess;
+  const hipError_t results[] = {PrepareScore<1>(), PrepareScore<2>(), PrepareScore<3>(), PrepareScore<4>()};
+  for (const hipError_t e : results) {
+    if (e != hipSuccess) return e;
+  }
+  for (const void* kernel : {reinterpret_cast<const void*>(&IndexerSelectKernel), reinterpret_cast<const void*>(&IndexKeyAppendKernel)}) {
+    hipFuncAttributes attributes;
+    if (hipError_t e = hipFuncGetAttributes(&attributes, kernel); e != hipSuccess) return e;
+  }
+  once.state[device] = 1;
+  return hipSuccess;
+}
 
 hipError_t LaunchIndexKeyAppend(const IndexKeyAppendArgs& args, hipStream_t stream) {
   if (args.num_tokens <= 0) return hipSuccess;
@@ -471,6 +496,7 @@ hipError_t LaunchIndexKeyAppend(const IndexKeyAppendArgs& args, hipStream_t stre
 
 hipError_t LaunchIndexer(const IndexerArgs& args, hipStream_t stream) {
   if (args.batch <= 0) return hipSuccess;
+  if (hipError_t e = PrepareIndexerKernels(); e != hipSuccess) return e;
   const int groups = (args.max_seq_len + kTokensPerGroup - 1) / kTokensPerGroup;
   if (args.max_seq_len > args.sparse_count) {
     const dim3 grid(groups, args.batch);

@@ -210,8 +210,19 @@ struct IndexKeyAppendArgs {
   int32_t num_tokens;
 };
 hipError_t LaunchIndexKeyAppend(const IndexKeyAppendArgs& args, hipStream_t stream);
-// One-time per-process kernel attribute setup (dynamic LDS above 64 KB).
+// Per device, once: loads this file's kernels onto the current device and sets the attributes they
+// need (dynamic LDS above 64 KB), so that no first launch pays for it. Idempotent and cheap after
+// the first call on a device; the attention launcher calls its own, the others are for a caller's
+// warm-up (mlakvPrepare).
 hipError_t PrepareAttnKernels();
+hipError_t PreparePagedCopyKernels();
+hipError_t PrepareIndexerKernels();
+hipError_t PrepareMxQuantKernels();
+// Shared by the four: runs `prepare` once per device (the current one), remembering its result.
+struct PerDeviceOnce {
+  static constexpr int kMaxDevices = 64;
+  int state[kMaxDevices] = {};  // 0: not yet, 1: done; guarded by the caller's mutex
+};
 // Device memory owned by the library for the split-KV partials of attention launches whose
 // caller brings no workspace: kAttnStaticScratchBytes per GPU, resolved on first use on the
 // current device. Launches that use it on one GPU share it.

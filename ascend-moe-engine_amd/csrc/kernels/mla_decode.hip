@@ -1500,12 +1500,20 @@ __global__ __launch_bounds__(kMergeHeads * 64) void MlaMergeKernel(AttnArgs a) {
   MergeHead<MXQ, false>(a, z, seq, h, a.max_units + seq, first_unit, partials, lane);
 }
 
+// Dynamic LDS above 64 KB needs the attribute per kernel and device (PrepareAttnKernels).
+template <bool FP8, bool ALIGNED, bool MXQ, bool SPARSE>
+hipError_t PrepareDecode() {
+  return hipFuncSetAttribute(reinterpret_cast<const void*>(&MlaDecodeKernel<FP8, ALIGNED, MXQ, SPARSE>),
+                             hipFuncAttributeMaxDynamicSharedMemorySize, Geom<FP8>::kLdsBytes);
+}
+template <bool MXQ, bool SPARSE>
+hipError_t PrepareMerge() {
+  hipFuncAttributes attributes;
+  return hipFuncGetAttributes(&attributes, reinterpret_cast<const void*>(&MlaMergeKernel<MXQ, SPARSE>));
+}
+
 template <bool FP8, bool ALIGNED, bool MXQ, bool SPARSE>
 hipError_t Launch(const AttnArgs& args, const dim3& grid, hipStream_t stream) {
-  // Dynamic LDS above 64 KB needs the attribute once per kernel and process.
-  static const hipError_t prepared = hipFuncSetAttribute(reinterpret_cast<const void*>(&MlaDecodeKernel<FP8, ALIGNED, MXQ, SPARSE>),
-                                                         hipFuncAttributeMaxDynamicSharedMemorySize, Geom<FP8>::kLdsBytes);
-  if (prepared != hipSuccess) return prepared;
   hipLaunchKernelGGL((MlaDecodeKernel<FP8, ALIGNED, MXQ, SPARSE>), grid, dim3(kThreads), Geom<FP8>::kLdsBytes, stream, args);
   return hipGetLastError();
 }
@@ -1544,7 +1552,27 @@ hipError_t SyncRegion(unsigned** region) {
 
 }  // namespace
 
-hipError_t PrepareAttnKernels() { return hipSuccess; }
+hipError_t PrepareAttnKernels() {
+  static std::mutex guard;
+  static PerDeviceOnce once;
+  int device = 0;
+  if (hipError_t e = hipGetDevice(&device); e != hipSuccess) return e;
+  if (device < 0 || device >= PerDeviceOnce::kMaxDevices) return hipErrorInvalidDevice;
+  std::lock_guard<std::mutex> lock(guard);
+  if (once.state[device] == 1) return hipSuccess;
+  const hipError_t results[] = {
+      PrepareDecode<false, true, false, false>(), PrepareDecode<false, false, false, false>(),
+      PrepareDecode<true, true, false, false>(),  PrepareDecode<true, false, false, false>(),
+      PrepareDecode<false, true, true, false>(),  PrepareDecode<false, false, true, false>(),
+      PrepareDecode<true, true, true, false>(),   PrepareDecode<true, false, true, false>(),
+      PrepareDecode<false, false, false, true>(), PrepareDecode<true, false, false, true>(),
+      PrepareMerge<false, false>(), PrepareMerge<true, false>(), PrepareMerge<false, true>()};
+  for (const hipError_t e : results) {
+    if (e != hipSuccess) return e;
+  }
+  once.state[device] = 1;
+  return hipSuccess;
+}
 
 // Whether any sequence of the launch is cut into several work units, i.e. whether partials will be
 // written that the merge has to put together. The host can tell when it knows the token counts:
@@ -1582,6 +1610,7 @@ bool AnySequenceSplit(const AttnArgs& a) {
 hipError_t LaunchAttnDecode(const AttnArgs& args_in, hipStream_t stream) {
   AttnArgs args = args_in;
   if (args.batch <= 0) return hipSuccess;
+  if (hipError_t e = PrepareAttnKernels(); e != hipSuccess) return e;
   const int head_groups = (args.heads + 63) / 64;
   const bool merge_in_launch = args.merge_in_launch && static_cast<int64_t>(args.batch) * head_groups <= kAttnSyncSequences;
   args.sync = nullptr;

@@ -36,6 +36,11 @@ __global__ __launch_bounds__(256) void MxQuantKernel(MxQuantArgs q) {
 
 }  // namespace
 
+hipError_t PrepareMxQuantKernels() {
+  hipFuncAttributes attributes;  // (no attribute to set: the call only loads the kernel onto the current device)
+  return hipFuncGetAttributes(&attributes, reinterpret_cast<const void*>(&MxQuantKernel));
+}
+
 hipError_t LaunchMxQuant(const MxQuantArgs& args, hipStream_t stream) {
   if (args.rows <= 0 || args.cols <= 0) return hipSuccess;
   const int64_t items = args.rows * (args.cols >> 3);

@@ -7,6 +7,8 @@
 // access (global_load/store_dwordx4), so a 1024-byte latent row is exactly one wave access
 // and eight 128-byte rope rows are another. The block-table entry and all row bases are
 // wave-uniform, so the address arithmetic stays in scalar registers.
+#include <mutex>
+
 #include "kernels.h"
 
 #include <hip/hip_ext.h>
@@ -722,6 +724,28 @@ hipError_t LaunchCopyBlocks(const CopyBlocksArgs& args, hipStream_t stream) {
     return hipErrorInvalidValue;
   }
   return hipGetLastError();
+}
+
+hipError_t PreparePagedCopyKernels() {
+  static std::mutex guard;
+  static PerDeviceOnce once;
+  int device = 0;
+  if (hipError_t e = hipGetDevice(&device); e != hipSuccess) return e;
+  if (device < 0 || device >= PerDeviceOnce::kMaxDevices) return hipErrorInvalidDevice;
+  std::lock_guard<std::mutex> lock(guard);
+  if (once.state[device] == 1) return hipSuccess;
+  const void* kernels[] = {
+      reinterpret_cast<const void*>(&AppendBf16Kernel<NoStepWords>), reinterpret_cast<const void*>(&AppendBf16Kernel<StepWords>),
+      reinterpret_cast<const void*>(&AppendFp8Kernel<NoStepWords>),  reinterpret_cast<const void*>(&AppendFp8Kernel<StepWords>),
+      reinterpret_cast<const void*>(&GatherBf16TileKernel<kGatherTileRows>), reinterpret_cast<const void*>(&GatherBf16Kernel),
+      reinterpret_cast<const void*>(&GatherFp8Kernel), reinterpret_cast<const void*>(&CopyBlocksKernel<64, 8>),
+      reinterpret_cast<const void*>(&CopyBlocksKernel<32, 4>), reinterpret_cast<const void*>(&StoreWordsKernel)};
+  for (const void* kernel : kernels) {
+    hipFuncAttributes attributes;
+    if (hipError_t e = hipFuncGetAttributes(&attributes, kernel); e != hipSuccess) return e;
+  }
+  once.state[device] = 1;
+  return hipSuccess;
 }
 
 }  // namespace mlakv

@@ -40,10 +40,10 @@ class StaticMemoryArena {
   StaticMemoryArena& operator=(const StaticMemoryArena&) = delete;
 
   ArenaHandle Reserve(const char* name, size_t bytes, size_t align = kArenaAlignBytes);
-  size_t reserved_bytes() const { return cursor_; }
+  size_t reserved_bytes() const { return next_offset_; }
 
   void Commit();
-  bool committed() const { return arena_ != nullptr; }
+  bool committed() const { return phase_ != Phase::kReserve; }
   void* Address(ArenaHandle handle) const;
   template <typename T>
   T* AddressAs(ArenaHandle handle) const {
@@ -54,34 +54,40 @@ class StaticMemoryArena {
 
   void NoteWorkspace(uint64_t bytes);
   void CommitWorkspace();
-  void* workspace() const { return workspace_; }
-  uint64_t workspace_bytes() const { return workspace_bytes_; }
+  void* workspace() const { return scratch_.base; }
+  uint64_t workspace_bytes() const { return scratch_.bytes; }
   void AssertWorkspaceFits(uint64_t bytes, const char* what) const;
 
   void Seal();
-  bool sealed() const { return sealed_; }
+  bool sealed() const { return phase_ == Phase::kSealed; }
 
-  const std::vector<ArenaReservation>& reservations() const { return reservations_; }
-  size_t arena_bytes() const { return arena_bytes_; }
-  const void* arena_base() const { return arena_; }
+  const std::vector<ArenaReservation>& reservations() const { return ledger_; }
+  size_t arena_bytes() const { return pool_.bytes; }
+  const void* arena_base() const { return pool_.base; }
   IDeviceBackend& backend() const { return backend_; }
 
   void ValidateAlignment() const;
   std::string DescribeLedger() const;
 
  private:
-  void RefuseIfSealed(const char* what) const;
-  void RequireCommitted(const char* what) const;
+  // RESERVE until Commit, BUILD until Seal, SEALED for good: one value instead of a latch per edge.
+  enum class Phase { kReserve, kBuild, kSealed };
+  // One device allocation owned by the arena.
+  struct Block {
+    void* base = nullptr;
+    size_t bytes = 0;
+  };
+  void CheckNotSealed(const char* call) const;  // throws in Phase::kSealed
+  void CheckBuilt(const char* call) const;      // throws in Phase::kReserve
+  const ArenaReservation& Entry(ArenaHandle handle) const;
 
   IDeviceBackend& backend_;
-  std::vector<ArenaReservation> reservations_;
-  size_t cursor_ = 0;
-  void* arena_ = nullptr;
-  size_t arena_bytes_ = 0;
-  void* workspace_ = nullptr;
-  uint64_t workspace_bytes_ = 0;
-  uint64_t workspace_high_water_ = 0;
-  bool sealed_ = false;
+  Phase phase_ = Phase::kReserve;
+  std::vector<ArenaReservation> ledger_;  // in request order; a handle is an index into it
+  size_t next_offset_ = 0;                // where the next reservation would start, before alignment
+  Block pool_;                            // what Commit allocated
+  Block scratch_;                         // the operators' shared workspace (CommitWorkspace)
+  uint64_t scratch_wanted_ = 0;           // largest NoteWorkspace so far
 };
 
 }  // namespace moe_hip

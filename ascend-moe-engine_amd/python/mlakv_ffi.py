@@ -91,6 +91,7 @@ _P = C.POINTER
 PROTOTYPES = {
     "mlakvGetLastError": (C.c_char_p, []),
     "mlakvDeviceCount": (_i32, []),
+    "mlakvPrepare": (_i32, []),
     "mlakvAppend": (_i32, [_P(CacheView), _i32, _i32, _vp, _i64, _i64, _vp, _i64, _i64, _vp, _i32, _vp]),
     "mlakvNormRopeAppend": (_i32, [_P(CacheView), _i32, _vp, _i64, _vp, C.c_double, _vp, _vp, _i64, _vp, _vp, _i32, _vp, _i64,
                                    _vp, _i64, _vp, _i64, _i64, _i32, _vp]),

@@ -39,6 +39,12 @@ typedef int32_t mlakvStatus;
 const char* mlakvGetLastError(void);
 /* Number of HIP devices visible; 0 without a GPU. Never fails. */
 int32_t mlakvDeviceCount(void);
+/* Warm-up for the current device: loads every kernel of the library onto it and sets the kernel
+ * attributes the launches need (dynamic LDS above 64 KB), so that the first launch of each
+ * operator inside a serving loop costs what the later ones cost. Optional (every launch makes
+ * sure of its own kernels), idempotent, allocates no device memory, enqueues nothing. The
+ * counterpart of what the reference pays once in aclInit / aclnnInit (src/core/acl_guard.cpp:22-46). */
+mlakvStatus mlakvPrepare(void);
 
 /* ------------------------------------------------------------------------- */
 /* Paged cache geometry                                                       */
@@ -157,7 +163,14 @@ mlakvStatus mlakvCopyBlocks(const mlakvCacheView* cache, int32_t layer_begin, in
  * launch merges (MLAKV_ATTN_MERGE_SECOND_LAUNCH, the default) or the same launch does
  * (MLAKV_ATTN_MERGE_IN_LAUNCH: contributors meet on counters the library keeps in a static device
  * array, with a bounded wait; measured no faster on MI355X, kept for callers that want one
- * launch). seq_lens[b] is read as min(max(seq_lens[b], 0), max_seq_len). */
+ * launch). seq_lens[b] is read as min(max(seq_lens[b], 0), max_seq_len).
+ * Limits of MLAKV_ATTN_MERGE_IN_LAUNCH: the counters are 16 regions per GPU, handed to the launches
+ * of a process in turn. Launches that are ordered (one stream, or streams joined by events) can be
+ * of any number; of launches that may run side by side on unordered streams at most 16 may be in
+ * flight on one GPU, or two of them share counters and merge wrongly. A region's words are zero
+ * between launches because the last contributor of every sequence clears them: a launch that is
+ * torn down midway (device reset, process kill) leaves them as they are for the next user of that
+ * region in the same process. The second-launch merge has neither limit. */
 #define MLAKV_ATTN_MERGE_AUTO 0
 #define MLAKV_ATTN_MERGE_IN_LAUNCH 1
 #define MLAKV_ATTN_MERGE_SECOND_LAUNCH 2

@@ -37,14 +37,28 @@ def _no_alloc(cache, q, table, lens, max_seq_len):
     out = torch.full((batch, heads, LATENT), float("nan"), dtype=torch.bfloat16, device="cuda")
     lse = torch.full((batch, heads), float("nan"), dtype=torch.float32, device="cuda")
     row = (LATENT + ROPE) * 2
-    before = torch.cuda.memory_allocated()
-    status = lib.mlakvAttnDecodeNoAlloc(C.byref(plan), C.byref(cache.view), 0, q.data_ptr(), heads * row, row,
-                                        q.data_ptr() + LATENT * 2, heads * row, row, table.data_ptr(), table.shape[1],
-                                        lens.data_ptr(), float(SCALE), out.data_ptr(), heads * LATENT * 2, LATENT * 2,
-                                        lse.data_ptr(), kt.stream_ptr())
-    ffi.check(status)
-    assert torch.cuda.memory_allocated() == before
+    def call():
+        ffi.check(lib.mlakvAttnDecodeNoAlloc(C.byref(plan), C.byref(cache.view), 0, q.data_ptr(), heads * row, row,
+                                             q.data_ptr() + LATENT * 2, heads * row, row, table.data_ptr(), table.shape[1],
+                                             lens.data_ptr(), float(SCALE), out.data_ptr(), heads * LATENT * 2, LATENT * 2,
+                                             lse.data_ptr(), kt.stream_ptr()))
+    # Once untimed: the kernels are loaded onto the device and the static array's address is resolved
+    # (one-time set-up, which may take device memory for the code). Then the call is bracketed with
+    # the driver's own count of free device memory (hipMemGetInfo): a hipMalloc inside the library
+    # would lower it, whatever torch's allocator knows; torch's counter is watched as well.
+    ffi.check(lib.mlakvPrepare())
+    call()
     torch.cuda.synchronize()
+    out.fill_(float("nan"))
+    lse.fill_(float("nan"))
+    torch.cuda.synchronize()
+    free_before, _ = torch.cuda.mem_get_info()
+    allocated_before = torch.cuda.memory_allocated()
+    call()
+    torch.cuda.synchronize()
+    free_after, _ = torch.cuda.mem_get_info()
+    assert free_after == free_before, f"free device memory went from {free_before} to {free_after} bytes across the call"
+    assert torch.cuda.memory_allocated() == allocated_before
     return out, lse, plan
 
 
