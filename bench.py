@@ -92,6 +92,8 @@ def parse_args():
     p.add_argument("--config5-pool-gb", type=float, default=200.0, help="KV pool of the configs[4] loop, in GB (clamped to free memory)")
     p.add_argument("--attn-merge", choices=["auto", "in", "second"], default="auto",
                    help="development aid: how the attention launches merge their partials (default: the planner's choice)")
+    p.add_argument("--attn-chunk-tiles", type=int, default=0, help="development aid: fixed tiles per work unit of the attention launches")
+    p.add_argument("--attn-work-groups", type=int, default=0, help="development aid: workgroups per head group of the attention launches")
     p.add_argument("--attn-host-lens", action="store_true",
                    help="development aid: pass the lengths from the host (mlakvAttnDecodeHostLens) where the batch allows")
     p.add_argument("--split-out", action="store_true", help="gather into separate latent/rope planes instead of 576-wide rows")
@@ -297,8 +299,8 @@ def bench_attention(args, torch, np, ffi, ctxs, fp8=False, heads=64, slices=8, i
                         pool_blocks=pool_blocks, seed=7, shuffle=1, dtype=ffi.DTYPE_FP8_E4M3 if fp8 else ffi.DTYPE_BF16)
     plan = ffi.AttnPlan()
     merge_mode = {"auto": ffi.ATTN_MERGE_AUTO, "in": ffi.ATTN_MERGE_IN_LAUNCH, "second": ffi.ATTN_MERGE_SECOND_LAUNCH}[args.attn_merge]
-    if merge_mode != ffi.ATTN_MERGE_AUTO:
-        options = ffi.AttnPlanOptions(0, 0, merge_mode, 0, 1 if sparse_k else 0)
+    if merge_mode != ffi.ATTN_MERGE_AUTO or args.attn_chunk_tiles or args.attn_work_groups:
+        options = ffi.AttnPlanOptions(args.attn_chunk_tiles, args.attn_work_groups, merge_mode, 0, 1 if sparse_k else 0)
         ffi.check(lib.mlakvAttnPlanInitEx(batch, heads, sparse_k or max_ctx, bs, cache.config.dtype, C.byref(options), C.byref(plan)))
     elif sparse_k:
         ffi.check(lib.mlakvAttnSparsePlanInit(batch, heads, sparse_k, bs, cache.config.dtype, C.byref(plan)))
