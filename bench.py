@@ -29,9 +29,10 @@ sys.path.insert(0, os.path.join(ROOT, "ascend-moe-engine_amd", "python"))
 sys.path.insert(0, os.path.join(ROOT, "oracle"))
 
 # HBM bytes per algorithmic byte of the gather kernel, from two rocprofv3 --pmc runs of this file
-# (FETCH_SIZE scaled by 2.000, WRITE_SIZE by 1.000, the factors a plain 1 GiB copy gives):
-# (1956.8 + 1956.7) MB measured per dispatch against 3912.4 MB algorithmic.
-GATHER_TRAFFIC_PER_ALGORITHMIC_BYTE = 1.0003
+# (FETCH_SIZE scaled by 2.000, WRITE_SIZE by 1.000, the factors a plain 1 GiB copy gives; figures in
+# profiles/bench_hbm_counters.md): (1556.12 + 1555.98) MB measured for the dispatch of 31,411 rows x
+# 43 layers against 3112.04 MB algorithmic.
+GATHER_TRAFFIC_PER_ALGORITHMIC_BYTE = 1.0000
 HBM_PEAK_GBPS = 8000.0      # MI355X HBM3E, published
 MFMA_BF16_PEAK_TFLOPS = 2500.0
 LATENT, ROPE, ROW = 512, 64, 576
