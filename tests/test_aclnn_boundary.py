@@ -280,6 +280,10 @@ def test_no_device_fails_loudly_instead_of_falling_back():
     with pytest.raises(ffi.MlakvError) as info:
         ffi.Arena(ffi.BACKEND_HIP)
     assert "no HIP device" in str(info.value)
+    # the warm-up reports the runtime's error as a status; it does not pretend to have prepared anything
+    lib = ffi.load()
+    assert lib.mlakvPrepare() == ffi.ERR_RUNTIME
+    assert b"mlakvPrepare" in lib.mlakvGetLastError()
 
 
 def test_mx_quant_plan_contract():
