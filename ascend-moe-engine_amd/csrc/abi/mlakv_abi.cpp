@@ -334,6 +334,7 @@ mlakvStatus mlakvCopyBlocks(const mlakvCacheView* cache, int32_t layer_begin, in
 namespace {
 
 constexpr int32_t kDefaultMergeSpinUs = 50;
+static_assert(MLAKV_ATTN_HEAD_BLOCK_TOKENS == mlakv::kAttnHeadBlockTokens, "the header states the kernel's staging size");
 
 // The largest unit (in tiles) whose block-table entries fit the kernel's LDS staging whatever
 // the unit's offset inside a block; a selection stages one entry per selected token.
@@ -384,7 +385,8 @@ mlakvStatus AttnPlanImpl(const char* who, int32_t batch, int32_t heads, int32_t 
   mlakvAttnPlanOptions chosen{};
   if (options != nullptr) chosen = *options;
   if (chosen.chunk_tiles < 0 || chosen.work_groups < 0 || chosen.work_groups > 65535 || chosen.merge_mode < 0 ||
-      chosen.merge_mode > MLAKV_ATTN_MERGE_SECOND_LAUNCH || chosen.merge_spin_us > 1000000) {
+      chosen.merge_mode > MLAKV_ATTN_MERGE_SECOND_LAUNCH || chosen.merge_spin_us > 1000000 || chosen.selection_units < 0 ||
+      chosen.selection_units > MLAKV_ATTN_UNITS_HEAD_BLOCK || (!sparse && chosen.selection_units != 0)) {
     return Fail(MLAKV_ERR_PARAM_INVALID, "%s: options outside their ranges", who);
   }
   const int64_t head_groups = (heads + 63) / 64;
@@ -417,7 +419,23 @@ mlakvStatus AttnPlanImpl(const char* who, int32_t batch, int32_t heads, int32_t 
   plan->merge_mode = chosen.merge_mode == MLAKV_ATTN_MERGE_IN_LAUNCH && fits ? MLAKV_ATTN_MERGE_IN_LAUNCH : MLAKV_ATTN_MERGE_SECOND_LAUNCH;
   plan->merge_spin_us = chosen.merge_spin_us == 0 ? kDefaultMergeSpinUs : (chosen.merge_spin_us < 0 ? -1 : chosen.merge_spin_us);
   plan->reserved = sparse ? 1 : 0;
-  plan->reserved2 = 0;
+  // Whole-selection units of 16 heads where they apply, unless the caller asked for properties of
+  // the split (a unit size, a workgroup count, a merge).
+  const bool head_block_fits = sparse && dtype == MLAKV_DTYPE_BF16 && max_seq_len <= MLAKV_ATTN_HEAD_BLOCK_TOKENS;
+  if (chosen.selection_units == MLAKV_ATTN_UNITS_HEAD_BLOCK && !head_block_fits) {
+    return Fail(MLAKV_ERR_PARAM_INVALID, "%s: whole-selection units of 16 heads take a bf16 cache and up to %d selected tokens", who,
+                MLAKV_ATTN_HEAD_BLOCK_TOKENS);
+  }
+  const bool split_asked = chosen.chunk_tiles != 0 || chosen.work_groups != 0 || chosen.merge_mode != 0;
+  // Measured on MI355X (batch 4 .. 128, 64 and 128 heads): a whole-selection unit streams a tile per
+  // 0.8 us after 5.5 us of set-up, so with one unit per CU it is ahead of the split up to 512
+  // selected tokens (8.5 against 12 us at 64, 12 against 19 us at 256, level at 512), with two
+  // units per CU up to 256, and behind beyond that.
+  const int64_t rounds = (static_cast<int64_t>(batch) * (heads / 16) + ComputeUnits() - 1) / ComputeUnits();
+  const bool head_block_pays = (rounds <= 1 && max_seq_len <= 512) || (rounds <= 2 && max_seq_len <= 256);
+  const bool head_block = head_block_fits && (chosen.selection_units == MLAKV_ATTN_UNITS_HEAD_BLOCK ||
+                                              (chosen.selection_units == MLAKV_ATTN_UNITS_AUTO && !split_asked && head_block_pays));
+  plan->selection_units = !sparse ? 0 : (head_block ? MLAKV_ATTN_UNITS_HEAD_BLOCK : MLAKV_ATTN_UNITS_SPLIT);
   plan->workspace_bytes = shape.workspace;
   return MLAKV_SUCCESS;
 }
@@ -435,7 +453,7 @@ mlakvStatus mlakvAttnPlanInitEx(int32_t batch, int32_t heads, int32_t max_seq_le
                                 const mlakvAttnPlanOptions* options, mlakvAttnPlan* plan) {
   const bool selection = options != nullptr && options->selection != 0;
   if (options != nullptr && (options->selection < 0 || options->selection > 1 || options->reserved[0] != 0 ||
-                             options->reserved[1] != 0 || options->reserved[2] != 0)) {
+                             options->reserved[1] != 0)) {
     return Fail(MLAKV_ERR_PARAM_INVALID, "mlakvAttnPlanInitEx: options outside their ranges");
   }
   if (selection && (max_seq_len <= 0 || max_seq_len > 2048)) {
@@ -498,7 +516,11 @@ mlakvStatus AttnDecodeImpl(const char* who, const mlakvAttnPlan* plan, const mla
   {
     const bool fields = plan->batch > 0 && plan->batch <= 65535 && plan->heads > 0 && plan->heads % 16 == 0 && plan->heads <= 128 &&
                         plan->max_seq_len > 0 && plan->block_size > 0 && plan->chunk_tiles >= 0 && plan->work_groups >= 1 &&
-                        plan->work_groups <= 65535 && (plan->reserved == 0 || plan->reserved == 1) && plan->reserved2 == 0 &&
+                        plan->work_groups <= 65535 && (plan->reserved == 0 || plan->reserved == 1) &&
+                        (plan->reserved == 0 ? plan->selection_units == 0
+                                             : (plan->selection_units == MLAKV_ATTN_UNITS_SPLIT ||
+                                                (plan->selection_units == MLAKV_ATTN_UNITS_HEAD_BLOCK && plan->dtype == MLAKV_DTYPE_BF16 &&
+                                                 plan->max_seq_len <= MLAKV_ATTN_HEAD_BLOCK_TOKENS))) &&
                         (plan->reserved == 0 || plan->max_seq_len <= 2048) &&
                         (plan->merge_mode == MLAKV_ATTN_MERGE_IN_LAUNCH || plan->merge_mode == MLAKV_ATTN_MERGE_SECOND_LAUNCH) &&
                         (plan->merge_spin_us == -1 || (plan->merge_spin_us > 0 && plan->merge_spin_us <= 1000000));
@@ -601,6 +623,7 @@ mlakvStatus AttnDecodeImpl(const char* who, const mlakvAttnPlan* plan, const mla
   args.spin_ticks = plan->merge_spin_us < 0 ? 0 : plan->merge_spin_us * 100;
   args.merge_in_launch = plan->merge_mode == MLAKV_ATTN_MERGE_IN_LAUNCH;
   args.fp8 = cache->dtype == MLAKV_DTYPE_FP8_E4M3;
+  args.head_block_units = plan->selection_units == MLAKV_ATTN_UNITS_HEAD_BLOCK;
   const hipError_t status = mlakv::LaunchAttnDecode(args, static_cast<hipStream_t>(stream));
   return status == hipSuccess ? MLAKV_SUCCESS : HipFail(status, who);
 }

@@ -127,6 +127,9 @@ struct AttnArgs {
   int32_t spin_ticks;         // bound of the in-launch merge's wait, in 10 ns ticks
   bool merge_in_launch;       // false: the merge is a second launch
   bool fp8;
+  // Selected-token attention only: a workgroup takes the whole selection of one sequence for one
+  // block of 16 heads (no partials, no merge); sparse_count <= kAttnHeadBlockTokens, bf16 cache.
+  bool head_block_units;
   unsigned* sync;             // set by the launcher: this launch's counters, null for a second-launch merge
   // Host-known lengths of a small batch travel here instead of through device memory: no upload,
   // no launch for it, and the kernels' first dependent load is gone. inline_count = 0: unused.
@@ -173,6 +176,7 @@ constexpr int kTileTokens = 32;
 constexpr int kAttnTableEntries = 512;     // block-table entries (or selected tokens) of one segment staged in LDS
 constexpr int kAttnBoundaryTiles = 4;      // what entering a sequence inside a work unit costs, in tiles (see MakeCut)
 constexpr int kAttnSyncSequences = 4096;   // (head group, sequence) pairs a launch can merge in place
+constexpr int kAttnHeadBlockTokens = 1024; // selected tokens a whole-sequence unit of 16 heads stages in LDS
 
 hipError_t LaunchAppend(const AppendArgs& args, hipStream_t stream);
 hipError_t LaunchNormRopeAppend(const NormRopeAppendArgs& args, hipStream_t stream);

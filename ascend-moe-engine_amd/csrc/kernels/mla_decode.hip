@@ -79,6 +79,7 @@ typedef __attribute__((ext_vector_type(2))) unsigned int u32x2;
 typedef __attribute__((ext_vector_type(4))) short s16x4;
 typedef __attribute__((ext_vector_type(8))) short s16x8;
 typedef __attribute__((ext_vector_type(2))) int i32x2;
+typedef unsigned long long u64;
 
 constexpr int kThreads = 512;
 constexpr int kWaves = kThreads / 64;
@@ -385,6 +386,47 @@ __device__ __forceinline__ bool IssueTileBf16(const AttnArgs& a, TileMap<ALIGNED
   return false;
 }
 
+// Selected-token tiles whose rows are all rows of the pool (no bad table entry among the staged
+// (block << slot_bits) | slot entries): the first P waves of the workgroup fetch the tile, wave w
+// the latent rows w, w + P, ... and eight rope rows (waves 4..7 for P = 8, as in IssueTileBf16,
+// every wave for P = 4), one rope row per eight lanes. No case distinction and no scalar address
+// chain: every lane forms the address of its 16 bytes itself, in units of 16 bytes with 24-bit
+// multiplies (PlainRowsAddressable says when that is exact). Entry `first + row` belongs to row
+// `row` of the tile; rows behind `last` repeat entry `last` (finite values that the softmax masks).
+__host__ __device__ __forceinline__ bool PlainRowsAddressable(const AttnArgs& a) {
+  const int64_t limit = int64_t{1} << 28;  // strides in 16-byte units below 2^24
+  return a.latent.block_stride < limit && a.rope.block_stride < limit && a.latent.row_stride < limit && a.rope.row_stride < limit &&
+         a.num_blocks <= (1 << 24) && a.num_blocks * a.latent.block_stride <= (int64_t{1} << 36) &&
+         a.num_blocks * a.rope.block_stride <= (int64_t{1} << 36);
+}
+template <int P>
+__device__ __forceinline__ void IssuePlainRowsBf16(const AttnArgs& a, const int* entries, int first, int last, int slot_bits, unsigned buf,
+                                                   int lane, int wave) {
+  using G = Geom<false>;
+  constexpr int kRows = kTileTokens / P;
+  const int rope_group = P == 4 ? wave : wave - kScoreWaves;
+  if (wave >= P) return;
+  const unsigned slot_mask = (1u << slot_bits) - 1u;
+  const unsigned lat_block16 = static_cast<unsigned>(a.latent.block_stride >> 4), lat_row16 = static_cast<unsigned>(a.latent.row_stride >> 4);
+  unsigned packed[kRows];
+#pragma unroll
+  for (int r = 0; r < kRows; ++r) packed[r] = static_cast<unsigned>(entries[min(first + wave + P * r, last)]);
+  unsigned rope_packed = 0u;
+  if (rope_group >= 0) rope_packed = static_cast<unsigned>(entries[min(first + 8 * rope_group + (lane >> 3), last)]);
+#pragma unroll
+  for (int r = 0; r < kRows; ++r) {
+    const int row = wave + P * r;
+    const unsigned off16 = __umul24(packed[r] >> slot_bits, lat_block16) + __umul24(packed[r] & slot_mask, lat_row16);
+    DirectLoad16PerLane(a.latent.base + (static_cast<u64>(off16) << 4) + ((lane ^ SwizzleLat(row)) << 4), buf + row * G::kLatRow);
+  }
+  if (rope_group >= 0) {
+    const unsigned rope_block16 = static_cast<unsigned>(a.rope.block_stride >> 4), rope_row16 = static_cast<unsigned>(a.rope.row_stride >> 4);
+    const unsigned off16 = __umul24(rope_packed >> slot_bits, rope_block16) + __umul24(rope_packed & slot_mask, rope_row16);
+    const int chunk = ((lane & 7) ^ SwizzleRope(8 * rope_group + (lane >> 3))) << 4;
+    DirectLoad16PerLane(a.rope.base + (static_cast<u64>(off16) << 4) + chunk, buf + G::kLatRegion + rope_group * 8 * G::kRopeRow);
+  }
+}
+
 // ---- FP8 tiles: direct global -> LDS, codes and row scales as they are in the cache -------------
 
 // Wave w of 8 owns the latent row pairs {2w, 2w+1} and {16+2w, 17+2w} (a 512-byte row is half a
@@ -479,8 +521,6 @@ __device__ __forceinline__ bf16x8 CodesToBf16(unsigned lo, unsigned hi) {
 // full. Waiting is bounded, and a share whose owner gave up (or has not claimed it by then) is
 // taken by the contributor that arrived last, so the launch finishes whatever the order in which
 // workgroups get to run.
-
-typedef unsigned long long u64;
 
 constexpr int kMergeHeads = 8;   // heads of one merge step: one per wave
 
@@ -1500,6 +1540,338 @@ __global__ __launch_bounds__(kMergeHeads * 64) void MlaMergeKernel(AttnArgs a) {
   MergeHead<MXQ, false>(a, z, seq, h, a.max_units + seq, first_unit, partials, lane);
 }
 
+// ---- selected-token attention in whole-sequence units of 16 heads ----------------------------
+//
+// A selection of a few hundred tokens is a dozen tiles. Cut into one unit per CU it is all fixed
+// cost: every workgroup fetches the 72-KB query of 64 heads for its two or three tiles and leaves
+// 64 KB of partials that a second launch reads back. Here a workgroup takes the whole selection
+// of one sequence for one block of 16 heads: an 18-KB query, no partials, no merge, the output
+// written once. The head blocks of a sequence run on one XCD at the same time, so the rows they
+// all read come from HBM once and from that L2 afterwards. Eight waves in two roles:
+//   score waves 0..3 fetch the tiles (the output waves' work per tile is the longer chain, so they
+//     issue no loads); wave (t, kh) multiplies token subtile t of the tile (16 tokens) with one
+//     half of the 18 k-steps for the 16 heads and leaves its 16 x 16 partial of S^T in LDS, one
+//     tile ahead of
+//   output waves 4..7, each of which adds the partials, runs the online softmax of all 16 heads
+//     itself (every output wave the same arithmetic on the same numbers, so the four agree on the
+//     reference maximum without exchanging it), forms P in registers as its MFMA operand and
+//     multiplies it with its 128 columns of V.
+// The tile ring, the operand layouts and the barrier per tile are those of the kernel above.
+constexpr int kHbWaves = kWaves, kHbThreads = kHbWaves * 64;
+constexpr int kHbLoaders = kScoreWaves;  // the waves that fetch the tiles when every row is a plain row
+struct GeomHeadBlock {
+  using T = Geom<false>;
+  static constexpr int kRing = 4;
+  static constexpr int kTableOff = kRing * T::kTileBytes;                          // int[kAttnHeadBlockTokens]: (block << slot_bits) | slot
+  static constexpr int kSOff = kTableOff + kAttnHeadBlockTokens * 4;               // S^T partials [2][4 waves][64 lanes] x 16 B
+  static constexpr int kEndOff = kSOff;  // int[2][kHbWaves], before the first S is written: where each wave saw the selection end, and whether it saw a bad table entry
+  static constexpr int kLdsBytes = kSOff + 2 * kScoreWaves * 64 * 16;
+  static_assert(kLdsBytes <= 160 * 1024, "one workgroup owns the LDS of a CU");
+  __device__ static __forceinline__ int Slot(int i) { return (i & 3) * T::kTileBytes; }
+};
+constexpr int kHeadBlockKSteps = kKSteps / 2;  // k-steps of one score wave
+
+__global__ __launch_bounds__(kHbThreads) void MlaSelectedHeadBlockKernel(AttnArgs a) {
+  using G = GeomHeadBlock;
+  using T = Geom<false>;
+  extern __shared__ __attribute__((aligned(16))) unsigned char lds[];
+  const unsigned lds_base = static_cast<unsigned>(reinterpret_cast<size_t>((__attribute__((address_space(3))) unsigned char*)lds));
+  const int tid = threadIdx.x;
+  const int lane = tid & 63, wave = Uniform(tid >> 6);
+  // Workgroups go to the XCDs round-robin by linear id: ids x, x + 8, x + 16, ... share XCD x, and
+  // the head blocks of a sequence are neighbours among them.
+  const int head_blocks = a.heads >> 4;  // heads is a multiple of 16
+  const int rest = blockIdx.x >> 3;
+  const int hb = rest % head_blocks;
+  const int seq = (rest / head_blocks) * kXcds + (blockIdx.x & (kXcds - 1));
+  if (seq >= a.batch) return;
+  const bool score_wave = wave < kScoreWaves;
+  const int hw = wave & (kScoreWaves - 1);
+  const int g = lane >> 4, i16 = lane & 15;
+  const int head = 16 * hb + i16;
+
+  // The selection ends at its first entry that is negative or not inside the context. Every
+  // thread resolves one or two entries to pool slots through the block table; the loads that the
+  // first tile's addresses depend on go out first, the query behind them.
+  int* table_lds = reinterpret_cast<int*>(lds + G::kTableOff);
+  int* end_lds = reinterpret_cast<int*>(lds + G::kEndOff);
+  const int context = static_cast<int>(
+      min(static_cast<int64_t>(max(Uniform(LiveLength(a, seq)), 0)), static_cast<int64_t>(a.table_stride) * a.block_size));
+  const int32_t* selection = a.sparse_indices + static_cast<int64_t>(seq) * a.sparse_seq_stride;
+  const int32_t* table_row = a.block_table + static_cast<int64_t>(seq) * a.table_stride;
+  const int slot_bits = a.block_size > 1 ? 32 - __builtin_clz(static_cast<unsigned>(a.block_size - 1)) : 0;
+  constexpr int kPerThread = (kAttnHeadBlockTokens + kHbThreads - 1) / kHbThreads;
+  int index[kPerThread];
+#pragma unroll
+  for (int j = 0; j < kPerThread; ++j) {
+    const int i = tid + kHbThreads * j;
+    index[j] = i < a.sparse_count ? selection[i] : -1;
+  }
+  // Q fragments of a score wave: lane (head i16, k-group g) holds Q[head][32 ks + 8 g .. +7] for the
+  // nine k-steps ks of its half.
+  bf16x8 q[kHeadBlockKSteps];
+  if (score_wave) {
+    const int kh = hw >> 1;
+    const char* q_latent = a.q_latent + seq * a.q_latent_seq_stride + head * a.q_latent_head_stride;
+    const char* q_rope = a.q_rope + seq * a.q_rope_seq_stride + head * a.q_rope_head_stride;
+#pragma unroll
+    for (int c = 0; c < kHeadBlockKSteps; ++c) {
+      const int d0 = 32 * (kHeadBlockKSteps * kh + c) + 8 * g;
+      const char* p = d0 < kLatentDim ? q_latent + d0 * 2 : q_rope + (d0 - kLatentDim) * 2;
+      q[c] = __builtin_bit_cast(bf16x8, GlobalLoad16(p));
+    }
+  } else {
+#pragma unroll
+    for (int c = 0; c < kHeadBlockKSteps; ++c) q[c] = __builtin_bit_cast(bf16x8, u32x4{0u, 0u, 0u, 0u});
+  }
+  int wave_end = a.sparse_count;
+  bool any_outside = false;  // a selected token behind a block-table entry that is not a block of the pool
+  const bool shift = (a.block_size & (a.block_size - 1)) == 0;
+#pragma unroll
+  for (int j = 0; j < kPerThread; ++j) {
+    const int i = tid + kHbThreads * j;
+    const bool good = index[j] >= 0 && index[j] < context;  // false behind the list's end as well
+    const u64 bad = __builtin_amdgcn_ballot_w64(!good);
+    if (bad != 0) wave_end = min(wave_end, kHbThreads * j + 64 * wave + static_cast<int>(__builtin_ctzll(bad)));
+    if (good && i < kAttnHeadBlockTokens) {
+      const int logical = shift ? index[j] >> slot_bits : index[j] / a.block_size;
+      const int entry = table_row[logical];
+      const bool inside = static_cast<unsigned>(entry) < static_cast<unsigned>(a.num_blocks);
+      table_lds[i] = inside ? (entry << slot_bits) | (index[j] - logical * a.block_size) : -1;
+      if (!inside) any_outside = true;
+    }
+  }
+  if (lane == 0) {
+    end_lds[wave] = wave_end;
+    end_lds[kHbWaves + wave] = __builtin_amdgcn_ballot_w64(any_outside) != 0 ? 1 : 0;
+  }
+  // Every role passes this statement with the query in hand: a wait of the compiler's for it further
+  // down would not know of the tile loads issued from inline assembly, and would wait for them all.
+#pragma unroll
+  for (int c = 0; c < kHeadBlockKSteps; ++c) asm volatile("" ::"v"(q[c]));
+  __syncthreads();
+  int seq_len = a.sparse_count, outside = 0;
+#pragma unroll
+  for (int w = 0; w < kHbWaves; ++w) {
+    seq_len = min(seq_len, end_lds[w]);
+    outside |= end_lds[kHbWaves + w];
+  }
+  seq_len = Uniform(seq_len);
+  // Every row a real row of the pool (the usual case) and strides that the per-lane address
+  // arithmetic covers: the score waves fetch the tiles; otherwise all eight waves do, one row at a
+  // time.
+  const bool plain_rows = Uniform(outside) == 0 && PlainRowsAddressable(a);
+  const int ntiles = (seq_len + kTileTokens - 1) / kTileTokens;
+  if (ntiles == 0) {  // nothing selected: zeros, lse = -inf
+    for (int h = wave; h < 16; h += kHbWaves) {
+      *reinterpret_cast<u32x4*>(a.out + seq * a.out_seq_stride + (16 * hb + h) * a.out_head_stride + lane * 16) = u32x4{0u, 0u, 0u, 0u};
+      if (a.lse != nullptr && lane == 0) a.lse[seq * a.heads + 16 * hb + h] = -__builtin_inff();
+    }
+    return;
+  }
+
+  TileMap<false> map;
+  map.entries = table_lds;
+  map.first_block = 0;
+  map.block_size = a.block_size;
+  map.seq_len = seq_len;
+  map.sparse = true;
+  map.first_pos = 0;
+  map.slot_bits = slot_bits;
+  map.tile_block = map.tile_slot0 = map.next_entry = map.next_slot0 = 0;
+  IssueLane il;
+  il.lat[0] = il.lat[1] = il.partner_lat[0] = il.partner_lat[1] = 0;  // (the row-at-a-time path forms these itself)
+  il.rope_chunk = ((lane & 7) ^ SwizzleRope(8 * (wave - kScoreWaves) + (lane >> 3))) << 4;
+  il.rope = 0;
+  // The head blocks of a sequence walk its tiles from different starting points (the order of the
+  // tiles only changes the rounding): at any time they ask for different rows, and what one has
+  // fetched the others find in the L2.
+  const int rotate = hb * ntiles / head_blocks;
+  const auto tile_of = [&](int i) __attribute__((always_inline)) { return i + rotate < ntiles ? i + rotate : i + rotate - ntiles; };
+  constexpr int kPlainLoads = kTileTokens / kHbLoaders + 1;  // a loader wave's loads per tile: eight latent rows and eight rope rows
+  const int per_tile = plain_rows ? (wave < kHbLoaders ? kPlainLoads : 0) : LoadsPerTile(wave);
+  int last_unknown = -1;  // newest tile issued with an unknown number of loads (a row that is not real)
+  int issued = 0;
+  const auto issue_next = [&]() __attribute__((always_inline)) {
+    if (issued < ntiles) {
+      if (plain_rows) {
+        IssuePlainRowsBf16<kHbLoaders>(a, table_lds, tile_of(issued) * kTileTokens, seq_len - 1, slot_bits, lds_base + G::Slot(issued), lane, wave);
+      } else if (!IssueTileBf16<false>(a, map, il, tile_of(issued), lds_base + G::Slot(issued), lds + G::Slot(issued), tid)) {
+        last_unknown = issued;
+      }
+      ++issued;
+    }
+  };
+  // Waits until tile t has landed: this wave's loads of the tiles issued after it may stay in flight
+  // (at most one tile here: the ring holds the tile in use, the next one and two on their way).
+  const auto wait_tile = [&](int t) __attribute__((always_inline)) {
+    if (per_tile == 0) return;
+    const int newer = last_unknown >= t ? 0 : max(0, issued - (t + 1)) * per_tile;
+    if (newer == 0) {
+      asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+    } else if (newer == kPlainLoads) {
+      asm volatile("s_waitcnt vmcnt(%0)" ::"n"(kPlainLoads) : "memory");
+    } else {
+      WaitLoads(newer);
+    }
+  };
+  // Top of iteration i, both roles: tile i + 1 has landed; the barrier publishes it together with
+  // S(i) and retires every wave's reads of tile i - 1, whose ring slot the next tile reuses.
+  const auto publish = [&](int i) __attribute__((always_inline)) {
+    if (i + 1 < ntiles) wait_tile(i + 1);
+    __syncthreads();
+  };
+  for (int t = 0; t < G::kRing - 1; ++t) issue_next();
+  wait_tile(0);
+  __syncthreads();
+
+  f32x4* s_lds = reinterpret_cast<f32x4*>(lds + G::kSOff) + lane;  // + (parity * kScoreWaves + score wave) * 64
+  if (score_wave) {
+    // ------------------------------------------------------------------ score waves
+    const int t = hw & 1;
+    const int k_lat = (16 * t + i16) * T::kLatRow, k_rope = T::kLatRegion + (16 * t + i16) * T::kRopeRow;
+    int k_e[4], kr_e[2];
+#pragma unroll
+    for (int j = 0; j < 4; ++j) k_e[j] = ((4 * j + g) ^ SwizzleLat(i16)) << 4;
+#pragma unroll
+    for (int j = 0; j < 2; ++j) kr_e[j] = ((4 * j + g) ^ SwizzleRope(i16)) << 4;
+    const auto score_tile = [&](int tile, auto kh_c) __attribute__((always_inline)) {
+      constexpr int kh = decltype(kh_c)::value;
+      const unsigned char* buf = lds + G::Slot(tile);
+      bf16x8 kf[kHeadBlockKSteps];
+      StaticFor<kHeadBlockKSteps>([&](auto c_c) __attribute__((always_inline)) {
+        constexpr int c = decltype(c_c)::value, ks = kHeadBlockKSteps * kh + c;
+        const int offset = ks < 16 ? k_lat + (ks >> 2) * 256 + k_e[ks & 3] : k_rope + kr_e[ks & 1];
+        kf[c] = *reinterpret_cast<const bf16x8*>(buf + offset);
+      });
+      f32x4 acc[3];
+#pragma unroll
+      for (int j = 0; j < 3; ++j) acc[j] = f32x4{0.f, 0.f, 0.f, 0.f};
+      StaticFor<kHeadBlockKSteps>([&](auto c_c) __attribute__((always_inline)) {
+        constexpr int c = decltype(c_c)::value;
+        acc[c % 3] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(kf[c], q[c], acc[c % 3], 0, 0, 0);
+      });
+      s_lds[((tile & 1) * kScoreWaves + hw) * 64] = acc[0] + acc[1] + acc[2];
+    };
+    const bool upper = (hw >> 1) != 0;  // wave-uniform: which half of the k-steps
+    const auto score = [&](int tile) __attribute__((always_inline)) {
+      if (upper) {
+        score_tile(tile, std::integral_constant<int, 1>{});
+      } else {
+        score_tile(tile, std::integral_constant<int, 0>{});
+      }
+    };
+    score(0);
+    for (int i = 0; i < ntiles; ++i) {
+      publish(i);
+      issue_next();
+      if (i + 1 < ntiles) score(i + 1);
+    }
+    __syncthreads();  // every output wave is through with the last tile (the ring becomes their staging space)
+  } else {
+    // ------------------------------------------------------------------ output waves
+    // bf16 V reads as in the kernel above: token = (16 +) 4g + i16/4, chunk = 2n + (i16 & 3) / 2, 8-byte half i16 & 1.
+    const int v_row = 4 * g + (i16 >> 2);
+    const int v_lane = v_row * T::kLatRow + (i16 & 1) * 8;
+    int v_e[8];
+#pragma unroll
+    for (int j = 0; j < 8; ++j) v_e[j] = ((2 * j + ((i16 & 3) >> 1)) ^ SwizzleLat(v_row)) << 4;
+    const auto v_fetch = [&](const unsigned char* buf, int n) __attribute__((always_inline)) {
+      const unsigned char* addr = buf + v_lane + (n >> 3) * 256 + v_e[n & 7];
+      const s16x4 lo = __builtin_amdgcn_ds_read_tr16_b64_v4i16((__attribute__((address_space(3))) s16x4*)(addr));
+      const s16x4 hi = __builtin_amdgcn_ds_read_tr16_b64_v4i16((__attribute__((address_space(3))) s16x4*)(addr + 16 * T::kLatRow));
+      return __builtin_bit_cast(bf16x8, __builtin_shufflevector(lo, hi, 0, 1, 2, 3, 4, 5, 6, 7));
+    };
+    constexpr int kDvPerWave = kDvTiles / (kWaves - kScoreWaves);  // 8 column tiles: columns [128 hw, 128 hw + 128)
+    f32x4 o[kDvPerWave];
+#pragma unroll
+    for (int n = 0; n < kDvPerWave; ++n) o[n] = f32x4{0.f, 0.f, 0.f, 0.f};
+    float m_ref = -__builtin_inff();  // reference maximum of the exponentials, log2 domain
+    float l_run = 0.0f;               // this lane's share of the running denominator
+
+    for (int i = 0; i < ntiles; ++i) {
+      publish(i);
+      issue_next();
+      const unsigned char* buf = lds + G::Slot(i);
+      const f32x4* s = s_lds + (i & 1) * kScoreWaves * 64;
+      const f32x4 s0 = s[0], s1 = s[64], s2 = s[128], s3 = s[192];
+      bf16x8 vf[kDvPerWave];
+      StaticFor<kDvPerWave>([&](auto n_c) __attribute__((always_inline)) {
+        constexpr int n = decltype(n_c)::value;
+        vf[n] = v_fetch(buf, kDvPerWave * hw + n);
+      });
+      // lane holds tokens 4g+j (x[0..3]) and 16+4g+j (x[4..7]) of head i16
+      float x[8];
+#pragma unroll
+      for (int j = 0; j < 4; ++j) {
+        x[j] = (s0[j] + s2[j]) * a.scale_log2;
+        x[4 + j] = (s1[j] + s3[j]) * a.scale_log2;
+      }
+      const int valid = seq_len - tile_of(i) * kTileTokens;  // >= 1
+      if (valid < kTileTokens) {                             // only the last tile of the selection
+#pragma unroll
+        for (int j = 0; j < 8; ++j) {
+          if (16 * (j >> 2) + 4 * g + (j & 3) >= valid) x[j] = -__builtin_inff();
+        }
+      }
+      float tile_max = fmaxf(fmaxf(fmaxf(x[0], x[1]), fmaxf(x[2], x[3])), fmaxf(fmaxf(x[4], x[5]), fmaxf(x[6], x[7])));
+      tile_max = MaxAcrossHalves(MaxAcrossRows16(tile_max));
+      // Move the reference only when some head's maximum outgrew it by more than the threshold.
+      if (__builtin_amdgcn_ballot_w64(tile_max > m_ref + kRescaleThreshold) != 0) {
+        const float m_new = fmaxf(m_ref, tile_max);  // finite: token 0 of the tile is valid
+        const float alpha = __builtin_amdgcn_exp2f(m_ref - m_new);
+        l_run *= alpha;
+        m_ref = m_new;
+        if (i != 0) {  // O is still zero on the first tile (and alpha is exp2(-inf - m) there)
+#pragma unroll
+          for (int n = 0; n < kDvPerWave; ++n) o[n] *= alpha;
+        }
+      }
+      bf16x8 p;
+      float sum = 0.0f;
+#pragma unroll
+      for (int j = 0; j < 8; ++j) {
+        const float e = __builtin_amdgcn_exp2f(x[j] - m_ref);
+        sum += e;
+        p[j] = static_cast<__bf16>(e);
+      }
+      l_run += sum;
+      StaticFor<kDvPerWave>([&](auto n_c) __attribute__((always_inline)) {
+        constexpr int n = decltype(n_c)::value;
+        o[n] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(vf[n], p, o[n], 0, 0, 0);
+      });
+    }
+    __syncthreads();  // every output wave is through with the last tile
+    const float l_total = SumAcrossHeadLanes(l_run);
+    const float inv = 1.0f / l_total;
+    if (hw == 0 && g == 0 && a.lse != nullptr) {
+      a.lse[seq * a.heads + head] = (m_ref + __builtin_amdgcn_logf(l_total)) * 0.6931471805599453f;  // v_log_f32 is log2
+    }
+    // The accumulators hold O^T (lane = head i16, four columns per 16-column tile); each wave turns
+    // its 256-byte slices of the 16 rows through its own part of the dead ring (row stride 272 B)
+    // and writes them 16 bytes per lane, four whole slices per instruction.
+    constexpr int kSliceBytes = kDvPerWave * 16 * 2;  // 256
+    constexpr int kStageRow = kSliceBytes + 16;
+    unsigned char* stage = lds + G::Slot(0) + hw * (16 * kStageRow);
+#pragma unroll
+    for (int n = 0; n < kDvPerWave; ++n) {
+      u32x2 packed;
+      packed.x = PackBf16(o[n][0] * inv, o[n][1] * inv);
+      packed.y = PackBf16(o[n][2] * inv, o[n][3] * inv);
+      *reinterpret_cast<u32x2*>(stage + i16 * kStageRow + (16 * n + 4 * g) * 2) = packed;
+    }
+    // Same wave wrote and reads: the LDS queue is in order, no barrier needed.
+    const int piece = lane & 15, sub = lane >> 4;
+    char* out0 = a.out + seq * a.out_seq_stride + (16 * hb) * a.out_head_stride + kSliceBytes * hw + piece * 16;
+#pragma unroll
+    for (int it = 0; it < 4; ++it) {
+      const int h = 4 * it + sub;
+      const u32x4 v = *reinterpret_cast<const u32x4*>(stage + h * kStageRow + piece * 16);
+      __builtin_nontemporal_store(v, reinterpret_cast<u32x4*>(out0 + h * a.out_head_stride));
+    }
+  }
+}
+
 // Dynamic LDS above 64 KB needs the attribute per kernel and device (PrepareAttnKernels).
 template <bool FP8, bool ALIGNED, bool MXQ, bool SPARSE>
 hipError_t PrepareDecode() {
@@ -1566,7 +1938,9 @@ hipError_t PrepareAttnKernels() {
       PrepareDecode<false, true, true, false>(),  PrepareDecode<false, false, true, false>(),
       PrepareDecode<true, true, true, false>(),   PrepareDecode<true, false, true, false>(),
       PrepareDecode<false, false, false, true>(), PrepareDecode<true, false, false, true>(),
-      PrepareMerge<false, false>(), PrepareMerge<true, false>(), PrepareMerge<false, true>()};
+      PrepareMerge<false, false>(), PrepareMerge<true, false>(), PrepareMerge<false, true>(),
+      hipFuncSetAttribute(reinterpret_cast<const void*>(&MlaSelectedHeadBlockKernel), hipFuncAttributeMaxDynamicSharedMemorySize,
+                          GeomHeadBlock::kLdsBytes)};
   for (const hipError_t e : results) {
     if (e != hipSuccess) return e;
   }
@@ -1627,6 +2001,13 @@ hipError_t LaunchAttnDecode(const AttnArgs& args_in, hipStream_t stream) {
     int slot_bits = 0;
     while ((int64_t{1} << slot_bits) < args.block_size) ++slot_bits;
     if ((static_cast<int64_t>(args.num_blocks) << slot_bits) > (int64_t{1} << 31)) return hipErrorInvalidValue;
+    if (args.head_block_units) {
+      if (args.fp8 || args.sparse_count > kAttnHeadBlockTokens || args.heads % 16 != 0 || args.out == nullptr) return hipErrorInvalidValue;
+      const int sequences_per_xcd = (args.batch + kXcds - 1) / kXcds;
+      const dim3 units(kXcds * (args.heads / 16) * sequences_per_xcd);
+      hipLaunchKernelGGL(MlaSelectedHeadBlockKernel, units, dim3(kHbThreads), GeomHeadBlock::kLdsBytes, stream, args);
+      return hipGetLastError();
+    }
     e = args.fp8 ? Launch<true, false, false, true>(args, grid, stream) : Launch<false, false, false, true>(args, grid, stream);
   } else {
     e = quantise ? LaunchByCache<true>(args, grid, stream) : LaunchByCache<false>(args, grid, stream);

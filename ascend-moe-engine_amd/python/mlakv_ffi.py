@@ -55,17 +55,19 @@ class AttnPlan(C.Structure):
     _fields_ = [
         ("batch", C.c_int32), ("heads", C.c_int32), ("max_seq_len", C.c_int32), ("block_size", C.c_int32),
         ("dtype", C.c_int32), ("chunk_tiles", C.c_int32), ("work_groups", C.c_int32), ("max_units", C.c_int32),
-        ("merge_mode", C.c_int32), ("merge_spin_us", C.c_int32), ("reserved", C.c_int32), ("reserved2", C.c_int32),
+        ("merge_mode", C.c_int32), ("merge_spin_us", C.c_int32), ("reserved", C.c_int32), ("selection_units", C.c_int32),
         ("workspace_bytes", C.c_uint64),
     ]
 
 
 class AttnPlanOptions(C.Structure):
     _fields_ = [("chunk_tiles", C.c_int32), ("work_groups", C.c_int32), ("merge_mode", C.c_int32), ("merge_spin_us", C.c_int32),
-                ("selection", C.c_int32), ("reserved", C.c_int32 * 3)]
+                ("selection", C.c_int32), ("selection_units", C.c_int32), ("reserved", C.c_int32 * 2)]
 
 
 ATTN_MERGE_AUTO, ATTN_MERGE_IN_LAUNCH, ATTN_MERGE_SECOND_LAUNCH = 0, 1, 2
+ATTN_UNITS_AUTO, ATTN_UNITS_SPLIT, ATTN_UNITS_HEAD_BLOCK = 0, 1, 2
+ATTN_HEAD_BLOCK_TOKENS = 1024
 
 
 class KvConfig(C.Structure):

@@ -186,7 +186,7 @@ typedef struct mlakvAttnPlan {
   int32_t merge_mode;      /* MLAKV_ATTN_MERGE_IN_LAUNCH or _SECOND_LAUNCH */
   int32_t merge_spin_us;   /* bound of the in-launch merge's wait for a sequence's other partials */
   int32_t reserved;        /* 1: made by mlakvAttnSparsePlanInit (max_seq_len holds sparse_count) */
-  int32_t reserved2;
+  int32_t selection_units; /* MLAKV_ATTN_UNITS_SPLIT or _HEAD_BLOCK (selected-token plans; 0 otherwise) */
   uint64_t workspace_bytes;
 } mlakvAttnPlan;
 
@@ -196,13 +196,26 @@ mlakvStatus mlakvAttnPlanInit(int32_t batch, int32_t heads, int32_t max_seq_len,
 /* The same with the planner's choices spelled out (tests and measurements use it to force many
  * small units, a single unit per sequence, the second-launch merge or a wait that gives up at
  * once); a zero field keeps the default. No reference counterpart. */
+/* How a selected-token launch cuts its work.
+ * SPLIT: the selections of the batch laid end to end and cut into one unit per CU, 64 heads per
+ *   unit; units that hold part of a selection leave partials that a merge puts together.
+ * HEAD_BLOCK: one unit = the whole selection of one sequence for 16 heads; nothing to merge and the
+ *   workspace stays untouched. bf16 caches, sparse_count up to MLAKV_ATTN_HEAD_BLOCK_TOKENS.
+ * AUTO takes HEAD_BLOCK where it applies and was measured ahead (up to 512 selected tokens while
+ * batch x heads / 16 units fit the CUs once, up to 256 while they fit twice), unless chunk_tiles,
+ * work_groups or merge_mode ask for properties of the split. */
+#define MLAKV_ATTN_UNITS_AUTO 0
+#define MLAKV_ATTN_UNITS_SPLIT 1
+#define MLAKV_ATTN_UNITS_HEAD_BLOCK 2
+#define MLAKV_ATTN_HEAD_BLOCK_TOKENS 1024
 typedef struct mlakvAttnPlanOptions {
   int32_t chunk_tiles;    /* tiles per work unit, fixed instead of derived from the live lengths */
   int32_t work_groups;    /* workgroups per group of 64 heads (default: CUs / head groups) */
   int32_t merge_mode;     /* MLAKV_ATTN_MERGE_* */
   int32_t merge_spin_us;  /* > 0: microseconds; < 0: do not wait at all (the last contributor merges) */
   int32_t selection;      /* 1: a plan for mlakvAttnDecodeSparse; max_seq_len then holds sparse_count */
-  int32_t reserved[3];    /* zero */
+  int32_t selection_units; /* MLAKV_ATTN_UNITS_* (selection plans only) */
+  int32_t reserved[2];    /* zero */
 } mlakvAttnPlanOptions;
 mlakvStatus mlakvAttnPlanInitEx(int32_t batch, int32_t heads, int32_t max_seq_len, int32_t block_size, int32_t dtype,
                                 const mlakvAttnPlanOptions* options, mlakvAttnPlan* plan);

@@ -121,14 +121,14 @@ def gather(cache, table, seq_lens, fused_out=False, layer_begin=0, layer_count=N
 
 
 def make_plan(batch, heads, max_seq_len, block_size, fp8, chunk_tiles=0, work_groups=0, merge_mode=0, merge_spin_us=0,
-              selection=False):
+              selection=False, selection_units=0):
     """The default plan, or one with the planner's choices forced (mlakvAttnPlanInitEx). With
     selection=True, max_seq_len is the length of the selection (mlakvAttnSparsePlanInit)."""
     lib = ffi.load()
     plan = ffi.AttnPlan()
     dtype = ffi.DTYPE_FP8_E4M3 if fp8 else ffi.DTYPE_BF16
-    if chunk_tiles or work_groups or merge_mode or merge_spin_us:
-        options = ffi.AttnPlanOptions(chunk_tiles, work_groups, merge_mode, merge_spin_us, 1 if selection else 0)
+    if chunk_tiles or work_groups or merge_mode or merge_spin_us or selection_units:
+        options = ffi.AttnPlanOptions(chunk_tiles, work_groups, merge_mode, merge_spin_us, 1 if selection else 0, selection_units)
         ffi.check(lib.mlakvAttnPlanInitEx(batch, heads, max_seq_len, block_size, dtype, C.byref(options), C.byref(plan)))
     elif selection:
         ffi.check(lib.mlakvAttnSparsePlanInit(batch, heads, max_seq_len, block_size, dtype, C.byref(plan)))

@@ -55,13 +55,52 @@ def test_selected_tokens_match_oracle(fp8, bs, k):
     q = kt.randn_bf16((len(ctxs), heads, LATENT + ROPE), seed=82).cuda()
     expected, expected_lse = kt.oracle_attention(cache, 0, q, table, ctxs, SCALE, sparse_indices=selection)
     table_d, lens_d, sel_d = kt.dev_i32(table), kt.dev_i32(ctxs), kt.dev_i32(selection)
-    for options in ({}, {"chunk_tiles": 1}, {"chunk_tiles": 100}, {"chunk_tiles": 3, "merge_mode": 1}):
+    whole = not fp8 and k <= 512   # where the default plan makes a unit a whole selection for 16 heads (24 units: far fewer than CUs)
+    for options in ({}, {"chunk_tiles": 1}, {"chunk_tiles": 100}, {"chunk_tiles": 3, "merge_mode": 1},
+                    {"selection_units": ffi.ATTN_UNITS_SPLIT}):
         out, lse, plan = kt.sparse_attention(cache, 0, q, table_d, lens_d, sel_d, SCALE, **options)
         assert plan.chunk_tiles * 32 <= 512  # a unit's selected tokens are staged in LDS, one entry each
+        assert plan.selection_units == (ffi.ATTN_UNITS_HEAD_BLOCK if whole and not options else ffi.ATTN_UNITS_SPLIT)
         _close(out, expected, 6e-2 if fp8 else 2e-2)
         live = np.array([min(n, k) > 0 for n in ctxs])
         assert np.abs(lse.cpu().numpy()[live] - expected_lse[live]).max() <= (6e-2 if fp8 else 2e-2)
         assert not out[3].any() and torch.isneginf(lse[3]).all()
+
+
+@pytest.mark.parametrize("batch,heads,bs,k", [(19, 128, 64, 1024), (8, 16, 16, 33), (3, 32, 48, 512), (9, 64, 128, 96)])
+def test_whole_selection_units_of_16_heads(batch, heads, bs, k):
+    """One workgroup per (sequence, 16 heads): selections of every length up to k (0, 1, multiples
+    of the 32-token tile and one beside them), more sequences than one round over the XCDs, against
+    the oracle and against the split units on the same inputs."""
+    rng = np.random.default_rng(700 + batch)
+    ctxs = [int(v) for v in rng.integers(1, 2 * k, size=batch)]
+    takes = [int(v) for v in rng.integers(0, k + 1, size=batch)]
+    takes[:4] = [k, 1, 32, 33][:min(4, batch)]
+    if batch > 4:
+        takes[4] = 0
+    ctxs = [max(c, t) for c, t in zip(ctxs, takes)]
+    cache, table = _setup(ctxs, bs, False, seed=70 + batch)
+    selection = np.full((batch, k), -1, dtype=np.int32)
+    for s, (n, take) in enumerate(zip(ctxs, takes)):
+        selection[s, :take] = rng.permutation(n)[:take]
+    q = kt.randn_bf16((batch, heads, LATENT + ROPE), seed=71 + batch).cuda()
+    expected, expected_lse = kt.oracle_attention(cache, 0, q, table, ctxs, SCALE, sparse_indices=selection)
+    table_d, lens_d, sel_d = kt.dev_i32(table), kt.dev_i32(ctxs), kt.dev_i32(selection)
+    out, lse, plan = kt.sparse_attention(cache, 0, q, table_d, lens_d, sel_d, SCALE, selection_units=ffi.ATTN_UNITS_HEAD_BLOCK)
+    assert plan.selection_units == ffi.ATTN_UNITS_HEAD_BLOCK
+    _close(out, expected, 2e-2)
+    live = np.array(takes) > 0
+    assert np.abs(lse.cpu().numpy()[live] - expected_lse[live]).max() <= 2e-2
+    assert not out[~torch.from_numpy(live).cuda()].any() and torch.isneginf(lse[~torch.from_numpy(live).cuda()]).all()
+    split, split_lse, _ = kt.sparse_attention(cache, 0, q, table_d, lens_d, sel_d, SCALE, selection_units=ffi.ATTN_UNITS_SPLIT)
+    peak = np.abs(expected).max()
+    assert (out.float() - split.float()).abs().max().item() <= 2 ** -6 * peak   # same tokens, same tiles; partials round to bf16 once more
+    assert (lse[torch.from_numpy(live).cuda()] - split_lse[torch.from_numpy(live).cuda()]).abs().max().item() <= 1e-3
+    # what the option refuses: FP8 caches and selections above the staging size
+    lib, refused = ffi.load(), ffi.AttnPlan()
+    for dtype, count in ((ffi.DTYPE_FP8_E4M3, 512), (ffi.DTYPE_BF16, ffi.ATTN_HEAD_BLOCK_TOKENS + 1)):
+        options = ffi.AttnPlanOptions(0, 0, 0, 0, 1, ffi.ATTN_UNITS_HEAD_BLOCK)
+        assert lib.mlakvAttnPlanInitEx(batch, heads, count, bs, dtype, C.byref(options), C.byref(refused)) == ffi.ERR_PARAM_INVALID
 
 
 def test_full_selection_equals_dense_and_order_does_not_matter():
