@@ -310,7 +310,9 @@ mlakvStatus mlakvAttnDecodeMxQuant(const mlakvAttnPlan* plan, const mlakvCacheVi
  *   sequence; sequence b attends to the cached rows at positions sparse_indices[b][0 .. n-1], where
  *   n is the number of entries before the first one that is negative or >= seq_lens[b]
  *   (n = 0: zeros, lse = -inf). Order does not matter; repeated positions count repeatedly.
- * The plan comes from mlakvAttnSparsePlanInit (sparse_count takes the place of max_seq_len). */
+ * The plan comes from mlakvAttnSparsePlanInit (sparse_count takes the place of max_seq_len); how
+ * it cuts the work (plan->selection_units) is described with MLAKV_ATTN_UNITS_* above. The
+ * workspace is required either way, and left untouched by whole-selection units. */
 mlakvStatus mlakvAttnSparsePlanInit(int32_t batch, int32_t heads, int32_t sparse_count, int32_t block_size, int32_t dtype,
                                     mlakvAttnPlan* plan);
 mlakvStatus mlakvAttnDecodeSparse(const mlakvAttnPlan* plan, const mlakvCacheView* cache, int32_t layer,
