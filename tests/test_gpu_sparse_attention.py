@@ -103,6 +103,41 @@ def test_whole_selection_units_of_16_heads(batch, heads, bs, k):
         assert lib.mlakvAttnPlanInitEx(batch, heads, count, bs, dtype, C.byref(options), C.byref(refused)) == ffi.ERR_PARAM_INVALID
 
 
+@pytest.mark.parametrize("fp8", [False, True])
+def test_table_entries_that_name_no_block_read_as_rows_of_zeros(fp8):
+    """A block-table entry outside [0, num_blocks) is never followed: its tokens count as rows of
+    zeros (score 0, nothing added to the output), in the whole-context kernel and in both kinds of
+    selected-token units. The oracle gets a table that points those entries at a block that was
+    never written (the cache starts as zeros)."""
+    bs, heads, k = 64, 32, 256
+    ctxs = [700, 300, 64]
+    cache, table = _setup(ctxs, bs, fp8, seed=60)
+    spare = sorted(set(range(cache.blocks)) - {int(b) for s, n in enumerate(ctxs) for b in table[s, :-(-n // bs)]})[0]
+    holes = [(0, 3, -1), (0, 10, cache.blocks + 7), (1, 0, 2 ** 31 - 1), (2, 0, -5)]
+    broken, zeroed = table.copy(), table.copy()
+    for s, logical, value in holes:
+        broken[s, logical], zeroed[s, logical] = value, spare
+    rng = np.random.default_rng(61)
+    selection = np.full((len(ctxs), k), -1, dtype=np.int32)
+    for s, n in enumerate(ctxs):
+        take = min(n, k)
+        selection[s, :take] = rng.permutation(n)[:take]
+    selection[0, :8] = 3 * bs + np.arange(8)            # tokens of a hole for certain, a whole tile row group
+    q = kt.randn_bf16((len(ctxs), heads, LATENT + ROPE), seed=62).cuda()
+    tol = 6e-2 if fp8 else 2e-2
+    lens_d, sel_d = kt.dev_i32(ctxs), kt.dev_i32(selection)
+    expected, expected_lse = kt.oracle_attention(cache, 0, q, zeroed, ctxs, SCALE)
+    out, lse, _ = kt.attention(cache, 0, q, kt.dev_i32(broken), lens_d, SCALE)
+    _close(out, expected, tol)
+    assert np.abs(lse.cpu().numpy() - expected_lse).max() <= tol
+    expected, expected_lse = kt.oracle_attention(cache, 0, q, zeroed, ctxs, SCALE, sparse_indices=selection)
+    for units in (ffi.ATTN_UNITS_SPLIT,) if fp8 else (ffi.ATTN_UNITS_SPLIT, ffi.ATTN_UNITS_HEAD_BLOCK):
+        out, lse, plan = kt.sparse_attention(cache, 0, q, kt.dev_i32(broken), lens_d, sel_d, SCALE, selection_units=units)
+        assert plan.selection_units == units
+        _close(out, expected, tol)
+        assert np.abs(lse.cpu().numpy() - expected_lse).max() <= tol
+
+
 def test_full_selection_equals_dense_and_order_does_not_matter():
     bs, heads, k = 64, 64, 512
     ctxs = [512, 300, 77]
