@@ -192,11 +192,39 @@ __global__ __launch_bounds__(kThreads) void AppendBf16Kernel(AppendArgs a, WORDS
 // Two quotients -> two E4M3 codes in the low half of a dword. v_cvt_pk_fp8_f32 rounds to nearest
 // even onto the OCP E4M3FN grid (subnormal grid 2^-9 below 2^-6 included): checked against a
 // software encoder over every float bit pattern below 464; beyond that it returns NaN, so the
-// clamp to +-448 provides the saturation for every finite input.
+// clamp to +-448 provides the saturation for every other number. A NaN keeps its sign and becomes
+// the format's NaN (a clamp made of minima and maxima would turn it into -448).
 __device__ __forceinline__ unsigned int E4m3EncodePair(float a, float b) {
+  const unsigned nan_a = ((__builtin_bit_cast(unsigned, a) >> 24) & 0x80u) | 0x7fu, nan_b = ((__builtin_bit_cast(unsigned, b) >> 24) & 0x80u) | 0x7fu;
+  const bool a_is_nan = a != a, b_is_nan = b != b;
   a = fminf(fmaxf(a, -448.0f), 448.0f);
   b = fminf(fmaxf(b, -448.0f), 448.0f);
-  return static_cast<unsigned int>(__builtin_amdgcn_cvt_pk_fp8_f32(a, b, 0, false)) & 0xffffu;
+  const unsigned codes = static_cast<unsigned int>(__builtin_amdgcn_cvt_pk_fp8_f32(a, b, 0, false)) & 0xffffu;
+  return (a_is_nan ? nan_a : codes & 0xffu) | ((b_is_nan ? nan_b : codes >> 8) << 8);
+}
+
+// Maximum over the 64 lanes, in every lane, of values that are neither negative nor NaN, without
+// the LDS crossbar: their bit patterns order like the values, so the steps are integer maxima, four
+// with data-parallel-primitive operands inside each row of 16 lanes (neighbour, other pair, mirrored
+// half, mirrored row), then v_permlane16_swap (odd and even rows) and v_permlane32_swap (the two
+// halves). A shuffle per step (ds_bpermute and a wait for it, six times in a row) and float maxima
+// that re-quiet their operands made the FP8 append arithmetic-bound.
+template <int CONTROL>
+__device__ __forceinline__ unsigned DppMaxU32(unsigned x) {
+  const int bits = static_cast<int>(x);
+  return max(x, static_cast<unsigned>(__builtin_amdgcn_update_dpp(bits, bits, CONTROL, 0xf, 0xf, true)));
+}
+__device__ __forceinline__ float WaveMaxNonNegative(float value) {
+  typedef __attribute__((ext_vector_type(2))) unsigned int u32x2_t;
+  unsigned x = __builtin_bit_cast(unsigned, value);
+  x = DppMaxU32<0xB1>(x);   // quad_perm [1,0,3,2]
+  x = DppMaxU32<0x4E>(x);   // quad_perm [2,3,0,1]
+  x = DppMaxU32<0x141>(x);  // row_half_mirror
+  x = DppMaxU32<0x140>(x);  // row_mirror
+  u32x2_t swapped = __builtin_amdgcn_permlane16_swap(x, x, false, false);
+  x = max(static_cast<unsigned>(swapped.x), static_cast<unsigned>(swapped.y));
+  swapped = __builtin_amdgcn_permlane32_swap(x, x, false, false);
+  return __builtin_bit_cast(float, max(static_cast<unsigned>(swapped.x), static_cast<unsigned>(swapped.y)));
 }
 
 // Quantises one row held by a wave (lane: 8 latent values, 1 rope value) and stores codes and
@@ -204,37 +232,59 @@ __device__ __forceinline__ unsigned int E4m3EncodePair(float a, float b) {
 // correctly rounded quotient.
 __device__ __forceinline__ void QuantizeRowAndStore(const AppendArgs& a, int layer, int block, int in_block, int lane,
                                                     const float (&x)[8], float y) {
-  float absmax = fabsf(y);
+  float absmax = fmaxf(0.0f, fabsf(y));  // a NaN never becomes the maximum (a row of nothing but NaNs has absmax 0)
 #pragma unroll
   for (int i = 0; i < 8; ++i) absmax = fmaxf(absmax, fabsf(x[i]));
-#pragma unroll
-  for (int offset = 32; offset >= 1; offset >>= 1) absmax = fmaxf(absmax, __shfl_xor(absmax, offset));
-  const float scale = absmax == 0.0f ? 1.0f : absmax / 448.0f;
+  absmax = WaveMaxNonNegative(absmax);
+  // The usual row: a maximum in [2^-100, the largest finite float] (as bit patterns, on the scalar
+  // unit: the value is the same in every lane).
+  const unsigned absmax_bits = __builtin_amdgcn_readfirstlane(__builtin_bit_cast(unsigned, absmax));
+  const bool usual = absmax_bits - 0x0d800000u <= 0x7f7fffffu - 0x0d800000u;
+  // scale = absmax / 448, correctly rounded. In the usual range three operations do it: with
+  // y = RN(1/448), q = absmax * y, then q + (absmax - 448 q) * y in one fused step each. absmax is a
+  // bf16 value; that the result equals the rounded quotient was checked for every one of the
+  // 29,184 bf16 values of that range in exact arithmetic (tests/test_oracle_formats.py).
+  float scale;
+  if (usual) {
+    const float y448 = __builtin_bit_cast(float, 0x3b124925u);
+    const float q0 = absmax * y448;
+    scale = __builtin_fmaf(__builtin_fmaf(-448.0f, q0, absmax), y448, q0);
+  } else {
+    scale = absmax == 0.0f ? 1.0f : absmax / 448.0f;
+  }
   // code = e4m3(x / scale) with the correctly rounded fp32 quotient. Nine divisions per lane made
-  // this kernel compute-bound, so the quotient is first taken as x * (1 / scale), which is within
-  // 2^-22 relative of the rounded quotient; the encoding is monotone, so if the two ends of that
-  // interval (widened to 2^-21) encode alike, so does the exact quotient. Only a lane that holds
-  // a value this close to a rounding boundary of the E4M3 grid (about one in 10^5 values) divides.
-  const float inverse = 1.0f / scale;
+  // this kernel compute-bound, so the quotient is first taken as x * r with r the hardware's
+  // reciprocal of the scale (within one unit in the last place): the product is within 2^-22
+  // relative of the rounded quotient (2^-23 from r, 2^-24 from each of the two roundings); the
+  // encoding is monotone, so if the two ends of that interval (widened to 2^-21) encode alike, so
+  // does the exact quotient. Only a lane that holds a value this close to a rounding boundary of
+  // the E4M3 grid (about one in 10^5 values) divides. A scale so small that its reciprocal leaves the
+  // normal range (the instruction reads a subnormal as zero) sends the whole row to the divisions,
+  // and so does an infinite one (quotients 0 and NaN). A usual row needs no clamp: its quotients
+  // stay below 448 (1 + 2^-21), which the conversion rounds to 448, and a NaN stays one.
+  const float inverse = __builtin_amdgcn_rcpf(scale);
   float q[9];
 #pragma unroll
-  for (int i = 0; i < 8; ++i) q[i] = fminf(fmaxf(x[i] * inverse, -448.0f), 448.0f);
-  q[8] = fminf(fmaxf(y * inverse, -448.0f), 448.0f);
+  for (int i = 0; i < 8; ++i) q[i] = x[i] * inverse;
+  q[8] = y * inverse;
   constexpr float kWiden = 4.76837158203125e-07f;  // 2^-21
-  unsigned below[5], above[5];
-#pragma unroll
-  for (int i = 0; i < 5; ++i) {
-    const float a = q[2 * i], b = i < 4 ? q[2 * i + 1] : 0.0f;
-    below[i] = static_cast<unsigned>(__builtin_amdgcn_cvt_pk_fp8_f32(__builtin_fmaf(a, -kWiden, a), __builtin_fmaf(b, -kWiden, b), 0, false)) & 0xffffu;
-    above[i] = static_cast<unsigned>(__builtin_amdgcn_cvt_pk_fp8_f32(__builtin_fmaf(a, kWiden, a), __builtin_fmaf(b, kWiden, b), 0, false)) & 0xffffu;
-  }
-  const bool settled = below[0] == above[0] && below[1] == above[1] && below[2] == above[2] && below[3] == above[3] && below[4] == above[4];
+  // four codes per dword: the conversion writes one half of its destination and keeps the other
+  const auto four_codes = [&](float widen, int i) __attribute__((always_inline)) {
+    const int low = __builtin_amdgcn_cvt_pk_fp8_f32(__builtin_fmaf(q[i], widen, q[i]), __builtin_fmaf(q[i + 1], widen, q[i + 1]), 0, false);
+    return static_cast<unsigned>(
+        __builtin_amdgcn_cvt_pk_fp8_f32(__builtin_fmaf(q[i + 2], widen, q[i + 2]), __builtin_fmaf(q[i + 3], widen, q[i + 3]), low, true));
+  };
+  const unsigned below_lo = four_codes(-kWiden, 0), below_hi = four_codes(-kWiden, 4);
+  const unsigned above_lo = four_codes(kWiden, 0), above_hi = four_codes(kWiden, 4);
+  const unsigned below_rope = static_cast<unsigned>(__builtin_amdgcn_cvt_pk_fp8_f32(__builtin_fmaf(q[8], -kWiden, q[8]), 0.0f, 0, false));
+  const unsigned above_rope = static_cast<unsigned>(__builtin_amdgcn_cvt_pk_fp8_f32(__builtin_fmaf(q[8], kWiden, q[8]), 0.0f, 0, false));
+  const bool settled = usual && below_lo == above_lo && below_hi == above_hi && ((below_rope ^ above_rope) & 0xffu) == 0u;
   u32x2 lq;
   unsigned int rq;
   if (settled) {
-    lq.x = below[0] | (below[1] << 16);
-    lq.y = below[2] | (below[3] << 16);
-    rq = below[4] & 0xffu;
+    lq.x = below_lo;
+    lq.y = below_hi;
+    rq = below_rope & 0xffu;
   } else {
     lq.x = E4m3EncodePair(x[0] / scale, x[1] / scale) | (E4m3EncodePair(x[2] / scale, x[3] / scale) << 16);
     lq.y = E4m3EncodePair(x[4] / scale, x[5] / scale) | (E4m3EncodePair(x[6] / scale, x[7] / scale) << 16);
@@ -264,6 +314,8 @@ __global__ __launch_bounds__(kThreads) void AppendFp8Kernel(AppendArgs a, WORDS 
   if (token0 >= a.num_tokens) return;
   int my_slot = -1;
   if (lane < kAppendRows && token0 + lane < a.num_tokens) my_slot = SlotOf(a, w, token0 + lane);
+  // the usual block sizes are powers of two: a shift then, not a division per row
+  const int block_shift = (a.block_size & (a.block_size - 1)) == 0 ? __builtin_ctz(static_cast<unsigned>(a.block_size)) : -1;
   u32x4 lv[kAppendRows];
   unsigned short rv[kAppendRows];
 #pragma unroll
@@ -276,7 +328,7 @@ __global__ __launch_bounds__(kThreads) void AppendFp8Kernel(AppendArgs a, WORDS 
   for (int i = 0; i < kAppendRows; ++i) {
     const int slot = __builtin_amdgcn_readlane(my_slot, i);
     if (slot < 0) continue;
-    const int block = slot / a.block_size;
+    const int block = block_shift >= 0 ? slot >> block_shift : slot / a.block_size;
     const int in_block = slot - block * a.block_size;
     if (block >= a.num_blocks) continue;
     float x[8];

@@ -369,6 +369,8 @@ def bench_attention(args, torch, np, ffi, ctxs, fp8=False, heads=64, slices=8, i
         return sustained_us(torch, fn, iters)
 
     us = timed_us(launch)
+    # the same launches with the lengths known on the host (what the aclnn face does for the reference's call)
+    us_host_lens = timed_us(launch_host_lens) if not sparse_k and batch <= 64 and not args.attn_host_lens else None
     mx = None
     if mx_quant:
         # the reference's next stage, block-32 MX quantisation of the output: fused into the
@@ -426,6 +428,9 @@ def bench_attention(args, torch, np, ffi, ctxs, fp8=False, heads=64, slices=8, i
         result["total_tokens"] = sum(ctxs)
     if mx is not None:
         result["mx_quant_output"] = mx
+    if us_host_lens is not None:
+        result["host_known_lengths"] = {"us_per_step": us_host_lens,
+                                        "what": "mlakvAttnDecodeHostLens: the lengths ride in the kernels' argument block, no device array is read"}
     cache.close()
     arena.close()
     return result

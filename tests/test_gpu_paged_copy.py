@@ -253,6 +253,75 @@ def test_fp8_quantize_on_append_and_dequant_gather_bit_exact(bs):
     assert bool(((x - y).abs() <= bound).all())
 
 
+def test_fp8_quantize_rows_at_the_edges_of_the_arithmetic_bit_exact():
+    """Rows where the quantiser's shortcuts do not apply or must not matter, against the oracle bit
+    for bit: magnitudes so small that the scale's reciprocal leaves the normal range (every lane
+    divides), subnormal bf16 values, NaNs beside finite values (a NaN never becomes the row's
+    maximum), a row of nothing but NaNs, infinities, quotients that sit exactly on rounding
+    boundaries of the E4M3 grid (ties go to even), the largest finite bf16."""
+    bs, layers = 16, 1
+    rng = np.random.default_rng(33)
+    rows = []
+    base = rng.standard_normal((LATENT + ROPE,)).astype(np.float32)
+    rows.append(base * np.float32(2.0 ** -112))                      # reciprocal of the scale overflows
+    rows.append(base * np.float32(2.0 ** -101))                      # just below the switch
+    rows.append(base * np.float32(2.0 ** -99))                       # just above it
+    rows.append(base * np.float32(2.0 ** -130))                      # subnormal values
+    with_nan = base.copy(); with_nan[[0, 513]] = np.nan; with_nan[[5, 575]] = np.copysign(np.nan, -1.0)   # both signs
+    rows.append(with_nan)
+    rows.append(np.full(LATENT + ROPE, np.nan, dtype=np.float32))
+    with_inf = base.copy(); with_inf[[7, 520]] = [np.inf, -np.inf]
+    rows.append(with_inf)
+    ties = np.zeros(LATENT + ROPE, dtype=np.float32)                  # absmax 448: scale exactly 1
+    grid = np.array([17, 19, 21, 23, 25, 27, 29, 31, 34, 36, 44, 52, 1.0625, 0.9375, 2.0 ** -9 * 1.5, 2.0 ** -9 * 2.5, 2.0 ** -10,
+                     3 * 2.0 ** -10, 416 + 16, 448], dtype=np.float32)
+    ties[:len(grid)] = grid; ties[100:100 + len(grid)] = -grid; ties[LATENT + 3] = 448.0; ties[LATENT + 4] = 17.0
+    rows.append(ties)
+    rows.append(ties * np.float32(3.0))                               # the same quotients behind a scale that is not a power of two
+    rows.append(base / np.abs(base).max() * np.float32(3.3895314e38))  # absmax = the largest finite bf16
+    data = torch.from_numpy(np.stack(rows)).to(torch.bfloat16)
+    total = data.shape[0]
+    blocks = -(-total // bs) + 1
+    table = kt.build_tables([total], bs, blocks, seed=5).table()
+    cache = kt.PagedCache(layers, blocks, bs, fp8=True)
+    latent_src, rope_src = data[None, :, :LATENT].contiguous().cuda(), data[None, :, LATENT:].contiguous().cuda()
+    slots = kt.slots_for(table, [total], bs)
+    kt.append(cache, latent_src, rope_src, kt.dev_i32(slots))
+    torch.cuda.synchronize()
+    lat, rop, scl = _oracle_planes(layers, blocks, bs, fp8=True)
+    orc.append_rows_fp8(lat[0], rop[0], scl[0], bs, kt.bits16(latent_src[0]), kt.bits16(rope_src[0]), slots)
+    assert cache.scale_np(0).tobytes() == scl[0].tobytes()
+    got_lat, got_rope = cache.latent_np(0).reshape(-1, LATENT), cache.rope_np(0).reshape(-1, ROPE)
+    for r, slot in enumerate(slots):
+        assert got_lat[slot].tobytes() == lat[0].reshape(-1, LATENT)[slot].tobytes(), r
+        assert got_rope[slot].tobytes() == rop[0].reshape(-1, ROPE)[slot].tobytes(), r
+    assert scl[0][slots[5]] == 1.0                                    # nothing but NaNs: absmax 0
+
+
+def test_fp8_scale_of_every_bf16_maximum_bit_exact():
+    """One row per positive finite bf16 value (and zero), that value its only non-zero element at a
+    varying column: the stored scale is the oracle's absmax / 448 for every possible maximum, and
+    the codes are the oracle's (the element itself encodes as 448)."""
+    bs = 64
+    values = np.arange(0, 0x7F80, dtype=np.uint32)             # bf16 bit patterns 0 .. largest finite
+    total = len(values)
+    data = np.zeros((total, LATENT + ROPE), dtype=np.uint16)
+    data[np.arange(total), (np.arange(total) * 37) % (LATENT + ROPE)] = values.astype(np.uint16)
+    src = torch.from_numpy(data.view(np.int16)).view(torch.bfloat16)
+    blocks = -(-total // bs) + 1
+    table = kt.build_tables([total], bs, blocks, seed=9).table()
+    cache = kt.PagedCache(1, blocks, bs, fp8=True)
+    latent_src, rope_src = src[None, :, :LATENT].contiguous().cuda(), src[None, :, LATENT:].contiguous().cuda()
+    slots = kt.slots_for(table, [total], bs)
+    kt.append(cache, latent_src, rope_src, kt.dev_i32(slots))
+    torch.cuda.synchronize()
+    lat, rop, scl = _oracle_planes(1, blocks, bs, fp8=True)
+    orc.append_rows_fp8(lat[0], rop[0], scl[0], bs, kt.bits16(latent_src[0]), kt.bits16(rope_src[0]), slots)
+    assert cache.scale_np(0).tobytes() == scl[0].tobytes()
+    assert cache.latent_np(0).tobytes() == lat[0].tobytes()
+    assert cache.rope_np(0).tobytes() == rop[0].tobytes()
+
+
 def test_fp8_compaction_moves_codes_and_scales():
     layers, bs, blocks = 2, 64, 12
     ctxs = [100, 64, 129]

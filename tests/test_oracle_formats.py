@@ -113,3 +113,38 @@ def test_splitmix64_known_answers(oracle):
     expected = [6457827717110365317, 3203168211198807973, 9817491932198370423, 4593380528125082431,
                 16408922859458223821]
     assert [oracle.kvo_splitmix64(C.byref(state)) for _ in range(5)] == expected
+
+
+def test_division_by_448_in_three_fused_steps_is_exact_for_every_bf16_maximum():
+    """The FP8 append kernel forms scale = absmax / 448 as q + (absmax - 448 q) y with y = RN(1/448)
+    and q = RN(absmax y), one fused multiply-add each (csrc/kernels/paged_copy.hip). absmax is a
+    bf16 value, so the claim that this equals the correctly rounded quotient is checked here for
+    every bf16 value the kernel sends down that path (2^-100 up to the largest finite one), in exact
+    rational arithmetic; the oracle's own scale (a float division) is compared on the way."""
+    from fractions import Fraction
+
+    def rn32(value):
+        guess = np.float32(float(value))          # correctly rounded to double, then to float: may be one step off
+        best = guess
+        for cand in (np.nextafter(guess, np.float32(np.inf)), np.nextafter(guess, np.float32(-np.inf))):
+            d_cand, d_best = abs(Fraction(float(cand)) - value), abs(Fraction(float(best)) - value)
+            if d_cand < d_best or (d_cand == d_best and (int(np.float32(cand).view(np.uint32)) & 1) == 0):
+                best = cand
+        return np.float32(best)
+
+    y = rn32(Fraction(1, 448))
+    assert int(y.view(np.uint32)) == 0x3B124925
+    Y = Fraction(float(y))
+    checked = 0
+    for bits in range(1, 0x7F80):
+        a = np.array([bits << 16], dtype=np.uint32).view(np.float32)[0]
+        if a < np.float32(2.0 ** -100):
+            continue
+        A = Fraction(float(a))
+        q0 = rn32(A * Y)
+        r0 = rn32(A - 448 * Fraction(float(q0)))
+        q1 = rn32(Fraction(float(q0)) + Fraction(float(r0)) * Y)
+        assert q1 == rn32(A / 448), hex(bits)
+        assert q1 == np.float32(a) / np.float32(448.0), hex(bits)     # what the oracle's division gives
+        checked += 1
+    assert checked == 29184
