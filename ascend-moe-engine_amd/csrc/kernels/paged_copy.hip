@@ -87,6 +87,14 @@ __device__ __forceinline__ unsigned int F32ToBf16(float v) {
   return bits >> 16;
 }
 
+// Two floats -> two bf16 in one dword, rounded to nearest even by the conversion instruction
+// (v_cvt_pk_bf16_f32; a NaN stays a quiet NaN of its sign).
+__device__ __forceinline__ unsigned int PackBf16Pair(float lo, float hi) {
+  typedef __attribute__((ext_vector_type(2))) __bf16 bf16x2_t;
+  const bf16x2_t packed = {static_cast<__bf16>(lo), static_cast<__bf16>(hi)};
+  return __builtin_bit_cast(unsigned int, packed);
+}
+
 // Eight E4M3 codes -> eight bf16, each decoded value times `scale`, rounded to nearest even.
 __device__ __forceinline__ u32x4 Dequant8(u32x2 codes, float scale) {
   const f32x2 a = __builtin_amdgcn_cvt_pk_f32_fp8(static_cast<int>(codes.x), false);
@@ -94,10 +102,10 @@ __device__ __forceinline__ u32x4 Dequant8(u32x2 codes, float scale) {
   const f32x2 c = __builtin_amdgcn_cvt_pk_f32_fp8(static_cast<int>(codes.y), false);
   const f32x2 d = __builtin_amdgcn_cvt_pk_f32_fp8(static_cast<int>(codes.y), true);
   u32x4 out;
-  out.x = F32ToBf16(a.x * scale) | (F32ToBf16(a.y * scale) << 16);
-  out.y = F32ToBf16(b.x * scale) | (F32ToBf16(b.y * scale) << 16);
-  out.z = F32ToBf16(c.x * scale) | (F32ToBf16(c.y * scale) << 16);
-  out.w = F32ToBf16(d.x * scale) | (F32ToBf16(d.y * scale) << 16);
+  out.x = PackBf16Pair(a.x * scale, a.y * scale);
+  out.y = PackBf16Pair(b.x * scale, b.y * scale);
+  out.z = PackBf16Pair(c.x * scale, c.y * scale);
+  out.w = PackBf16Pair(d.x * scale, d.y * scale);
   return out;
 }
 

@@ -296,6 +296,16 @@ def test_fp8_quantize_rows_at_the_edges_of_the_arithmetic_bit_exact():
         assert got_lat[slot].tobytes() == lat[0].reshape(-1, LATENT)[slot].tobytes(), r
         assert got_rope[slot].tobytes() == rop[0].reshape(-1, ROPE)[slot].tobytes(), r
     assert scl[0][slots[5]] == 1.0                                    # nothing but NaNs: absmax 0
+    # and back through the dequantising gather: bit for bit where the oracle's value is a number, a NaN
+    # where it is one (0 x inf has the sign of the machine's default NaN, which differs between the two)
+    table_d = kt.dev_i32(table)
+    got_latent, got_rope = kt.gather(cache, table_d, kt.dev_i32([total]))
+    exp_latent, exp_rope = orc.gather_rows_fp8(lat[0], rop[0], scl[0], bs, table, [total])
+    for got, expected in ((kt.bits16(got_latent[0]), exp_latent), (kt.bits16(got_rope[0]), exp_rope)):
+        got, expected = got.reshape(-1), expected.reshape(-1)
+        is_nan = (expected & 0x7FFF) > 0x7F80
+        assert np.array_equal(got[~is_nan], expected[~is_nan])
+        assert ((got[is_nan] & 0x7FFF) > 0x7F80).all() and is_nan.sum() >= 4
 
 
 def test_fp8_scale_of_every_bf16_maximum_bit_exact():
