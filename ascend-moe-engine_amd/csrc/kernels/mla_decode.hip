@@ -386,45 +386,13 @@ __device__ __forceinline__ bool IssueTileBf16(const AttnArgs& a, TileMap<ALIGNED
   return false;
 }
 
-// Selected-token tiles whose rows are all rows of the pool (no bad table entry among the staged
-// (block << slot_bits) | slot entries): the first P waves of the workgroup fetch the tile, wave w
-// the latent rows w, w + P, ... and eight rope rows (waves 4..7 for P = 8, as in IssueTileBf16,
-// every wave for P = 4), one rope row per eight lanes. No case distinction and no scalar address
-// chain: every lane forms the address of its 16 bytes itself, in units of 16 bytes with 24-bit
-// multiplies (PlainRowsAddressable says when that is exact). Entry `first + row` belongs to row
-// `row` of the tile; rows behind `last` repeat entry `last` (finite values that the softmax masks).
+// Whether a row's start inside its plane can be formed in 16-byte units with 24-bit multiplies
+// and held in 32 bits (what the whole-selection units of 16 heads stage per selected token).
 __host__ __device__ __forceinline__ bool PlainRowsAddressable(const AttnArgs& a) {
   const int64_t limit = int64_t{1} << 28;  // strides in 16-byte units below 2^24
   return a.latent.block_stride < limit && a.rope.block_stride < limit && a.latent.row_stride < limit && a.rope.row_stride < limit &&
          a.num_blocks <= (1 << 24) && a.num_blocks * a.latent.block_stride <= (int64_t{1} << 36) &&
          a.num_blocks * a.rope.block_stride <= (int64_t{1} << 36);
-}
-template <int P>
-__device__ __forceinline__ void IssuePlainRowsBf16(const AttnArgs& a, const int* entries, int first, int last, int slot_bits, unsigned buf,
-                                                   int lane, int wave) {
-  using G = Geom<false>;
-  constexpr int kRows = kTileTokens / P;
-  const int rope_group = P == 4 ? wave : wave - kScoreWaves;
-  if (wave >= P) return;
-  const unsigned slot_mask = (1u << slot_bits) - 1u;
-  const unsigned lat_block16 = static_cast<unsigned>(a.latent.block_stride >> 4), lat_row16 = static_cast<unsigned>(a.latent.row_stride >> 4);
-  unsigned packed[kRows];
-#pragma unroll
-  for (int r = 0; r < kRows; ++r) packed[r] = static_cast<unsigned>(entries[min(first + wave + P * r, last)]);
-  unsigned rope_packed = 0u;
-  if (rope_group >= 0) rope_packed = static_cast<unsigned>(entries[min(first + 8 * rope_group + (lane >> 3), last)]);
-#pragma unroll
-  for (int r = 0; r < kRows; ++r) {
-    const int row = wave + P * r;
-    const unsigned off16 = __umul24(packed[r] >> slot_bits, lat_block16) + __umul24(packed[r] & slot_mask, lat_row16);
-    DirectLoad16PerLane(a.latent.base + (static_cast<u64>(off16) << 4) + ((lane ^ SwizzleLat(row)) << 4), buf + row * G::kLatRow);
-  }
-  if (rope_group >= 0) {
-    const unsigned rope_block16 = static_cast<unsigned>(a.rope.block_stride >> 4), rope_row16 = static_cast<unsigned>(a.rope.row_stride >> 4);
-    const unsigned off16 = __umul24(rope_packed >> slot_bits, rope_block16) + __umul24(rope_packed & slot_mask, rope_row16);
-    const int chunk = ((lane & 7) ^ SwizzleRope(8 * rope_group + (lane >> 3))) << 4;
-    DirectLoad16PerLane(a.rope.base + (static_cast<u64>(off16) << 4) + chunk, buf + G::kLatRegion + rope_group * 8 * G::kRopeRow);
-  }
 }
 
 // ---- FP8 tiles: direct global -> LDS, codes and row scales as they are in the cache -------------
@@ -1562,8 +1530,8 @@ constexpr int kHbLoaders = kScoreWaves;  // the waves that fetch the tiles when 
 struct GeomHeadBlock {
   using T = Geom<false>;
   static constexpr int kRing = 4;
-  static constexpr int kTableOff = kRing * T::kTileBytes;                          // int[kAttnHeadBlockTokens]: (block << slot_bits) | slot
-  static constexpr int kSOff = kTableOff + kAttnHeadBlockTokens * 4;               // S^T partials [2][4 waves][64 lanes] x 16 B
+  static constexpr int kTableOff = kRing * T::kTileBytes;                          // unsigned[2][kAttnHeadBlockTokens]: where a selected token's latent and rope rows start, in 16-byte units from the plane's base
+  static constexpr int kSOff = kTableOff + 2 * kAttnHeadBlockTokens * 4;           // S^T partials [2][4 waves][64 lanes] x 16 B
   static constexpr int kEndOff = kSOff;  // int[2][kHbWaves], before the first S is written: where each wave saw the selection end, and whether it saw a bad table entry
   static constexpr int kLdsBytes = kSOff + 2 * kScoreWaves * 64 * 16;
   static_assert(kLdsBytes <= 160 * 1024, "one workgroup owns the LDS of a CU");
@@ -1575,7 +1543,7 @@ __global__ __launch_bounds__(kHbThreads) void MlaSelectedHeadBlockKernel(AttnArg
   using G = GeomHeadBlock;
   using T = Geom<false>;
   extern __shared__ __attribute__((aligned(16))) unsigned char lds[];
-  const unsigned lds_base = static_cast<unsigned>(reinterpret_cast<size_t>((__attribute__((address_space(3))) unsigned char*)lds));
+  const unsigned lds_base = Uniform(static_cast<unsigned>(reinterpret_cast<size_t>((__attribute__((address_space(3))) unsigned char*)lds)));
   const int tid = threadIdx.x;
   const int lane = tid & 63, wave = Uniform(tid >> 6);
   // Workgroups go to the XCDs round-robin by linear id: ids x, x + 8, x + 16, ... share XCD x, and
@@ -1593,7 +1561,9 @@ __global__ __launch_bounds__(kHbThreads) void MlaSelectedHeadBlockKernel(AttnArg
   // The selection ends at its first entry that is negative or not inside the context. Every
   // thread resolves one or two entries to pool slots through the block table; the loads that the
   // first tile's addresses depend on go out first, the query behind them.
-  int* table_lds = reinterpret_cast<int*>(lds + G::kTableOff);
+  unsigned* latent_rows = reinterpret_cast<unsigned*>(lds + G::kTableOff);
+  unsigned* rope_rows = latent_rows + kAttnHeadBlockTokens;
+  constexpr unsigned kNoRow = 0xffffffffu;  // a selected token behind a block-table entry that is not a block of the pool
   int* end_lds = reinterpret_cast<int*>(lds + G::kEndOff);
   const int context = static_cast<int>(
       min(static_cast<int64_t>(max(Uniform(LiveLength(a, seq)), 0)), static_cast<int64_t>(a.table_stride) * a.block_size));
@@ -1625,8 +1595,12 @@ __global__ __launch_bounds__(kHbThreads) void MlaSelectedHeadBlockKernel(AttnArg
     for (int c = 0; c < kHeadBlockKSteps; ++c) q[c] = __builtin_bit_cast(bf16x8, u32x4{0u, 0u, 0u, 0u});
   }
   int wave_end = a.sparse_count;
-  bool any_outside = false;  // a selected token behind a block-table entry that is not a block of the pool
+  bool any_outside = false;
   const bool shift = (a.block_size & (a.block_size - 1)) == 0;
+  // Row starts in 16-byte units, by 24-bit multiplies (the launcher sends pools that these do not
+  // cover to the split units: PlainRowsAddressable).
+  const unsigned lat_block16 = static_cast<unsigned>(a.latent.block_stride >> 4), lat_row16 = static_cast<unsigned>(a.latent.row_stride >> 4);
+  const unsigned rope_block16 = static_cast<unsigned>(a.rope.block_stride >> 4), rope_row16 = static_cast<unsigned>(a.rope.row_stride >> 4);
 #pragma unroll
   for (int j = 0; j < kPerThread; ++j) {
     const int i = tid + kHbThreads * j;
@@ -1637,7 +1611,9 @@ __global__ __launch_bounds__(kHbThreads) void MlaSelectedHeadBlockKernel(AttnArg
       const int logical = shift ? index[j] >> slot_bits : index[j] / a.block_size;
       const int entry = table_row[logical];
       const bool inside = static_cast<unsigned>(entry) < static_cast<unsigned>(a.num_blocks);
-      table_lds[i] = inside ? (entry << slot_bits) | (index[j] - logical * a.block_size) : -1;
+      const unsigned block = static_cast<unsigned>(entry), in_block = static_cast<unsigned>(index[j] - logical * a.block_size);
+      latent_rows[i] = inside ? __umul24(block, lat_block16) + __umul24(in_block, lat_row16) : kNoRow;
+      rope_rows[i] = inside ? __umul24(block, rope_block16) + __umul24(in_block, rope_row16) : kNoRow;
       if (!inside) any_outside = true;
     }
   }
@@ -1657,10 +1633,8 @@ __global__ __launch_bounds__(kHbThreads) void MlaSelectedHeadBlockKernel(AttnArg
     outside |= end_lds[kHbWaves + w];
   }
   seq_len = Uniform(seq_len);
-  // Every row a real row of the pool (the usual case) and strides that the per-lane address
-  // arithmetic covers: the score waves fetch the tiles; otherwise all eight waves do, one row at a
-  // time.
-  const bool plain_rows = Uniform(outside) == 0 && PlainRowsAddressable(a);
+  // Every row a real row of the pool (the usual case): the tile loads need no case distinction.
+  const bool plain_rows = Uniform(outside) == 0;
   const int ntiles = (seq_len + kTileTokens - 1) / kTileTokens;
   if (ntiles == 0) {  // nothing selected: zeros, lse = -inf
     for (int h = wave; h < 16; h += kHbWaves) {
@@ -1670,34 +1644,57 @@ __global__ __launch_bounds__(kHbThreads) void MlaSelectedHeadBlockKernel(AttnArg
     return;
   }
 
-  TileMap<false> map;
-  map.entries = table_lds;
-  map.first_block = 0;
-  map.block_size = a.block_size;
-  map.seq_len = seq_len;
-  map.sparse = true;
-  map.first_pos = 0;
-  map.slot_bits = slot_bits;
-  map.tile_block = map.tile_slot0 = map.next_entry = map.next_slot0 = 0;
-  IssueLane il;
-  il.lat[0] = il.lat[1] = il.partner_lat[0] = il.partner_lat[1] = 0;  // (the row-at-a-time path forms these itself)
-  il.rope_chunk = ((lane & 7) ^ SwizzleRope(8 * (wave - kScoreWaves) + (lane >> 3))) << 4;
-  il.rope = 0;
   // The head blocks of a sequence walk its tiles from different starting points (the order of the
   // tiles only changes the rounding): at any time they ask for different rows, and what one has
   // fetched the others find in the L2.
   const int rotate = hb * ntiles / head_blocks;
   const auto tile_of = [&](int i) __attribute__((always_inline)) { return i + rotate < ntiles ? i + rotate : i + rotate - ntiles; };
-  constexpr int kPlainLoads = kTileTokens / kHbLoaders + 1;  // a loader wave's loads per tile: eight latent rows and eight rope rows
-  const int per_tile = plain_rows ? (wave < kHbLoaders ? kPlainLoads : 0) : LoadsPerTile(wave);
+  // The score waves fetch the tiles: wave w the latent rows w, w + 4, ... (one row per load: lane L
+  // asks for the 16 bytes that belong at 16 L of the swizzled LDS row) and the rope rows 8 w .. 8 w + 7
+  // (one load, a row per eight lanes). A lane's address is the plane's base, its own chunk and the
+  // row's staged start; positions behind the selection's end repeat its last row (finite values
+  // that the softmax masks). A row that is not a row of the pool becomes zeros.
+  constexpr int kRowsPerLoader = kTileTokens / kHbLoaders, kPlainLoads = kRowsPerLoader + 1;
+  const char* lat_lane[4];
+#pragma unroll
+  for (int j = 0; j < 4; ++j) lat_lane[j] = a.latent.base + ((lane ^ SwizzleLat(wave + kHbLoaders * j)) << 4);
+  const char* rope_lane = a.rope.base + (((lane & 7) ^ SwizzleRope(8 * wave + (lane >> 3))) << 4);
+  const int per_tile = wave < kHbLoaders ? kPlainLoads : 0;
   int last_unknown = -1;  // newest tile issued with an unknown number of loads (a row that is not real)
   int issued = 0;
   const auto issue_next = [&]() __attribute__((always_inline)) {
     if (issued < ntiles) {
-      if (plain_rows) {
-        IssuePlainRowsBf16<kHbLoaders>(a, table_lds, tile_of(issued) * kTileTokens, seq_len - 1, slot_bits, lds_base + G::Slot(issued), lane, wave);
-      } else if (!IssueTileBf16<false>(a, map, il, tile_of(issued), lds_base + G::Slot(issued), lds + G::Slot(issued), tid)) {
-        last_unknown = issued;
+      if (wave < kHbLoaders) {
+        const int first = tile_of(issued) * kTileTokens, last = seq_len - 1;
+        const unsigned buf = lds_base + G::Slot(issued);
+        unsigned starts[kRowsPerLoader];
+#pragma unroll
+        for (int r = 0; r < kRowsPerLoader; ++r) starts[r] = latent_rows[min(first + wave + kHbLoaders * r, last)];
+        const unsigned rope_start = rope_rows[min(first + 8 * wave + (lane >> 3), last)];
+        if (plain_rows) {
+#pragma unroll
+          for (int r = 0; r < kRowsPerLoader; ++r) {
+            DirectLoad16PerLane(lat_lane[r & 3] + (static_cast<u64>(starts[r]) << 4), buf + (wave + kHbLoaders * r) * T::kLatRow);
+          }
+          DirectLoad16PerLane(rope_lane + (static_cast<u64>(rope_start) << 4), buf + T::kLatRegion + wave * 8 * T::kRopeRow);
+        } else {
+          unsigned char* tile = lds + G::Slot(issued);
+#pragma unroll
+          for (int r = 0; r < kRowsPerLoader; ++r) {
+            const int row = wave + kHbLoaders * r;
+            if (Uniform(starts[r]) != kNoRow) {
+              DirectLoad16PerLane(lat_lane[r & 3] + (static_cast<u64>(starts[r]) << 4), buf + row * T::kLatRow);
+            } else {
+              *reinterpret_cast<u32x4*>(tile + row * T::kLatRow + lane * 16) = u32x4{0u, 0u, 0u, 0u};
+            }
+          }
+          if (rope_start != kNoRow) {
+            DirectLoad16PerLane(rope_lane + (static_cast<u64>(rope_start) << 4), buf + T::kLatRegion + wave * 8 * T::kRopeRow);
+          } else {
+            *reinterpret_cast<u32x4*>(tile + T::kLatRegion + wave * 8 * T::kRopeRow + lane * 16) = u32x4{0u, 0u, 0u, 0u};
+          }
+          last_unknown = issued;
+        }
       }
       ++issued;
     }
@@ -1706,13 +1703,14 @@ __global__ __launch_bounds__(kHbThreads) void MlaSelectedHeadBlockKernel(AttnArg
   // (at most one tile here: the ring holds the tile in use, the next one and two on their way).
   const auto wait_tile = [&](int t) __attribute__((always_inline)) {
     if (per_tile == 0) return;
-    const int newer = last_unknown >= t ? 0 : max(0, issued - (t + 1)) * per_tile;
-    if (newer == 0) {
-      asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
-    } else if (newer == kPlainLoads) {
+    // (two newer tiles in the prologue, one in the loop, none at the end)
+    const int newer_tiles = last_unknown >= t ? 0 : issued - (t + 1);
+    if (newer_tiles >= 2) {
+      asm volatile("s_waitcnt vmcnt(%0)" ::"n"(2 * kPlainLoads) : "memory");
+    } else if (newer_tiles == 1) {
       asm volatile("s_waitcnt vmcnt(%0)" ::"n"(kPlainLoads) : "memory");
     } else {
-      WaitLoads(newer);
+      asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
     }
   };
   // Top of iteration i, both roles: tile i + 1 has landed; the barrier publishes it together with
@@ -2001,7 +1999,8 @@ hipError_t LaunchAttnDecode(const AttnArgs& args_in, hipStream_t stream) {
     int slot_bits = 0;
     while ((int64_t{1} << slot_bits) < args.block_size) ++slot_bits;
     if ((static_cast<int64_t>(args.num_blocks) << slot_bits) > (int64_t{1} << 31)) return hipErrorInvalidValue;
-    if (args.head_block_units) {
+    // (a pool whose rows the 32-bit starts of the whole-selection units cannot address goes to the split units)
+    if (args.head_block_units && PlainRowsAddressable(args)) {
       if (args.fp8 || args.sparse_count > kAttnHeadBlockTokens || args.heads % 16 != 0 || args.out == nullptr) return hipErrorInvalidValue;
       const int sequences_per_xcd = (args.batch + kXcds - 1) / kXcds;
       const dim3 units(kXcds * (args.heads / 16) * sequences_per_xcd);
