@@ -107,7 +107,7 @@ template <int HB>
 __global__ __launch_bounds__(kScoreThreads) void IndexerScoreKernel(IndexerArgs a) {
   extern __shared__ __attribute__((aligned(16))) unsigned char lds[];
   const unsigned lds_base = static_cast<unsigned>(reinterpret_cast<size_t>((__attribute__((address_space(3))) unsigned char*)lds));
-  constexpr int kQueryBytes = HB * 16 * kIndexDim;
+  constexpr int kQueryBytes = HB * 16 * kIndexDim * 2;  // the query as bf16: converted once per workgroup, not once per wavefront
   const int seq = blockIdx.y;
   const int lane = threadIdx.x & 63, wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
   const int r = lane & 15, g = lane >> 4;
@@ -120,31 +120,40 @@ __global__ __launch_bounds__(kScoreThreads) void IndexerScoreKernel(IndexerArgs 
   const int raw_len = a.seq_lens[seq];
   const int limit = a.max_seq_len;  // the caller's table rows address at least this many positions (checked on the host)
 
-  // Query codes: HB * 16 rows, eight per load instruction, the instructions dealt to the waves.
-  for (int j = wave; j < 2 * HB; j += kScoreThreads / 64) {
-    const int head = 8 * j + (lane >> 3);
-    const char* src = a.query + seq * a.query_seq_stride + head * a.query_head_stride + (((lane & 7) ^ Swizzle(head)) << 4);
-    DirectLoad16PerLane(src, lds_base + j * 1024);
+  // Query codes: HB * 16 rows of 128, eight rows per wavefront (16 codes per lane) for the first
+  // 2 HB wavefronts; they go to LDS as bf16 further down, with the rest of this round of loads.
+  static_assert(2 * HB <= kScoreThreads / 64, "one load of query codes per wavefront at most");
+  const bool converts_query = wave < 2 * HB;
+  const int query_head = 8 * wave + (lane >> 3);
+  u32x4 query_codes = {0u, 0u, 0u, 0u};
+  if (converts_query) {
+    query_codes = *reinterpret_cast<const u32x4*>(a.query + seq * a.query_seq_stride + query_head * a.query_head_stride + (lane & 7) * 16);
   }
   // wave-uniform: whether the weight and scale rows of every sequence start on 8 and 16 bytes
   const bool rows_aligned = ((reinterpret_cast<uintptr_t>(a.weights) | static_cast<uintptr_t>(a.weights_seq_stride)) & 7) == 0 &&
                             ((reinterpret_cast<uintptr_t>(a.query_scale) | static_cast<uintptr_t>(a.query_scale_seq_stride) * 4) & 15) == 0;
-  float w[HB][4];  // heads 16 hb + 4 g + j: the rows this lane holds of every product
+  // Head weights and query scales of heads 16 hb + 4 g + j, the rows this lane holds of every
+  // product: four consecutive heads are 8 bytes of weights and 16 bytes of scales. All of them are
+  // asked for here, with the query and the table entries, and turned into w[][] only below, once
+  // everything of this round has been asked for: used one block at a time they cost a memory
+  // latency per block of heads before the first key was asked for.
+  float w[HB][4];
+  u32x2 weight_pairs[HB];
+  f32x4 scale_fours[HB];
+  if (rows_aligned) {
 #pragma unroll
-  for (int hb = 0; hb < HB; ++hb) {
-    // four consecutive heads: 8 bytes of weights, 16 bytes of scales
-    const char* weights = a.weights + seq * a.weights_seq_stride + (16 * hb + 4 * g) * 2;
-    const float* scales = a.query_scale + seq * a.query_scale_seq_stride + 16 * hb + 4 * g;
-    if (rows_aligned) {
-      const u32x2 pair = *reinterpret_cast<const u32x2*>(weights);
-      const f32x4 four = *reinterpret_cast<const f32x4*>(scales);
-      w[hb][0] = Bf16BitsToF32(pair.x & 0xffffu) * four[0];
-      w[hb][1] = Bf16BitsToF32(pair.x >> 16) * four[1];
-      w[hb][2] = Bf16BitsToF32(pair.y & 0xffffu) * four[2];
-      w[hb][3] = Bf16BitsToF32(pair.y >> 16) * four[3];
-    } else {
+    for (int hb = 0; hb < HB; ++hb) {
+      weight_pairs[hb] = *reinterpret_cast<const u32x2*>(a.weights + seq * a.weights_seq_stride + (16 * hb + 4 * g) * 2);
+      scale_fours[hb] = *reinterpret_cast<const f32x4*>(a.query_scale + seq * a.query_scale_seq_stride + 16 * hb + 4 * g);
+    }
+  } else {
 #pragma unroll
-      for (int j = 0; j < 4; ++j) w[hb][j] = Bf16BitsToF32(reinterpret_cast<const unsigned short*>(weights)[j]) * scales[j];
+    for (int hb = 0; hb < HB; ++hb) {
+      const unsigned short* weights = reinterpret_cast<const unsigned short*>(a.weights + seq * a.weights_seq_stride + (16 * hb + 4 * g) * 2);
+      const float* scales = a.query_scale + seq * a.query_scale_seq_stride + 16 * hb + 4 * g;
+      weight_pairs[hb] = u32x2{static_cast<unsigned>(weights[0]) | (static_cast<unsigned>(weights[1]) << 16),
+                               static_cast<unsigned>(weights[2]) | (static_cast<unsigned>(weights[3]) << 16)};
+      scale_fours[hb] = f32x4{scales[0], scales[1], scales[2], scales[3]};
     }
   }
 
@@ -172,6 +181,21 @@ __global__ __launch_bounds__(kScoreThreads) void IndexerScoreKernel(IndexerArgs 
     }
   };
 
+#pragma unroll
+  for (int hb = 0; hb < HB; ++hb) {
+    w[hb][0] = Bf16BitsToF32(weight_pairs[hb].x & 0xffffu) * scale_fours[hb][0];
+    w[hb][1] = Bf16BitsToF32(weight_pairs[hb].x >> 16) * scale_fours[hb][1];
+    w[hb][2] = Bf16BitsToF32(weight_pairs[hb].y & 0xffffu) * scale_fours[hb][2];
+    w[hb][3] = Bf16BitsToF32(weight_pairs[hb].y >> 16) * scale_fours[hb][3];
+  }
+  // The query as bf16, 256 bytes per head, 16-byte piece p of head h at position p ^ (h % 16): the
+  // sixteen heads that the lanes of an MFMA operand read together fall into sixteen bank groups.
+  if (converts_query) {
+    unsigned char* row = lds + query_head * (kIndexDim * 2);
+    const int piece = 2 * (lane & 7), turn = query_head & 15;
+    *reinterpret_cast<bf16x8*>(row + ((piece ^ turn) << 4)) = CodesToBf16(query_codes.x, query_codes.y);
+    *reinterpret_cast<bf16x8*>(row + (((piece + 1) ^ turn) << 4)) = CodesToBf16(query_codes.z, query_codes.w);
+  }
   const int seq_len = min(raw_len, a.max_seq_len);
   if (seq_len <= a.sparse_count || group0 >= seq_len) {  // the whole workgroup; short sequences select everything without scores
     asm volatile("s_waitcnt vmcnt(0)" ::: "memory");  // no load may land in LDS that is no longer this workgroup's
@@ -203,16 +227,10 @@ __global__ __launch_bounds__(kScoreThreads) void IndexerScoreKernel(IndexerArgs 
     locate(lane, &block, &slot);
     my_scale = a.key_scale_base[block * a.key_scale_block_stride + slot];
   }
-  // Loads return in issue order: query, keys (two loads per group of 16 tokens), the scale. A
-  // group is scored while the later ones are still on their way: a wave that asked for keys has
-  // nine newer loads behind its query rows, so all but seven of them done means the query landed.
-  // A wave past the end of its sequence asked for no keys and waits for everything it issued.
-  if (wave_in_range && token0 < seq_len) {
-    asm volatile("s_waitcnt vmcnt(7)" ::: "memory");
-  } else {
-    asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
-  }
-  __syncthreads();  // the query rows the other waves fetched
+  // Loads return in issue order: keys (two loads per group of 16 tokens), then the scale. A group
+  // is scored while the later ones are still on their way. A wave past the end of its sequence
+  // asked for no keys.
+  __syncthreads();  // the query rows the other waves converted
   if (token0 >= seq_len) return;
 
   const unsigned char* q_lds = lds;
@@ -220,17 +238,15 @@ __global__ __launch_bounds__(kScoreThreads) void IndexerScoreKernel(IndexerArgs 
   bf16x8 q[HB][4];
 #pragma unroll
   for (int hb = 0; hb < HB; ++hb) {
-    const int head = 16 * hb + r;
-    const u32x4 lo = *reinterpret_cast<const u32x4*>(q_lds + head * kIndexDim + (((2 * g) ^ Swizzle(head)) << 4));
-    const u32x4 hi = *reinterpret_cast<const u32x4*>(q_lds + head * kIndexDim + (((2 * g + 1) ^ Swizzle(head)) << 4));
-    q[hb][0] = CodesToBf16(lo.x, lo.y);
-    q[hb][1] = CodesToBf16(lo.z, lo.w);
-    q[hb][2] = CodesToBf16(hi.x, hi.y);
-    q[hb][3] = CodesToBf16(hi.z, hi.w);
+#pragma unroll
+    for (int s = 0; s < 4; ++s) {
+      q[hb][s] = *reinterpret_cast<const bf16x8*>(q_lds + (16 * hb + r) * (kIndexDim * 2) + (((4 * g + s) ^ r) << 4));
+    }
   }
   float mine = 0.0f;  // score of token 16 g + r before its key scale
 #pragma unroll
   for (int rg = 0; rg < 4; ++rg) {
+    if (rg == 0) asm volatile("s_waitcnt vmcnt(7)" ::: "memory");
     if (rg == 1) asm volatile("s_waitcnt vmcnt(5)" ::: "memory");
     if (rg == 2) asm volatile("s_waitcnt vmcnt(3)" ::: "memory");
     if (rg == 3) asm volatile("s_waitcnt vmcnt(1)" ::: "memory");
@@ -275,6 +291,19 @@ __device__ __forceinline__ void LoadKeys(const unsigned short* keys, int first, 
   }
 }
 
+// Inclusive prefix sum over the 64 lanes with data-parallel-primitive moves (no LDS crossbar, no
+// wait per step): four shifted adds inside each row of 16 lanes, then lane 15 of rows 0 and 2 onto
+// rows 1 and 3, then lane 31 onto the upper half. Lanes a move does not reach add zero.
+__device__ __forceinline__ int WaveInclusiveScan(int v) {
+  v += __builtin_amdgcn_update_dpp(0, v, 0x111, 0xf, 0xf, false);  // row_shr:1
+  v += __builtin_amdgcn_update_dpp(0, v, 0x112, 0xf, 0xf, false);  // row_shr:2
+  v += __builtin_amdgcn_update_dpp(0, v, 0x114, 0xf, 0xf, false);  // row_shr:4
+  v += __builtin_amdgcn_update_dpp(0, v, 0x118, 0xf, 0xf, false);  // row_shr:8
+  v += __builtin_amdgcn_update_dpp(0, v, 0x142, 0xa, 0xf, false);  // row_bcast:15 into rows 1 and 3
+  v += __builtin_amdgcn_update_dpp(0, v, 0x143, 0xc, 0xf, false);  // row_bcast:31 into rows 2 and 3
+  return v;
+}
+
 // The byte value that holds the `wanted`-th largest entry of a 256-bin histogram, and the number
 // of entries above that bin, found by the first wavefront (four bins per lane, a suffix sum over
 // the lanes) and handed to everyone through `result`.
@@ -286,13 +315,9 @@ __device__ __forceinline__ void FindBin(const int* histogram, int wanted, int* r
       bins[i] = histogram[4 * tid + i];
       mine += bins[i];
     }
-    int suffix = mine;  // inclusive sum over this lane and the lanes above it
-#pragma unroll
-    for (int offset = 1; offset < 64; offset <<= 1) {
-      const int higher = __shfl_down(suffix, offset);
-      if (tid + offset < 64) suffix += higher;
-    }
-    int above = suffix - mine;
+    // the sum over the lanes above this one: everything minus this lane's inclusive prefix
+    const int inclusive = WaveInclusiveScan(mine);
+    int above = __builtin_amdgcn_readlane(inclusive, 63) - inclusive;
 #pragma unroll
     for (int i = 3; i >= 0; --i) {
       if (above < wanted && wanted <= above + bins[i]) {
@@ -379,12 +404,7 @@ __global__ __launch_bounds__(kSelectThreads) void IndexerSelectKernel(IndexerArg
     }
     // exclusive prefix over the threads of both counts at once (each below 2^16 per pass)
     const int packed = greater | (equal << 16);
-    int inclusive = packed;
-#pragma unroll
-    for (int offset = 1; offset < 64; offset <<= 1) {
-      const int below = __shfl_up(inclusive, offset);
-      if (lane >= offset) inclusive += below;
-    }
+    const int inclusive = WaveInclusiveScan(packed);
     __syncthreads();  // wave_counts of the previous pass have been read
     if (lane == 63) wave_counts[wave] = inclusive;
     __syncthreads();
@@ -455,13 +475,13 @@ __global__ __launch_bounds__(256) void IndexKeyAppendKernel(IndexKeyAppendArgs a
 // Dynamic LDS above 64 KB needs the attribute per kernel and device (PrepareIndexerKernels).
 template <int HB>
 hipError_t PrepareScore() {
-  constexpr int kLdsBytes = HB * 16 * kIndexDim + kTokensPerGroup * kIndexDim;
+  constexpr int kLdsBytes = HB * 16 * kIndexDim * 2 + kTokensPerGroup * kIndexDim;
   return hipFuncSetAttribute(reinterpret_cast<const void*>(&IndexerScoreKernel<HB>), hipFuncAttributeMaxDynamicSharedMemorySize, kLdsBytes);
 }
 
 template <int HB>
 hipError_t LaunchScore(const IndexerArgs& args, const dim3& grid, hipStream_t stream) {
-  constexpr int kLdsBytes = HB * 16 * kIndexDim + kTokensPerGroup * kIndexDim;  // query codes + the keys of eight waves
+  constexpr int kLdsBytes = HB * 16 * kIndexDim * 2 + kTokensPerGroup * kIndexDim;  // the query as bf16 + the key codes of eight waves
   hipLaunchKernelGGL(IndexerScoreKernel<HB>, grid, dim3(kScoreThreads), kLdsBytes, stream, args);
   return hipGetLastError();
 }
