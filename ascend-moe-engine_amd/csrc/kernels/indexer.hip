@@ -335,8 +335,8 @@ __device__ __forceinline__ void FindBin(const int* histogram, int wanted, int* r
 // order. (Measured at 8192 keys: this 7.1 us; 256 threads of 32 keys 10.0 us; sixteen one-bit
 // counting rounds 14 us; one atomic per key with a serial bin search 31.6 us.)
 __global__ __launch_bounds__(kSelectThreads) void IndexerSelectKernel(IndexerArgs a) {
-  __shared__ int histogram[256];
-  __shared__ int found[2];
+  __shared__ int histograms[2][256];  // of the high bytes, then of the low bytes among the keys with the high byte found
+  __shared__ int founds[2][2];
   __shared__ int wave_counts[kSelectWaves];
   const int seq = blockIdx.x, tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
   const int n = max(min(a.seq_lens[seq], a.max_seq_len), 0);
@@ -352,10 +352,14 @@ __global__ __launch_bounds__(kSelectThreads) void IndexerSelectKernel(IndexerArg
   LoadKeys(keys, tid * kKeysPerThread, n, first);
 
   int prefix = 0, wanted = k;  // the bytes of the k-th largest key decided so far; how many of the candidates are wanted
+  // both histograms are cleared here and each round has its own result words, so a round is two
+  // barriers: the counts complete, the bin found
+  if (tid < 512) histograms[tid >> 8][tid & 255] = 0;
+  __syncthreads();
 #pragma unroll
   for (int shift = 8; shift >= 0; shift -= 8) {
-    for (int i = tid; i < 256; i += kSelectThreads) histogram[i] = 0;
-    __syncthreads();
+    int* histogram = histograms[shift == 8 ? 0 : 1];
+    int* found = founds[shift == 8 ? 0 : 1];
     for (int pass = 0; pass < passes; ++pass) {
       int more[kKeysPerThread];
       if (pass > 0) LoadKeys(keys, pass * kKeysPerPass + tid * kKeysPerThread, n, more);
@@ -383,7 +387,6 @@ __global__ __launch_bounds__(kSelectThreads) void IndexerSelectKernel(IndexerArg
     __syncthreads();
     prefix = shift == 8 ? found[0] : (prefix << 8) | found[0];
     wanted -= found[1];
-    __syncthreads();
   }
   const int threshold = prefix, equal_wanted = wanted, greater_total = k - wanted;
 
