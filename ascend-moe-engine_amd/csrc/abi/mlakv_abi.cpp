@@ -386,7 +386,7 @@ mlakvStatus AttnPlanImpl(const char* who, int32_t batch, int32_t heads, int32_t 
   if (options != nullptr) chosen = *options;
   if (chosen.chunk_tiles < 0 || chosen.work_groups < 0 || chosen.work_groups > 65535 || chosen.merge_mode < 0 ||
       chosen.merge_mode > MLAKV_ATTN_MERGE_SECOND_LAUNCH || chosen.merge_spin_us > 1000000 || chosen.selection_units < 0 ||
-      chosen.selection_units > MLAKV_ATTN_UNITS_HEAD_BLOCK || (!sparse && chosen.selection_units != 0)) {
+      chosen.selection_units > MLAKV_ATTN_UNITS_HEAD_BLOCK_HALVES || (!sparse && chosen.selection_units != 0)) {
     return Fail(MLAKV_ERR_PARAM_INVALID, "%s: options outside their ranges", who);
   }
   const int64_t head_groups = (heads + 63) / 64;
@@ -422,20 +422,36 @@ mlakvStatus AttnPlanImpl(const char* who, int32_t batch, int32_t heads, int32_t 
   // Whole-selection units of 16 heads where they apply, unless the caller asked for properties of
   // the split (a unit size, a workgroup count, a merge).
   const bool head_block_fits = sparse && dtype == MLAKV_DTYPE_BF16 && max_seq_len <= MLAKV_ATTN_HEAD_BLOCK_TOKENS;
-  if (chosen.selection_units == MLAKV_ATTN_UNITS_HEAD_BLOCK && !head_block_fits) {
+  const bool head_block_asked = chosen.selection_units == MLAKV_ATTN_UNITS_HEAD_BLOCK || chosen.selection_units == MLAKV_ATTN_UNITS_HEAD_BLOCK_HALVES;
+  if (head_block_asked && !head_block_fits) {
     return Fail(MLAKV_ERR_PARAM_INVALID, "%s: whole-selection units of 16 heads take a bf16 cache and up to %d selected tokens", who,
                 MLAKV_ATTN_HEAD_BLOCK_TOKENS);
   }
+  // Halved units leave two partials of 16 rows per (sequence, 16 heads) in the workspace and meet on
+  // one of the library's counters each.
+  const int64_t pairs = static_cast<int64_t>(batch) * (heads / 16);
+  const bool halves_fit = head_block_fits && pairs <= 2 * mlakv::kAttnSyncSequences &&
+                          pairs * 32 <= shape.head_groups * (shape.units + batch) * 64;
+  if (chosen.selection_units == MLAKV_ATTN_UNITS_HEAD_BLOCK_HALVES && !halves_fit) {
+    return Fail(MLAKV_ERR_PARAM_INVALID, "%s: halved whole-selection units take up to %d (sequence, 16 heads) pairs whose partials fit the workspace",
+                who, 2 * mlakv::kAttnSyncSequences);
+  }
   const bool split_asked = chosen.chunk_tiles != 0 || chosen.work_groups != 0 || chosen.merge_mode != 0;
   // Measured on MI355X (batch 4 .. 128, 64 and 128 heads): a whole-selection unit streams a tile per
-  // 0.8 us after 5.5 us of set-up, so with one unit per CU it is ahead of the split up to 512
+  // 0.7 us after 5.5 us of set-up, so with one unit per CU it is ahead of the split up to 512
   // selected tokens (8.5 against 12 us at 64, 12 against 19 us at 256, level at 512), with two
-  // units per CU up to 256, and behind beyond that.
+  // units per CU up to 256, and behind beyond that. While two workgroups per unit still fit the CUs
+  // once, halving the units pays from 257 selected tokens (the exchange costs what four tiles do:
+  // 11.5 us either way at 256) to 768 (15.2 against 17.5 us at 512, 18.9 against 21.0 us for the
+  // split at 768; the split is ahead again at 1024).
   const int64_t rounds = (static_cast<int64_t>(batch) * (heads / 16) + ComputeUnits() - 1) / ComputeUnits();
   const bool head_block_pays = (rounds <= 1 && max_seq_len <= 512) || (rounds <= 2 && max_seq_len <= 256);
   const bool head_block = head_block_fits && (chosen.selection_units == MLAKV_ATTN_UNITS_HEAD_BLOCK ||
                                               (chosen.selection_units == MLAKV_ATTN_UNITS_AUTO && !split_asked && head_block_pays));
-  plan->selection_units = !sparse ? 0 : (head_block ? MLAKV_ATTN_UNITS_HEAD_BLOCK : MLAKV_ATTN_UNITS_SPLIT);
+  const bool halves_pay = 2 * pairs <= ComputeUnits() && max_seq_len > 256 && max_seq_len <= 768;
+  const bool halves = chosen.selection_units == MLAKV_ATTN_UNITS_HEAD_BLOCK_HALVES ||
+                      (chosen.selection_units == MLAKV_ATTN_UNITS_AUTO && !split_asked && halves_fit && halves_pay);
+  plan->selection_units = !sparse ? 0 : (halves ? MLAKV_ATTN_UNITS_HEAD_BLOCK_HALVES : (head_block ? MLAKV_ATTN_UNITS_HEAD_BLOCK : MLAKV_ATTN_UNITS_SPLIT));
   plan->workspace_bytes = shape.workspace;
   return MLAKV_SUCCESS;
 }
@@ -519,8 +535,9 @@ mlakvStatus AttnDecodeImpl(const char* who, const mlakvAttnPlan* plan, const mla
                         plan->work_groups <= 65535 && (plan->reserved == 0 || plan->reserved == 1) &&
                         (plan->reserved == 0 ? plan->selection_units == 0
                                              : (plan->selection_units == MLAKV_ATTN_UNITS_SPLIT ||
-                                                (plan->selection_units == MLAKV_ATTN_UNITS_HEAD_BLOCK && plan->dtype == MLAKV_DTYPE_BF16 &&
-                                                 plan->max_seq_len <= MLAKV_ATTN_HEAD_BLOCK_TOKENS))) &&
+                                                ((plan->selection_units == MLAKV_ATTN_UNITS_HEAD_BLOCK ||
+                                                  plan->selection_units == MLAKV_ATTN_UNITS_HEAD_BLOCK_HALVES) &&
+                                                 plan->dtype == MLAKV_DTYPE_BF16 && plan->max_seq_len <= MLAKV_ATTN_HEAD_BLOCK_TOKENS))) &&
                         (plan->reserved == 0 || plan->max_seq_len <= 2048) &&
                         (plan->merge_mode == MLAKV_ATTN_MERGE_IN_LAUNCH || plan->merge_mode == MLAKV_ATTN_MERGE_SECOND_LAUNCH) &&
                         (plan->merge_spin_us == -1 || (plan->merge_spin_us > 0 && plan->merge_spin_us <= 1000000));
@@ -623,7 +640,7 @@ mlakvStatus AttnDecodeImpl(const char* who, const mlakvAttnPlan* plan, const mla
   args.spin_ticks = plan->merge_spin_us < 0 ? 0 : plan->merge_spin_us * 100;
   args.merge_in_launch = plan->merge_mode == MLAKV_ATTN_MERGE_IN_LAUNCH;
   args.fp8 = cache->dtype == MLAKV_DTYPE_FP8_E4M3;
-  args.head_block_units = plan->selection_units == MLAKV_ATTN_UNITS_HEAD_BLOCK;
+  args.head_block_units = plan->selection_units == MLAKV_ATTN_UNITS_HEAD_BLOCK ? 1 : (plan->selection_units == MLAKV_ATTN_UNITS_HEAD_BLOCK_HALVES ? 2 : 0);
   const hipError_t status = mlakv::LaunchAttnDecode(args, static_cast<hipStream_t>(stream));
   return status == hipSuccess ? MLAKV_SUCCESS : HipFail(status, who);
 }

@@ -128,8 +128,9 @@ struct AttnArgs {
   bool merge_in_launch;       // false: the merge is a second launch
   bool fp8;
   // Selected-token attention only: a workgroup takes the whole selection of one sequence for one
-  // block of 16 heads (no partials, no merge); sparse_count <= kAttnHeadBlockTokens, bf16 cache.
-  bool head_block_units;
+  // block of 16 heads (1: no partials, no merge), or two workgroups take half of it each and the
+  // second to finish combines the two (2); sparse_count <= kAttnHeadBlockTokens, bf16 cache. 0: the split units.
+  int32_t head_block_units;
   unsigned* sync;             // set by the launcher: this launch's counters, null for a second-launch merge
   // Host-known lengths of a small batch travel here instead of through device memory: no upload,
   // no launch for it, and the kernels' first dependent load is gone. inline_count = 0: unused.

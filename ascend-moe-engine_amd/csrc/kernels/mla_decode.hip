@@ -1525,6 +1525,15 @@ __global__ __launch_bounds__(kMergeHeads * 64) void MlaMergeKernel(AttnArgs a) {
 //     reference maximum without exchanging it), forms P in registers as its MFMA operand and
 //     multiplies it with its 128 columns of V.
 // The tile ring, the operand layouts and the barrier per tile are those of the kernel above.
+//
+// HALVES: two workgroups per (sequence, 16 heads), neighbours on one XCD, each with one half of the
+// selection's tiles, so that twice as many CUs (and twice as many rows in flight) work on a launch
+// that has fewer units than the chip has CUs. Each leaves its normalised partial (bf16 rows and a
+// log2-domain LSE per head, agent-scope stores) in the workspace and counts itself on the pair's
+// word; the one that finds the other's count there reads that partial back, combines it with what
+// it still holds in registers (fp32) and writes the output. Nobody waits: the first to arrive
+// leaves. The pair's word is zero between launches (the second to arrive clears it). A selection
+// of a single tile is taken by the first workgroup alone.
 constexpr int kHbWaves = kWaves, kHbThreads = kHbWaves * 64;
 constexpr int kHbLoaders = kScoreWaves;  // the waves that fetch the tiles when every row is a plain row
 struct GeomHeadBlock {
@@ -1539,6 +1548,7 @@ struct GeomHeadBlock {
 };
 constexpr int kHeadBlockKSteps = kKSteps / 2;  // k-steps of one score wave
 
+template <bool HALVES>
 __global__ __launch_bounds__(kHbThreads) void MlaSelectedHeadBlockKernel(AttnArgs a) {
   using G = GeomHeadBlock;
   using T = Geom<false>;
@@ -1550,8 +1560,10 @@ __global__ __launch_bounds__(kHbThreads) void MlaSelectedHeadBlockKernel(AttnArg
   // the head blocks of a sequence are neighbours among them.
   const int head_blocks = a.heads >> 4;  // heads is a multiple of 16
   const int rest = blockIdx.x >> 3;
-  const int hb = rest % head_blocks;
-  const int seq = (rest / head_blocks) * kXcds + (blockIdx.x & (kXcds - 1));
+  const int half = HALVES ? rest & 1 : 0;
+  const int unit = HALVES ? rest >> 1 : rest;
+  const int hb = unit % head_blocks;
+  const int seq = (unit / head_blocks) * kXcds + (blockIdx.x & (kXcds - 1));
   if (seq >= a.batch) return;
   const bool score_wave = wave < kScoreWaves;
   const int hw = wave & (kScoreWaves - 1);
@@ -1635,7 +1647,12 @@ __global__ __launch_bounds__(kHbThreads) void MlaSelectedHeadBlockKernel(AttnArg
   seq_len = Uniform(seq_len);
   // Every row a real row of the pool (the usual case): the tile loads need no case distinction.
   const bool plain_rows = Uniform(outside) == 0;
-  const int ntiles = (seq_len + kTileTokens - 1) / kTileTokens;
+  const int all_tiles = (seq_len + kTileTokens - 1) / kTileTokens;
+  // two workgroups share a selection of at least two tiles: the first ceil(all / 2), then the rest
+  const bool shared = HALVES && all_tiles >= 2;
+  if (HALVES && !shared && half != 0) return;
+  const int first_tile = shared && half != 0 ? (all_tiles + 1) >> 1 : 0;
+  const int ntiles = shared ? (half != 0 ? all_tiles >> 1 : (all_tiles + 1) >> 1) : all_tiles;
   if (ntiles == 0) {  // nothing selected: zeros, lse = -inf
     for (int h = wave; h < 16; h += kHbWaves) {
       *reinterpret_cast<u32x4*>(a.out + seq * a.out_seq_stride + (16 * hb + h) * a.out_head_stride + lane * 16) = u32x4{0u, 0u, 0u, 0u};
@@ -1648,7 +1665,9 @@ __global__ __launch_bounds__(kHbThreads) void MlaSelectedHeadBlockKernel(AttnArg
   // tiles only changes the rounding): at any time they ask for different rows, and what one has
   // fetched the others find in the L2.
   const int rotate = hb * ntiles / head_blocks;
-  const auto tile_of = [&](int i) __attribute__((always_inline)) { return i + rotate < ntiles ? i + rotate : i + rotate - ntiles; };
+  const auto tile_of = [&](int i) __attribute__((always_inline)) {
+    return first_tile + (i + rotate < ntiles ? i + rotate : i + rotate - ntiles);
+  };
   // The score waves fetch the tiles: wave w the latent rows w, w + 4, ... (one row per load: lane L
   // asks for the 16 bytes that belong at 16 L of the swizzled LDS row) and the rope rows 8 w .. 8 w + 7
   // (one load, a row per eight lanes). A lane's address is the plane's base, its own chunk and the
@@ -1766,6 +1785,10 @@ __global__ __launch_bounds__(kHbThreads) void MlaSelectedHeadBlockKernel(AttnArg
       if (i + 1 < ntiles) score(i + 1);
     }
     __syncthreads();  // every output wave is through with the last tile (the ring becomes their staging space)
+    if (shared) {     // the output waves' two barriers around the count on the pair's word
+      __syncthreads();
+      __syncthreads();
+    }
   } else {
     // ------------------------------------------------------------------ output waves
     // bf16 V reads as in the kernel above: token = (16 +) 4g + i16/4, chunk = 2n + (i16 & 3) / 2, 8-byte half i16 & 1.
@@ -1842,30 +1865,78 @@ __global__ __launch_bounds__(kHbThreads) void MlaSelectedHeadBlockKernel(AttnArg
     __syncthreads();  // every output wave is through with the last tile
     const float l_total = SumAcrossHeadLanes(l_run);
     const float inv = 1.0f / l_total;
-    if (hw == 0 && g == 0 && a.lse != nullptr) {
-      a.lse[seq * a.heads + head] = (m_ref + __builtin_amdgcn_logf(l_total)) * 0.6931471805599453f;  // v_log_f32 is log2
-    }
+    float lse2 = m_ref + __builtin_amdgcn_logf(l_total);  // v_log_f32 is log2
+#pragma unroll
+    for (int n = 0; n < kDvPerWave; ++n) o[n] *= inv;
     // The accumulators hold O^T (lane = head i16, four columns per 16-column tile); each wave turns
     // its 256-byte slices of the 16 rows through its own part of the dead ring (row stride 272 B)
     // and writes them 16 bytes per lane, four whole slices per instruction.
     constexpr int kSliceBytes = kDvPerWave * 16 * 2;  // 256
     constexpr int kStageRow = kSliceBytes + 16;
     unsigned char* stage = lds + G::Slot(0) + hw * (16 * kStageRow);
-#pragma unroll
-    for (int n = 0; n < kDvPerWave; ++n) {
-      u32x2 packed;
-      packed.x = PackBf16(o[n][0] * inv, o[n][1] * inv);
-      packed.y = PackBf16(o[n][2] * inv, o[n][3] * inv);
-      *reinterpret_cast<u32x2*>(stage + i16 * kStageRow + (16 * n + 4 * g) * 2) = packed;
-    }
-    // Same wave wrote and reads: the LDS queue is in order, no barrier needed.
     const int piece = lane & 15, sub = lane >> 4;
+    // (same wave writes and reads the staging rows: the LDS queue is in order, no barrier needed)
+    const auto rows_of_o = [&](u32x4 (&v)[4]) __attribute__((always_inline)) {
+#pragma unroll
+      for (int n = 0; n < kDvPerWave; ++n) {
+        u32x2 packed;
+        packed.x = PackBf16(o[n][0], o[n][1]);
+        packed.y = PackBf16(o[n][2], o[n][3]);
+        *reinterpret_cast<u32x2*>(stage + i16 * kStageRow + (16 * n + 4 * g) * 2) = packed;
+      }
+#pragma unroll
+      for (int it = 0; it < 4; ++it) v[it] = *reinterpret_cast<const u32x4*>(stage + (4 * it + sub) * kStageRow + piece * 16);
+    };
+    u32x4 v[4];
+    if (shared) {
+      // this half's partial: 16 rows of 1 KB and 16 LSEs, at (pair, half) of the workspace
+      const int pair = seq * head_blocks + hb;
+      const int64_t row0 = static_cast<int64_t>(2 * pair + half) * 16, other0 = static_cast<int64_t>(2 * pair + (half ^ 1)) * 16;
+      rows_of_o(v);
+      char* mine = a.partial_out + row0 * (kLatentDim * 2) + kSliceBytes * hw + piece * 16;
+#pragma unroll
+      for (int it = 0; it < 4; ++it) StoreAgent16(mine + (4 * it + sub) * (kLatentDim * 2), v[it]);
+      if (hw == 0 && g == 0) StoreAgentF32(a.partial_lse + row0 + i16, lse2);
+      asm volatile("s_waitcnt vmcnt(0)" ::: "memory");  // this wave's partial stores are complete
+      __syncthreads();                                  // every wave's are
+      unsigned* arrived_lds = reinterpret_cast<unsigned*>(lds + G::kSOff);
+      if (hw == 0 && lane == 0) *arrived_lds = __hip_atomic_fetch_add(a.sync + pair, 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+      __syncthreads();
+      if (Uniform(*arrived_lds) == 0u) return;  // the other half will find this partial
+      if (hw == 0 && lane == 0) __hip_atomic_store(a.sync + pair, 0u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+      const float lse2_other = LoadAgentF32(a.partial_lse + other0 + i16);
+      const char* theirs = a.partial_out + other0 * (kLatentDim * 2) + kSliceBytes * hw + piece * 16;
+#pragma unroll
+      for (int it = 0; it < 4; ++it) v[it] = LoadAgent16(theirs + (4 * it + sub) * (kLatentDim * 2));
+      asm volatile("s_waitcnt vmcnt(0)" : "+v"(v[0]), "+v"(v[1]), "+v"(v[2]), "+v"(v[3]) : : "memory");
+#pragma unroll
+      for (int it = 0; it < 4; ++it) *reinterpret_cast<u32x4*>(stage + (4 * it + sub) * kStageRow + piece * 16) = v[it];
+      // Whichever half arrives second, the result is the same: both partials enter as the bf16
+      // rows that were stored, the first half's term first.
+      const float top = fmaxf(lse2, lse2_other);
+      const float w_mine = __builtin_amdgcn_exp2f(lse2 - top), w_theirs = __builtin_amdgcn_exp2f(lse2_other - top);
+      const float inv_w = 1.0f / (w_mine + w_theirs);
+      const bool second_half = half != 0;
+      const float c_first = (second_half ? w_theirs : w_mine) * inv_w, c_second = (second_half ? w_mine : w_theirs) * inv_w;
+#pragma unroll
+      for (int n = 0; n < kDvPerWave; ++n) {
+        const u32x2 packed = *reinterpret_cast<const u32x2*>(stage + i16 * kStageRow + (16 * n + 4 * g) * 2);
+        const float theirs[4] = {__builtin_bit_cast(float, packed.x << 16), __builtin_bit_cast(float, packed.x & 0xffff0000u),
+                                 __builtin_bit_cast(float, packed.y << 16), __builtin_bit_cast(float, packed.y & 0xffff0000u)};
+#pragma unroll
+        for (int j = 0; j < 4; ++j) {
+          const float mine = static_cast<float>(static_cast<__bf16>(o[n][j]));
+          o[n][j] = (second_half ? theirs[j] : mine) * c_first + (second_half ? mine : theirs[j]) * c_second;
+        }
+      }
+      lse2 = top + __builtin_amdgcn_logf(w_mine + w_theirs);
+    }
+    if (hw == 0 && g == 0 && a.lse != nullptr) a.lse[seq * a.heads + head] = lse2 * 0.6931471805599453f;
+    rows_of_o(v);
     char* out0 = a.out + seq * a.out_seq_stride + (16 * hb) * a.out_head_stride + kSliceBytes * hw + piece * 16;
 #pragma unroll
     for (int it = 0; it < 4; ++it) {
-      const int h = 4 * it + sub;
-      const u32x4 v = *reinterpret_cast<const u32x4*>(stage + h * kStageRow + piece * 16);
-      __builtin_nontemporal_store(v, reinterpret_cast<u32x4*>(out0 + h * a.out_head_stride));
+      __builtin_nontemporal_store(v[it], reinterpret_cast<u32x4*>(out0 + (4 * it + sub) * a.out_head_stride));
     }
   }
 }
@@ -1937,7 +2008,9 @@ hipError_t PrepareAttnKernels() {
       PrepareDecode<true, true, true, false>(),   PrepareDecode<true, false, true, false>(),
       PrepareDecode<false, false, false, true>(), PrepareDecode<true, false, false, true>(),
       PrepareMerge<false, false>(), PrepareMerge<true, false>(), PrepareMerge<false, true>(),
-      hipFuncSetAttribute(reinterpret_cast<const void*>(&MlaSelectedHeadBlockKernel), hipFuncAttributeMaxDynamicSharedMemorySize,
+      hipFuncSetAttribute(reinterpret_cast<const void*>(&MlaSelectedHeadBlockKernel<false>), hipFuncAttributeMaxDynamicSharedMemorySize,
+                          GeomHeadBlock::kLdsBytes),
+      hipFuncSetAttribute(reinterpret_cast<const void*>(&MlaSelectedHeadBlockKernel<true>), hipFuncAttributeMaxDynamicSharedMemorySize,
                           GeomHeadBlock::kLdsBytes)};
   for (const hipError_t e : results) {
     if (e != hipSuccess) return e;
@@ -2000,11 +2073,22 @@ hipError_t LaunchAttnDecode(const AttnArgs& args_in, hipStream_t stream) {
     while ((int64_t{1} << slot_bits) < args.block_size) ++slot_bits;
     if ((static_cast<int64_t>(args.num_blocks) << slot_bits) > (int64_t{1} << 31)) return hipErrorInvalidValue;
     // (a pool whose rows the 32-bit starts of the whole-selection units cannot address goes to the split units)
-    if (args.head_block_units && PlainRowsAddressable(args)) {
+    if (args.head_block_units != 0 && PlainRowsAddressable(args)) {
       if (args.fp8 || args.sparse_count > kAttnHeadBlockTokens || args.heads % 16 != 0 || args.out == nullptr) return hipErrorInvalidValue;
       const int sequences_per_xcd = (args.batch + kXcds - 1) / kXcds;
-      const dim3 units(kXcds * (args.heads / 16) * sequences_per_xcd);
-      hipLaunchKernelGGL(MlaSelectedHeadBlockKernel, units, dim3(kHbThreads), GeomHeadBlock::kLdsBytes, stream, args);
+      const int64_t pairs = static_cast<int64_t>(args.batch) * (args.heads / 16);
+      // Two workgroups per unit meet on one word each of this launch's counters and leave their
+      // partials in the first 2 x 16 x pairs rows of the workspace.
+      const bool halves = args.head_block_units == 2 && pairs <= kAttnSyncSequences * 2 && args.partial_out != nullptr &&
+                          pairs * 32 <= static_cast<int64_t>(head_groups) * (args.max_units + args.batch) * 64;
+      if (halves) {
+        if (hipError_t sync_error = SyncRegion(&args.sync); sync_error != hipSuccess) return sync_error;
+        const dim3 units(kXcds * (args.heads / 16) * 2 * sequences_per_xcd);
+        hipLaunchKernelGGL(MlaSelectedHeadBlockKernel<true>, units, dim3(kHbThreads), GeomHeadBlock::kLdsBytes, stream, args);
+      } else {
+        const dim3 units(kXcds * (args.heads / 16) * sequences_per_xcd);
+        hipLaunchKernelGGL(MlaSelectedHeadBlockKernel<false>, units, dim3(kHbThreads), GeomHeadBlock::kLdsBytes, stream, args);
+      }
       return hipGetLastError();
     }
     e = args.fp8 ? Launch<true, false, false, true>(args, grid, stream) : Launch<false, false, false, true>(args, grid, stream);

@@ -66,7 +66,7 @@ class AttnPlanOptions(C.Structure):
 
 
 ATTN_MERGE_AUTO, ATTN_MERGE_IN_LAUNCH, ATTN_MERGE_SECOND_LAUNCH = 0, 1, 2
-ATTN_UNITS_AUTO, ATTN_UNITS_SPLIT, ATTN_UNITS_HEAD_BLOCK = 0, 1, 2
+ATTN_UNITS_AUTO, ATTN_UNITS_SPLIT, ATTN_UNITS_HEAD_BLOCK, ATTN_UNITS_HEAD_BLOCK_HALVES = 0, 1, 2, 3
 ATTN_HEAD_BLOCK_TOKENS = 1024
 
 

@@ -91,7 +91,7 @@ def parse_args():
     p.add_argument("--attention-only", action="store_true", help="development aid: time only the attention configurations")
     p.add_argument("--config5-only", action="store_true", help="development aid: run only the continuous-batching loop of configs[4]")
     p.add_argument("--config5-pool-gb", type=float, default=200.0, help="KV pool of the configs[4] loop, in GB (clamped to free memory)")
-    p.add_argument("--attn-units", choices=["auto", "split", "head-block"], default="auto",
+    p.add_argument("--attn-units", choices=["auto", "split", "head-block", "halves"], default="auto",
                    help="development aid: how the selected-token attention cuts its work (MLAKV_ATTN_UNITS_*)")
     p.add_argument("--attn-merge", choices=["auto", "in", "second"], default="auto",
                    help="development aid: how the attention launches merge their partials (default: the planner's choice)")
@@ -302,7 +302,7 @@ def bench_attention(args, torch, np, ffi, ctxs, fp8=False, heads=64, slices=8, i
                         pool_blocks=pool_blocks, seed=7, shuffle=1, dtype=ffi.DTYPE_FP8_E4M3 if fp8 else ffi.DTYPE_BF16)
     plan = ffi.AttnPlan()
     merge_mode = {"auto": ffi.ATTN_MERGE_AUTO, "in": ffi.ATTN_MERGE_IN_LAUNCH, "second": ffi.ATTN_MERGE_SECOND_LAUNCH}[args.attn_merge]
-    units = {"auto": ffi.ATTN_UNITS_AUTO, "split": ffi.ATTN_UNITS_SPLIT, "head-block": ffi.ATTN_UNITS_HEAD_BLOCK}[args.attn_units] if sparse_k else 0
+    units = {"auto": ffi.ATTN_UNITS_AUTO, "split": ffi.ATTN_UNITS_SPLIT, "head-block": ffi.ATTN_UNITS_HEAD_BLOCK, "halves": ffi.ATTN_UNITS_HEAD_BLOCK_HALVES}[args.attn_units] if sparse_k else 0
     if merge_mode != ffi.ATTN_MERGE_AUTO or args.attn_chunk_tiles or args.attn_work_groups or units:
         options = ffi.AttnPlanOptions(args.attn_chunk_tiles, args.attn_work_groups, merge_mode, 0, 1 if sparse_k else 0, units)
         ffi.check(lib.mlakvAttnPlanInitEx(batch, heads, sparse_k or max_ctx, bs, cache.config.dtype, C.byref(options), C.byref(plan)))
@@ -418,6 +418,8 @@ def bench_attention(args, torch, np, ffi, ctxs, fp8=False, heads=64, slices=8, i
         "mfma_frac_of_bf16_peak": flops / (us * 1e-6) / 1e12 / MFMA_BF16_PEAK_TFLOPS,
         "work_groups": int(plan.work_groups), "max_units": int(plan.max_units),
         "merge": ("none (a unit holds a whole selection for 16 heads)" if plan.selection_units == ffi.ATTN_UNITS_HEAD_BLOCK
+                  else "in launch, pairs (two workgroups per selection and 16 heads; the second to finish combines)"
+                  if plan.selection_units == ffi.ATTN_UNITS_HEAD_BLOCK_HALVES
                   else "in launch" if plan.merge_mode == ffi.ATTN_MERGE_IN_LAUNCH else "second launch"),
         "workspace_bytes": int(plan.workspace_bytes), "timing": "250 ms of back-to-back launches untimed, then at least 100 ms of them timed",
     }

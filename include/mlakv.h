@@ -186,7 +186,7 @@ typedef struct mlakvAttnPlan {
   int32_t merge_mode;      /* MLAKV_ATTN_MERGE_IN_LAUNCH or _SECOND_LAUNCH */
   int32_t merge_spin_us;   /* bound of the in-launch merge's wait for a sequence's other partials */
   int32_t reserved;        /* 1: made by mlakvAttnSparsePlanInit (max_seq_len holds sparse_count) */
-  int32_t selection_units; /* MLAKV_ATTN_UNITS_SPLIT or _HEAD_BLOCK (selected-token plans; 0 otherwise) */
+  int32_t selection_units; /* MLAKV_ATTN_UNITS_SPLIT, _HEAD_BLOCK or _HEAD_BLOCK_HALVES (selected-token plans; 0 otherwise) */
   uint64_t workspace_bytes;
 } mlakvAttnPlan;
 
@@ -201,12 +201,19 @@ mlakvStatus mlakvAttnPlanInit(int32_t batch, int32_t heads, int32_t max_seq_len,
  *   unit; units that hold part of a selection leave partials that a merge puts together.
  * HEAD_BLOCK: one unit = the whole selection of one sequence for 16 heads; nothing to merge and the
  *   workspace stays untouched. bf16 caches, sparse_count up to MLAKV_ATTN_HEAD_BLOCK_TOKENS.
- * AUTO takes HEAD_BLOCK where it applies and was measured ahead (up to 512 selected tokens while
- * batch x heads / 16 units fit the CUs once, up to 256 while they fit twice), unless chunk_tiles,
- * work_groups or merge_mode ask for properties of the split. */
+ * HEAD_BLOCK_HALVES: the same unit taken by two workgroups, half of the selection's tiles each; each
+ *   leaves a partial (16 rows) in the workspace and counts itself on a word of the library's
+ *   counters (those of MLAKV_ATTN_MERGE_IN_LAUNCH, with their limit on launches in flight); the
+ *   second to finish combines the two inside the launch, nobody waits. Up to 8192 (sequence, 16
+ *   heads) pairs.
+ * AUTO, unless chunk_tiles, work_groups or merge_mode ask for properties of the split, takes what
+ * was measured ahead: HEAD_BLOCK_HALVES from 257 to 768 selected tokens while two workgroups per
+ * unit fit the CUs once; else HEAD_BLOCK up to 512 selected tokens while batch x heads / 16 units
+ * fit the CUs once and up to 256 while they fit twice; else SPLIT. */
 #define MLAKV_ATTN_UNITS_AUTO 0
 #define MLAKV_ATTN_UNITS_SPLIT 1
 #define MLAKV_ATTN_UNITS_HEAD_BLOCK 2
+#define MLAKV_ATTN_UNITS_HEAD_BLOCK_HALVES 3
 #define MLAKV_ATTN_HEAD_BLOCK_TOKENS 1024
 typedef struct mlakvAttnPlanOptions {
   int32_t chunk_tiles;    /* tiles per work unit, fixed instead of derived from the live lengths */
@@ -312,7 +319,8 @@ mlakvStatus mlakvAttnDecodeMxQuant(const mlakvAttnPlan* plan, const mlakvCacheVi
  *   (n = 0: zeros, lse = -inf). Order does not matter; repeated positions count repeatedly.
  * The plan comes from mlakvAttnSparsePlanInit (sparse_count takes the place of max_seq_len); how
  * it cuts the work (plan->selection_units) is described with MLAKV_ATTN_UNITS_* above. The
- * workspace is required either way, and left untouched by whole-selection units. */
+ * workspace is required either way; whole-selection units leave it untouched, halved ones use
+ * its first 2 KB x batch x heads. */
 mlakvStatus mlakvAttnSparsePlanInit(int32_t batch, int32_t heads, int32_t sparse_count, int32_t block_size, int32_t dtype,
                                     mlakvAttnPlan* plan);
 mlakvStatus mlakvAttnDecodeSparse(const mlakvAttnPlan* plan, const mlakvCacheView* cache, int32_t layer,

@@ -274,15 +274,22 @@ def test_thin_abi_argument_validation_without_a_device():
     assert sparse.reserved == 1 and sparse.max_seq_len == 512 and sparse.chunk_tiles == 0
     assert decode(sparse) == ffi.ERR_PARAM_INVALID        # a selection plan handed to the whole-context entry
     # how a selection plan cuts its work: whole selections for 16 heads while batch x heads / 16 units
-    # fit the CUs once (up to 512 selected tokens) or twice (up to 256), bf16 only; the split otherwise
+    # fit the CUs once (up to 512 selected tokens) or twice (up to 256), two workgroups per unit from
+    # 257 to 768 selected tokens while those fit the CUs once, bf16 only; the split otherwise
     if lib.mlakvDeviceCount() == 0:                       # (planning without a device assumes the 256 CUs of an MI355X)
-        for batch, heads, count, dtype, expected in ((32, 64, 512, ffi.DTYPE_BF16, ffi.ATTN_UNITS_HEAD_BLOCK),
+        for batch, heads, count, dtype, expected in ((32, 64, 512, ffi.DTYPE_BF16, ffi.ATTN_UNITS_HEAD_BLOCK_HALVES),
+                                                     (32, 64, 256, ffi.DTYPE_BF16, ffi.ATTN_UNITS_HEAD_BLOCK),
+                                                     (32, 64, 257, ffi.DTYPE_BF16, ffi.ATTN_UNITS_HEAD_BLOCK_HALVES),
+                                                     (32, 64, 768, ffi.DTYPE_BF16, ffi.ATTN_UNITS_HEAD_BLOCK_HALVES),
+                                                     (32, 64, 769, ffi.DTYPE_BF16, ffi.ATTN_UNITS_SPLIT),
+                                                     (16, 128, 512, ffi.DTYPE_BF16, ffi.ATTN_UNITS_HEAD_BLOCK_HALVES),
+                                                     (33, 64, 512, ffi.DTYPE_BF16, ffi.ATTN_UNITS_HEAD_BLOCK),
                                                      (64, 64, 512, ffi.DTYPE_BF16, ffi.ATTN_UNITS_HEAD_BLOCK),
                                                      (65, 64, 512, ffi.DTYPE_BF16, ffi.ATTN_UNITS_SPLIT),
                                                      (128, 64, 256, ffi.DTYPE_BF16, ffi.ATTN_UNITS_HEAD_BLOCK),
                                                      (128, 64, 257, ffi.DTYPE_BF16, ffi.ATTN_UNITS_SPLIT),
                                                      (128, 128, 128, ffi.DTYPE_BF16, ffi.ATTN_UNITS_SPLIT),
-                                                     (32, 64, 513, ffi.DTYPE_BF16, ffi.ATTN_UNITS_SPLIT),
+                                                     (64, 64, 513, ffi.DTYPE_BF16, ffi.ATTN_UNITS_SPLIT),
                                                      (32, 64, 512, ffi.DTYPE_FP8_E4M3, ffi.ATTN_UNITS_SPLIT)):
             assert lib.mlakvAttnSparsePlanInit(batch, heads, count, 64, dtype, C.byref(sparse)) == 0
             assert sparse.selection_units == expected, (batch, heads, count, dtype)
@@ -290,6 +297,15 @@ def test_thin_abi_argument_validation_without_a_device():
     assert lib.mlakvAttnPlanInitEx(128, 128, 1024, 64, ffi.DTYPE_BF16, C.byref(forced), C.byref(sparse)) == 0
     assert sparse.selection_units == ffi.ATTN_UNITS_HEAD_BLOCK
     assert lib.mlakvAttnPlanInitEx(32, 64, 1025, 64, ffi.DTYPE_BF16, C.byref(forced), C.byref(sparse)) == ffi.ERR_PARAM_INVALID
+    halved = ffi.AttnPlanOptions(0, 0, 0, 0, 1, ffi.ATTN_UNITS_HEAD_BLOCK_HALVES)
+    assert lib.mlakvAttnPlanInitEx(128, 128, 64, 64, ffi.DTYPE_BF16, C.byref(halved), C.byref(sparse)) == 0
+    assert sparse.selection_units == ffi.ATTN_UNITS_HEAD_BLOCK_HALVES
+    assert lib.mlakvAttnPlanInitEx(32, 64, 512, 64, ffi.DTYPE_FP8_E4M3, C.byref(halved), C.byref(sparse)) == ffi.ERR_PARAM_INVALID
+    assert lib.mlakvAttnPlanInitEx(2048, 128, 64, 64, ffi.DTYPE_BF16, C.byref(halved), C.byref(sparse)) == ffi.ERR_PARAM_INVALID  # more pairs than counters
+    for option in ({"chunk_tiles": 2}, {"work_groups": 64}, {"merge_mode": ffi.ATTN_MERGE_SECOND_LAUNCH}):   # properties of the split
+        asked = ffi.AttnPlanOptions(option.get("chunk_tiles", 0), option.get("work_groups", 0), option.get("merge_mode", 0), 0, 1, 0)
+        assert lib.mlakvAttnPlanInitEx(32, 64, 512, 64, ffi.DTYPE_BF16, C.byref(asked), C.byref(sparse)) == 0
+        assert sparse.selection_units == ffi.ATTN_UNITS_SPLIT, option
     dense_option = ffi.AttnPlanOptions(0, 0, 0, 0, 0, ffi.ATTN_UNITS_SPLIT)   # the option belongs to selection plans
     assert lib.mlakvAttnPlanInitEx(32, 64, 2048, 64, ffi.DTYPE_BF16, C.byref(dense_option), C.byref(sparse)) == ffi.ERR_PARAM_INVALID
     assert lib.mlakvAttnPlanInit(32, 64, 2048, 64, ffi.DTYPE_BF16, C.byref(sparse)) == 0 and sparse.selection_units == 0

@@ -55,12 +55,15 @@ def test_selected_tokens_match_oracle(fp8, bs, k):
     q = kt.randn_bf16((len(ctxs), heads, LATENT + ROPE), seed=82).cuda()
     expected, expected_lse = kt.oracle_attention(cache, 0, q, table, ctxs, SCALE, sparse_indices=selection)
     table_d, lens_d, sel_d = kt.dev_i32(table), kt.dev_i32(ctxs), kt.dev_i32(selection)
-    whole = not fp8 and k <= 512   # where the default plan makes a unit a whole selection for 16 heads (24 units: far fewer than CUs)
+    # what the default plan does with 24 units, far fewer than CUs: a whole selection for 16 heads up
+    # to 256 selected tokens, two workgroups per unit from there to 768, the split beyond and for FP8
+    default_units = (ffi.ATTN_UNITS_SPLIT if fp8 or k > 768 else
+                     ffi.ATTN_UNITS_HEAD_BLOCK_HALVES if k > 256 else ffi.ATTN_UNITS_HEAD_BLOCK)
     for options in ({}, {"chunk_tiles": 1}, {"chunk_tiles": 100}, {"chunk_tiles": 3, "merge_mode": 1},
                     {"selection_units": ffi.ATTN_UNITS_SPLIT}):
         out, lse, plan = kt.sparse_attention(cache, 0, q, table_d, lens_d, sel_d, SCALE, **options)
         assert plan.chunk_tiles * 32 <= 512  # a unit's selected tokens are staged in LDS, one entry each
-        assert plan.selection_units == (ffi.ATTN_UNITS_HEAD_BLOCK if whole and not options else ffi.ATTN_UNITS_SPLIT)
+        assert plan.selection_units == (ffi.ATTN_UNITS_SPLIT if options else default_units)
         _close(out, expected, 6e-2 if fp8 else 2e-2)
         live = np.array([min(n, k) > 0 for n in ctxs])
         assert np.abs(lse.cpu().numpy()[live] - expected_lse[live]).max() <= (6e-2 if fp8 else 2e-2)
@@ -96,6 +99,33 @@ def test_whole_selection_units_of_16_heads(batch, heads, bs, k):
     peak = np.abs(expected).max()
     assert (out.float() - split.float()).abs().max().item() <= 2 ** -6 * peak   # same tokens, same tiles; partials round to bf16 once more
     assert (lse[torch.from_numpy(live).cuda()] - split_lse[torch.from_numpy(live).cuda()]).abs().max().item() <= 1e-3
+    # two workgroups per unit, each with half of the tiles, the second to finish combining the two
+    halves, halves_lse, halves_plan = kt.sparse_attention(cache, 0, q, table_d, lens_d, sel_d, SCALE,
+                                                          selection_units=ffi.ATTN_UNITS_HEAD_BLOCK_HALVES)
+    assert halves_plan.selection_units == ffi.ATTN_UNITS_HEAD_BLOCK_HALVES
+    _close(halves, expected, 2e-2)
+    assert np.abs(halves_lse.cpu().numpy()[live] - expected_lse[live]).max() <= 2e-2
+    assert (halves.float() - out.float()).abs().max().item() <= 2 ** -6 * peak
+    assert not halves[~torch.from_numpy(live).cuda()].any() and torch.isneginf(halves_lse[~torch.from_numpy(live).cuda()]).all()
+    # Launch after launch (more of them than the library has sets of counters), alternating with a
+    # shorter selection whose pairs split differently: every pair's counter is back at zero and no
+    # partial of an earlier launch is taken for a new one; whichever half finishes second, the
+    # result is the same to the bit.
+    shorter = selection.copy()
+    shorter[:, k // 3:] = -1
+    shorter_d = kt.dev_i32(shorter)
+    shorter_expected, _ = kt.oracle_attention(cache, 0, q, table, ctxs, SCALE, sparse_indices=shorter)
+    shorter_first = None
+    for launch in range(40):
+        if launch % 2 == 0:
+            again, again_lse, _ = kt.sparse_attention(cache, 0, q, table_d, lens_d, sel_d, SCALE, selection_units=ffi.ATTN_UNITS_HEAD_BLOCK_HALVES)
+            assert torch.equal(again, halves) and torch.equal(again_lse, halves_lse), launch
+        else:
+            again, _, _ = kt.sparse_attention(cache, 0, q, table_d, lens_d, shorter_d, SCALE, selection_units=ffi.ATTN_UNITS_HEAD_BLOCK_HALVES)
+            if shorter_first is None:
+                shorter_first = again
+                _close(again, shorter_expected, 2e-2)
+            assert torch.equal(again, shorter_first), launch
     # what the option refuses: FP8 caches and selections above the staging size
     lib, refused = ffi.load(), ffi.AttnPlan()
     for dtype, count in ((ffi.DTYPE_FP8_E4M3, 512), (ffi.DTYPE_BF16, ffi.ATTN_HEAD_BLOCK_TOKENS + 1)):
@@ -131,7 +161,7 @@ def test_table_entries_that_name_no_block_read_as_rows_of_zeros(fp8):
     _close(out, expected, tol)
     assert np.abs(lse.cpu().numpy() - expected_lse).max() <= tol
     expected, expected_lse = kt.oracle_attention(cache, 0, q, zeroed, ctxs, SCALE, sparse_indices=selection)
-    for units in (ffi.ATTN_UNITS_SPLIT,) if fp8 else (ffi.ATTN_UNITS_SPLIT, ffi.ATTN_UNITS_HEAD_BLOCK):
+    for units in (ffi.ATTN_UNITS_SPLIT,) if fp8 else (ffi.ATTN_UNITS_SPLIT, ffi.ATTN_UNITS_HEAD_BLOCK, ffi.ATTN_UNITS_HEAD_BLOCK_HALVES):
         out, lse, plan = kt.sparse_attention(cache, 0, q, kt.dev_i32(broken), lens_d, sel_d, SCALE, selection_units=units)
         assert plan.selection_units == units
         _close(out, expected, tol)
