@@ -352,7 +352,7 @@ struct PlanShape {
 // What follows from a plan's own fields; the launch recomputes it to refuse a plan that was not
 // made by the init functions.
 PlanShape ShapeOf(int32_t batch, int32_t heads, int32_t max_seq_len, int32_t block_size, bool sparse, int32_t chunk_tiles,
-                  int32_t work_groups) {
+                  int32_t work_groups, bool halved_units) {
   PlanShape shape;
   shape.max_tiles = (static_cast<int64_t>(max_seq_len) + mlakv::kTileTokens - 1) / mlakv::kTileTokens;
   shape.head_groups = (heads + 63) / 64;
@@ -368,6 +368,10 @@ PlanShape ShapeOf(int32_t batch, int32_t heads, int32_t max_seq_len, int32_t blo
   const uint64_t rows = static_cast<uint64_t>(shape.head_groups) * static_cast<uint64_t>(shape.units + batch) * 64;
   // bf16 partial outputs, then fp32 partial log-sum-exps
   shape.workspace = rows * mlakv::kLatentDim * 2 + ((rows * sizeof(float) + 255) & ~255ull);
+  // Halved whole-selection units: two partials of 16 rows per (sequence, 16 heads) and, behind the
+  // rows of all of them, their LSEs (2 x 4 x 16 floats each).
+  const uint64_t halved = static_cast<uint64_t>(batch) * (heads / 16) * (32 * mlakv::kLatentDim * 2 + 2 * 4 * 16 * sizeof(float));
+  if (halved_units && halved > shape.workspace) shape.workspace = halved;
   return shape;
 }
 
@@ -399,7 +403,7 @@ mlakvStatus AttnPlanImpl(const char* who, int32_t batch, int32_t heads, int32_t 
   }
   int32_t chunk_tiles = chosen.chunk_tiles;
   if (chunk_tiles > cap) chunk_tiles = static_cast<int32_t>(cap);
-  const PlanShape shape = ShapeOf(batch, heads, max_seq_len, block_size, sparse, chunk_tiles, work_groups);
+  PlanShape shape = ShapeOf(batch, heads, max_seq_len, block_size, sparse, chunk_tiles, work_groups, false);
   if (shape.units > (int64_t{1} << 30)) return Fail(MLAKV_ERR_PARAM_INVALID, "%s: too many work units (%lld)", who, static_cast<long long>(shape.units));
   plan->batch = batch;
   plan->heads = heads;
@@ -427,14 +431,13 @@ mlakvStatus AttnPlanImpl(const char* who, int32_t batch, int32_t heads, int32_t 
     return Fail(MLAKV_ERR_PARAM_INVALID, "%s: whole-selection units of 16 heads take a bf16 cache and up to %d selected tokens", who,
                 MLAKV_ATTN_HEAD_BLOCK_TOKENS);
   }
-  // Halved units leave two partials of 16 rows per (sequence, 16 heads) in the workspace and meet on
-  // one of the library's counters each.
+  // Halved units leave two partials of 16 rows (and their LSEs, another half row) per (sequence,
+  // 16 heads) in the workspace and meet on four of the library's counters each.
   const int64_t pairs = static_cast<int64_t>(batch) * (heads / 16);
-  const bool halves_fit = head_block_fits && pairs <= 2 * mlakv::kAttnSyncSequences &&
-                          pairs * 32 <= shape.head_groups * (shape.units + batch) * 64;
+  const bool halves_fit = head_block_fits && pairs * 4 <= 2 * mlakv::kAttnSyncSequences;
   if (chosen.selection_units == MLAKV_ATTN_UNITS_HEAD_BLOCK_HALVES && !halves_fit) {
-    return Fail(MLAKV_ERR_PARAM_INVALID, "%s: halved whole-selection units take up to %d (sequence, 16 heads) pairs whose partials fit the workspace",
-                who, 2 * mlakv::kAttnSyncSequences);
+    return Fail(MLAKV_ERR_PARAM_INVALID, "%s: halved whole-selection units take up to %d (sequence, 16 heads) pairs", who,
+                mlakv::kAttnSyncSequences / 2);
   }
   const bool split_asked = chosen.chunk_tiles != 0 || chosen.work_groups != 0 || chosen.merge_mode != 0;
   // Measured on MI355X (batch 4 .. 128, 64 and 128 heads): a whole-selection unit streams a tile per
@@ -452,6 +455,7 @@ mlakvStatus AttnPlanImpl(const char* who, int32_t batch, int32_t heads, int32_t 
   const bool halves = chosen.selection_units == MLAKV_ATTN_UNITS_HEAD_BLOCK_HALVES ||
                       (chosen.selection_units == MLAKV_ATTN_UNITS_AUTO && !split_asked && halves_fit && halves_pay);
   plan->selection_units = !sparse ? 0 : (halves ? MLAKV_ATTN_UNITS_HEAD_BLOCK_HALVES : (head_block ? MLAKV_ATTN_UNITS_HEAD_BLOCK : MLAKV_ATTN_UNITS_SPLIT));
+  if (halves) shape = ShapeOf(batch, heads, max_seq_len, block_size, sparse, chunk_tiles, work_groups, true);
   plan->workspace_bytes = shape.workspace;
   return MLAKV_SUCCESS;
 }
@@ -544,7 +548,7 @@ mlakvStatus AttnDecodeImpl(const char* who, const mlakvAttnPlan* plan, const mla
     bool sane = fields;
     if (fields) {
       const PlanShape shape = ShapeOf(plan->batch, plan->heads, plan->max_seq_len, plan->block_size, plan->reserved == 1,
-                                      plan->chunk_tiles, plan->work_groups);
+                                      plan->chunk_tiles, plan->work_groups, plan->selection_units == MLAKV_ATTN_UNITS_HEAD_BLOCK_HALVES);
       sane = plan->chunk_tiles <= shape.cap && plan->max_units == shape.units && plan->workspace_bytes == shape.workspace &&
              (plan->merge_mode != MLAKV_ATTN_MERGE_IN_LAUNCH ||
               (static_cast<int64_t>(plan->batch) * shape.head_groups <= mlakv::kAttnSyncSequences && shape.units < 65535));

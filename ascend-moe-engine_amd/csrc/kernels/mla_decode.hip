@@ -1528,12 +1528,13 @@ __global__ __launch_bounds__(kMergeHeads * 64) void MlaMergeKernel(AttnArgs a) {
 //
 // HALVES: two workgroups per (sequence, 16 heads), neighbours on one XCD, each with one half of the
 // selection's tiles, so that twice as many CUs (and twice as many rows in flight) work on a launch
-// that has fewer units than the chip has CUs. Each leaves its normalised partial (bf16 rows and a
-// log2-domain LSE per head, agent-scope stores) in the workspace and counts itself on the pair's
-// word; the one that finds the other's count there reads that partial back, combines it with what
-// it still holds in registers (fp32) and writes the output. Nobody waits: the first to arrive
-// leaves. The pair's word is zero between launches (the second to arrive clears it). A selection
-// of a single tile is taken by the first workgroup alone.
+// that has fewer units than the chip has CUs. The exchange is a matter between the two output waves
+// that hold the same 128 columns, one in each workgroup: each leaves its normalised slice (bf16
+// rows and a log2-domain LSE per head, agent-scope stores) in the workspace and counts itself on
+// the word of (pair, slice); the one that finds the other's count there reads that slice back,
+// combines the two and writes the output. Nobody waits, no barrier is involved: the first to
+// arrive leaves. The words are zero between launches (the second to arrive clears its word). A
+// selection of a single tile is taken by the first workgroup alone.
 constexpr int kHbWaves = kWaves, kHbThreads = kHbWaves * 64;
 constexpr int kHbLoaders = kScoreWaves;  // the waves that fetch the tiles when every row is a plain row
 struct GeomHeadBlock {
@@ -1785,10 +1786,6 @@ __global__ __launch_bounds__(kHbThreads) void MlaSelectedHeadBlockKernel(AttnArg
       if (i + 1 < ntiles) score(i + 1);
     }
     __syncthreads();  // every output wave is through with the last tile (the ring becomes their staging space)
-    if (shared) {     // the output waves' two barriers around the count on the pair's word
-      __syncthreads();
-      __syncthreads();
-    }
   } else {
     // ------------------------------------------------------------------ output waves
     // bf16 V reads as in the kernel above: token = (16 +) 4g + i16/4, chunk = 2n + (i16 & 3) / 2, 8-byte half i16 & 1.
@@ -1889,22 +1886,23 @@ __global__ __launch_bounds__(kHbThreads) void MlaSelectedHeadBlockKernel(AttnArg
     };
     u32x4 v[4];
     if (shared) {
-      // this half's partial: 16 rows of 1 KB and 16 LSEs, at (pair, half) of the workspace
+      // This half's partial at (pair, half) of the workspace: 16 rows of 1 KB, and behind the rows
+      // of all pairs the 16 LSEs once per slice, so that each wave's count covers what its partner reads.
       const int pair = seq * head_blocks + hb;
       const int64_t row0 = static_cast<int64_t>(2 * pair + half) * 16, other0 = static_cast<int64_t>(2 * pair + (half ^ 1)) * 16;
+      float* lses = reinterpret_cast<float*>(a.partial_out + static_cast<int64_t>(a.batch) * head_blocks * 32 * (kLatentDim * 2));
       rows_of_o(v);
       char* mine = a.partial_out + row0 * (kLatentDim * 2) + kSliceBytes * hw + piece * 16;
 #pragma unroll
       for (int it = 0; it < 4; ++it) StoreAgent16(mine + (4 * it + sub) * (kLatentDim * 2), v[it]);
-      if (hw == 0 && g == 0) StoreAgentF32(a.partial_lse + row0 + i16, lse2);
+      if (g == 0) StoreAgentF32(lses + (row0 * 4 + 16 * hw) + i16, lse2);
       asm volatile("s_waitcnt vmcnt(0)" ::: "memory");  // this wave's partial stores are complete
-      __syncthreads();                                  // every wave's are
-      unsigned* arrived_lds = reinterpret_cast<unsigned*>(lds + G::kSOff);
-      if (hw == 0 && lane == 0) *arrived_lds = __hip_atomic_fetch_add(a.sync + pair, 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-      __syncthreads();
-      if (Uniform(*arrived_lds) == 0u) return;  // the other half will find this partial
-      if (hw == 0 && lane == 0) __hip_atomic_store(a.sync + pair, 0u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-      const float lse2_other = LoadAgentF32(a.partial_lse + other0 + i16);
+      unsigned* word = a.sync + 4 * pair + hw;
+      unsigned arrived = 0u;
+      if (lane == 0) arrived = __hip_atomic_fetch_add(word, 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+      if (Uniform(arrived) == 0u) return;  // the other half's wave will find this slice
+      if (lane == 0) __hip_atomic_store(word, 0u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+      const float lse2_other = LoadAgentF32(lses + (other0 * 4 + 16 * hw) + i16);
       const char* theirs = a.partial_out + other0 * (kLatentDim * 2) + kSliceBytes * hw + piece * 16;
 #pragma unroll
       for (int it = 0; it < 4; ++it) v[it] = LoadAgent16(theirs + (4 * it + sub) * (kLatentDim * 2));
@@ -2077,10 +2075,10 @@ hipError_t LaunchAttnDecode(const AttnArgs& args_in, hipStream_t stream) {
       if (args.fp8 || args.sparse_count > kAttnHeadBlockTokens || args.heads % 16 != 0 || args.out == nullptr) return hipErrorInvalidValue;
       const int sequences_per_xcd = (args.batch + kXcds - 1) / kXcds;
       const int64_t pairs = static_cast<int64_t>(args.batch) * (args.heads / 16);
-      // Two workgroups per unit meet on one word each of this launch's counters and leave their
-      // partials in the first 2 x 16 x pairs rows of the workspace.
-      const bool halves = args.head_block_units == 2 && pairs <= kAttnSyncSequences * 2 && args.partial_out != nullptr &&
-                          pairs * 32 <= static_cast<int64_t>(head_groups) * (args.max_units + args.batch) * 64;
+      // Two workgroups per unit meet on four words each of this launch's counters and leave their
+      // partials in the first 2 x 16 x pairs rows of the workspace, the LSEs behind them (the plan
+      // sizes the workspace for that).
+      const bool halves = args.head_block_units == 2 && pairs * 4 <= kAttnSyncSequences * 2 && args.partial_out != nullptr;
       if (halves) {
         if (hipError_t sync_error = SyncRegion(&args.sync); sync_error != hipSuccess) return sync_error;
         const dim3 units(kXcds * (args.heads / 16) * 2 * sequences_per_xcd);

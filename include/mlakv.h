@@ -204,7 +204,7 @@ mlakvStatus mlakvAttnPlanInit(int32_t batch, int32_t heads, int32_t max_seq_len,
  * HEAD_BLOCK_HALVES: the same unit taken by two workgroups, half of the selection's tiles each; each
  *   leaves a partial (16 rows) in the workspace and counts itself on a word of the library's
  *   counters (those of MLAKV_ATTN_MERGE_IN_LAUNCH, with their limit on launches in flight); the
- *   second to finish combines the two inside the launch, nobody waits. Up to 8192 (sequence, 16
+ *   second to finish combines the two inside the launch, nobody waits. Up to 2048 (sequence, 16
  *   heads) pairs.
  * AUTO, unless chunk_tiles, work_groups or merge_mode ask for properties of the split, takes what
  * was measured ahead: HEAD_BLOCK_HALVES from 257 to 768 selected tokens while two workgroups per
@@ -320,7 +320,7 @@ mlakvStatus mlakvAttnDecodeMxQuant(const mlakvAttnPlan* plan, const mlakvCacheVi
  * The plan comes from mlakvAttnSparsePlanInit (sparse_count takes the place of max_seq_len); how
  * it cuts the work (plan->selection_units) is described with MLAKV_ATTN_UNITS_* above. The
  * workspace is required either way; whole-selection units leave it untouched, halved ones use
- * its first 2 KB x batch x heads. */
+ * its first 2112 bytes x batch x heads. */
 mlakvStatus mlakvAttnSparsePlanInit(int32_t batch, int32_t heads, int32_t sparse_count, int32_t block_size, int32_t dtype,
                                     mlakvAttnPlan* plan);
 mlakvStatus mlakvAttnDecodeSparse(const mlakvAttnPlan* plan, const mlakvCacheView* cache, int32_t layer,
