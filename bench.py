@@ -91,6 +91,8 @@ def parse_args():
     p.add_argument("--attention-only", action="store_true", help="development aid: time only the attention configurations")
     p.add_argument("--config5-only", action="store_true", help="development aid: run only the continuous-batching loop of configs[4]")
     p.add_argument("--config5-pool-gb", type=float, default=200.0, help="KV pool of the configs[4] loop, in GB (clamped to free memory)")
+    p.add_argument("--attn-merge-spin-us", type=int, default=0,
+                   help="development aid: bound of the in-launch merge's wait (0: the plan's default, -1: never wait)")
     p.add_argument("--attn-units", choices=["auto", "split", "head-block", "halves"], default="auto",
                    help="development aid: how the selected-token attention cuts its work (MLAKV_ATTN_UNITS_*)")
     p.add_argument("--attn-merge", choices=["auto", "in", "second"], default="auto",
@@ -304,7 +306,7 @@ def bench_attention(args, torch, np, ffi, ctxs, fp8=False, heads=64, slices=8, i
     merge_mode = {"auto": ffi.ATTN_MERGE_AUTO, "in": ffi.ATTN_MERGE_IN_LAUNCH, "second": ffi.ATTN_MERGE_SECOND_LAUNCH}[args.attn_merge]
     units = {"auto": ffi.ATTN_UNITS_AUTO, "split": ffi.ATTN_UNITS_SPLIT, "head-block": ffi.ATTN_UNITS_HEAD_BLOCK, "halves": ffi.ATTN_UNITS_HEAD_BLOCK_HALVES}[args.attn_units] if sparse_k else 0
     if merge_mode != ffi.ATTN_MERGE_AUTO or args.attn_chunk_tiles or args.attn_work_groups or units:
-        options = ffi.AttnPlanOptions(args.attn_chunk_tiles, args.attn_work_groups, merge_mode, 0, 1 if sparse_k else 0, units)
+        options = ffi.AttnPlanOptions(args.attn_chunk_tiles, args.attn_work_groups, merge_mode, args.attn_merge_spin_us, 1 if sparse_k else 0, units)
         ffi.check(lib.mlakvAttnPlanInitEx(batch, heads, sparse_k or max_ctx, bs, cache.config.dtype, C.byref(options), C.byref(plan)))
     elif sparse_k:
         ffi.check(lib.mlakvAttnSparsePlanInit(batch, heads, sparse_k, bs, cache.config.dtype, C.byref(plan)))
