@@ -133,6 +133,52 @@ def test_whole_selection_units_of_16_heads(batch, heads, bs, k):
         assert lib.mlakvAttnPlanInitEx(batch, heads, count, bs, dtype, C.byref(options), C.byref(refused)) == ffi.ERR_PARAM_INVALID
 
 
+def test_halved_units_side_by_side_on_two_streams():
+    """Launches of halved units on two unordered streams, back to back without a host wait between
+    them: each launch has counters of its own (the library hands them out in turn), so the two
+    streams' pairs never meet on one word, and every launch gives the bytes its stream's inputs
+    give alone."""
+    import ctypes as C
+    lib = ffi.load()
+    bs, heads, k = 64, 64, 512
+    ctxs = [4000, 2500, 600, 3000, 513, 1900, 2047, 800]
+    cache, table = _setup(ctxs, bs, False, seed=90)
+    table_d, lens_d = kt.dev_i32(table), kt.dev_i32(ctxs)
+    rng = np.random.default_rng(91)
+    row = (LATENT + ROPE) * 2
+    lanes = []
+    for lane in range(2):
+        selection = np.full((len(ctxs), k), -1, dtype=np.int32)
+        for s, n in enumerate(ctxs):
+            take = min(n, k) - 7 * lane * s          # the two streams' selections end at different tiles
+            selection[s, :take] = rng.permutation(n)[:take]
+        q = kt.randn_bf16((len(ctxs), heads, LATENT + ROPE), seed=92 + lane).cuda()
+        sel_d = kt.dev_i32(selection)
+        alone, alone_lse, plan = kt.sparse_attention(cache, 0, q, table_d, lens_d, sel_d, SCALE,
+                                                     selection_units=ffi.ATTN_UNITS_HEAD_BLOCK_HALVES)
+        expected, _ = kt.oracle_attention(cache, 0, q, table, ctxs, SCALE, sparse_indices=selection)
+        _close(alone, expected, 2e-2)
+        lanes.append({"q": q, "sel": sel_d, "alone": alone, "alone_lse": alone_lse, "plan": plan, "stream": torch.cuda.Stream(),
+                      "workspace": torch.empty(int(plan.workspace_bytes), dtype=torch.uint8, device="cuda"),
+                      "outs": [torch.full_like(alone, float("nan")) for _ in range(24)],
+                      "lses": [torch.full_like(alone_lse, float("nan")) for _ in range(24)]})
+    torch.cuda.synchronize()
+    for launch in range(24):
+        for lane in lanes:
+            q, plan = lane["q"], lane["plan"]
+            ffi.check(lib.mlakvAttnDecodeSparse(C.byref(plan), C.byref(cache.view), 0, q.data_ptr(), heads * row, row,
+                                                q.data_ptr() + LATENT * 2, heads * row, row, table_d.data_ptr(), table_d.shape[1],
+                                                lens_d.data_ptr(), lane["sel"].data_ptr(), lane["sel"].stride(0), float(SCALE),
+                                                lane["outs"][launch].data_ptr(), heads * LATENT * 2, LATENT * 2,
+                                                lane["lses"][launch].data_ptr(), lane["workspace"].data_ptr(),
+                                                int(plan.workspace_bytes), C.c_void_p(lane["stream"].cuda_stream)))
+    torch.cuda.synchronize()
+    for lane in lanes:
+        for launch in range(24):
+            assert torch.equal(lane["outs"][launch], lane["alone"]), launch
+            assert torch.equal(lane["lses"][launch], lane["alone_lse"]), launch
+
+
 @pytest.mark.parametrize("fp8", [False, True])
 def test_table_entries_that_name_no_block_read_as_rows_of_zeros(fp8):
     """A block-table entry outside [0, num_blocks) is never followed: its tokens count as rows of
