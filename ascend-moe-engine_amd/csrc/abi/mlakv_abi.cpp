@@ -425,10 +425,10 @@ mlakvStatus AttnPlanImpl(const char* who, int32_t batch, int32_t heads, int32_t 
   plan->reserved = sparse ? 1 : 0;
   // Whole-selection units of 16 heads where they apply, unless the caller asked for properties of
   // the split (a unit size, a workgroup count, a merge).
-  const bool head_block_fits = sparse && dtype == MLAKV_DTYPE_BF16 && max_seq_len <= MLAKV_ATTN_HEAD_BLOCK_TOKENS;
+  const bool head_block_fits = sparse && max_seq_len <= MLAKV_ATTN_HEAD_BLOCK_TOKENS;
   const bool head_block_asked = chosen.selection_units == MLAKV_ATTN_UNITS_HEAD_BLOCK || chosen.selection_units == MLAKV_ATTN_UNITS_HEAD_BLOCK_HALVES;
   if (head_block_asked && !head_block_fits) {
-    return Fail(MLAKV_ERR_PARAM_INVALID, "%s: whole-selection units of 16 heads take a bf16 cache and up to %d selected tokens", who,
+    return Fail(MLAKV_ERR_PARAM_INVALID, "%s: whole-selection units of 16 heads take up to %d selected tokens", who,
                 MLAKV_ATTN_HEAD_BLOCK_TOKENS);
   }
   // Halved units leave two partials of 16 rows (and their LSEs, another half row) per (sequence,
@@ -448,10 +448,16 @@ mlakvStatus AttnPlanImpl(const char* who, int32_t batch, int32_t heads, int32_t 
   // 11.5 us either way at 256) to 768 (15.2 against 17.5 us at 512, 18.9 against 21.0 us for the
   // split at 768; the split is ahead again at 1024).
   const int64_t rounds = (static_cast<int64_t>(batch) * (heads / 16) + ComputeUnits() - 1) / ComputeUnits();
-  const bool head_block_pays = (rounds <= 1 && max_seq_len <= 512) || (rounds <= 2 && max_seq_len <= 256);
+  // FP8 caches (same shapes): the split converts every K tile in four waves and is behind the whole
+  // units at every measured size (batch 64, 512 selected tokens: 26.6 against 19.2 us; batch 128,
+  // 1024: 63.8 against 63.1), the halved units ahead of both from 257 tokens on (batch 32, 512:
+  // 19.7 / 17.3 / 15.2 us; 1024: 24.7 / 28.6 / 22.1).
+  const bool fp8 = dtype == MLAKV_DTYPE_FP8_E4M3;
+  const bool head_block_pays = fp8 ? (rounds <= 4 || max_seq_len <= 256)
+                                   : ((rounds <= 1 && max_seq_len <= 512) || (rounds <= 2 && max_seq_len <= 256));
   const bool head_block = head_block_fits && (chosen.selection_units == MLAKV_ATTN_UNITS_HEAD_BLOCK ||
                                               (chosen.selection_units == MLAKV_ATTN_UNITS_AUTO && !split_asked && head_block_pays));
-  const bool halves_pay = 2 * pairs <= ComputeUnits() && max_seq_len > 256 && max_seq_len <= 768;
+  const bool halves_pay = 2 * pairs <= ComputeUnits() && max_seq_len > 256 && (fp8 || max_seq_len <= 768);
   const bool halves = chosen.selection_units == MLAKV_ATTN_UNITS_HEAD_BLOCK_HALVES ||
                       (chosen.selection_units == MLAKV_ATTN_UNITS_AUTO && !split_asked && halves_fit && halves_pay);
   plan->selection_units = !sparse ? 0 : (halves ? MLAKV_ATTN_UNITS_HEAD_BLOCK_HALVES : (head_block ? MLAKV_ATTN_UNITS_HEAD_BLOCK : MLAKV_ATTN_UNITS_SPLIT));
@@ -541,7 +547,7 @@ mlakvStatus AttnDecodeImpl(const char* who, const mlakvAttnPlan* plan, const mla
                                              : (plan->selection_units == MLAKV_ATTN_UNITS_SPLIT ||
                                                 ((plan->selection_units == MLAKV_ATTN_UNITS_HEAD_BLOCK ||
                                                   plan->selection_units == MLAKV_ATTN_UNITS_HEAD_BLOCK_HALVES) &&
-                                                 plan->dtype == MLAKV_DTYPE_BF16 && plan->max_seq_len <= MLAKV_ATTN_HEAD_BLOCK_TOKENS))) &&
+                                                 plan->max_seq_len <= MLAKV_ATTN_HEAD_BLOCK_TOKENS))) &&
                         (plan->reserved == 0 || plan->max_seq_len <= 2048) &&
                         (plan->merge_mode == MLAKV_ATTN_MERGE_IN_LAUNCH || plan->merge_mode == MLAKV_ATTN_MERGE_SECOND_LAUNCH) &&
                         (plan->merge_spin_us == -1 || (plan->merge_spin_us > 0 && plan->merge_spin_us <= 1000000));

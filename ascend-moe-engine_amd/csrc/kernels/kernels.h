@@ -129,7 +129,7 @@ struct AttnArgs {
   bool fp8;
   // Selected-token attention only: a workgroup takes the whole selection of one sequence for one
   // block of 16 heads (1: no partials, no merge), or two workgroups take half of it each and the
-  // second to finish combines the two (2); sparse_count <= kAttnHeadBlockTokens, bf16 cache. 0: the split units.
+  // second to finish combines the two (2); sparse_count <= kAttnHeadBlockTokens. 0: the split units.
   int32_t head_block_units;
   unsigned* sync;             // set by the launcher: this launch's counters, null for a second-launch merge
   // Host-known lengths of a small batch travel here instead of through device memory: no upload,

@@ -177,6 +177,13 @@ __device__ __forceinline__ void DirectLoad16PerLane(const char* lane_pointer, un
                : "v"(lane_pointer), "s"(__builtin_amdgcn_readfirstlane(lds_wave_base))
                : "memory", "m0");
 }
+// (four bytes per lane: lane L's dword lands at lds_wave_base + 4 * L)
+__device__ __forceinline__ void DirectLoad4PerLane(const char* lane_pointer, unsigned lds_wave_base) {
+  asm volatile("s_mov_b32 m0, %1\n\ts_nop 0\n\tglobal_load_lds_dword %0, off"
+               :
+               : "v"(lane_pointer), "s"(__builtin_amdgcn_readfirstlane(lds_wave_base))
+               : "memory", "m0");
+}
 // Waits until at most `newer` of this wave's vector-memory loads are outstanding (loads complete
 // in issue order; the count is an immediate of s_waitcnt, hence the switch).
 __device__ __forceinline__ void WaitLoads(int newer) {
@@ -391,8 +398,10 @@ __device__ __forceinline__ bool IssueTileBf16(const AttnArgs& a, TileMap<ALIGNED
 __host__ __device__ __forceinline__ bool PlainRowsAddressable(const AttnArgs& a) {
   const int64_t limit = int64_t{1} << 28;  // strides in 16-byte units below 2^24
   return a.latent.block_stride < limit && a.rope.block_stride < limit && a.latent.row_stride < limit && a.rope.row_stride < limit &&
-         a.num_blocks <= (1 << 24) && a.num_blocks * a.latent.block_stride <= (int64_t{1} << 36) &&
-         a.num_blocks * a.rope.block_stride <= (int64_t{1} << 36);
+         a.num_blocks <= (1 << 24) && a.num_blocks * a.latent.block_stride < (int64_t{1} << 36) &&
+         a.num_blocks * a.rope.block_stride < (int64_t{1} << 36) &&
+         // (FP8: a row's scale, in 4-byte units from its plane's base)
+         (!a.fp8 || a.num_blocks * a.scale.block_stride < (int64_t{1} << 34));
 }
 
 // ---- FP8 tiles: direct global -> LDS, codes and row scales as they are in the cache -------------
@@ -1537,22 +1546,28 @@ __global__ __launch_bounds__(kMergeHeads * 64) void MlaMergeKernel(AttnArgs a) {
 // selection of a single tile is taken by the first workgroup alone.
 constexpr int kHbWaves = kWaves, kHbThreads = kHbWaves * 64;
 constexpr int kHbLoaders = kScoreWaves;  // the waves that fetch the tiles when every row is a plain row
+template <bool FP8>
 struct GeomHeadBlock {
-  using T = Geom<false>;
-  static constexpr int kRing = 4;
-  static constexpr int kTableOff = kRing * T::kTileBytes;                          // unsigned[2][kAttnHeadBlockTokens]: where a selected token's latent and rope rows start, in 16-byte units from the plane's base
-  static constexpr int kSOff = kTableOff + 2 * kAttnHeadBlockTokens * 4;           // S^T partials [2][4 waves][64 lanes] x 16 B
+  using T = Geom<FP8>;
+  static constexpr int kRing = FP8 ? 7 : 4;    // an FP8 tile is half the bytes: seven of them, five on their way
+  static constexpr int kTables = FP8 ? 3 : 2;  // FP8: the row's scale as well, in 4-byte units
+  static constexpr int kTableOff = kRing * T::kTileBytes;                          // unsigned[kTables][kAttnHeadBlockTokens]: where a selected token's latent and rope rows start, in 16-byte units from the plane's base
+  static constexpr int kSOff = kTableOff + kTables * kAttnHeadBlockTokens * 4;     // S^T partials [2][4 waves][64 lanes] x 16 B
   static constexpr int kEndOff = kSOff;  // int[2][kHbWaves], before the first S is written: where each wave saw the selection end, and whether it saw a bad table entry
   static constexpr int kLdsBytes = kSOff + 2 * kScoreWaves * 64 * 16;
   static_assert(kLdsBytes <= 160 * 1024, "one workgroup owns the LDS of a CU");
-  __device__ static __forceinline__ int Slot(int i) { return (i & 3) * T::kTileBytes; }
+  __device__ static __forceinline__ int Slot(int i) { return (kRing == 4 ? (i & 3) : (i % kRing)) * T::kTileBytes; }
 };
-constexpr int kHeadBlockKSteps = kKSteps / 2;  // k-steps of one score wave
+// k-steps of one score wave: half of the 18 for bf16 tiles; FP8 codes are read 16 at a time (two
+// k-steps), so the nine reads of a token are split five and four.
+template <bool FP8>
+constexpr int kHeadBlockKSteps = FP8 ? 10 : kKSteps / 2;
 
-template <bool HALVES>
+template <bool HALVES, bool FP8>
 __global__ __launch_bounds__(kHbThreads) void MlaSelectedHeadBlockKernel(AttnArgs a) {
-  using G = GeomHeadBlock;
-  using T = Geom<false>;
+  using G = GeomHeadBlock<FP8>;
+  using T = Geom<FP8>;
+  constexpr int kQSteps = kHeadBlockKSteps<FP8>;
   extern __shared__ __attribute__((aligned(16))) unsigned char lds[];
   const unsigned lds_base = Uniform(static_cast<unsigned>(reinterpret_cast<size_t>((__attribute__((address_space(3))) unsigned char*)lds)));
   const int tid = threadIdx.x;
@@ -1576,6 +1591,7 @@ __global__ __launch_bounds__(kHbThreads) void MlaSelectedHeadBlockKernel(AttnArg
   // first tile's addresses depend on go out first, the query behind them.
   unsigned* latent_rows = reinterpret_cast<unsigned*>(lds + G::kTableOff);
   unsigned* rope_rows = latent_rows + kAttnHeadBlockTokens;
+  unsigned* scale_rows = rope_rows + kAttnHeadBlockTokens;  // FP8 only
   constexpr unsigned kNoRow = 0xffffffffu;  // a selected token behind a block-table entry that is not a block of the pool
   int* end_lds = reinterpret_cast<int*>(lds + G::kEndOff);
   const int context = static_cast<int>(
@@ -1591,21 +1607,26 @@ __global__ __launch_bounds__(kHbThreads) void MlaSelectedHeadBlockKernel(AttnArg
     index[j] = i < a.sparse_count ? selection[i] : -1;
   }
   // Q fragments of a score wave: lane (head i16, k-group g) holds Q[head][32 ks + 8 g .. +7] for the
-  // nine k-steps ks of its half.
-  bf16x8 q[kHeadBlockKSteps];
+  // nine k-steps ks of its half. FP8: the code reads cover k = 64 kp + 16 g .. + 15 (two k-steps),
+  // the first half of the waves takes reads kp = 0 .. 4, the second kp = 5 .. 8 (8 is the rope row).
+  bf16x8 q[kQSteps];
   if (score_wave) {
     const int kh = hw >> 1;
     const char* q_latent = a.q_latent + seq * a.q_latent_seq_stride + head * a.q_latent_head_stride;
     const char* q_rope = a.q_rope + seq * a.q_rope_seq_stride + head * a.q_rope_head_stride;
 #pragma unroll
-    for (int c = 0; c < kHeadBlockKSteps; ++c) {
-      const int d0 = 32 * (kHeadBlockKSteps * kh + c) + 8 * g;
+    for (int c = 0; c < kQSteps; ++c) {
+      const int d0 = FP8 ? 64 * (5 * kh + (c >> 1)) + 16 * g + 8 * (c & 1) : 32 * (kQSteps * kh + c) + 8 * g;
       const char* p = d0 < kLatentDim ? q_latent + d0 * 2 : q_rope + (d0 - kLatentDim) * 2;
-      q[c] = __builtin_bit_cast(bf16x8, GlobalLoad16(p));
+      if (d0 < kLatentDim + kRopeDim) {  // (the second half of the FP8 reads has four of them)
+        q[c] = __builtin_bit_cast(bf16x8, GlobalLoad16(p));
+      } else {
+        q[c] = __builtin_bit_cast(bf16x8, u32x4{0u, 0u, 0u, 0u});
+      }
     }
   } else {
 #pragma unroll
-    for (int c = 0; c < kHeadBlockKSteps; ++c) q[c] = __builtin_bit_cast(bf16x8, u32x4{0u, 0u, 0u, 0u});
+    for (int c = 0; c < kQSteps; ++c) q[c] = __builtin_bit_cast(bf16x8, u32x4{0u, 0u, 0u, 0u});
   }
   int wave_end = a.sparse_count;
   bool any_outside = false;
@@ -1614,6 +1635,7 @@ __global__ __launch_bounds__(kHbThreads) void MlaSelectedHeadBlockKernel(AttnArg
   // cover to the split units: PlainRowsAddressable).
   const unsigned lat_block16 = static_cast<unsigned>(a.latent.block_stride >> 4), lat_row16 = static_cast<unsigned>(a.latent.row_stride >> 4);
   const unsigned rope_block16 = static_cast<unsigned>(a.rope.block_stride >> 4), rope_row16 = static_cast<unsigned>(a.rope.row_stride >> 4);
+  const unsigned scale_block4 = FP8 ? static_cast<unsigned>(a.scale.block_stride >> 2) : 0u;
 #pragma unroll
   for (int j = 0; j < kPerThread; ++j) {
     const int i = tid + kHbThreads * j;
@@ -1627,6 +1649,7 @@ __global__ __launch_bounds__(kHbThreads) void MlaSelectedHeadBlockKernel(AttnArg
       const unsigned block = static_cast<unsigned>(entry), in_block = static_cast<unsigned>(index[j] - logical * a.block_size);
       latent_rows[i] = inside ? __umul24(block, lat_block16) + __umul24(in_block, lat_row16) : kNoRow;
       rope_rows[i] = inside ? __umul24(block, rope_block16) + __umul24(in_block, rope_row16) : kNoRow;
+      if constexpr (FP8) scale_rows[i] = inside ? block * scale_block4 + in_block : kNoRow;
       if (!inside) any_outside = true;
     }
   }
@@ -1637,7 +1660,7 @@ __global__ __launch_bounds__(kHbThreads) void MlaSelectedHeadBlockKernel(AttnArg
   // Every role passes this statement with the query in hand: a wait of the compiler's for it further
   // down would not know of the tile loads issued from inline assembly, and would wait for them all.
 #pragma unroll
-  for (int c = 0; c < kHeadBlockKSteps; ++c) asm volatile("" ::"v"(q[c]));
+  for (int c = 0; c < kQSteps; ++c) asm volatile("" ::"v"(q[c]));
   __syncthreads();
   int seq_len = a.sparse_count, outside = 0;
 #pragma unroll
@@ -1674,11 +1697,26 @@ __global__ __launch_bounds__(kHbThreads) void MlaSelectedHeadBlockKernel(AttnArg
   // (one load, a row per eight lanes). A lane's address is the plane's base, its own chunk and the
   // row's staged start; positions behind the selection's end repeat its last row (finite values
   // that the softmax masks). A row that is not a row of the pool becomes zeros.
-  constexpr int kRowsPerLoader = kTileTokens / kHbLoaders, kPlainLoads = kRowsPerLoader + 1;
+  // FP8 tiles: a load covers two latent rows of 512 bytes (wave w the row pairs w, w + 4, w + 8,
+  // w + 12), waves 0 and 1 add sixteen 64-byte rope rows each, waves 2 and 3 the 32 row scales (a
+  // dword per lane; both waves, the same bytes, so that every wave has the same count of loads).
+  constexpr int kRowsPerLoader = FP8 ? 4 : kTileTokens / kHbLoaders, kPlainLoads = kRowsPerLoader + 1;
+  int lat_row[4];  // FP8: the tile row behind each of this lane's latent loads
   const char* lat_lane[4];
 #pragma unroll
-  for (int j = 0; j < 4; ++j) lat_lane[j] = a.latent.base + ((lane ^ SwizzleLat(wave + kHbLoaders * j)) << 4);
-  const char* rope_lane = a.rope.base + (((lane & 7) ^ SwizzleRope(8 * wave + (lane >> 3))) << 4);
+  for (int j = 0; j < 4; ++j) {
+    if constexpr (FP8) {
+      lat_row[j] = 2 * (wave + kHbLoaders * j) + (lane >> 5);
+      lat_lane[j] = a.latent.base + (((lane & 31) ^ SwizzleLat8(lat_row[j])) << 4);
+    } else {
+      lat_row[j] = 0;
+      lat_lane[j] = a.latent.base + ((lane ^ SwizzleLat(wave + kHbLoaders * j)) << 4);
+    }
+  }
+  // the lane's row of the fifth load: a rope row (waves 0, 1 for FP8), or the token whose scale it fetches
+  const int extra_row = FP8 ? (wave < 2 ? 16 * wave + (lane >> 2) : (lane & 31)) : 8 * wave + (lane >> 3);
+  const char* rope_lane = FP8 ? a.rope.base + (((lane & 3) ^ SwizzleRope8(extra_row)) << 4)
+                              : a.rope.base + (((lane & 7) ^ SwizzleRope(extra_row)) << 4);
   const int per_tile = wave < kHbLoaders ? kPlainLoads : 0;
   int last_unknown = -1;  // newest tile issued with an unknown number of loads (a row that is not real)
   int issued = 0;
@@ -1687,50 +1725,98 @@ __global__ __launch_bounds__(kHbThreads) void MlaSelectedHeadBlockKernel(AttnArg
       if (wave < kHbLoaders) {
         const int first = tile_of(issued) * kTileTokens, last = seq_len - 1;
         const unsigned buf = lds_base + G::Slot(issued);
-        unsigned starts[kRowsPerLoader];
+        unsigned char* tile = lds + G::Slot(issued);
+        if constexpr (FP8) {
+          unsigned starts[4];
 #pragma unroll
-        for (int r = 0; r < kRowsPerLoader; ++r) starts[r] = latent_rows[min(first + wave + kHbLoaders * r, last)];
-        const unsigned rope_start = rope_rows[min(first + 8 * wave + (lane >> 3), last)];
-        if (plain_rows) {
+          for (int r = 0; r < 4; ++r) starts[r] = latent_rows[min(first + lat_row[r], last)];
+          const bool scale_wave = wave >= 2;
+          const unsigned extra_start = (scale_wave ? scale_rows : rope_rows)[min(first + extra_row, last)];
+          const unsigned extra_dst = scale_wave ? buf + T::kScaleOff : buf + T::kLatRegion + wave * 16 * T::kRopeRow;
+          const char* extra_src = scale_wave ? a.scale.base + (static_cast<u64>(extra_start) << 2) : rope_lane + (static_cast<u64>(extra_start) << 4);
+          if (plain_rows) {
 #pragma unroll
-          for (int r = 0; r < kRowsPerLoader; ++r) {
-            DirectLoad16PerLane(lat_lane[r & 3] + (static_cast<u64>(starts[r]) << 4), buf + (wave + kHbLoaders * r) * T::kLatRow);
-          }
-          DirectLoad16PerLane(rope_lane + (static_cast<u64>(rope_start) << 4), buf + T::kLatRegion + wave * 8 * T::kRopeRow);
-        } else {
-          unsigned char* tile = lds + G::Slot(issued);
-#pragma unroll
-          for (int r = 0; r < kRowsPerLoader; ++r) {
-            const int row = wave + kHbLoaders * r;
-            if (Uniform(starts[r]) != kNoRow) {
-              DirectLoad16PerLane(lat_lane[r & 3] + (static_cast<u64>(starts[r]) << 4), buf + row * T::kLatRow);
-            } else {
-              *reinterpret_cast<u32x4*>(tile + row * T::kLatRow + lane * 16) = u32x4{0u, 0u, 0u, 0u};
+            for (int r = 0; r < 4; ++r) {
+              DirectLoad16PerLane(lat_lane[r] + (static_cast<u64>(starts[r]) << 4), buf + 2 * (wave + kHbLoaders * r) * T::kLatRow);
             }
+            if (scale_wave) {
+              DirectLoad4PerLane(extra_src, extra_dst);
+            } else {
+              DirectLoad16PerLane(extra_src, extra_dst);
+            }
+          } else {
+#pragma unroll
+            for (int r = 0; r < 4; ++r) {
+              if (starts[r] != kNoRow) {
+                DirectLoad16PerLane(lat_lane[r] + (static_cast<u64>(starts[r]) << 4), buf + 2 * (wave + kHbLoaders * r) * T::kLatRow);
+              } else {
+                *reinterpret_cast<u32x4*>(tile + 2 * (wave + kHbLoaders * r) * T::kLatRow + lane * 16) = u32x4{0u, 0u, 0u, 0u};
+              }
+            }
+            if (scale_wave) {
+              if (extra_start != kNoRow) {
+                DirectLoad4PerLane(extra_src, extra_dst);
+              } else {
+                reinterpret_cast<float*>(tile + T::kScaleOff)[lane] = 0.0f;
+              }
+            } else if (extra_start != kNoRow) {
+              DirectLoad16PerLane(extra_src, extra_dst);
+            } else {
+              *reinterpret_cast<u32x4*>(tile + T::kLatRegion + wave * 16 * T::kRopeRow + lane * 16) = u32x4{0u, 0u, 0u, 0u};
+            }
+            last_unknown = issued;
           }
-          if (rope_start != kNoRow) {
+        } else {
+          unsigned starts[kRowsPerLoader];
+#pragma unroll
+          for (int r = 0; r < kRowsPerLoader; ++r) starts[r] = latent_rows[min(first + wave + kHbLoaders * r, last)];
+          const unsigned rope_start = rope_rows[min(first + extra_row, last)];
+          if (plain_rows) {
+#pragma unroll
+            for (int r = 0; r < kRowsPerLoader; ++r) {
+              DirectLoad16PerLane(lat_lane[r & 3] + (static_cast<u64>(starts[r]) << 4), buf + (wave + kHbLoaders * r) * T::kLatRow);
+            }
             DirectLoad16PerLane(rope_lane + (static_cast<u64>(rope_start) << 4), buf + T::kLatRegion + wave * 8 * T::kRopeRow);
           } else {
-            *reinterpret_cast<u32x4*>(tile + T::kLatRegion + wave * 8 * T::kRopeRow + lane * 16) = u32x4{0u, 0u, 0u, 0u};
+#pragma unroll
+            for (int r = 0; r < kRowsPerLoader; ++r) {
+              const int row = wave + kHbLoaders * r;
+              if (Uniform(starts[r]) != kNoRow) {
+                DirectLoad16PerLane(lat_lane[r & 3] + (static_cast<u64>(starts[r]) << 4), buf + row * T::kLatRow);
+              } else {
+                *reinterpret_cast<u32x4*>(tile + row * T::kLatRow + lane * 16) = u32x4{0u, 0u, 0u, 0u};
+              }
+            }
+            if (rope_start != kNoRow) {
+              DirectLoad16PerLane(rope_lane + (static_cast<u64>(rope_start) << 4), buf + T::kLatRegion + wave * 8 * T::kRopeRow);
+            } else {
+              *reinterpret_cast<u32x4*>(tile + T::kLatRegion + wave * 8 * T::kRopeRow + lane * 16) = u32x4{0u, 0u, 0u, 0u};
+            }
+            last_unknown = issued;
           }
-          last_unknown = issued;
         }
       }
       ++issued;
     }
   };
   // Waits until tile t has landed: this wave's loads of the tiles issued after it may stay in flight
-  // (at most one tile here: the ring holds the tile in use, the next one and two on their way).
+  // (the ring holds the tile in use, the next one and the rest on their way: up to kRing - 2 newer
+  // tiles in the prologue, one fewer in the loop, none at the end).
   const auto wait_tile = [&](int t) __attribute__((always_inline)) {
     if (per_tile == 0) return;
-    // (two newer tiles in the prologue, one in the loop, none at the end)
     const int newer_tiles = last_unknown >= t ? 0 : issued - (t + 1);
-    if (newer_tiles >= 2) {
-      asm volatile("s_waitcnt vmcnt(%0)" ::"n"(2 * kPlainLoads) : "memory");
+    if (newer_tiles <= 0) {
+      asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
     } else if (newer_tiles == 1) {
       asm volatile("s_waitcnt vmcnt(%0)" ::"n"(kPlainLoads) : "memory");
+    } else if (newer_tiles == 2 || G::kRing == 4) {
+      asm volatile("s_waitcnt vmcnt(%0)" ::"n"(2 * kPlainLoads) : "memory");
+    } else if (newer_tiles == 3) {
+      asm volatile("s_waitcnt vmcnt(%0)" ::"n"(3 * kPlainLoads) : "memory");
+    } else if (newer_tiles == 4) {
+      asm volatile("s_waitcnt vmcnt(%0)" ::"n"(4 * kPlainLoads) : "memory");
     } else {
-      asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+      asm volatile("s_waitcnt vmcnt(%0)" ::"n"(5 * kPlainLoads) : "memory");
     }
   };
   // Top of iteration i, both roles: tile i + 1 has landed; the barrier publishes it together with
@@ -1753,22 +1839,42 @@ __global__ __launch_bounds__(kHbThreads) void MlaSelectedHeadBlockKernel(AttnArg
     for (int j = 0; j < 4; ++j) k_e[j] = ((4 * j + g) ^ SwizzleLat(i16)) << 4;
 #pragma unroll
     for (int j = 0; j < 2; ++j) kr_e[j] = ((4 * j + g) ^ SwizzleRope(i16)) << 4;
+    // FP8: read kp fetches the 16 codes k = 64 kp + 16 g .. + 15 of token 16 t + i16 (two k-steps):
+    // chunk (4 kp + g) ^ swizzle(token) of the 512-byte row; kp = 8 is the rope row. The products
+    // are of the codes as they are: the row's scale meets the sums in the output waves.
+    const int k8_lat = (16 * t + i16) * T::kLatRow + ((g ^ SwizzleLat8(16 * t + i16)) << 4);
+    const int k8_rope = T::kLatRegion + (16 * t + i16) * T::kRopeRow + ((g ^ SwizzleRope8(16 * t + i16)) << 4);
     const auto score_tile = [&](int tile, auto kh_c) __attribute__((always_inline)) {
       constexpr int kh = decltype(kh_c)::value;
       const unsigned char* buf = lds + G::Slot(tile);
-      bf16x8 kf[kHeadBlockKSteps];
-      StaticFor<kHeadBlockKSteps>([&](auto c_c) __attribute__((always_inline)) {
-        constexpr int c = decltype(c_c)::value, ks = kHeadBlockKSteps * kh + c;
-        const int offset = ks < 16 ? k_lat + (ks >> 2) * 256 + k_e[ks & 3] : k_rope + kr_e[ks & 1];
-        kf[c] = *reinterpret_cast<const bf16x8*>(buf + offset);
-      });
       f32x4 acc[3];
 #pragma unroll
       for (int j = 0; j < 3; ++j) acc[j] = f32x4{0.f, 0.f, 0.f, 0.f};
-      StaticFor<kHeadBlockKSteps>([&](auto c_c) __attribute__((always_inline)) {
-        constexpr int c = decltype(c_c)::value;
-        acc[c % 3] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(kf[c], q[c], acc[c % 3], 0, 0, 0);
-      });
+      if constexpr (FP8) {
+        constexpr int kReads = kh == 0 ? 5 : 4;
+        u32x4 codes[kReads];
+        StaticFor<kReads>([&](auto c_c) __attribute__((always_inline)) {
+          constexpr int c = decltype(c_c)::value, kp = 5 * kh + c;
+          codes[c] = *reinterpret_cast<const u32x4*>(buf + (kp < 8 ? (k8_lat ^ (kp << 6)) : k8_rope));
+        });
+        StaticFor<kReads>([&](auto c_c) __attribute__((always_inline)) {
+          constexpr int c = decltype(c_c)::value;
+          acc[(2 * c) % 3] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(CodesToBf16(codes[c].x, codes[c].y), q[2 * c], acc[(2 * c) % 3], 0, 0, 0);
+          acc[(2 * c + 1) % 3] =
+              __builtin_amdgcn_mfma_f32_16x16x32_bf16(CodesToBf16(codes[c].z, codes[c].w), q[2 * c + 1], acc[(2 * c + 1) % 3], 0, 0, 0);
+        });
+      } else {
+        bf16x8 kf[kQSteps];
+        StaticFor<kQSteps>([&](auto c_c) __attribute__((always_inline)) {
+          constexpr int c = decltype(c_c)::value, ks = kQSteps * kh + c;
+          const int offset = ks < 16 ? k_lat + (ks >> 2) * 256 + k_e[ks & 3] : k_rope + kr_e[ks & 1];
+          kf[c] = *reinterpret_cast<const bf16x8*>(buf + offset);
+        });
+        StaticFor<kQSteps>([&](auto c_c) __attribute__((always_inline)) {
+          constexpr int c = decltype(c_c)::value;
+          acc[c % 3] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(kf[c], q[c], acc[c % 3], 0, 0, 0);
+        });
+      }
       s_lds[((tile & 1) * kScoreWaves + hw) * 64] = acc[0] + acc[1] + acc[2];
     };
     const bool upper = (hw >> 1) != 0;  // wave-uniform: which half of the k-steps
@@ -1794,11 +1900,20 @@ __global__ __launch_bounds__(kHbThreads) void MlaSelectedHeadBlockKernel(AttnArg
     int v_e[8];
 #pragma unroll
     for (int j = 0; j < 8; ++j) v_e[j] = ((2 * j + ((i16 & 3) >> 1)) ^ SwizzleLat(v_row)) << 4;
+    // FP8 V reads as in the kernel above (ds_read_b64_tr_b8): as a source, lane j of a 16-lane group
+    // addresses bytes 16 n + 8 (j & 1) .. + 7 of the row of token 4 g + (j >> 1 & 3) + 16 (j >> 3).
+    const int v8_token = 4 * g + ((i16 >> 1) & 3) + 16 * (i16 >> 3);
+    const int v8_base = v8_token * Geom<true>::kLatRow + (SwizzleLat8(v8_token) << 4) + 8 * (i16 & 1);
     const auto v_fetch = [&](const unsigned char* buf, int n) __attribute__((always_inline)) {
-      const unsigned char* addr = buf + v_lane + (n >> 3) * 256 + v_e[n & 7];
-      const s16x4 lo = __builtin_amdgcn_ds_read_tr16_b64_v4i16((__attribute__((address_space(3))) s16x4*)(addr));
-      const s16x4 hi = __builtin_amdgcn_ds_read_tr16_b64_v4i16((__attribute__((address_space(3))) s16x4*)(addr + 16 * T::kLatRow));
-      return __builtin_bit_cast(bf16x8, __builtin_shufflevector(lo, hi, 0, 1, 2, 3, 4, 5, 6, 7));
+      if constexpr (FP8) {
+        const i32x2 codes = __builtin_amdgcn_ds_read_tr8_b64_v2i32((__attribute__((address_space(3))) i32x2*)(buf + (v8_base ^ (n << 4))));
+        return CodesToBf16(static_cast<unsigned>(codes.x), static_cast<unsigned>(codes.y));
+      } else {
+        const unsigned char* addr = buf + v_lane + (n >> 3) * 256 + v_e[n & 7];
+        const s16x4 lo = __builtin_amdgcn_ds_read_tr16_b64_v4i16((__attribute__((address_space(3))) s16x4*)(addr));
+        const s16x4 hi = __builtin_amdgcn_ds_read_tr16_b64_v4i16((__attribute__((address_space(3))) s16x4*)(addr + 16 * T::kLatRow));
+        return __builtin_bit_cast(bf16x8, __builtin_shufflevector(lo, hi, 0, 1, 2, 3, 4, 5, 6, 7));
+      }
     };
     constexpr int kDvPerWave = kDvTiles / (kWaves - kScoreWaves);  // 8 column tiles: columns [128 hw, 128 hw + 128)
     f32x4 o[kDvPerWave];
@@ -1824,6 +1939,17 @@ __global__ __launch_bounds__(kHbThreads) void MlaSelectedHeadBlockKernel(AttnArg
       for (int j = 0; j < 4; ++j) {
         x[j] = (s0[j] + s2[j]) * a.scale_log2;
         x[4 + j] = (s1[j] + s3[j]) * a.scale_log2;
+      }
+      f32x4 row_scale[2] = {f32x4{1.f, 1.f, 1.f, 1.f}, f32x4{1.f, 1.f, 1.f, 1.f}};  // FP8: of tokens 4g+j and 16+4g+j
+      if constexpr (FP8) {  // the codes were multiplied unscaled
+        const float* scales = reinterpret_cast<const float*>(buf + T::kScaleOff);
+        row_scale[0] = *reinterpret_cast<const f32x4*>(scales + 4 * g);
+        row_scale[1] = *reinterpret_cast<const f32x4*>(scales + 16 + 4 * g);
+#pragma unroll
+        for (int j = 0; j < 4; ++j) {
+          x[j] *= row_scale[0][j];
+          x[4 + j] *= row_scale[1][j];
+        }
       }
       const int valid = seq_len - tile_of(i) * kTileTokens;  // >= 1
       if (valid < kTileTokens) {                             // only the last tile of the selection
@@ -1851,7 +1977,7 @@ __global__ __launch_bounds__(kHbThreads) void MlaSelectedHeadBlockKernel(AttnArg
       for (int j = 0; j < 8; ++j) {
         const float e = __builtin_amdgcn_exp2f(x[j] - m_ref);
         sum += e;
-        p[j] = static_cast<__bf16>(e);
+        p[j] = static_cast<__bf16>(FP8 ? e * row_scale[j >> 2][j & 3] : e);  // V = codes x the row's scale
       }
       l_run += sum;
       StaticFor<kDvPerWave>([&](auto n_c) __attribute__((always_inline)) {
@@ -1945,6 +2071,16 @@ hipError_t PrepareDecode() {
   return hipFuncSetAttribute(reinterpret_cast<const void*>(&MlaDecodeKernel<FP8, ALIGNED, MXQ, SPARSE>),
                              hipFuncAttributeMaxDynamicSharedMemorySize, Geom<FP8>::kLdsBytes);
 }
+template <bool HALVES, bool FP8>
+hipError_t PrepareHeadBlock() {
+  return hipFuncSetAttribute(reinterpret_cast<const void*>(&MlaSelectedHeadBlockKernel<HALVES, FP8>),
+                             hipFuncAttributeMaxDynamicSharedMemorySize, GeomHeadBlock<FP8>::kLdsBytes);
+}
+template <bool HALVES, bool FP8>
+hipError_t LaunchHeadBlock(const AttnArgs& args, const dim3& units, hipStream_t stream) {
+  hipLaunchKernelGGL((MlaSelectedHeadBlockKernel<HALVES, FP8>), units, dim3(kHbThreads), GeomHeadBlock<FP8>::kLdsBytes, stream, args);
+  return hipGetLastError();
+}
 template <bool MXQ, bool SPARSE>
 hipError_t PrepareMerge() {
   hipFuncAttributes attributes;
@@ -2006,10 +2142,7 @@ hipError_t PrepareAttnKernels() {
       PrepareDecode<true, true, true, false>(),   PrepareDecode<true, false, true, false>(),
       PrepareDecode<false, false, false, true>(), PrepareDecode<true, false, false, true>(),
       PrepareMerge<false, false>(), PrepareMerge<true, false>(), PrepareMerge<false, true>(),
-      hipFuncSetAttribute(reinterpret_cast<const void*>(&MlaSelectedHeadBlockKernel<false>), hipFuncAttributeMaxDynamicSharedMemorySize,
-                          GeomHeadBlock::kLdsBytes),
-      hipFuncSetAttribute(reinterpret_cast<const void*>(&MlaSelectedHeadBlockKernel<true>), hipFuncAttributeMaxDynamicSharedMemorySize,
-                          GeomHeadBlock::kLdsBytes)};
+      PrepareHeadBlock<false, false>(), PrepareHeadBlock<true, false>(), PrepareHeadBlock<false, true>(), PrepareHeadBlock<true, true>()};
   for (const hipError_t e : results) {
     if (e != hipSuccess) return e;
   }
@@ -2072,7 +2205,7 @@ hipError_t LaunchAttnDecode(const AttnArgs& args_in, hipStream_t stream) {
     if ((static_cast<int64_t>(args.num_blocks) << slot_bits) > (int64_t{1} << 31)) return hipErrorInvalidValue;
     // (a pool whose rows the 32-bit starts of the whole-selection units cannot address goes to the split units)
     if (args.head_block_units != 0 && PlainRowsAddressable(args)) {
-      if (args.fp8 || args.sparse_count > kAttnHeadBlockTokens || args.heads % 16 != 0 || args.out == nullptr) return hipErrorInvalidValue;
+      if (args.sparse_count > kAttnHeadBlockTokens || args.heads % 16 != 0 || args.out == nullptr) return hipErrorInvalidValue;
       const int sequences_per_xcd = (args.batch + kXcds - 1) / kXcds;
       const int64_t pairs = static_cast<int64_t>(args.batch) * (args.heads / 16);
       // Two workgroups per unit meet on four words each of this launch's counters and leave their
@@ -2082,12 +2215,10 @@ hipError_t LaunchAttnDecode(const AttnArgs& args_in, hipStream_t stream) {
       if (halves) {
         if (hipError_t sync_error = SyncRegion(&args.sync); sync_error != hipSuccess) return sync_error;
         const dim3 units(kXcds * (args.heads / 16) * 2 * sequences_per_xcd);
-        hipLaunchKernelGGL(MlaSelectedHeadBlockKernel<true>, units, dim3(kHbThreads), GeomHeadBlock::kLdsBytes, stream, args);
-      } else {
-        const dim3 units(kXcds * (args.heads / 16) * sequences_per_xcd);
-        hipLaunchKernelGGL(MlaSelectedHeadBlockKernel<false>, units, dim3(kHbThreads), GeomHeadBlock::kLdsBytes, stream, args);
+        return args.fp8 ? LaunchHeadBlock<true, true>(args, units, stream) : LaunchHeadBlock<true, false>(args, units, stream);
       }
-      return hipGetLastError();
+      const dim3 units(kXcds * (args.heads / 16) * sequences_per_xcd);
+      return args.fp8 ? LaunchHeadBlock<false, true>(args, units, stream) : LaunchHeadBlock<false, false>(args, units, stream);
     }
     e = args.fp8 ? Launch<true, false, false, true>(args, grid, stream) : Launch<false, false, false, true>(args, grid, stream);
   } else {

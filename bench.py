@@ -836,6 +836,8 @@ def attention_suite(args, torch, np, ffi):
     out["attention_sparse"] = bench_attention(args, torch, np, ffi, [8192] * 32, slices=4, sparse_k=512,
                                               label="selected-token decode (index_topk 512 of 8192)",
                                               traffic_ratio=ATTENTION_TRAFFIC["attention_sparse"])
+    out["attention_sparse_fp8"] = bench_attention(args, torch, np, ffi, [8192] * 32, slices=4, sparse_k=512, fp8=True,
+                                                  label="selected-token decode over an FP8 cache (index_topk 512 of 8192)")
     out["indexer"] = bench_indexer(args, torch, np, ffi)
     # The pair as a decode step would run it (indexer, then attention over its selection), against
     # the bytes the pair has to move: B * ctx * 132 of index keys and scales, B * k * 1152 of selected rows.

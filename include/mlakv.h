@@ -200,16 +200,19 @@ mlakvStatus mlakvAttnPlanInit(int32_t batch, int32_t heads, int32_t max_seq_len,
  * SPLIT: the selections of the batch laid end to end and cut into one unit per CU, 64 heads per
  *   unit; units that hold part of a selection leave partials that a merge puts together.
  * HEAD_BLOCK: one unit = the whole selection of one sequence for 16 heads; nothing to merge and the
- *   workspace stays untouched. bf16 caches, sparse_count up to MLAKV_ATTN_HEAD_BLOCK_TOKENS.
+ *   workspace stays untouched. sparse_count up to MLAKV_ATTN_HEAD_BLOCK_TOKENS.
  * HEAD_BLOCK_HALVES: the same unit taken by two workgroups, half of the selection's tiles each; each
  *   leaves a partial (16 rows) in the workspace and counts itself on a word of the library's
  *   counters (those of MLAKV_ATTN_MERGE_IN_LAUNCH, with their limit on launches in flight); the
  *   second to finish combines the two inside the launch, nobody waits. Up to 2048 (sequence, 16
  *   heads) pairs.
  * AUTO, unless chunk_tiles, work_groups or merge_mode ask for properties of the split, takes what
- * was measured ahead: HEAD_BLOCK_HALVES from 257 to 768 selected tokens while two workgroups per
- * unit fit the CUs once; else HEAD_BLOCK up to 512 selected tokens while batch x heads / 16 units
- * fit the CUs once and up to 256 while they fit twice; else SPLIT. */
+ * was measured ahead. bf16 caches: HEAD_BLOCK_HALVES from 257 to 768 selected tokens while two
+ * workgroups per unit fit the CUs once; else HEAD_BLOCK up to 512 selected tokens while batch x
+ * heads / 16 units fit the CUs once and up to 256 while they fit twice; else SPLIT. FP8 caches:
+ * HEAD_BLOCK_HALVES from 257 selected tokens while two workgroups per unit fit the CUs once; else
+ * HEAD_BLOCK while the units fit the CUs four times (beyond that up to 256 selected tokens); else
+ * SPLIT. */
 #define MLAKV_ATTN_UNITS_AUTO 0
 #define MLAKV_ATTN_UNITS_SPLIT 1
 #define MLAKV_ATTN_UNITS_HEAD_BLOCK 2

@@ -290,7 +290,13 @@ def test_thin_abi_argument_validation_without_a_device():
                                                      (128, 64, 257, ffi.DTYPE_BF16, ffi.ATTN_UNITS_SPLIT),
                                                      (128, 128, 128, ffi.DTYPE_BF16, ffi.ATTN_UNITS_SPLIT),
                                                      (64, 64, 513, ffi.DTYPE_BF16, ffi.ATTN_UNITS_SPLIT),
-                                                     (32, 64, 512, ffi.DTYPE_FP8_E4M3, ffi.ATTN_UNITS_SPLIT)):
+                                                     (32, 64, 512, ffi.DTYPE_FP8_E4M3, ffi.ATTN_UNITS_HEAD_BLOCK_HALVES),
+                                                     (32, 64, 1024, ffi.DTYPE_FP8_E4M3, ffi.ATTN_UNITS_HEAD_BLOCK_HALVES),
+                                                     (32, 64, 256, ffi.DTYPE_FP8_E4M3, ffi.ATTN_UNITS_HEAD_BLOCK),
+                                                     (128, 64, 1024, ffi.DTYPE_FP8_E4M3, ffi.ATTN_UNITS_HEAD_BLOCK),
+                                                     (512, 64, 256, ffi.DTYPE_FP8_E4M3, ffi.ATTN_UNITS_HEAD_BLOCK),
+                                                     (512, 64, 257, ffi.DTYPE_FP8_E4M3, ffi.ATTN_UNITS_SPLIT),
+                                                     (32, 64, 1025, ffi.DTYPE_FP8_E4M3, ffi.ATTN_UNITS_SPLIT)):
             assert lib.mlakvAttnSparsePlanInit(batch, heads, count, 64, dtype, C.byref(sparse)) == 0
             assert sparse.selection_units == expected, (batch, heads, count, dtype)
     forced = ffi.AttnPlanOptions(0, 0, 0, 0, 1, ffi.ATTN_UNITS_HEAD_BLOCK)
@@ -300,7 +306,9 @@ def test_thin_abi_argument_validation_without_a_device():
     halved = ffi.AttnPlanOptions(0, 0, 0, 0, 1, ffi.ATTN_UNITS_HEAD_BLOCK_HALVES)
     assert lib.mlakvAttnPlanInitEx(128, 128, 64, 64, ffi.DTYPE_BF16, C.byref(halved), C.byref(sparse)) == 0
     assert sparse.selection_units == ffi.ATTN_UNITS_HEAD_BLOCK_HALVES
-    assert lib.mlakvAttnPlanInitEx(32, 64, 512, 64, ffi.DTYPE_FP8_E4M3, C.byref(halved), C.byref(sparse)) == ffi.ERR_PARAM_INVALID
+    assert lib.mlakvAttnPlanInitEx(32, 64, 512, 64, ffi.DTYPE_FP8_E4M3, C.byref(halved), C.byref(sparse)) == 0
+    assert sparse.selection_units == ffi.ATTN_UNITS_HEAD_BLOCK_HALVES
+    assert lib.mlakvAttnPlanInitEx(32, 64, 1025, 64, ffi.DTYPE_FP8_E4M3, C.byref(halved), C.byref(sparse)) == ffi.ERR_PARAM_INVALID
     assert lib.mlakvAttnPlanInitEx(2048, 128, 64, 64, ffi.DTYPE_BF16, C.byref(halved), C.byref(sparse)) == ffi.ERR_PARAM_INVALID  # more pairs than counters
     for option in ({"chunk_tiles": 2}, {"work_groups": 64}, {"merge_mode": ffi.ATTN_MERGE_SECOND_LAUNCH}):   # properties of the split
         asked = ffi.AttnPlanOptions(option.get("chunk_tiles", 0), option.get("work_groups", 0), option.get("merge_mode", 0), 0, 1, 0)
