@@ -53,7 +53,8 @@ ATTENTION_TRAFFIC = {
     "attention": {"ratio": 1.429, "source": _TRAFFIC_SOURCE},        # 114.27 MB against 79.96 MB
     "attention_fp8": {"ratio": 1.254, "source": _TRAFFIC_SOURCE},    # 221.43 MB against 176.52 MB
     "attention_long": {"ratio": 1.060, "source": _TRAFFIC_SOURCE},   # 952.84 MB against 898.64 MB
-    "attention_sparse": {"ratio": 1.320, "source": _TRAFFIC_SOURCE}, # 30.90 MB against 23.41 MB (one dispatch: halved whole-selection units)
+    "attention_sparse": {"ratio": 1.322, "source": _TRAFFIC_SOURCE}, # 30.96 MB against 23.41 MB (one dispatch: halved whole-selection units)
+    "attention_sparse_fp8": {"ratio": 1.613, "source": _TRAFFIC_SOURCE}, # 22.65 MB against 14.04 MB
     "indexer": {"ratio": 1.094, "source": _TRAFFIC_SOURCE},          # 38.24 MB against 34.96 MB
 }
 # Host orchestration of the reference's own 43-layer decode step (its mock build: every operator
@@ -837,7 +838,8 @@ def attention_suite(args, torch, np, ffi):
                                               label="selected-token decode (index_topk 512 of 8192)",
                                               traffic_ratio=ATTENTION_TRAFFIC["attention_sparse"])
     out["attention_sparse_fp8"] = bench_attention(args, torch, np, ffi, [8192] * 32, slices=4, sparse_k=512, fp8=True,
-                                                  label="selected-token decode over an FP8 cache (index_topk 512 of 8192)")
+                                                  label="selected-token decode over an FP8 cache (index_topk 512 of 8192)",
+                                                  traffic_ratio=ATTENTION_TRAFFIC["attention_sparse_fp8"])
     out["indexer"] = bench_indexer(args, torch, np, ffi)
     # The pair as a decode step would run it (indexer, then attention over its selection), against
     # the bytes the pair has to move: B * ctx * 132 of index keys and scales, B * k * 1152 of selected rows.
