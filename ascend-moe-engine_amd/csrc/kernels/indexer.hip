@@ -18,6 +18,9 @@
 
 #include "kernels.h"
 
+// (the direct global -> LDS loads name M0, which they set themselves, in their clobber lists)
+#pragma clang diagnostic ignored "-Winline-asm"
+
 namespace mlakv {
 namespace {
 
