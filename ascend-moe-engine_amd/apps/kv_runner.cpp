@@ -46,6 +46,7 @@ struct Options {
   bool prompt_from_ids = false;
   bool verbose = false;
   bool dry_run = false;
+  bool graph = false;  // decode steps after the first token replay one recorded step
   bool help = false;
 };
 
@@ -85,6 +86,8 @@ void PrintUsage() {
       "  --device <id>             GPU (default 0)\n"
       "  --seed <n>                seed of the synthetic stage outputs\n"
       "  --dry-run                 size and report, decode nothing\n"
+      "  --graph                   record one decode step (stream capture) after the first token and\n"
+      "                            replay it for every later token: one launch per step for the host\n"
       "  --report <path>           write the report there as well as to stdout\n"
       "  --diag-json <path>        structured diagnostics (also for dry runs)\n"
       "  --stats-json <path>       machine-readable run stats after a decode\n"
@@ -152,6 +155,7 @@ Options Parse(int argc, char** argv) {
     else if (flag == "--report") o.report_path = value();
     else if (flag == "--verbose") o.verbose = true;
     else if (flag == "--dry-run") o.dry_run = true;
+    else if (flag == "--graph") o.graph = true;
     else if (flag == "--synthetic-weights") {}  // the only kind of input this runner has
     else if (flag == "--weights" || flag == "--config" || flag == "--prompt" || flag == "--vram-slots" || flag == "--moe-path" ||
              flag == "--moe-backend" || flag == "--gating-norm-type" || flag == "--dense-group-size" || flag == "--routed-coverage") {
@@ -288,6 +292,7 @@ int Run(int argc, char** argv) {
   const size_t off_gather_rope = reserve(2 * static_cast<size_t>(steps) * kRope);
   const size_t off_latent = reserve(latent_stride * static_cast<size_t>(o.layers));
   const size_t off_rope = reserve(rope_stride * static_cast<size_t>(o.layers));
+  const size_t off_live = reserve(4);  // the live length as the attention reads it when steps are replayed
   const size_t arena_bytes = align_up(cursor);
   char* arena = nullptr;
   uint64_t device_allocations = 0;
@@ -384,16 +389,27 @@ int Run(int argc, char** argv) {
   uint16_t* readback = nullptr;
   RUNNER_CHECK(aclrtMallocHost(reinterpret_cast<void**>(&readback), 2 * kHeads * kLatent));
 
-  uint64_t launches = 0, host_synchronizations = 0, generated = 0;
-  double enqueue_seconds = 0.0;
-  const auto decode_step = [&](int64_t position) {
-    const auto begin = std::chrono::steady_clock::now();
-    mailbox[position] = static_cast<int32_t>(position);  // slot = position (pipeline.cpp:517); a word per step
-    RUNNER_CHECK(aclrtMemcpyAsync(arena + off_slot, 4, mailbox + position, 4, ACL_MEMCPY_HOST_TO_DEVICE, stream));
-    const int64_t live = position + 1;
-    RUNNER_CHECK(aclnnMlaKvSetSeqLens(ex_attention, &live, 1));
+  // Replayed steps: a recorded step cannot take its position, its length or its input rows from
+  // host arguments, so the length is read from device memory (a word of the arena, written by a
+  // copy from a pinned word as the slot is) and the step's inputs come from one pinned staging area.
+  int32_t* live_words = nullptr;   // a word per step (eager steps), like the slot mailbox
+  int32_t* replay_words = nullptr; // [slot, length] of the step being replayed
+  uint16_t* replay_inputs = nullptr;
+  if (o.graph) {
+    RUNNER_CHECK(aclrtMallocHost(reinterpret_cast<void**>(&live_words), 4 * static_cast<size_t>(steps)));
+    RUNNER_CHECK(aclrtMallocHost(reinterpret_cast<void**>(&replay_words), 8));
+    RUNNER_CHECK(aclrtMallocHost(reinterpret_cast<void**>(&replay_inputs), 2 * per_item * static_cast<size_t>(o.layers)));
+    RUNNER_CHECK(aclnnMlaKvBindSeqLens(ex_attention, reinterpret_cast<const int32_t*>(arena + off_live)));
+  }
+
+  uint64_t launches = 0, host_synchronizations = 0, generated = 0, replayed_steps = 0;
+  double enqueue_seconds = 0.0, replay_host_seconds = 0.0;
+  // One step's work on the stream; `slot_word`, `live_word` and `step_inputs` are pinned host memory.
+  const auto enqueue_step = [&](const int32_t* slot_word, const int32_t* live_word, const uint16_t* step_inputs) {
+    RUNNER_CHECK(aclrtMemcpyAsync(arena + off_slot, 4, slot_word, 4, ACL_MEMCPY_HOST_TO_DEVICE, stream));
+    if (live_word != nullptr) RUNNER_CHECK(aclrtMemcpyAsync(arena + off_live, 4, live_word, 4, ACL_MEMCPY_HOST_TO_DEVICE, stream));
     for (int64_t layer = 0; layer < o.layers; ++layer) {
-      const uint16_t* item = inputs + per_item * static_cast<size_t>(position * o.layers + layer);
+      const uint16_t* item = step_inputs + per_item * static_cast<size_t>(layer);
       RUNNER_CHECK(aclrtMemcpyAsync(arena + off_normed, 2 * per_item, item, 2 * per_item, ACL_MEMCPY_HOST_TO_DEVICE, stream));
       char* latent = arena + off_latent + latent_stride * static_cast<size_t>(layer);
       char* rope = arena + off_rope + rope_stride * static_cast<size_t>(layer);
@@ -404,9 +420,39 @@ int Run(int argc, char** argv) {
       RUNNER_CHECK(aclSetTensorAddr(ex_attention, 25, rope_cache_view, rope));        // kFiaKeyRope
       RUNNER_CHECK(aclnnScatterPaKvCache(workspace, ws_scatter, ex_scatter, stream));
       RUNNER_CHECK(aclnnFusedInferAttentionScoreV5(workspace, ws_attention, ex_attention, stream));
-      launches += 2;
     }
+  };
+  uint64_t eager_steps = 0;
+  const auto decode_step = [&](int64_t position) {
+    const auto begin = std::chrono::steady_clock::now();
+    mailbox[position] = static_cast<int32_t>(position);  // slot = position (pipeline.cpp:517); a word per step
+    const int64_t live = position + 1;
+    if (o.graph) {
+      live_words[position] = static_cast<int32_t>(live);
+    } else {
+      RUNNER_CHECK(aclnnMlaKvSetSeqLens(ex_attention, &live, 1));
+    }
+    enqueue_step(mailbox + position, o.graph ? live_words + position : nullptr, inputs + per_item * static_cast<size_t>(position * o.layers));
+    launches += 2 * static_cast<uint64_t>(o.layers);
+    ++eager_steps;
     enqueue_seconds += std::chrono::duration<double>(std::chrono::steady_clock::now() - begin).count();
+  };
+  aclmdlRI recorded_step = nullptr;
+  const auto replay_step = [&](int64_t position) {
+    const auto begin = std::chrono::steady_clock::now();
+    if (recorded_step == nullptr) {  // record: the same calls, from the staging words and rows
+      RUNNER_CHECK(aclmdlRICaptureBegin(stream, ACL_MODEL_RI_CAPTURE_MODE_GLOBAL));
+      enqueue_step(replay_words, replay_words + 1, replay_inputs);
+      RUNNER_CHECK(aclmdlRICaptureEnd(stream, &recorded_step));
+    }
+    // (the previous step's readback has been waited for: the staging area is free)
+    replay_words[0] = static_cast<int32_t>(position);
+    replay_words[1] = static_cast<int32_t>(position + 1);
+    std::memcpy(replay_inputs, inputs + per_item * static_cast<size_t>(position * o.layers), 2 * per_item * static_cast<size_t>(o.layers));
+    RUNNER_CHECK(aclmdlRIExecuteAsync(recorded_step, stream));
+    launches += 2 * static_cast<uint64_t>(o.layers);
+    ++replayed_steps;
+    replay_host_seconds += std::chrono::duration<double>(std::chrono::steady_clock::now() - begin).count();
   };
   const auto read_token = [&]() {  // where the reference reads the argmax back: one synchronisation per generated token
     RUNNER_CHECK(aclrtMemcpyAsync(readback, 2 * kHeads * kLatent, arena + off_out, 2 * kHeads * kLatent, ACL_MEMCPY_DEVICE_TO_HOST, stream));
@@ -421,10 +467,20 @@ int Run(int argc, char** argv) {
   read_token();
   const auto first_token_time = std::chrono::steady_clock::now();
   for (int64_t i = 1; i < o.max_new_tokens && position < o.max_context; ++i) {
-    decode_step(position++);
+    if (o.graph) {
+      replay_step(position++);
+    } else {
+      decode_step(position++);
+    }
     read_token();
   }
   const auto decode_end = std::chrono::steady_clock::now();
+  // FNV-1a over the last step's attention output (64 heads x 512 bf16): the same for the same seed
+  // and flags whether the steps were enqueued call by call or replayed.
+  uint64_t output_hash = 0xcbf29ce484222325ull;
+  for (size_t i = 0; i < 2 * static_cast<size_t>(kHeads * kLatent); ++i) {
+    output_hash = (output_hash ^ reinterpret_cast<const unsigned char*>(readback)[i]) * 0x100000001b3ull;
+  }
   const double ttft_seconds = std::chrono::duration<double>(first_token_time - decode_start).count();
   const double decode_span_seconds = std::chrono::duration<double>(decode_end - first_token_time).count();
   const double total_seconds = std::chrono::duration<double>(decode_end - decode_start).count();
@@ -463,7 +519,12 @@ int Run(int argc, char** argv) {
   report << "steps " << position << ", layers " << o.layers << ", launches " << launches << "\n"
          << "timing: ttft " << ttft_seconds << " s (prefill of " << o.prompt_tokens << " single-token steps + first readback), tpot "
          << tpot_seconds << " s, total " << total_seconds << " s\n"
-         << "host time per step (enqueue only) " << enqueue_seconds / static_cast<double>(position) * 1e3 << " ms\n"
+         << "host time per step (enqueue only) " << enqueue_seconds / static_cast<double>(eager_steps) * 1e3 << " ms over "
+         << eager_steps << " steps enqueued call by call\n"
+         << (replayed_steps > 0 ? "replayed " + std::to_string(replayed_steps) + " steps from one recorded step: host time per replayed step " +
+                                      std::to_string(replay_host_seconds / static_cast<double>(replayed_steps) * 1e3) +
+                                      " ms (staging the step's inputs, one launch; the first includes the recording)\n"
+                                : std::string())
          << "host synchronizations " << host_synchronizations << " (one per generated-token readback)\n"
          << "allocations inside a step " << allocations_in_step << " (must be 0); descriptors 0 (must be 0)\n"
          << "gathered " << position << " rows x " << o.layers << " layers through the block table: " << mismatched_rows
@@ -491,7 +552,10 @@ int Run(int argc, char** argv) {
           << "  \"total_seconds\": " << total_seconds << ",\n"
           << "  \"device_slots\": 0,\n  \"slot_bytes\": 0,\n"
           << "  \"backbone_bytes\": " << arena_bytes << ",\n"
-          << "  \"host_enqueue_seconds_per_step\": " << enqueue_seconds / static_cast<double>(position) << ",\n"
+          << "  \"host_enqueue_seconds_per_step\": " << enqueue_seconds / static_cast<double>(eager_steps) << ",\n"
+          << "  \"replayed_steps\": " << replayed_steps << ",\n"
+          << "  \"host_seconds_per_replayed_step\": " << (replayed_steps > 0 ? replay_host_seconds / static_cast<double>(replayed_steps) : 0.0) << ",\n"
+          << "  \"last_output_fnv1a\": \"" << std::hex << output_hash << std::dec << "\",\n"
           << "  \"gathered_rows\": " << position * o.layers << ",\n"
           << "  \"gathered_rows_mismatched\": " << mismatched_rows << "\n"
           << "}\n";
@@ -517,6 +581,12 @@ int Run(int argc, char** argv) {
   }
   aclDestroyIntArray(actual_seq_q);
   aclDestroyIntArray(actual_seq_kv);
+  if (recorded_step != nullptr) RUNNER_CHECK(aclmdlRIDestroy(recorded_step));
+  if (o.graph) {
+    aclrtFreeHost(live_words);
+    aclrtFreeHost(replay_words);
+    aclrtFreeHost(replay_inputs);
+  }
   aclrtFreeHost(readback);
   aclrtFreeHost(mailbox);
   aclrtFreeHost(inputs);

@@ -369,6 +369,44 @@ aclError aclrtGetMemInfo(aclrtMemAttr, size_t* free_bytes, size_t* total_bytes) 
   return status == hipSuccess ? ACL_SUCCESS : RtFail(status, "aclrtGetMemInfo");
 }
 
+// ---- stream capture ------------------------------------------------------------------------
+
+aclError aclmdlRICaptureBegin(aclrtStream stream, aclmdlRICaptureMode mode) {
+  SHIM_REQUIRE(stream != nullptr, ACL_ERROR_INVALID_PARAM, "aclmdlRICaptureBegin: a stream of its own is needed (not the null stream)");
+  hipStreamCaptureMode hip_mode;
+  switch (mode) {
+    case ACL_MODEL_RI_CAPTURE_MODE_GLOBAL: hip_mode = hipStreamCaptureModeGlobal; break;
+    case ACL_MODEL_RI_CAPTURE_MODE_THREAD_LOCAL: hip_mode = hipStreamCaptureModeThreadLocal; break;
+    case ACL_MODEL_RI_CAPTURE_MODE_RELAXED: hip_mode = hipStreamCaptureModeRelaxed; break;
+    default: return Fail(ACL_ERROR_INVALID_PARAM, "aclmdlRICaptureBegin: unknown capture mode %d", static_cast<int>(mode));
+  }
+  const hipError_t status = hipStreamBeginCapture(static_cast<hipStream_t>(stream), hip_mode);
+  return status == hipSuccess ? ACL_SUCCESS : RtFail(status, "aclmdlRICaptureBegin");
+}
+aclError aclmdlRICaptureEnd(aclrtStream stream, aclmdlRI* model_ri) {
+  SHIM_REQUIRE(stream != nullptr && model_ri != nullptr, ACL_ERROR_INVALID_PARAM, "aclmdlRICaptureEnd: null stream or output");
+  *model_ri = nullptr;
+  hipGraph_t graph = nullptr;
+  hipError_t status = hipStreamEndCapture(static_cast<hipStream_t>(stream), &graph);
+  if (status != hipSuccess || graph == nullptr) return RtFail(status == hipSuccess ? hipErrorUnknown : status, "aclmdlRICaptureEnd");
+  hipGraphExec_t exec = nullptr;
+  status = hipGraphInstantiate(&exec, graph, nullptr, nullptr, 0);
+  (void)hipGraphDestroy(graph);
+  if (status != hipSuccess) return RtFail(status, "aclmdlRICaptureEnd (instantiate)");
+  *model_ri = exec;
+  return ACL_SUCCESS;
+}
+aclError aclmdlRIExecuteAsync(aclmdlRI model_ri, aclrtStream stream) {
+  SHIM_REQUIRE(model_ri != nullptr, ACL_ERROR_INVALID_PARAM, "aclmdlRIExecuteAsync: null recording");
+  const hipError_t status = hipGraphLaunch(static_cast<hipGraphExec_t>(model_ri), static_cast<hipStream_t>(stream));
+  return status == hipSuccess ? ACL_SUCCESS : RtFail(status, "aclmdlRIExecuteAsync");
+}
+aclError aclmdlRIDestroy(aclmdlRI model_ri) {
+  if (model_ri == nullptr) return ACL_SUCCESS;
+  const hipError_t status = hipGraphExecDestroy(static_cast<hipGraphExec_t>(model_ri));
+  return status == hipSuccess ? ACL_SUCCESS : RtFail(status, "aclmdlRIDestroy");
+}
+
 // ---- descriptor engine ------------------------------------------------------------------
 
 aclTensor* aclCreateTensor(const int64_t* view_dims, uint64_t view_dims_num, aclDataType dtype, const int64_t* view_strides,

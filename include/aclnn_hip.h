@@ -106,6 +106,27 @@ aclError aclrtSynchronizeStreamWithTimeout(aclrtStream stream, int32_t timeout_m
 aclError aclrtSynchronizeEvent(aclrtEvent event);
 aclError aclrtGetMemInfo(aclrtMemAttr attr, size_t* free_bytes, size_t* total_bytes);
 
+/* ---- stream capture: a step enqueued once, replayed as one launch ----
+ * The names and argument lists of CANN's capture interface (aclmdlRICaptureBegin / CaptureEnd /
+ * ExecuteAsync / Destroy); the reference does not call it (its loop enqueues every operator every
+ * step, src/pipeline/pipeline.cpp:390-416), so nothing of the reference binds to these. Served by a
+ * HIP graph: everything enqueued on `stream` between Begin and End (operator launches, asynchronous
+ * copies to or from pinned host memory) is recorded instead of run; ExecuteAsync enqueues the whole
+ * recording on a stream. Addresses and host-side arguments are those of the recording; what changes
+ * from replay to replay has to live in memory the recording reads (a pinned host word copied by a
+ * recorded aclrtMemcpyAsync, device lengths bound with aclnnMlaKvBindSeqLens). The first launch of
+ * every operator on a device must have happened before Begin (it sets up the kernels). */
+typedef void* aclmdlRI;
+typedef enum {
+  ACL_MODEL_RI_CAPTURE_MODE_GLOBAL = 0,
+  ACL_MODEL_RI_CAPTURE_MODE_THREAD_LOCAL = 1,
+  ACL_MODEL_RI_CAPTURE_MODE_RELAXED = 2
+} aclmdlRICaptureMode;
+aclError aclmdlRICaptureBegin(aclrtStream stream, aclmdlRICaptureMode mode);
+aclError aclmdlRICaptureEnd(aclrtStream stream, aclmdlRI* model_ri);
+aclError aclmdlRIExecuteAsync(aclmdlRI model_ri, aclrtStream stream);
+aclError aclmdlRIDestroy(aclmdlRI model_ri);
+
 /* ---- descriptor engine (mock/include/aclnn/acl_meta.h:59-90) ----
  * Dims and strides count ELEMENTS. The getters return arrays allocated with new[]; the
  * caller releases them with delete[] (src/memory/static_arena.cpp:181-188). A tensor list owns

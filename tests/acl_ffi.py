@@ -27,6 +27,8 @@ PROTOTYPES = {
     "aclrtRecordEvent": (_i32, [_vp, _vp]), "aclrtStreamWaitEvent": (_i32, [_vp, _vp]), "aclrtSynchronizeStream": (_i32, [_vp]),
     "aclrtSynchronizeStreamWithTimeout": (_i32, [_vp, _i32]), "aclrtSynchronizeEvent": (_i32, [_vp]),
     "aclrtGetMemInfo": (_i32, [_i32, _P(C.c_size_t), _P(C.c_size_t)]),
+    "aclmdlRICaptureBegin": (_i32, [_vp, _i32]), "aclmdlRICaptureEnd": (_i32, [_vp, _P(_vp)]),
+    "aclmdlRIExecuteAsync": (_i32, [_vp, _vp]), "aclmdlRIDestroy": (_i32, [_vp]),
     "aclCreateTensor": (_vp, [_P(_i64), _u64, _i32, _P(_i64), _i64, _i32, _P(_i64), _u64, _vp]),
     "aclDestroyTensor": (_i32, [_vp]),
     "aclGetViewShape": (_i32, [_vp, _P(_P(_i64)), _P(_u64)]), "aclGetStorageShape": (_i32, [_vp, _P(_P(_i64)), _P(_u64)]),
