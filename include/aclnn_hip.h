@@ -107,9 +107,10 @@ aclError aclrtSynchronizeEvent(aclrtEvent event);
 aclError aclrtGetMemInfo(aclrtMemAttr attr, size_t* free_bytes, size_t* total_bytes);
 
 /* ---- stream capture: a step enqueued once, replayed as one launch ----
- * The names and argument lists of CANN's capture interface (aclmdlRICaptureBegin / CaptureEnd /
- * ExecuteAsync / Destroy); the reference does not call it (its loop enqueues every operator every
- * step, src/pipeline/pipeline.cpp:390-416), so nothing of the reference binds to these. Served by a
+ * Named after CANN's stream-capture entry points (aclmdlRICaptureBegin / CaptureEnd / ExecuteAsync /
+ * Destroy; CANN is not installed here, so the match with its headers is unchecked). The reference
+ * does not call them (its loop enqueues every operator every step, src/pipeline/pipeline.cpp:390-416),
+ * so nothing of the reference binds to these. Served by a
  * HIP graph: everything enqueued on `stream` between Begin and End (operator launches, asynchronous
  * copies to or from pinned host memory) is recorded instead of run; ExecuteAsync enqueues the whole
  * recording on a stream. Addresses and host-side arguments are those of the recording; what changes
