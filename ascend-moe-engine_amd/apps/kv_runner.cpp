@@ -475,11 +475,21 @@ int Run(int argc, char** argv) {
     read_token();
   }
   const auto decode_end = std::chrono::steady_clock::now();
-  // FNV-1a over the last step's attention output (64 heads x 512 bf16): the same for the same seed
-  // and flags whether the steps were enqueued call by call or replayed.
+  // The last step's attention output (64 heads x 512 bf16) in two figures: FNV-1a over its bytes
+  // (the same for the same seed and flags as long as the same kernels run) and the sum of the
+  // magnitudes (which kernels that round differently agree on to a fraction of a percent: a step
+  // whose lengths the host passes by value may take the short-context units where a replayed step,
+  // whose length lives in device memory, takes the 64-head kernel).
   uint64_t output_hash = 0xcbf29ce484222325ull;
   for (size_t i = 0; i < 2 * static_cast<size_t>(kHeads * kLatent); ++i) {
     output_hash = (output_hash ^ reinterpret_cast<const unsigned char*>(readback)[i]) * 0x100000001b3ull;
+  }
+  double output_l1 = 0.0;
+  for (size_t i = 0; i < static_cast<size_t>(kHeads * kLatent); ++i) {
+    const uint32_t bits = static_cast<uint32_t>(readback[i]) << 16;
+    float value;
+    std::memcpy(&value, &bits, 4);
+    output_l1 += std::fabs(static_cast<double>(value));
   }
   const double ttft_seconds = std::chrono::duration<double>(first_token_time - decode_start).count();
   const double decode_span_seconds = std::chrono::duration<double>(decode_end - first_token_time).count();
@@ -556,6 +566,7 @@ int Run(int argc, char** argv) {
           << "  \"replayed_steps\": " << replayed_steps << ",\n"
           << "  \"host_seconds_per_replayed_step\": " << (replayed_steps > 0 ? replay_host_seconds / static_cast<double>(replayed_steps) : 0.0) << ",\n"
           << "  \"last_output_fnv1a\": \"" << std::hex << output_hash << std::dec << "\",\n"
+          << "  \"last_output_l1\": " << std::setprecision(12) << output_l1 << ",\n"
           << "  \"gathered_rows\": " << position * o.layers << ",\n"
           << "  \"gathered_rows_mismatched\": " << mismatched_rows << "\n"
           << "}\n";

@@ -375,6 +375,26 @@ PlanShape ShapeOf(int32_t batch, int32_t heads, int32_t max_seq_len, int32_t blo
   return shape;
 }
 
+// How a whole-context launch whose longest context is `bound` tokens cuts its work: 0 = the
+// 64-head kernel's flat cut, 1 = one workgroup per (sequence, 16 heads), 2 = two. Measured on
+// MI355X, bf16 and FP8 caches alike (64 heads unless said; us, 64-head kernel / one workgroup per
+// unit / two): batch 1 .. 32 (and 16 x 128, 64 x 16 heads), 128 tokens 14.5-16.8 / 8.3-8.5 / 8.7-9.9;
+// 256: 17.0-19.2 / 10.3-11.4 / 10.1-11.6; 512: 16.4-21.4 / 15.4-17.7 / 12.8-15.0; 768: 16.5-22.5 /
+// 20.8-24.0 / 15.5-18.7; 1024: 16.7-25.6 / 26.1-29.6 / 18.3-22.9. Batch 48, 64 (32 x 128): 256:
+// 21.1-22.9 / 12.0-12.8; 512: 21.3-23.9 / 17.9-20.3; 768: 23.7-26.8 / 24.4-37.5. Batch 96, 128
+// (64 x 128), two rounds of units: 256: 24.8-27.6 / 21.1-24.6; 384: 27.5-30.4 / 27.2-32.1. Batch 256:
+// 128: 29.0 / 31.8.
+int32_t ShortContextUnits(const mlakvAttnPlan* plan, int32_t bound) {
+  if (plan->selection_units == MLAKV_ATTN_UNITS_SPLIT || bound > MLAKV_ATTN_HEAD_BLOCK_TOKENS) return 0;
+  if (plan->selection_units == MLAKV_ATTN_UNITS_HEAD_BLOCK) return 1;
+  if (plan->selection_units == MLAKV_ATTN_UNITS_HEAD_BLOCK_HALVES) return 2;
+  const int64_t pairs = static_cast<int64_t>(plan->batch) * (plan->heads / 16);
+  if (2 * pairs <= ComputeUnits()) return bound <= 256 ? 1 : (bound <= 768 ? 2 : 0);
+  if (pairs <= ComputeUnits()) return bound <= 512 ? 1 : 0;
+  if (pairs <= 2 * ComputeUnits()) return bound <= 256 ? 1 : 0;
+  return 0;
+}
+
 mlakvStatus AttnPlanImpl(const char* who, int32_t batch, int32_t heads, int32_t max_seq_len, int32_t block_size,
                          int32_t dtype, bool sparse, const mlakvAttnPlanOptions* options, mlakvAttnPlan* plan) {
   if (plan == nullptr) return Fail(MLAKV_ERR_PARAM_NULLPTR, "%s: plan is null", who);
@@ -390,7 +410,7 @@ mlakvStatus AttnPlanImpl(const char* who, int32_t batch, int32_t heads, int32_t 
   if (options != nullptr) chosen = *options;
   if (chosen.chunk_tiles < 0 || chosen.work_groups < 0 || chosen.work_groups > 65535 || chosen.merge_mode < 0 ||
       chosen.merge_mode > MLAKV_ATTN_MERGE_SECOND_LAUNCH || chosen.merge_spin_us > 1000000 || chosen.selection_units < 0 ||
-      chosen.selection_units > MLAKV_ATTN_UNITS_HEAD_BLOCK_HALVES || (!sparse && chosen.selection_units != 0)) {
+      chosen.selection_units > MLAKV_ATTN_UNITS_HEAD_BLOCK_HALVES) {
     return Fail(MLAKV_ERR_PARAM_INVALID, "%s: options outside their ranges", who);
   }
   const int64_t head_groups = (heads + 63) / 64;
@@ -427,7 +447,7 @@ mlakvStatus AttnPlanImpl(const char* who, int32_t batch, int32_t heads, int32_t 
   // the split (a unit size, a workgroup count, a merge).
   const bool head_block_fits = sparse && max_seq_len <= MLAKV_ATTN_HEAD_BLOCK_TOKENS;
   const bool head_block_asked = chosen.selection_units == MLAKV_ATTN_UNITS_HEAD_BLOCK || chosen.selection_units == MLAKV_ATTN_UNITS_HEAD_BLOCK_HALVES;
-  if (head_block_asked && !head_block_fits) {
+  if (sparse && head_block_asked && !head_block_fits) {
     return Fail(MLAKV_ERR_PARAM_INVALID, "%s: whole-selection units of 16 heads take up to %d selected tokens", who,
                 MLAKV_ATTN_HEAD_BLOCK_TOKENS);
   }
@@ -435,7 +455,7 @@ mlakvStatus AttnPlanImpl(const char* who, int32_t batch, int32_t heads, int32_t 
   // 16 heads) in the workspace and meet on four of the library's counters each.
   const int64_t pairs = static_cast<int64_t>(batch) * (heads / 16);
   const bool halves_fit = head_block_fits && pairs * 4 <= 2 * mlakv::kAttnSyncSequences;
-  if (chosen.selection_units == MLAKV_ATTN_UNITS_HEAD_BLOCK_HALVES && !halves_fit) {
+  if (sparse && chosen.selection_units == MLAKV_ATTN_UNITS_HEAD_BLOCK_HALVES && !halves_fit) {
     return Fail(MLAKV_ERR_PARAM_INVALID, "%s: halved whole-selection units take up to %d (sequence, 16 heads) pairs", who,
                 mlakv::kAttnSyncSequences / 2);
   }
@@ -458,9 +478,20 @@ mlakvStatus AttnPlanImpl(const char* who, int32_t batch, int32_t heads, int32_t 
   const bool head_block = head_block_fits && (chosen.selection_units == MLAKV_ATTN_UNITS_HEAD_BLOCK ||
                                               (chosen.selection_units == MLAKV_ATTN_UNITS_AUTO && !split_asked && head_block_pays));
   const bool halves_pay = 2 * pairs <= ComputeUnits() && max_seq_len > 256 && (fp8 || max_seq_len <= 768);
-  const bool halves = chosen.selection_units == MLAKV_ATTN_UNITS_HEAD_BLOCK_HALVES ||
-                      (chosen.selection_units == MLAKV_ATTN_UNITS_AUTO && !split_asked && halves_fit && halves_pay);
-  plan->selection_units = !sparse ? 0 : (halves ? MLAKV_ATTN_UNITS_HEAD_BLOCK_HALVES : (head_block ? MLAKV_ATTN_UNITS_HEAD_BLOCK : MLAKV_ATTN_UNITS_SPLIT));
+  const bool halves = sparse && (chosen.selection_units == MLAKV_ATTN_UNITS_HEAD_BLOCK_HALVES ||
+                                 (chosen.selection_units == MLAKV_ATTN_UNITS_AUTO && !split_asked && halves_fit && halves_pay));
+  if (sparse) {
+    plan->selection_units = halves ? MLAKV_ATTN_UNITS_HEAD_BLOCK_HALVES : (head_block ? MLAKV_ATTN_UNITS_HEAD_BLOCK : MLAKV_ATTN_UNITS_SPLIT);
+  } else {
+    // A whole-context plan keeps what was asked for: AUTO lets every launch choose by the lengths it
+    // can see (ShortContextUnits), SPLIT keeps the 64-head kernel, the other two need a context the
+    // units can stage. Properties of the split pin the split.
+    if ((chosen.selection_units == MLAKV_ATTN_UNITS_HEAD_BLOCK || chosen.selection_units == MLAKV_ATTN_UNITS_HEAD_BLOCK_HALVES) &&
+        (max_seq_len > MLAKV_ATTN_HEAD_BLOCK_TOKENS || (chosen.selection_units == MLAKV_ATTN_UNITS_HEAD_BLOCK_HALVES && pairs * 4 > 2 * mlakv::kAttnSyncSequences))) {
+      return Fail(MLAKV_ERR_PARAM_INVALID, "%s: whole-context units of 16 heads take contexts of up to %d tokens", who, MLAKV_ATTN_HEAD_BLOCK_TOKENS);
+    }
+    plan->selection_units = chosen.selection_units == MLAKV_ATTN_UNITS_AUTO && split_asked ? MLAKV_ATTN_UNITS_SPLIT : chosen.selection_units;
+  }
   if (halves) shape = ShapeOf(batch, heads, max_seq_len, block_size, sparse, chunk_tiles, work_groups, true);
   plan->workspace_bytes = shape.workspace;
   return MLAKV_SUCCESS;
@@ -543,7 +574,10 @@ mlakvStatus AttnDecodeImpl(const char* who, const mlakvAttnPlan* plan, const mla
     const bool fields = plan->batch > 0 && plan->batch <= 65535 && plan->heads > 0 && plan->heads % 16 == 0 && plan->heads <= 128 &&
                         plan->max_seq_len > 0 && plan->block_size > 0 && plan->chunk_tiles >= 0 && plan->work_groups >= 1 &&
                         plan->work_groups <= 65535 && (plan->reserved == 0 || plan->reserved == 1) &&
-                        (plan->reserved == 0 ? plan->selection_units == 0
+                        (plan->reserved == 0 ? (plan->selection_units == MLAKV_ATTN_UNITS_AUTO || plan->selection_units == MLAKV_ATTN_UNITS_SPLIT ||
+                                                ((plan->selection_units == MLAKV_ATTN_UNITS_HEAD_BLOCK ||
+                                                  plan->selection_units == MLAKV_ATTN_UNITS_HEAD_BLOCK_HALVES) &&
+                                                 plan->max_seq_len <= MLAKV_ATTN_HEAD_BLOCK_TOKENS))
                                              : (plan->selection_units == MLAKV_ATTN_UNITS_SPLIT ||
                                                 ((plan->selection_units == MLAKV_ATTN_UNITS_HEAD_BLOCK ||
                                                   plan->selection_units == MLAKV_ATTN_UNITS_HEAD_BLOCK_HALVES) &&
@@ -554,7 +588,8 @@ mlakvStatus AttnDecodeImpl(const char* who, const mlakvAttnPlan* plan, const mla
     bool sane = fields;
     if (fields) {
       const PlanShape shape = ShapeOf(plan->batch, plan->heads, plan->max_seq_len, plan->block_size, plan->reserved == 1,
-                                      plan->chunk_tiles, plan->work_groups, plan->selection_units == MLAKV_ATTN_UNITS_HEAD_BLOCK_HALVES);
+                                      plan->chunk_tiles, plan->work_groups,
+                                      plan->reserved == 1 && plan->selection_units == MLAKV_ATTN_UNITS_HEAD_BLOCK_HALVES);
       sane = plan->chunk_tiles <= shape.cap && plan->max_units == shape.units && plan->workspace_bytes == shape.workspace &&
              (plan->merge_mode != MLAKV_ATTN_MERGE_IN_LAUNCH ||
               (static_cast<int64_t>(plan->batch) * shape.head_groups <= mlakv::kAttnSyncSequences && shape.units < 65535));
@@ -651,6 +686,24 @@ mlakvStatus AttnDecodeImpl(const char* who, const mlakvAttnPlan* plan, const mla
   args.merge_in_launch = plan->merge_mode == MLAKV_ATTN_MERGE_IN_LAUNCH;
   args.fp8 = cache->dtype == MLAKV_DTYPE_FP8_E4M3;
   args.head_block_units = plan->selection_units == MLAKV_ATTN_UNITS_HEAD_BLOCK ? 1 : (plan->selection_units == MLAKV_ATTN_UNITS_HEAD_BLOCK_HALVES ? 2 : 0);
+  if (!sparse) {
+    // A whole context that is short: the units of the selected-token attention (one workgroup, or
+    // two, per sequence and 16 heads; no selection, every position of the context) are ahead of the
+    // 64-head kernel, whose work units are all fixed cost at that size. What the launch can see of
+    // the lengths decides: the values themselves when they ride in the argument block, else the
+    // plan's bound.
+    int32_t bound = args.max_tokens;
+    if (host_lens != nullptr) {
+      bound = 0;
+      for (int32_t i = 0; i < plan->batch; ++i) bound = std::max(bound, std::min(std::max(host_lens[i], 0), args.max_tokens));
+    }
+    args.head_block_units = quant != nullptr ? 0 : ShortContextUnits(plan, bound);
+    if (args.head_block_units == 2) {  // (the halves' partials must fit what the plan sized for the split)
+      const uint64_t halved = static_cast<uint64_t>(plan->batch) * (plan->heads / 16) * (32 * mlakv::kLatentDim * 2 + 2 * 4 * 16 * sizeof(float));
+      if (halved > plan->workspace_bytes) args.head_block_units = 1;
+    }
+    args.sparse_count = args.head_block_units != 0 ? std::max(bound, 1) : 0;
+  }
   const hipError_t status = mlakv::LaunchAttnDecode(args, static_cast<hipStream_t>(stream));
   return status == hipSuccess ? MLAKV_SUCCESS : HipFail(status, who);
 }

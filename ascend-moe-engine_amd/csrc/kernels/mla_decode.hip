@@ -1604,7 +1604,8 @@ __global__ __launch_bounds__(kHbThreads) void MlaSelectedHeadBlockKernel(AttnArg
 #pragma unroll
   for (int j = 0; j < kPerThread; ++j) {
     const int i = tid + kHbThreads * j;
-    index[j] = i < a.sparse_count ? selection[i] : -1;
+    // (no selection: the sequence's own positions 0 .. context - 1, a whole context of up to sparse_count tokens)
+    index[j] = i < a.sparse_count ? (a.sparse_indices != nullptr ? selection[i] : i) : -1;
   }
   // Q fragments of a score wave: lane (head i16, k-group g) holds Q[head][32 ks + 8 g .. +7] for the
   // nine k-steps ks of its half. FP8: the code reads cover k = 64 kp + 16 g .. + 15 (two k-steps),
@@ -2183,6 +2184,23 @@ bool AnySequenceSplit(const AttnArgs& a) {
   return false;
 }
 
+// Whole-selection units of 16 heads, one workgroup per unit or two (head_block_units 1 / 2).
+static hipError_t LaunchHeadBlockUnits(AttnArgs& args, hipStream_t stream) {
+  const int sequences_per_xcd = (args.batch + kXcds - 1) / kXcds;
+  const int64_t pairs = static_cast<int64_t>(args.batch) * (args.heads / 16);
+  // Two workgroups per unit meet on four words each of this launch's counters and leave their
+  // partials in the first 2 x 16 x pairs rows of the workspace, the LSEs behind them (the plan
+  // sizes the workspace for that).
+  const bool halves = args.head_block_units == 2 && pairs * 4 <= kAttnSyncSequences * 2 && args.partial_out != nullptr;
+  if (halves) {
+    if (hipError_t sync_error = SyncRegion(&args.sync); sync_error != hipSuccess) return sync_error;
+    const dim3 units(kXcds * (args.heads / 16) * 2 * sequences_per_xcd);
+    return args.fp8 ? LaunchHeadBlock<true, true>(args, units, stream) : LaunchHeadBlock<true, false>(args, units, stream);
+  }
+  const dim3 units(kXcds * (args.heads / 16) * sequences_per_xcd);
+  return args.fp8 ? LaunchHeadBlock<false, true>(args, units, stream) : LaunchHeadBlock<false, false>(args, units, stream);
+}
+
 hipError_t LaunchAttnDecode(const AttnArgs& args_in, hipStream_t stream) {
   AttnArgs args = args_in;
   if (args.batch <= 0) return hipSuccess;
@@ -2206,21 +2224,14 @@ hipError_t LaunchAttnDecode(const AttnArgs& args_in, hipStream_t stream) {
     // (a pool whose rows the 32-bit starts of the whole-selection units cannot address goes to the split units)
     if (args.head_block_units != 0 && PlainRowsAddressable(args)) {
       if (args.sparse_count > kAttnHeadBlockTokens || args.heads % 16 != 0 || args.out == nullptr) return hipErrorInvalidValue;
-      const int sequences_per_xcd = (args.batch + kXcds - 1) / kXcds;
-      const int64_t pairs = static_cast<int64_t>(args.batch) * (args.heads / 16);
-      // Two workgroups per unit meet on four words each of this launch's counters and leave their
-      // partials in the first 2 x 16 x pairs rows of the workspace, the LSEs behind them (the plan
-      // sizes the workspace for that).
-      const bool halves = args.head_block_units == 2 && pairs * 4 <= kAttnSyncSequences * 2 && args.partial_out != nullptr;
-      if (halves) {
-        if (hipError_t sync_error = SyncRegion(&args.sync); sync_error != hipSuccess) return sync_error;
-        const dim3 units(kXcds * (args.heads / 16) * 2 * sequences_per_xcd);
-        return args.fp8 ? LaunchHeadBlock<true, true>(args, units, stream) : LaunchHeadBlock<true, false>(args, units, stream);
-      }
-      const dim3 units(kXcds * (args.heads / 16) * sequences_per_xcd);
-      return args.fp8 ? LaunchHeadBlock<false, true>(args, units, stream) : LaunchHeadBlock<false, false>(args, units, stream);
+      return LaunchHeadBlockUnits(args, stream);
     }
     e = args.fp8 ? Launch<true, false, false, true>(args, grid, stream) : Launch<false, false, false, true>(args, grid, stream);
+  } else if (args.head_block_units != 0 && !quantise && args.out != nullptr && args.heads % 16 == 0 && args.sparse_count > 0 &&
+             args.sparse_count <= kAttnHeadBlockTokens && PlainRowsAddressable(args)) {
+    // a whole context of up to sparse_count tokens in the units of the selected-token attention: no
+    // selection, a sequence attends to its own positions
+    return LaunchHeadBlockUnits(args, stream);
   } else {
     e = quantise ? LaunchByCache<true>(args, grid, stream) : LaunchByCache<false>(args, grid, stream);
   }

@@ -186,7 +186,8 @@ typedef struct mlakvAttnPlan {
   int32_t merge_mode;      /* MLAKV_ATTN_MERGE_IN_LAUNCH or _SECOND_LAUNCH */
   int32_t merge_spin_us;   /* bound of the in-launch merge's wait for a sequence's other partials */
   int32_t reserved;        /* 1: made by mlakvAttnSparsePlanInit (max_seq_len holds sparse_count) */
-  int32_t selection_units; /* MLAKV_ATTN_UNITS_SPLIT, _HEAD_BLOCK or _HEAD_BLOCK_HALVES (selected-token plans; 0 otherwise) */
+  int32_t selection_units; /* selected-token plans: MLAKV_ATTN_UNITS_SPLIT, _HEAD_BLOCK or _HEAD_BLOCK_HALVES, fixed by the plan;
+                            * whole-context plans: what the options asked for, MLAKV_ATTN_UNITS_AUTO = every launch chooses */
   uint64_t workspace_bytes;
 } mlakvAttnPlan;
 
@@ -212,7 +213,18 @@ mlakvStatus mlakvAttnPlanInit(int32_t batch, int32_t heads, int32_t max_seq_len,
  * heads / 16 units fit the CUs once and up to 256 while they fit twice; else SPLIT. FP8 caches:
  * HEAD_BLOCK_HALVES from 257 selected tokens while two workgroups per unit fit the CUs once; else
  * HEAD_BLOCK while the units fit the CUs four times (beyond that up to 256 selected tokens); else
- * SPLIT. */
+ * SPLIT.
+ * Whole-context plans (mlakvAttnPlanInit[Ex] without `selection`) use the same units for short
+ * contexts: a unit then takes every position of its sequence. AUTO decides at every launch from
+ * the longest context the launch can see -- the lengths themselves with mlakvAttnDecodeHostLens,
+ * the plan's max_seq_len with lengths in device memory: while two workgroups per unit fit the CUs
+ * once, HEAD_BLOCK up to 256 tokens and HEAD_BLOCK_HALVES up to 768; while one per unit fits,
+ * HEAD_BLOCK up to 512; while they fit twice, up to 256; the 64-head kernel otherwise, for the
+ * quantising entry point and whenever
+ * chunk_tiles, work_groups or merge_mode ask for properties of the split. SPLIT keeps the 64-head
+ * kernel always; HEAD_BLOCK and HEAD_BLOCK_HALVES ask for the units (max_seq_len up to
+ * MLAKV_ATTN_HEAD_BLOCK_TOKENS). The two kinds of kernel round differently (both inside the stated
+ * tolerance), so launches of one plan that see different lengths may differ in the last bits. */
 #define MLAKV_ATTN_UNITS_AUTO 0
 #define MLAKV_ATTN_UNITS_SPLIT 1
 #define MLAKV_ATTN_UNITS_HEAD_BLOCK 2
@@ -224,7 +236,7 @@ typedef struct mlakvAttnPlanOptions {
   int32_t merge_mode;     /* MLAKV_ATTN_MERGE_* */
   int32_t merge_spin_us;  /* > 0: microseconds; < 0: do not wait at all (the last contributor merges) */
   int32_t selection;      /* 1: a plan for mlakvAttnDecodeSparse; max_seq_len then holds sparse_count */
-  int32_t selection_units; /* MLAKV_ATTN_UNITS_* (selection plans only) */
+  int32_t selection_units; /* MLAKV_ATTN_UNITS_* */
   int32_t reserved[2];    /* zero */
 } mlakvAttnPlanOptions;
 mlakvStatus mlakvAttnPlanInitEx(int32_t batch, int32_t heads, int32_t max_seq_len, int32_t block_size, int32_t dtype,

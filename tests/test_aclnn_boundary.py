@@ -314,8 +314,18 @@ def test_thin_abi_argument_validation_without_a_device():
         asked = ffi.AttnPlanOptions(option.get("chunk_tiles", 0), option.get("work_groups", 0), option.get("merge_mode", 0), 0, 1, 0)
         assert lib.mlakvAttnPlanInitEx(32, 64, 512, 64, ffi.DTYPE_BF16, C.byref(asked), C.byref(sparse)) == 0
         assert sparse.selection_units == ffi.ATTN_UNITS_SPLIT, option
-    dense_option = ffi.AttnPlanOptions(0, 0, 0, 0, 0, ffi.ATTN_UNITS_SPLIT)   # the option belongs to selection plans
-    assert lib.mlakvAttnPlanInitEx(32, 64, 2048, 64, ffi.DTYPE_BF16, C.byref(dense_option), C.byref(sparse)) == ffi.ERR_PARAM_INVALID
+    # whole-context plans keep what was asked for (AUTO: every launch chooses); the units need a context they can stage
+    dense_option = ffi.AttnPlanOptions(0, 0, 0, 0, 0, ffi.ATTN_UNITS_SPLIT)
+    assert lib.mlakvAttnPlanInitEx(32, 64, 2048, 64, ffi.DTYPE_BF16, C.byref(dense_option), C.byref(sparse)) == 0
+    assert sparse.selection_units == ffi.ATTN_UNITS_SPLIT and sparse.reserved == 0
+    for units in (ffi.ATTN_UNITS_HEAD_BLOCK, ffi.ATTN_UNITS_HEAD_BLOCK_HALVES):
+        dense_option = ffi.AttnPlanOptions(0, 0, 0, 0, 0, units)
+        assert lib.mlakvAttnPlanInitEx(32, 64, 1025, 64, ffi.DTYPE_BF16, C.byref(dense_option), C.byref(sparse)) == ffi.ERR_PARAM_INVALID
+        assert lib.mlakvAttnPlanInitEx(32, 64, 1024, 64, ffi.DTYPE_BF16, C.byref(dense_option), C.byref(sparse)) == 0
+        assert sparse.selection_units == units
+    dense_option = ffi.AttnPlanOptions(2, 0, 0, 0, 0, 0)                      # a property of the split pins the split
+    assert lib.mlakvAttnPlanInitEx(32, 64, 256, 64, ffi.DTYPE_BF16, C.byref(dense_option), C.byref(sparse)) == 0
+    assert sparse.selection_units == ffi.ATTN_UNITS_SPLIT
     assert lib.mlakvAttnPlanInit(32, 64, 2048, 64, ffi.DTYPE_BF16, C.byref(sparse)) == 0 and sparse.selection_units == 0
     altered = ffi.AttnPlan.from_buffer_copy(sparse)
     altered.selection_units = ffi.ATTN_UNITS_HEAD_BLOCK   # a whole-context plan that claims a selection's units

@@ -217,6 +217,66 @@ def test_maximum_context_single_sequence_many_chunks(fp8):
         _assert_close(out[:1, :16], expected, TOL_BF16)
 
 
+@pytest.mark.parametrize("fp8", [False, True])
+def test_short_whole_contexts_in_units_of_16_heads(fp8):
+    """A whole-context launch whose longest context the launch can see is short takes the units of
+    the selected-token attention (no selection: every position of the sequence): asked for by the
+    plan, chosen by the default plan from its own bound, and chosen by a launch with host-known
+    lengths under a plan made for long contexts. Against the oracle, against the 64-head kernel, and
+    the quantising entry point (which keeps the 64-head kernel) against its own bf16 output."""
+    import ctypes as C
+    lib = ffi.load()
+    bs, heads = 64, 64
+    tol = TOL_FP8 if fp8 else TOL_BF16
+    for ctxs in ([1, 0, 250, 64, 33, 256, 65, 129], [300, 512, 1, 0, 97], [1000, 1024, 3]):
+        blocks = sum(-(-c // bs) for c in ctxs) + 4
+        table = kt.build_tables(ctxs, bs, blocks, seed=91, max_blocks=2048 // bs).table()   # rows wide enough for a 2048-token plan
+        cache = kt.PagedCache(1, blocks, bs, fp8=fp8)
+        _fill_cache(cache, ctxs, table, seed=92, outliers=0.01 if fp8 else 0.0)
+        q = kt.randn_bf16((len(ctxs), heads, LATENT + ROPE), seed=93).cuda()
+        tab, lens = kt.dev_i32(table), kt.dev_i32(ctxs)
+        expected, expected_lse = kt.oracle_attention(cache, 0, q, table, ctxs, SCALE)
+        live = np.array(ctxs) > 0
+        split, split_lse, plan = kt.attention(cache, 0, q, tab, lens, SCALE, selection_units=ffi.ATTN_UNITS_SPLIT)
+        assert plan.selection_units == ffi.ATTN_UNITS_SPLIT
+        _assert_close(split, expected, tol)
+        peak = np.abs(expected).max()
+        for units in (ffi.ATTN_UNITS_AUTO, ffi.ATTN_UNITS_HEAD_BLOCK, ffi.ATTN_UNITS_HEAD_BLOCK_HALVES):
+            out, lse, plan = kt.attention(cache, 0, q, tab, lens, SCALE, selection_units=units)
+            assert plan.selection_units == units
+            _assert_close(out, expected, tol)
+            assert np.abs(lse.cpu().numpy()[live] - expected_lse[live]).max() <= tol
+            assert not out[~torch.from_numpy(live).cuda()].any() and torch.isneginf(lse[~torch.from_numpy(live).cuda()]).all()
+            assert (out.float() - split.float()).abs().max().item() <= 2 ** -5 * peak
+            if units != ffi.ATTN_UNITS_AUTO or max(ctxs) <= 768:   # the units ran: not the 64-head kernel's bits
+                assert not torch.equal(out, split)
+            else:
+                assert torch.equal(out, split)
+        # a plan for long contexts, the lengths by value: the launch sees that they are short
+        long_plan = kt.make_plan(len(ctxs), heads, 2048, bs, fp8)
+        ws = torch.empty(int(long_plan.workspace_bytes), dtype=torch.uint8, device="cuda")
+        by_value, by_value_lse = torch.full_like(split, float("nan")), torch.full_like(split_lse, float("nan"))
+        in_memory = torch.full_like(split, float("nan"))
+        host = (C.c_int32 * len(ctxs))(*ctxs)
+        row = (LATENT + ROPE) * 2
+        head_args = (C.byref(long_plan), C.byref(cache.view), 0, q.data_ptr(), heads * row, row, q.data_ptr() + LATENT * 2, heads * row, row,
+                     tab.data_ptr(), tab.shape[1])
+        ffi.check(lib.mlakvAttnDecodeHostLens(*head_args, C.cast(host, C.c_void_p), SCALE, by_value.data_ptr(), heads * LATENT * 2, LATENT * 2,
+                                              by_value_lse.data_ptr(), ws.data_ptr(), ws.numel(), kt.stream_ptr()))
+        ffi.check(lib.mlakvAttnDecode(*head_args, lens.data_ptr(), SCALE, in_memory.data_ptr(), heads * LATENT * 2, LATENT * 2, None,
+                                      ws.data_ptr(), ws.numel(), kt.stream_ptr()))
+        torch.cuda.synchronize()
+        _assert_close(by_value, expected, tol)
+        _assert_close(in_memory, expected, tol)
+        assert torch.equal(in_memory, split)                       # lengths in device memory: the plan's bound decides
+        assert torch.equal(by_value, split) == (max(ctxs) > 768)   # by value: the lengths themselves
+        # the quantising entry point keeps the 64-head kernel
+        _, _, _, codes, scales = kt.attention(cache, 0, q, tab, lens, SCALE, quant=True, want_out=False)
+        _, _, _, codes_split, scales_split = kt.attention(cache, 0, q, tab, lens, SCALE, quant=True, want_out=False,
+                                                          selection_units=ffi.ATTN_UNITS_SPLIT)
+        assert torch.equal(codes, codes_split) and torch.equal(scales, scales_split)
+
+
 def test_host_lengths_in_the_argument_block_give_the_same_bits():
     """mlakvAttnDecodeHostLens against mlakvAttnDecode with the same lengths in device memory: the
     kernels only read the lengths from another place, so every output bit agrees; split and
