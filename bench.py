@@ -305,7 +305,8 @@ def bench_attention(args, torch, np, ffi, ctxs, fp8=False, heads=64, slices=8, i
                         pool_blocks=pool_blocks, seed=7, shuffle=1, dtype=ffi.DTYPE_FP8_E4M3 if fp8 else ffi.DTYPE_BF16)
     plan = ffi.AttnPlan()
     merge_mode = {"auto": ffi.ATTN_MERGE_AUTO, "in": ffi.ATTN_MERGE_IN_LAUNCH, "second": ffi.ATTN_MERGE_SECOND_LAUNCH}[args.attn_merge]
-    units = {"auto": ffi.ATTN_UNITS_AUTO, "split": ffi.ATTN_UNITS_SPLIT, "head-block": ffi.ATTN_UNITS_HEAD_BLOCK, "halves": ffi.ATTN_UNITS_HEAD_BLOCK_HALVES}[args.attn_units] if sparse_k else 0
+    units = {"auto": ffi.ATTN_UNITS_AUTO, "split": ffi.ATTN_UNITS_SPLIT, "head-block": ffi.ATTN_UNITS_HEAD_BLOCK,
+             "halves": ffi.ATTN_UNITS_HEAD_BLOCK_HALVES}[args.attn_units] if sparse_k or max_ctx <= ffi.ATTN_HEAD_BLOCK_TOKENS else 0
     if merge_mode != ffi.ATTN_MERGE_AUTO or args.attn_chunk_tiles or args.attn_work_groups or units:
         options = ffi.AttnPlanOptions(args.attn_chunk_tiles, args.attn_work_groups, merge_mode, args.attn_merge_spin_us, 1 if sparse_k else 0, units)
         ffi.check(lib.mlakvAttnPlanInitEx(batch, heads, sparse_k or max_ctx, bs, cache.config.dtype, C.byref(options), C.byref(plan)))
@@ -423,6 +424,9 @@ def bench_attention(args, torch, np, ffi, ctxs, fp8=False, heads=64, slices=8, i
         "merge": ("none (a unit holds a whole selection for 16 heads)" if plan.selection_units == ffi.ATTN_UNITS_HEAD_BLOCK
                   else "in launch, pairs (two workgroups per selection and 16 heads; the second to finish combines)"
                   if plan.selection_units == ffi.ATTN_UNITS_HEAD_BLOCK_HALVES
+                  else "chosen per launch: units of 16 heads (no partials, or pairs combined in the launch) while the longest context "
+                       "the launch can see is short, else the 64-head kernel with a second launch"
+                  if not sparse_k and plan.selection_units == ffi.ATTN_UNITS_AUTO and max_ctx <= ffi.ATTN_HEAD_BLOCK_TOKENS
                   else "in launch" if plan.merge_mode == ffi.ATTN_MERGE_IN_LAUNCH else "second launch"),
         "workspace_bytes": int(plan.workspace_bytes), "timing": "250 ms of back-to-back launches untimed, then at least 100 ms of them timed",
     }
@@ -834,6 +838,8 @@ def attention_suite(args, torch, np, ffi):
         args, torch, np, ffi, draw_contexts(np, "lognormal_4096_cap_32768", 128, CONTEXT_SEED), slices=2, iters=16,
         label="configs[4] decode attention of one layer", distribution="lognormal (median 4096, sigma 1.0, cap 32768)",
         traffic_ratio=ATTENTION_TRAFFIC["attention_long"])
+    # short whole contexts: the launch takes the units of the selected-token attention (every position of the sequence)
+    out["attention_short"] = bench_attention(args, torch, np, ffi, [512] * 32, slices=8, label="whole contexts of 512 tokens")
     out["attention_sparse"] = bench_attention(args, torch, np, ffi, [8192] * 32, slices=4, sparse_k=512,
                                               label="selected-token decode (index_topk 512 of 8192)",
                                               traffic_ratio=ATTENTION_TRAFFIC["attention_sparse"])
