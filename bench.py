@@ -839,7 +839,7 @@ def attention_suite(args, torch, np, ffi):
         label="configs[4] decode attention of one layer", distribution="lognormal (median 4096, sigma 1.0, cap 32768)",
         traffic_ratio=ATTENTION_TRAFFIC["attention_long"])
     # short whole contexts: the launch takes the units of the selected-token attention (every position of the sequence)
-    out["attention_short"] = bench_attention(args, torch, np, ffi, [512] * 32, slices=8, label="whole contexts of 512 tokens")
+    out["attention_short"] = bench_attention(args, torch, np, ffi, [256] * 32, slices=8, label="whole contexts of 256 tokens")
     out["attention_sparse"] = bench_attention(args, torch, np, ffi, [8192] * 32, slices=4, sparse_k=512,
                                               label="selected-token decode (index_topk 512 of 8192)",
                                               traffic_ratio=ATTENTION_TRAFFIC["attention_sparse"])
