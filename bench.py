@@ -53,7 +53,8 @@ ATTENTION_TRAFFIC = {
     "attention": {"ratio": 1.429, "source": _TRAFFIC_SOURCE},        # 114.27 MB against 79.96 MB
     "attention_fp8": {"ratio": 1.254, "source": _TRAFFIC_SOURCE},    # 221.43 MB against 176.52 MB
     "attention_long": {"ratio": 1.060, "source": _TRAFFIC_SOURCE},   # 952.84 MB against 898.64 MB
-    "attention_sparse": {"ratio": 1.322, "source": _TRAFFIC_SOURCE}, # 30.96 MB against 23.41 MB (one dispatch: halved whole-selection units)
+    "attention_sparse": {"ratio": 1.320, "source": _TRAFFIC_SOURCE}, # 30.90 MB against 23.41 MB (one dispatch: halved whole-selection units)
+    "attention_short": {"ratio": 1.018, "source": _TRAFFIC_SOURCE},  # 14.14 MB against 13.89 MB (one dispatch, no partials)
     "attention_sparse_fp8": {"ratio": 1.613, "source": _TRAFFIC_SOURCE}, # 22.65 MB against 14.04 MB
     "indexer": {"ratio": 1.094, "source": _TRAFFIC_SOURCE},          # 38.24 MB against 34.96 MB
 }
@@ -839,7 +840,8 @@ def attention_suite(args, torch, np, ffi):
         label="configs[4] decode attention of one layer", distribution="lognormal (median 4096, sigma 1.0, cap 32768)",
         traffic_ratio=ATTENTION_TRAFFIC["attention_long"])
     # short whole contexts: the launch takes the units of the selected-token attention (every position of the sequence)
-    out["attention_short"] = bench_attention(args, torch, np, ffi, [256] * 32, slices=8, label="whole contexts of 256 tokens")
+    out["attention_short"] = bench_attention(args, torch, np, ffi, [256] * 32, slices=8, label="whole contexts of 256 tokens",
+                                             traffic_ratio=ATTENTION_TRAFFIC["attention_short"])
     out["attention_sparse"] = bench_attention(args, torch, np, ffi, [8192] * 32, slices=4, sparse_k=512,
                                               label="selected-token decode (index_topk 512 of 8192)",
                                               traffic_ratio=ATTENTION_TRAFFIC["attention_sparse"])
