@@ -427,8 +427,9 @@ int Run(int argc, char** argv) {
     const auto begin = std::chrono::steady_clock::now();
     mailbox[position] = static_cast<int32_t>(position);  // slot = position (pipeline.cpp:517); a word per step
     const int64_t live = position + 1;
-    if (o.graph) {
+    if (o.graph) {  // the length lives in device memory; the launch chooses its kernels by the bound it is told
       live_words[position] = static_cast<int32_t>(live);
+      RUNNER_CHECK(aclnnMlaKvSetSeqLenBound(ex_attention, live));
     } else {
       RUNNER_CHECK(aclnnMlaKvSetSeqLens(ex_attention, &live, 1));
     }
@@ -438,12 +439,23 @@ int Run(int argc, char** argv) {
     enqueue_seconds += std::chrono::duration<double>(std::chrono::steady_clock::now() - begin).count();
   };
   aclmdlRI recorded_step = nullptr;
+  int64_t recorded_bound = 0;  // the context length the recording's kernels were chosen for
+  uint64_t recordings = 0;
   const auto replay_step = [&](int64_t position) {
     const auto begin = std::chrono::steady_clock::now();
-    if (recorded_step == nullptr) {  // record: the same calls, from the staging words and rows
+    if (recorded_step == nullptr || position + 1 > recorded_bound) {
+      // Record: the same calls, from the staging words and rows. A recording fixes the kernels of
+      // its launches, and short contexts have faster ones, so it is made for the next size where
+      // the choice changes and made again when the context outgrows it.
+      if (recorded_step != nullptr) RUNNER_CHECK(aclmdlRIDestroy(recorded_step));
+      recorded_step = nullptr;
+      recorded_bound = position + 1 <= 256 ? 256 : (position + 1 <= 768 ? 768 : o.max_context);
+      recorded_bound = std::min(recorded_bound, o.max_context);
+      RUNNER_CHECK(aclnnMlaKvSetSeqLenBound(ex_attention, recorded_bound));
       RUNNER_CHECK(aclmdlRICaptureBegin(stream, ACL_MODEL_RI_CAPTURE_MODE_GLOBAL));
       enqueue_step(replay_words, replay_words + 1, replay_inputs);
       RUNNER_CHECK(aclmdlRICaptureEnd(stream, &recorded_step));
+      ++recordings;
     }
     // (the previous step's readback has been waited for: the staging area is free)
     replay_words[0] = static_cast<int32_t>(position);
@@ -531,9 +543,10 @@ int Run(int argc, char** argv) {
          << tpot_seconds << " s, total " << total_seconds << " s\n"
          << "host time per step (enqueue only) " << enqueue_seconds / static_cast<double>(eager_steps) * 1e3 << " ms over "
          << eager_steps << " steps enqueued call by call\n"
-         << (replayed_steps > 0 ? "replayed " + std::to_string(replayed_steps) + " steps from one recorded step: host time per replayed step " +
+         << (replayed_steps > 0 ? "replayed " + std::to_string(replayed_steps) + " steps from " + std::to_string(recordings) +
+                                      " recording(s) of a step (one per range of context lengths with kernels of its own): host time per replayed step " +
                                       std::to_string(replay_host_seconds / static_cast<double>(replayed_steps) * 1e3) +
-                                      " ms (staging the step's inputs, one launch; the first includes the recording)\n"
+                                      " ms (staging the step's inputs, one launch; recording included)\n"
                                 : std::string())
          << "host synchronizations " << host_synchronizations << " (one per generated-token readback)\n"
          << "allocations inside a step " << allocations_in_step << " (must be 0); descriptors 0 (must be 0)\n"
@@ -564,6 +577,7 @@ int Run(int argc, char** argv) {
           << "  \"backbone_bytes\": " << arena_bytes << ",\n"
           << "  \"host_enqueue_seconds_per_step\": " << enqueue_seconds / static_cast<double>(eager_steps) << ",\n"
           << "  \"replayed_steps\": " << replayed_steps << ",\n"
+          << "  \"recordings\": " << recordings << ",\n"
           << "  \"host_seconds_per_replayed_step\": " << (replayed_steps > 0 ? replay_host_seconds / static_cast<double>(replayed_steps) : 0.0) << ",\n"
           << "  \"last_output_fnv1a\": \"" << std::hex << output_hash << std::dec << "\",\n"
           << "  \"last_output_l1\": " << std::setprecision(12) << output_l1 << ",\n"

@@ -143,6 +143,7 @@ struct aclOpExecutor {
   uint64_t workspace_bytes = 0;
   uint64_t lens_offset = 0;  // attention: where the int32 lengths live inside the workspace
   const int32_t* bound_lens = nullptr;
+  int32_t bound_longest = -1;  // the caller's word for the longest of the bound lengths; -1: none given
   std::vector<int32_t> host_lens;  // plan-time kv lengths, or those of the latest aclnnMlaKvSetSeqLens
 };
 
@@ -1015,11 +1016,15 @@ aclnnStatus aclnnFusedInferAttentionScoreV5(void* workspace, uint64_t workspace_
                                             static_cast<const int32_t*>(e->slots[14].addresses[0]), e->table_width, e->host_lens.data(),
                                             e->scale, e->slots[31].addresses[0], e->out_token_stride, e->out_head_stride, lse, workspace,
                                             e->plan.workspace_bytes, stream)
-                  : mlakvAttnDecode(&e->plan, &view, 0, e->slots[0].addresses[0], e->q_token_stride, e->q_head_stride,
-                                    e->slots[24].addresses[0], e->qr_token_stride, e->qr_head_stride,
-                                    static_cast<const int32_t*>(e->slots[14].addresses[0]), e->table_width, device_lens, e->scale,
-                                    e->slots[31].addresses[0], e->out_token_stride, e->out_head_stride, lse, workspace,
-                                    e->plan.workspace_bytes, stream);
+                  // (lengths in device memory; a bound the caller gave for them decides the kernels)
+                  : mlakvAttnDecodeBounded(&e->plan, &view, 0, e->slots[0].addresses[0], e->q_token_stride, e->q_head_stride,
+                                           e->slots[24].addresses[0], e->qr_token_stride, e->qr_head_stride,
+                                           static_cast<const int32_t*>(e->slots[14].addresses[0]), e->table_width, device_lens,
+                                           e->bound_lens == nullptr ? *std::max_element(e->host_lens.begin(), e->host_lens.end())  // staged from the host values
+                                                                    : (e->bound_longest >= 0 ? e->bound_longest : e->max_seq_len),
+                                           e->scale,
+                                           e->slots[31].addresses[0], e->out_token_stride, e->out_head_stride, lse, workspace,
+                                           e->plan.workspace_bytes, stream);
   if (status == MLAKV_SUCCESS) e->launched = true;
   return status;
 }
@@ -1044,6 +1049,17 @@ aclnnStatus aclnnMlaKvBindSeqLens(aclOpExecutor* executor, const int32_t* device
   SHIM_REQUIRE(AsExecutor(executor) && executor->kind == OpKind::kAttention, ACLNN_ERR_PARAM_INVALID,
                "aclnnMlaKvBindSeqLens: not an attention executor");
   executor->bound_lens = device_seq_lens;
+  executor->bound_longest = -1;
+  return ACLNN_SUCCESS;
+}
+
+aclnnStatus aclnnMlaKvSetSeqLenBound(aclOpExecutor* executor, int64_t longest) {
+  const char* who = "aclnnMlaKvSetSeqLenBound";
+  SHIM_REQUIRE(executor, ACLNN_ERR_PARAM_NULLPTR, "%s: null executor", who);
+  SHIM_REQUIRE(AsExecutor(executor) && executor->kind == OpKind::kAttention, ACLNN_ERR_PARAM_INVALID, "%s: not an attention executor", who);
+  SHIM_REQUIRE(longest >= -1 && longest <= executor->max_seq_len, ACLNN_ERR_PARAM_INVALID, "%s: bound %lld outside [-1, %d]", who,
+               static_cast<long long>(longest), executor->max_seq_len);
+  executor->bound_longest = static_cast<int32_t>(longest);
   return ACLNN_SUCCESS;
 }
 

@@ -536,7 +536,7 @@ mlakvStatus AttnDecodeImpl(const char* who, const mlakvAttnPlan* plan, const mla
                            int32_t table_stride, const int32_t* seq_lens, double scale, void* out, int64_t out_seq_stride,
                            int64_t out_head_stride, const mlakvMxQuantOut* quant, const int32_t* sparse_indices,
                            int64_t sparse_indices_seq_stride, float* lse, void* workspace, uint64_t workspace_bytes,
-                           void* stream, const int32_t* host_lens = nullptr) {
+                           void* stream, const int32_t* host_lens = nullptr, int32_t longest = -1) {
   if (plan == nullptr) return Fail(MLAKV_ERR_PARAM_NULLPTR, "%s: plan is null", who);
   if (host_lens != nullptr) {
     if (plan->batch > mlakv::kAttnInlineLens) {
@@ -692,7 +692,7 @@ mlakvStatus AttnDecodeImpl(const char* who, const mlakvAttnPlan* plan, const mla
     // 64-head kernel, whose work units are all fixed cost at that size. What the launch can see of
     // the lengths decides: the values themselves when they ride in the argument block, else the
     // plan's bound.
-    int32_t bound = args.max_tokens;
+    int32_t bound = longest >= 0 ? std::min(longest, args.max_tokens) : args.max_tokens;  // (the caller's word for lengths in device memory)
     if (host_lens != nullptr) {
       bound = 0;
       for (int32_t i = 0; i < plan->batch; ++i) bound = std::max(bound, std::min(std::max(host_lens[i], 0), args.max_tokens));
@@ -721,6 +721,20 @@ mlakvStatus mlakvAttnDecode(const mlakvAttnPlan* plan, const mlakvCacheView* cac
   return AttnDecodeImpl("mlakvAttnDecode", plan, cache, layer, q_latent, q_latent_seq_stride, q_latent_head_stride, q_rope,
                         q_rope_seq_stride, q_rope_head_stride, block_table, table_stride, seq_lens, scale, out, out_seq_stride,
                         out_head_stride, nullptr, nullptr, 0, lse, workspace, workspace_bytes, stream);
+}
+
+mlakvStatus mlakvAttnDecodeBounded(const mlakvAttnPlan* plan, const mlakvCacheView* cache, int32_t layer, const void* q_latent,
+                                   int64_t q_latent_seq_stride, int64_t q_latent_head_stride, const void* q_rope,
+                                   int64_t q_rope_seq_stride, int64_t q_rope_head_stride, const int32_t* block_table,
+                                   int32_t table_stride, const int32_t* seq_lens, int32_t longest, double scale, void* out,
+                                   int64_t out_seq_stride, int64_t out_head_stride, float* lse, void* workspace,
+                                   uint64_t workspace_bytes, void* stream) {
+  const char* who = "mlakvAttnDecodeBounded";
+  if (out == nullptr) return Fail(MLAKV_ERR_PARAM_NULLPTR, "%s: the output is required", who);
+  if (longest < 0) return Fail(MLAKV_ERR_PARAM_INVALID, "%s: the bound of the lengths must not be negative", who);
+  return AttnDecodeImpl(who, plan, cache, layer, q_latent, q_latent_seq_stride, q_latent_head_stride, q_rope, q_rope_seq_stride,
+                        q_rope_head_stride, block_table, table_stride, seq_lens, scale, out, out_seq_stride, out_head_stride, nullptr,
+                        nullptr, 0, lse, workspace, workspace_bytes, stream, nullptr, longest);
 }
 
 mlakvStatus mlakvAttnDecodeHostLens(const mlakvAttnPlan* plan, const mlakvCacheView* cache, int32_t layer, const void* q_latent,

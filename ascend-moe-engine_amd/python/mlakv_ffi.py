@@ -107,6 +107,8 @@ PROTOTYPES = {
                                C.c_double, _vp, _i64, _i64, _vp, _vp, _u64, _vp]),
     "mlakvAttnDecodeHostLens": (_i32, [_P(AttnPlan), _P(CacheView), _i32, _vp, _i64, _i64, _vp, _i64, _i64, _vp, _i32, _vp,
                                        C.c_double, _vp, _i64, _i64, _vp, _vp, _u64, _vp]),
+    "mlakvAttnDecodeBounded": (_i32, [_P(AttnPlan), _P(CacheView), _i32, _vp, _i64, _i64, _vp, _i64, _i64, _vp, _i32, _vp, _i32,
+                                      C.c_double, _vp, _i64, _i64, _vp, _vp, _u64, _vp]),
     "mlakvAttnDecodeNoAlloc": (_i32, [_P(AttnPlan), _P(CacheView), _i32, _vp, _i64, _i64, _vp, _i64, _i64, _vp, _i32, _vp,
                                       C.c_double, _vp, _i64, _i64, _vp, _vp]),
     "mlakvAttnDecodeMxQuant": (_i32, [_P(AttnPlan), _P(CacheView), _i32, _vp, _i64, _i64, _vp, _i64, _i64, _vp, _i32, _vp,

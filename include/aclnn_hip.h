@@ -260,6 +260,12 @@ aclnnStatus aclnnMlaKvSetSeqLens(aclOpExecutor* executor, const int64_t* seq_len
  * lengths to a planned attention executor; it then replaces the host values, with no per-launch
  * copy. NULL unbinds. */
 aclnnStatus aclnnMlaKvBindSeqLens(aclOpExecutor* executor, const int32_t* device_seq_lens);
+/* EXTENSION (no reference counterpart, as above). With lengths bound to device memory the launch
+ * cannot see them and chooses its kernels for the reserved context. A caller that knows a bound the
+ * lengths stay under (a recorded step's loop knows its position) says so here: `longest` then
+ * decides the kernels (short contexts have faster ones), and a device length above it is read as
+ * `longest`. -1 withdraws the bound; binding another array withdraws it too. */
+aclnnStatus aclnnMlaKvSetSeqLenBound(aclOpExecutor* executor, int64_t longest);
 
 #ifdef __cplusplus
 }

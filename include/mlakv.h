@@ -252,6 +252,19 @@ mlakvStatus mlakvAttnDecode(const mlakvAttnPlan* plan, const mlakvCacheView* cac
                             void* out, int64_t out_seq_stride, int64_t out_head_stride, float* lse, void* workspace,
                             uint64_t workspace_bytes, void* stream);
 
+/* mlakvAttnDecode for a caller that keeps the lengths in device memory (a recorded step reads them
+ * there) and still knows, on the host, a bound they stay under: `longest` >= seq_lens[b] for every
+ * sequence when the launch runs. The launch chooses its kernels by `longest` as
+ * mlakvAttnDecodeHostLens does by the lengths themselves (short contexts: the units of 16 heads).
+ * The bound is the caller's word: a length above it is read as `longest`. No reference
+ * counterpart. */
+mlakvStatus mlakvAttnDecodeBounded(const mlakvAttnPlan* plan, const mlakvCacheView* cache, int32_t layer,
+                                   const void* q_latent, int64_t q_latent_seq_stride, int64_t q_latent_head_stride,
+                                   const void* q_rope, int64_t q_rope_seq_stride, int64_t q_rope_head_stride,
+                                   const int32_t* block_table, int32_t table_stride, const int32_t* seq_lens, int32_t longest,
+                                   double scale, void* out, int64_t out_seq_stride, int64_t out_head_stride, float* lse,
+                                   void* workspace, uint64_t workspace_bytes, void* stream);
+
 /* mlakvAttnDecode for a caller that knows the live lengths on the host (the engine's decode loop
  * does: src/pipeline/pipeline.cpp:515-519 derives the position on the host): host_seq_lens holds
  * plan->batch values, at most MLAKV_ATTN_HOST_LENS_MAX; they are copied into the kernels' argument

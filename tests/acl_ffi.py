@@ -45,7 +45,7 @@ PROTOTYPES = {
     "aclnnFusedInferAttentionScoreV5": (_i32, [_vp, _u64, _vp, _vp]),
     "aclnnGatherPaKvCacheGetWorkspaceSize": (_i32, [_vp] * 7 + [_i64, _P(_u64), _P(_vp)]),
     "aclnnGatherPaKvCache": (_i32, [_vp, _u64, _vp, _vp]),
-    "aclnnMlaKvBindSeqLens": (_i32, [_vp, _vp]),
+    "aclnnMlaKvBindSeqLens": (_i32, [_vp, _vp]), "aclnnMlaKvSetSeqLenBound": (_i32, [_vp, _i64]),
     "aclnnMlaKvSetSeqLens": (_i32, [_vp, _vp, _u64]),
     "aclnnDynamicMxQuantGetWorkspaceSize": (_i32, [_vp, _i64, C.c_char_p, _i64, _i64, _i64, _vp, _vp, _P(_u64), _P(_vp)]),
     "aclnnDynamicMxQuant": (_i32, [_vp, _u64, _vp, _vp]),

@@ -265,7 +265,12 @@ def test_short_whole_contexts_in_units_of_16_heads(fp8):
                                               by_value_lse.data_ptr(), ws.data_ptr(), ws.numel(), kt.stream_ptr()))
         ffi.check(lib.mlakvAttnDecode(*head_args, lens.data_ptr(), SCALE, in_memory.data_ptr(), heads * LATENT * 2, LATENT * 2, None,
                                       ws.data_ptr(), ws.numel(), kt.stream_ptr()))
+        # the lengths in device memory and the caller's word for their bound: as by value
+        bounded = torch.full_like(split, float("nan"))
+        ffi.check(lib.mlakvAttnDecodeBounded(*head_args, lens.data_ptr(), max(ctxs), SCALE, bounded.data_ptr(), heads * LATENT * 2, LATENT * 2,
+                                             None, ws.data_ptr(), ws.numel(), kt.stream_ptr()))
         torch.cuda.synchronize()
+        assert torch.equal(bounded, by_value)
         _assert_close(by_value, expected, tol)
         _assert_close(in_memory, expected, tol)
         assert torch.equal(in_memory, split)                       # lengths in device memory: the plan's bound decides
