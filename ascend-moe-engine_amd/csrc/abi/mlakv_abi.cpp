@@ -697,10 +697,44 @@ mlakvStatus AttnDecodeImpl(const char* who, const mlakvAttnPlan* plan, const mla
       bound = 0;
       for (int32_t i = 0; i < plan->batch; ++i) bound = std::max(bound, std::min(std::max(host_lens[i], 0), args.max_tokens));
     }
-    args.head_block_units = quant != nullptr ? 0 : ShortContextUnits(plan, bound);
-    if (args.head_block_units == 2) {  // (the halves' partials must fit what the plan sized for the split)
-      const uint64_t halved = static_cast<uint64_t>(plan->batch) * (plan->heads / 16) * (32 * mlakv::kLatentDim * 2 + 2 * 4 * 16 * sizeof(float));
-      if (halved > plan->workspace_bytes) args.head_block_units = 1;
+    args.head_block_units = ShortContextUnits(plan, bound);
+    const uint64_t halved = static_cast<uint64_t>(plan->batch) * (plan->heads / 16) * (32 * mlakv::kLatentDim * 2 + 2 * 4 * 16 * sizeof(float));
+    if (args.head_block_units == 2 && halved > plan->workspace_bytes) args.head_block_units = 1;  // (the halves' partials must fit what the plan sized for the split)
+    if (quant != nullptr && args.head_block_units != 0) {
+      // The units have no quantising epilogue: they write bf16 rows (the caller's, or rows of the
+      // workspace behind the halves' partials) and the standalone quantiser follows in the same
+      // stream; its codes are those of the fused epilogue, by construction of both from the bf16 rows.
+      const uint64_t rows_offset = args.head_block_units == 2 ? ((halved + 255) & ~255ull) : 0;
+      const uint64_t rows_bytes = static_cast<uint64_t>(plan->batch) * plan->heads * mlakv::kLatentDim * 2;
+      const bool own_rows = out == nullptr;
+      const bool uniform = (own_rows || out_seq_stride == plan->heads * out_head_stride) &&
+                           quant->codes_seq_stride == plan->heads * quant->codes_head_stride &&
+                           quant->scales_seq_stride == plan->heads * quant->scales_head_stride;
+      if (!uniform || (own_rows && rows_offset + rows_bytes > plan->workspace_bytes)) {
+        args.head_block_units = 0;
+      } else {
+        if (own_rows) {
+          args.out = static_cast<char*>(workspace) + rows_offset;
+          args.out_seq_stride = static_cast<int64_t>(plan->heads) * mlakv::kLatentDim * 2;
+          args.out_head_stride = mlakv::kLatentDim * 2;
+        }
+        args.out_codes = nullptr;
+        args.out_scales = nullptr;
+        args.sparse_count = std::max(bound, 1);
+        hipError_t status = mlakv::LaunchAttnDecode(args, static_cast<hipStream_t>(stream));
+        if (status != hipSuccess) return HipFail(status, who);
+        mlakv::MxQuantArgs quantise{};
+        quantise.x = args.out;
+        quantise.x_row_stride = args.out_head_stride;
+        quantise.codes = static_cast<char*>(quant->codes);
+        quantise.codes_row_stride = quant->codes_head_stride;
+        quantise.scales = static_cast<char*>(quant->scales);
+        quantise.scales_row_stride = quant->scales_head_stride;
+        quantise.rows = static_cast<int64_t>(plan->batch) * plan->heads;
+        quantise.cols = mlakv::kLatentDim;
+        status = mlakv::LaunchMxQuant(quantise, static_cast<hipStream_t>(stream));
+        return status == hipSuccess ? MLAKV_SUCCESS : HipFail(status, who);
+      }
     }
     args.sparse_count = args.head_block_units != 0 ? std::max(bound, 1) : 0;
   }

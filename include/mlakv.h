@@ -219,8 +219,7 @@ mlakvStatus mlakvAttnPlanInit(int32_t batch, int32_t heads, int32_t max_seq_len,
  * the longest context the launch can see -- the lengths themselves with mlakvAttnDecodeHostLens,
  * the plan's max_seq_len with lengths in device memory: while two workgroups per unit fit the CUs
  * once, HEAD_BLOCK up to 256 tokens and HEAD_BLOCK_HALVES up to 768; while one per unit fits,
- * HEAD_BLOCK up to 512; while they fit twice, up to 256; the 64-head kernel otherwise, for the
- * quantising entry point and whenever
+ * HEAD_BLOCK up to 512; while they fit twice, up to 256; the 64-head kernel otherwise and whenever
  * chunk_tiles, work_groups or merge_mode ask for properties of the split. SPLIT keeps the 64-head
  * kernel always; HEAD_BLOCK and HEAD_BLOCK_HALVES ask for the units (max_seq_len up to
  * MLAKV_ATTN_HEAD_BLOCK_TOKENS). The two kinds of kernel round differently (both inside the stated

@@ -275,11 +275,16 @@ def test_short_whole_contexts_in_units_of_16_heads(fp8):
         _assert_close(in_memory, expected, tol)
         assert torch.equal(in_memory, split)                       # lengths in device memory: the plan's bound decides
         assert torch.equal(by_value, split) == (max(ctxs) > 768)   # by value: the lengths themselves
-        # the quantising entry point keeps the 64-head kernel
+        # the quantising entry point makes the same choice and quantises the units' bf16 rows (held in
+        # the workspace when the caller wants no bf16 output) with the standalone quantiser
+        plain, _, _ = kt.attention(cache, 0, q, tab, lens, SCALE)
         _, _, _, codes, scales = kt.attention(cache, 0, q, tab, lens, SCALE, quant=True, want_out=False)
-        _, _, _, codes_split, scales_split = kt.attention(cache, 0, q, tab, lens, SCALE, quant=True, want_out=False,
-                                                          selection_units=ffi.ATTN_UNITS_SPLIT)
-        assert torch.equal(codes, codes_split) and torch.equal(scales, scales_split)
+        with_out, _, _, codes_too, scales_too = kt.attention(cache, 0, q, tab, lens, SCALE, quant=True)
+        want_codes, want_scales = orc.mx_quant_rows(kt.bits16(plain).reshape(-1, LATENT))
+        assert torch.equal(with_out, plain)
+        for got_codes, got_scales in ((codes, scales), (codes_too, scales_too)):
+            assert np.array_equal(got_scales.cpu().numpy().reshape(-1, LATENT // 32), want_scales)
+            assert np.array_equal(got_codes.cpu().numpy().reshape(-1, LATENT), want_codes)
 
 
 def test_host_lengths_in_the_argument_block_give_the_same_bits():

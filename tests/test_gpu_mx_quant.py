@@ -96,10 +96,9 @@ def test_attention_epilogue_equals_quantising_the_bf16_output(fp8, options):
     # planner's choice; sequences split over units (the merge quantises); whole sequences per unit
     # (the kernel's own epilogue quantises); the merge inside the launch
     table_d, lens_d = kt.dev_i32(table), kt.dev_i32(ctxs)
-    # (the quantising entry point always runs the 64-head kernel; the plain one is pinned to it here:
-    # contexts this short would otherwise go to the units of 16 heads, which round differently)
-    pinned = options or {"selection_units": ffi.ATTN_UNITS_SPLIT}
-    out, lse, plan = kt.attention(cache, 0, q, table_d, lens_d, SCALE, **pinned)
+    # (with the planner's choice, contexts this short go to the units of 16 heads in both entry points;
+    # the quantising one then runs the standalone quantiser behind them)
+    out, lse, plan = kt.attention(cache, 0, q, table_d, lens_d, SCALE, **options)
     out_q, lse_q, _, codes, scales = kt.attention(cache, 0, q, table_d, lens_d, SCALE, quant=True, **options)
     assert torch.equal(out_q, out) and torch.equal(lse_q, lse)       # the bf16 output is unchanged by the epilogue
     want_codes, want_scales = orc.mx_quant_rows(kt.bits16(out).reshape(-1, LATENT))
